@@ -1,0 +1,183 @@
+/*
+ * karume_hip.h — C ABI of libkarume_hip.so, the gfx950 (MI355X, wave64) backend for the
+ * Karume IR runtime's int4 `linear`, states-form `attention` and `state_append` ops.
+ *
+ * The reference has no FFI: every op reaches the device as a WebGPU DispatchRecipe = a
+ * params struct + an ordered list of buffer bindings + a grid
+ * (packages/runtime/src/runtime/recipe.ts:87-96).  Each entry point below takes exactly what
+ * the corresponding recipe carries — the params words as scalar arguments, the bindings as
+ * device addresses — so a Deno host can `Deno.dlopen` this library and call it where the
+ * reference would have pushed the recipe.  Citations are `path:line` in the reference tree.
+ *
+ * Conventions
+ *  - every function returns int32: 0 = ok, negative = error class (below).  The text of the
+ *    last error of a context is available from krm_last_error().
+ *  - `krm_buf` is a raw device address (uint64).  Offsets are applied by the caller
+ *    (address + bytes).  The caller owns every buffer; the library owns its context, its
+ *    stream and whatever scratch it allocated itself.
+ *  - launches are asynchronous on the context's stream; krm_buf_download and krm_sync fence.
+ *  - host pointers are only read/written during the call.
+ *  - one context = one stream, externally serialised (the reference serialises runs per
+ *    Session, packages/runtime/src/runtime/generation-context.ts:103-106).  The device is set
+ *    on entry of every call, so calls may come from any OS thread.
+ *  - nothing is approximated silently: an unsupported combination is rejected before launch.
+ */
+#ifndef KARUME_HIP_H
+#define KARUME_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct krm_ctx krm_ctx;
+typedef uint64_t krm_buf;
+typedef struct krm_event krm_event;
+
+/* Error classes; they mirror the reference's public error types
+ * (packages/runtime/mod.ts:25-35,112). */
+#define KRM_OK 0
+#define KRM_ERR_VALIDATION (-1)    /* GpuValidationError: shapes / attrs / alignment rejected */
+#define KRM_ERR_OUT_OF_MEMORY (-2) /* GpuOutOfMemoryError */
+#define KRM_ERR_DEVICE_LOST (-3)   /* GpuDeviceLostError: the HIP runtime reported a failure */
+#define KRM_ERR_EXECUTION (-4)     /* ExecutionError: contract of a run violated (P+Q > C ...) */
+
+/* Element encodings of activation / scale / KV-slot buffers. */
+#define KRM_F32 0
+#define KRM_F16 1
+
+/* `linear` arithmetic, the reference's SessionOptions.linearCompute
+ * (packages/runtime/src/runtime/session-types.ts:127-195):
+ *   KRM_COMPUTE_F32  — f32 products and f32 accumulation for every M (the reference default);
+ *   KRM_COMPUTE_F16  — rows M > 16 go to the fp16 MFMA GEMM (x rounded to fp16, integer
+ *                      weight codes exact in fp16, group scale applied to f32 partial sums).
+ * M <= 16 always runs the bandwidth-bound GEMV with f32 accumulation. */
+#define KRM_COMPUTE_F32 0
+#define KRM_COMPUTE_F16 1
+
+/* ---- context (acquireGpu / GpuContext.destroy, packages/runtime/mod.ts:13-113) ---------- */
+int32_t krm_ctx_create(int32_t device, krm_ctx** out);
+/* Same, but launches go to an existing hipStream_t (0 = the device's default stream); the
+ * stream stays owned by the caller. */
+int32_t krm_ctx_create_on_stream(int32_t device, void* hip_stream, krm_ctx** out);
+int32_t krm_ctx_destroy(krm_ctx* ctx);
+/* Text of the last error on `ctx` (or of the last context-less failure when ctx is NULL).
+ * Valid until the next failing call on the same context. */
+const char* krm_last_error(krm_ctx* ctx);
+/* Fence: returns when everything queued on the context's stream has finished. */
+int32_t krm_sync(krm_ctx* ctx);
+/* Library identification: "karume-hip <version> gfx950". */
+const char* krm_version(void);
+
+/* ---- buffers (createBuffer / queue.writeBuffer / readback mapAsync,
+ *      packages/runtime/src/runtime/executor.ts:870-896,1272) ------------------------------ */
+int32_t krm_buf_alloc(krm_ctx* ctx, size_t bytes, krm_buf* out);
+int32_t krm_buf_free(krm_ctx* ctx, krm_buf buf);
+int32_t krm_buf_upload(krm_ctx* ctx, krm_buf dst, size_t dst_offset, const void* host,
+                       size_t bytes);
+int32_t krm_buf_download(krm_ctx* ctx, krm_buf src, size_t src_offset, void* host, size_t bytes);
+/* State slots are zero-initialised at creation
+ * (packages/runtime/tests/gpu_state_execution_test.ts:159-164). */
+int32_t krm_buf_zero(krm_ctx* ctx, krm_buf dst, size_t dst_offset, size_t bytes);
+
+/* ---- timing (timestamp-query diagnostics, packages/runtime/src/gpu/submit.ts:54-63) ------ */
+int32_t krm_event_create(krm_ctx* ctx, krm_event** out);
+int32_t krm_event_record(krm_ctx* ctx, krm_event* ev);
+/* Waits for `stop`, then writes the milliseconds between the two recorded events. */
+int32_t krm_event_elapsed_ms(krm_ctx* ctx, krm_event* start, krm_event* stop, float* ms);
+int32_t krm_event_destroy(krm_ctx* ctx, krm_event* ev);
+
+/* ---- int4 storage (packages/runtime/src/format/i4.ts:63-118,
+ *      packages/runtime/src/kernels/weight-storage.ts:152-187) ------------------------------
+ * Expands packed int4 `w` ([rows, width] elements, 2 per byte, element 2j = low nibble,
+ * stored u = q + 8) into f32: out[i] = f32(u - 8) * scale[row*(width/group) + (i%width)/group],
+ * one f32 multiply — bit-identical to decodeI4.  Requires group >= 1, width % group == 0,
+ * (rows*width) % 8 == 0 and 4-byte aligned `w`. */
+int32_t krm_dequant_i4(krm_ctx* ctx, krm_buf w, krm_buf scales, krm_buf out_f32, uint64_t rows,
+                       uint64_t width, uint32_t group, int32_t scale_dtype);
+
+/* ---- linear with int4 weights (bindings 1-5 + Dims{m,n,k}:
+ *      packages/runtime/src/kernels/gemm.ts:115,315-327,1223-1227;
+ *      builder packages/runtime/src/runtime/recipe-builder.ts:1311-1392) --------------------
+ * out[m, n] = (sum_k x[m,k] * dequant(w)[n,k]) + bias[n]
+ *   x      [m, k]  io_dtype, row-major
+ *   w      [n, k]  packed int4, k contiguous (k/2 bytes per row)
+ *   scales [n, k/group]  scale_dtype
+ *   bias   [n]     io_dtype, or 0 for "no bias" (the reference always binds one; zeros)
+ *   out    [m, n]  io_dtype
+ * group must be a power of two >= 16 dividing k (docs/ir-v1.md:135-150).
+ * The kernel is a pure function of (m, n, k, group, dtypes, compute); for m <= 16 a row of
+ * `out` does not depend on the other rows in the call (same reduction order for every m). */
+int32_t krm_linear_i4(krm_ctx* ctx, krm_buf x, krm_buf w, krm_buf scales, krm_buf bias,
+                      krm_buf out, uint32_t m, uint32_t n, uint32_t k, uint32_t group,
+                      int32_t io_dtype, int32_t scale_dtype, int32_t compute);
+
+/* ---- states-form attention (Params 10 words + Lengths{past,query} + bindings:
+ *      packages/runtime/src/kernels/state-attention.ts:169-180,190-193,284-294,476-487;
+ *      builder packages/runtime/src/runtime/recipe-builder.ts:1856-2002;
+ *      contract docs/ir-v1.md:296-351) -------------------------------------------------------
+ * One call replaces the reference's three dispatches (QK -> row stats -> PV); the score
+ * matrix is never materialised.
+ *   q      [B, H,   M, D]  io_dtype
+ *   ins_k  [B, Hkv, M, D]  io_dtype   this step's keys   (valid rows: first `query`)
+ *   ins_v  [B, Hkv, M, D]  io_dtype   this step's values
+ *   slot_k [B, Hkv, C, D]  kv_dtype   past keys   (logical column c < past lives in physical
+ *   slot_v [B, Hkv, C, D]  kv_dtype   past values  row c, or c % window when window > 0)
+ *   out    [B, H,   M, D]  io_dtype   rows >= query are written as exact +0
+ * Row r attends to logical columns c with c <= past + r and (window == 0 or
+ * past + r - c < window); kv plane of (b, h) is floor((b*H + h) / (H/Hkv)).
+ * `half_scale` multiplies q AND k (IR attr `scale`; sqrt(1/sqrt(D)) for the usual 1/sqrt(D)).
+ * Rejected before launch: H % Hkv != 0, query < 1 or > M, window > C, window == 0 with
+ * past + query > C (packages/runtime/src/kernels/state-attention.ts:588-636,
+ * packages/runtime/src/runtime/recipe.ts:273-280).
+ * `workspace` holds split-K partials; ask krm_attention_state_workspace for its size. */
+int32_t krm_attention_state_workspace(uint32_t batch, uint32_t heads, uint32_t kv_heads,
+                                      uint32_t chunk_rows, uint32_t depth, uint32_t window,
+                                      uint32_t max_past, uint32_t max_query, size_t* bytes);
+int32_t krm_attention_state(krm_ctx* ctx, krm_buf q, krm_buf ins_k, krm_buf ins_v,
+                            krm_buf slot_k, krm_buf slot_v, krm_buf out, uint32_t batch,
+                            uint32_t heads, uint32_t kv_heads, uint32_t chunk_rows,
+                            uint32_t depth, uint32_t capacity, uint32_t window,
+                            float half_scale, uint32_t past, uint32_t query, int32_t io_dtype,
+                            int32_t kv_dtype, krm_buf workspace, size_t workspace_bytes);
+
+/* ---- state_append (packages/runtime/src/kernels/state-append.ts:47-96,120-173;
+ *      builder packages/runtime/src/runtime/recipe-builder.ts:2011-2048) --------------------
+ * Copies the first `query` rows of x[kv_planes, M, D] (x_dtype) into
+ * slot[kv_planes, C, D] (slot_dtype) at physical row (past+row) or (past+row) % window.
+ * Rows >= query are never written.  With window > 0 and query > window only the last
+ * logical row mapping to a physical row is written.  f32 -> f16 rounds to nearest even.
+ * Must be issued after every reader of the slot in the same step (docs/ir-v1.md:345-348). */
+int32_t krm_state_append(krm_ctx* ctx, krm_buf x, krm_buf slot, uint32_t kv_planes,
+                         uint32_t chunk_rows, uint32_t depth, uint32_t capacity,
+                         uint32_t window, uint32_t past, uint32_t query, int32_t x_dtype,
+                         int32_t slot_dtype);
+
+/* ---- ragged decode batch (no counterpart in the reference, which runs one sequence at a
+ *      time: docs/decisions/0066-generation-context-state-slots.md:130-135) -----------------
+ * `nseq` sequences, one query row each, packed along the slot's row axis:
+ *   q      [nseq, H, D]            io_dtype
+ *   ins_k  [nseq, Hkv, D]          io_dtype   this step's key per sequence
+ *   ins_v  [nseq, Hkv, D]          io_dtype
+ *   slot_k [Hkv, total_rows, D]    kv_dtype   sequence i owns rows [cu_seqlens[i], cu_seqlens[i+1])
+ *   slot_v [Hkv, total_rows, D]    kv_dtype
+ *   out    [nseq, H, D]            io_dtype
+ * `cu_seqlens` is a HOST array of nseq+1 ascending row offsets (cu_seqlens[0] >= 0,
+ * cu_seqlens[nseq] <= total_rows); sequence i has past_i = cu[i+1]-cu[i] rows in the slot and
+ * attends to those plus its own ins row (window = 0).  Each sequence's result is
+ * bit-identical to krm_attention_state run on that sequence alone. */
+int32_t krm_attention_varlen_workspace(uint32_t nseq, uint32_t heads, uint32_t kv_heads,
+                                       uint32_t depth, uint64_t total_rows, size_t* bytes);
+int32_t krm_attention_varlen(krm_ctx* ctx, krm_buf q, krm_buf ins_k, krm_buf ins_v,
+                             krm_buf slot_k, krm_buf slot_v, krm_buf out,
+                             const int32_t* cu_seqlens, uint32_t nseq, uint32_t heads,
+                             uint32_t kv_heads, uint32_t depth, uint64_t total_rows,
+                             float half_scale, int32_t io_dtype, int32_t kv_dtype,
+                             krm_buf workspace, size_t workspace_bytes);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* KARUME_HIP_H */

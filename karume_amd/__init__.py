@@ -1,0 +1,18 @@
+"""karume_amd — MI355X (gfx950) backend for the Karume IR runtime's int4 ``linear``,
+states-form ``attention`` and ``state_append`` ops.
+
+The compute lives in ``lib/libkarume_hip.so`` (hand-written HIP, built by
+``python -m karume_amd.build``) behind the C ABI of ``include/karume_hip.h``; this package is
+the host-side mirror of the reference's interface for those ops.
+"""
+from .format_i4 import I4Error, check_int4, group_scale_shape, pack_int4
+from .runtime import (COMPUTE_F16, COMPUTE_F32, F16, F32, DeviceBuffer, ExecutionError,
+                      GpuContext, GpuDeviceLostError, GpuEvent, GpuOutOfMemoryError,
+                      GpuValidationError, KarumeError, acquire_gpu, dtype_code, version)
+
+__all__ = [
+    "I4Error", "check_int4", "group_scale_shape", "pack_int4",
+    "COMPUTE_F16", "COMPUTE_F32", "F16", "F32", "DeviceBuffer", "ExecutionError", "GpuContext",
+    "GpuDeviceLostError", "GpuEvent", "GpuOutOfMemoryError", "GpuValidationError", "KarumeError",
+    "acquire_gpu", "dtype_code", "version",
+]

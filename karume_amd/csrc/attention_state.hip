@@ -1,0 +1,775 @@
+// states-form attention over the KV state slots for gfx950.
+//
+// Contract (packages/runtime/src/kernels/state-attention.ts:1-113, docs/ir-v1.md:296-351):
+// logical columns [0, P+Q); column c < P is read from the slot at physical row c (or c % W for
+// a sliding window), column c >= P from this step's ins row c - P; output row r attends to
+// c <= P + r and, with a window, P + r - c < W; kv plane = floor((b*H + h) / r); rows >= Q
+// are written as exact 0; the half-scale multiplies q and k.
+//
+// The reference materialises S, reduces row statistics and multiplies by V in three
+// dispatches.  Here one launch streams K and V once with an online softmax:
+//  * decode (Q = 1, M = 1): split-K.  A workgroup owns one KV head and one range of past
+//    columns, loads that range's K and V with 16-byte coalesced loads, scores all r query
+//    heads of the KV head against it (the KV bytes are read once, not r times), and writes
+//    (max, sum, weighted V) partials that a second small kernel merges in split order.
+//    The column partition depends only on the number of past columns, the head dim and the
+//    slot dtype, so a sequence gives the same bits alone or inside a ragged batch.
+//  * everything else (prefill chunks, pad rows, head dims the fast path does not cover):
+//    a generic kernel, one workgroup per (plane, row).
+#include "krm_internal.h"
+
+#include <cmath>
+
+using namespace krm;
+
+namespace {
+
+constexpr int kThreads = 256;
+constexpr int kDecodeIter = 8;  // K/V rows each lane group walks per split
+
+template <typename T>
+__device__ inline float ld_f32(const T* p, size_t i);
+template <>
+__device__ inline float ld_f32<float>(const float* p, size_t i) { return p[i]; }
+template <>
+__device__ inline float ld_f32<__half>(const __half* p, size_t i) { return __half2float(p[i]); }
+template <typename T>
+__device__ inline void st_f32(T* p, size_t i, float v);
+template <>
+__device__ inline void st_f32<float>(float* p, size_t i, float v) { p[i] = v; }
+template <>
+__device__ inline void st_f32<__half>(__half* p, size_t i, float v) { p[i] = __float2half_rn(v); }
+
+// first logical column a row with causal limit `limit` may see (0 for a full context)
+__host__ __device__ inline uint64_t window_low(uint32_t window, uint64_t limit) {
+  return (window && limit + 1 > window) ? limit + 1 - window : 0;
+}
+
+// ------------------------------------------------------------------------------ generic
+
+struct GenericArgs {
+  uint32_t heads, kv_heads, chunk_rows, depth, capacity, window, past, query;
+  float scale;
+};
+
+// One workgroup per (plane z = b*H + h, row).  Columns are walked 256 at a time: a thread
+// scores one column (serial dot over D), the block folds the chunk into the running
+// (max, sum), then threads switch to one output dim each and add the chunk's P*V.
+template <typename XT, typename ST>
+__global__ __launch_bounds__(kThreads) void attention_generic_kernel(
+    const XT* __restrict__ q, const XT* __restrict__ ins_k, const XT* __restrict__ ins_v,
+    const ST* __restrict__ slot_k, const ST* __restrict__ slot_v, XT* __restrict__ out,
+    GenericArgs a) {
+  __shared__ float s_q[1024];
+  __shared__ float s_p[kThreads];
+  __shared__ float s_red[kThreads / kWave];
+  __shared__ float s_bcast;
+
+  const uint32_t z = blockIdx.x;
+  const uint32_t row = blockIdx.y;
+  const uint32_t tid = threadIdx.x;
+  const uint32_t D = a.depth;
+  const size_t q_base = ((size_t)z * a.chunk_rows + row) * D;
+
+  if (row >= a.query) {  // pad row: exact zeros, nothing is read
+    for (uint32_t d = tid; d < D; d += kThreads) st_f32<XT>(out, q_base + d, 0.0f);
+    return;
+  }
+  const uint32_t kv_plane = z / (a.heads / a.kv_heads);
+  const uint64_t limit = (uint64_t)a.past + row;
+  const uint64_t lo = window_low(a.window, limit);
+  const uint64_t count = limit - lo + 1;  // >= 1: the row always sees its own column
+
+  for (uint32_t d = tid; d < D; d += kThreads) s_q[d] = ld_f32<XT>(q, q_base + d) * a.scale;
+  __syncthreads();
+
+  float run_max = -INFINITY, run_sum = 0.f;
+  float acc[4] = {0.f, 0.f, 0.f, 0.f};  // output dims tid, tid+256, ... (D <= 1024)
+
+  for (uint64_t c0 = 0; c0 < count; c0 += kThreads) {
+    const uint64_t col = lo + c0 + tid;
+    const bool valid = c0 + tid < count;
+    float score = -INFINITY;
+    if (valid) {
+      float dot = 0.f;
+      if (col < a.past) {
+        const uint64_t prow = a.window ? col % a.window : col;
+        const ST* kp = slot_k + ((size_t)kv_plane * a.capacity + prow) * D;
+        for (uint32_t d = 0; d < D; ++d) dot = fmaf(s_q[d], ld_f32<ST>(kp, d) * a.scale, dot);
+      } else {
+        const XT* kp = ins_k + ((size_t)kv_plane * a.chunk_rows + (col - a.past)) * D;
+        for (uint32_t d = 0; d < D; ++d) dot = fmaf(s_q[d], ld_f32<XT>(kp, d) * a.scale, dot);
+      }
+      score = dot;
+    }
+    // chunk max
+    float m = score;
+    for (int off = 32; off > 0; off >>= 1) m = fmaxf(m, __shfl_xor(m, off, kWave));
+    if ((tid & (kWave - 1)) == 0) s_red[tid >> 6] = m;
+    __syncthreads();
+    if (tid == 0) {
+      float t = s_red[0];
+      for (int i = 1; i < kThreads / kWave; ++i) t = fmaxf(t, s_red[i]);
+      s_bcast = fmaxf(t, run_max);
+    }
+    __syncthreads();
+    const float new_max = s_bcast;  // finite: every chunk holds at least one valid column
+    const float alpha = expf(run_max - new_max);  // exp(-inf) = 0 on the first chunk
+    const float p = valid ? expf(score - new_max) : 0.f;
+    s_p[tid] = p;
+    float s = p;
+    for (int off = 32; off > 0; off >>= 1) s += __shfl_xor(s, off, kWave);
+    __syncthreads();  // s_p complete; s_red free to reuse
+    if ((tid & (kWave - 1)) == 0) s_red[tid >> 6] = s;
+    __syncthreads();
+    float chunk_sum = 0.f;
+    for (int i = 0; i < kThreads / kWave; ++i) chunk_sum += s_red[i];
+    run_sum = run_sum * alpha + chunk_sum;
+    run_max = new_max;
+
+    const uint32_t ncols = (uint32_t)((count - c0) < kThreads ? (count - c0) : kThreads);
+#pragma unroll
+    for (int slot = 0; slot < 4; ++slot) {
+      const uint32_t d = tid + slot * kThreads;
+      if (d >= D) break;
+      float sum = 0.f;
+      for (uint32_t c = 0; c < ncols; ++c) {
+        const uint64_t vc = lo + c0 + c;
+        float v;
+        if (vc < a.past) {
+          const uint64_t prow = a.window ? vc % a.window : vc;
+          v = ld_f32<ST>(slot_v, ((size_t)kv_plane * a.capacity + prow) * D + d);
+        } else {
+          v = ld_f32<XT>(ins_v, ((size_t)kv_plane * a.chunk_rows + (vc - a.past)) * D + d);
+        }
+        sum = fmaf(s_p[c], v, sum);
+      }
+      acc[slot] = acc[slot] * alpha + sum;
+    }
+    __syncthreads();  // before s_p / s_red are overwritten
+  }
+  const float inv = 1.0f / run_sum;  // run_sum >= 1: the max column contributes exp(0)
+#pragma unroll
+  for (int slot = 0; slot < 4; ++slot) {
+    const uint32_t d = tid + slot * kThreads;
+    if (d < D) st_f32<XT>(out, q_base + d, acc[slot] * inv);
+  }
+}
+
+// ------------------------------------------------------------------------------ decode
+
+// Sum over the LPR consecutive lanes that share one K/V row; all of them get the total.
+template <int LPR>
+__device__ inline float group_sum(float v) {
+  if constexpr (LPR >= 2) {
+    int t = __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0xB1, 0xf, 0xf, true);
+    v += __builtin_bit_cast(float, t);  // quad_perm [1,0,3,2]
+  }
+  if constexpr (LPR >= 4) {
+    int t = __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x4E, 0xf, 0xf, true);
+    v += __builtin_bit_cast(float, t);  // quad_perm [2,3,0,1]
+  }
+  if constexpr (LPR >= 8) {
+    int t = __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x141, 0xf, 0xf, true);
+    v += __builtin_bit_cast(float, t);  // row_half_mirror
+  }
+  if constexpr (LPR >= 16) {
+    int t = __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x140, 0xf, 0xf, true);
+    v += __builtin_bit_cast(float, t);  // row_mirror
+  }
+  if constexpr (LPR >= 32) v += __shfl_xor(v, 16, kWave);
+  if constexpr (LPR >= 64) v += __shfl_xor(v, 32, kWave);
+  return v;
+}
+
+template <typename ST>
+struct RowChunk;  // 16 bytes of a K/V row
+template <>
+struct RowChunk<__half> {
+  static constexpr int E = 8;
+  __device__ static inline void unpack(const uint4& raw, float (&f)[8]) {
+    const __half2* h = reinterpret_cast<const __half2*>(&raw);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const float2 v = __half22float2(h[i]);
+      f[2 * i] = v.x;
+      f[2 * i + 1] = v.y;
+    }
+  }
+};
+template <>
+struct RowChunk<float> {
+  static constexpr int E = 4;
+  __device__ static inline void unpack(const uint4& raw, float (&f)[4]) {
+    f[0] = __uint_as_float(raw.x);
+    f[1] = __uint_as_float(raw.y);
+    f[2] = __uint_as_float(raw.z);
+    f[3] = __uint_as_float(raw.w);
+  }
+};
+
+struct DecodeArgs {
+  uint32_t heads, kv_heads;
+  uint32_t window;           // 0 = full context
+  uint32_t past;             // single sequence: P.  ragged batch: unused
+  uint64_t slot_batch_stride;  // elements between batches of the slot (0 for a ragged batch)
+  uint64_t slot_plane_stride;  // elements between kv heads of the slot
+  float scale;
+  uint32_t nseq;             // ragged batch: sequences; single: batch
+  const int32_t* cu_rows;    // ragged batch: [nseq+1] first slot row of each sequence
+  const int32_t* split_prefix;  // ragged batch: [nseq+1] first global split of each sequence
+};
+
+__host__ __device__ inline uint32_t decode_split_columns(uint32_t lanes_per_row) {
+  return kDecodeIter * (kThreads / lanes_per_row);
+}
+__host__ __device__ inline uint32_t decode_splits(uint64_t slot_columns, uint32_t split_columns) {
+  const uint64_t n = (slot_columns + split_columns - 1) / split_columns;
+  return n ? (uint32_t)n : 1u;
+}
+
+// Workgroup = (split, kv head, batch | -): 256 threads = G groups of LPR lanes; a group owns
+// one K/V row per iteration, a lane 16 bytes of it.
+template <typename XT, typename ST, int R, int LPR, bool RAGGED>
+__global__ __launch_bounds__(kThreads) void attention_decode_kernel(
+    const XT* __restrict__ q, const XT* __restrict__ ins_k, const XT* __restrict__ ins_v,
+    const ST* __restrict__ slot_k, const ST* __restrict__ slot_v, XT* __restrict__ out,
+    float* __restrict__ ws_ml, float* __restrict__ ws_acc, DecodeArgs a) {
+  constexpr int E = RowChunk<ST>::E;
+  constexpr int D = LPR * E;
+  constexpr int G = kThreads / LPR;
+  constexpr int kWaves = kThreads / kWave;
+  __shared__ float s_max[kWaves][R];
+  __shared__ float s_sum[kWaves][R];
+  __shared__ float s_acc[kWaves][R][D];
+
+  const int tid = threadIdx.x;
+  const int sub = tid % LPR;   // which 16 bytes of the row
+  const int group = tid / LPR;
+  const int wave = tid >> 6;
+  const uint32_t hk = blockIdx.y;
+
+  uint32_t seq, split, nsplit, first_split;
+  uint64_t past, row_base;
+  if constexpr (RAGGED) {
+    // binary search: last sequence whose first split is <= blockIdx.x
+    uint32_t lo_i = 0, hi_i = a.nseq;
+    while (hi_i - lo_i > 1) {
+      const uint32_t mid = (lo_i + hi_i) >> 1;
+      if ((uint32_t)a.split_prefix[mid] <= blockIdx.x) lo_i = mid; else hi_i = mid;
+    }
+    seq = lo_i;
+    first_split = (uint32_t)a.split_prefix[seq];
+    nsplit = (uint32_t)a.split_prefix[seq + 1] - first_split;
+    split = blockIdx.x - first_split;
+    row_base = (uint64_t)a.cu_rows[seq];
+    past = (uint64_t)a.cu_rows[seq + 1] - row_base;
+  } else {
+    seq = blockIdx.z;
+    past = a.past;
+    row_base = 0;
+    const uint64_t low = window_low(a.window, past);
+    nsplit = decode_splits(past - low, kDecodeIter * G);
+    split = blockIdx.x;
+    first_split = seq * nsplit;
+  }
+  const uint64_t low = window_low(a.window, past);  // limit of row 0 is `past`
+  const uint64_t c_begin = low + (uint64_t)split * (kDecodeIter * G);
+  const uint64_t c_end = (c_begin + kDecodeIter * G < past) ? c_begin + kDecodeIter * G : past;
+  const bool last = split + 1 == nsplit;
+
+  const size_t slot_base = (size_t)seq * a.slot_batch_stride + (size_t)hk * a.slot_plane_stride;
+  const ST* kslot = slot_k + slot_base;
+  const ST* vslot = slot_v + slot_base;
+
+  // requests first: K rows, V rows, this step's row (last split only)
+  uint4 kraw[kDecodeIter], vraw[kDecodeIter];
+  bool valid[kDecodeIter];
+#pragma unroll
+  for (int it = 0; it < kDecodeIter; ++it) {
+    const uint64_t col = c_begin + (uint64_t)it * G + group;
+    valid[it] = col < c_end;
+    kraw[it] = make_uint4(0, 0, 0, 0);
+    if (valid[it]) {
+      const uint64_t prow = row_base + (a.window ? col % a.window : col);
+      kraw[it] = *reinterpret_cast<const uint4*>(kslot + prow * D + sub * E);
+    }
+  }
+#pragma unroll
+  for (int it = 0; it < kDecodeIter; ++it) {
+    const uint64_t col = c_begin + (uint64_t)it * G + group;
+    vraw[it] = make_uint4(0, 0, 0, 0);
+    if (valid[it]) {
+      const uint64_t prow = row_base + (a.window ? col % a.window : col);
+      vraw[it] = *reinterpret_cast<const uint4*>(vslot + prow * D + sub * E);
+    }
+  }
+  const bool own = last && group == 0;  // the lanes that also take this step's own column
+  float kx[E], vx[E];
+  {
+    const size_t ins_base = ((size_t)seq * a.kv_heads + hk) * D + sub * E;
+#pragma unroll
+    for (int e = 0; e < E; ++e) {
+      kx[e] = own ? ld_f32<XT>(ins_k, ins_base + e) : 0.f;
+      vx[e] = own ? ld_f32<XT>(ins_v, ins_base + e) : 0.f;
+    }
+  }
+  float qf[R][E];
+#pragma unroll
+  for (int h = 0; h < R; ++h) {
+    const size_t q_base = ((size_t)seq * a.heads + (size_t)hk * R + h) * D + sub * E;
+#pragma unroll
+    for (int e = 0; e < E; ++e) qf[h][e] = (ld_f32<XT>(q, q_base + e) * a.scale) * a.scale;
+  }
+
+  // scores
+  float sc[kDecodeIter + 1][R];
+#pragma unroll
+  for (int it = 0; it < kDecodeIter; ++it) {
+    float kf[E];
+    RowChunk<ST>::unpack(kraw[it], kf);
+#pragma unroll
+    for (int h = 0; h < R; ++h) {
+      float part = 0.f;
+#pragma unroll
+      for (int e = 0; e < E; ++e) part = fmaf(qf[h][e], kf[e], part);
+      part = group_sum<LPR>(part);
+      sc[it][h] = valid[it] ? part : -INFINITY;
+    }
+  }
+#pragma unroll
+  for (int h = 0; h < R; ++h) {
+    float part = 0.f;
+#pragma unroll
+    for (int e = 0; e < E; ++e) part = fmaf(qf[h][e], kx[e], part);
+    part = group_sum<LPR>(part);
+    sc[kDecodeIter][h] = own ? part : -INFINITY;
+  }
+
+  // block max per head
+  float mx[R];
+#pragma unroll
+  for (int h = 0; h < R; ++h) {
+    float m = sc[0][h];
+#pragma unroll
+    for (int it = 1; it <= kDecodeIter; ++it) m = fmaxf(m, sc[it][h]);
+#pragma unroll
+    for (int off = LPR; off < kWave; off <<= 1) m = fmaxf(m, __shfl_xor(m, off, kWave));
+    if ((tid & (kWave - 1)) == 0) s_max[wave][h] = m;
+  }
+  __syncthreads();
+#pragma unroll
+  for (int h = 0; h < R; ++h) {
+    float m = s_max[0][h];
+#pragma unroll
+    for (int w = 1; w < kWaves; ++w) m = fmaxf(m, s_max[w][h]);
+    mx[h] = m;  // finite: a split always holds at least one column
+  }
+
+  // weights, their sum, and the weighted V rows
+  float acc[R][E];
+  float sum[R];
+#pragma unroll
+  for (int h = 0; h < R; ++h) {
+    sum[h] = 0.f;
+#pragma unroll
+    for (int e = 0; e < E; ++e) acc[h][e] = 0.f;
+  }
+#pragma unroll
+  for (int it = 0; it <= kDecodeIter; ++it) {
+    float vf[E];
+    if (it < kDecodeIter) {
+      RowChunk<ST>::unpack(vraw[it < kDecodeIter ? it : 0], vf);
+    } else {
+#pragma unroll
+      for (int e = 0; e < E; ++e) vf[e] = vx[e];
+    }
+#pragma unroll
+    for (int h = 0; h < R; ++h) {
+      const float p = expf(sc[it][h] - mx[h]);  // exp(-inf) = 0 for columns outside the split
+      sum[h] += p;
+#pragma unroll
+      for (int e = 0; e < E; ++e) acc[h][e] = fmaf(p, vf[e], acc[h][e]);
+    }
+  }
+  // fold the groups of a wave (lanes with equal `sub`), then the waves through LDS
+#pragma unroll
+  for (int h = 0; h < R; ++h) {
+#pragma unroll
+    for (int off = LPR; off < kWave; off <<= 1) {
+      sum[h] += __shfl_xor(sum[h], off, kWave);
+#pragma unroll
+      for (int e = 0; e < E; ++e) acc[h][e] += __shfl_xor(acc[h][e], off, kWave);
+    }
+    if ((tid & (kWave - 1)) < LPR) {
+#pragma unroll
+      for (int e = 0; e < E; ++e) s_acc[wave][h][sub * E + e] = acc[h][e];
+      if (sub == 0) s_sum[wave][h] = sum[h];
+    }
+  }
+  __syncthreads();
+
+  const uint32_t gsplit = first_split + split;
+  for (int o = tid; o < R * D; o += kThreads) {
+    const int h = o / D, d = o - h * D;
+    float total = s_acc[0][h][d];
+    float l = s_sum[0][h];
+#pragma unroll
+    for (int w = 1; w < kWaves; ++w) {
+      total += s_acc[w][h][d];
+      l += s_sum[w][h];
+    }
+    const uint32_t head = hk * R + h;
+    if (nsplit == 1) {
+      st_f32<XT>(out, ((size_t)seq * a.heads + head) * D + d, total / l);
+    } else {
+      const size_t slot_index = (size_t)gsplit * a.heads + head;
+      ws_acc[slot_index * D + d] = total;
+      if (d == 0) {
+        float m = s_max[0][h];
+#pragma unroll
+        for (int w = 1; w < kWaves; ++w) m = fmaxf(m, s_max[w][h]);
+        ws_ml[slot_index * 2] = m;
+        ws_ml[slot_index * 2 + 1] = l;
+      }
+    }
+  }
+}
+
+// Merge of the split partials of one (sequence, head), in ascending split order.
+template <typename XT, bool RAGGED>
+__global__ __launch_bounds__(128) void attention_combine_kernel(
+    const float* __restrict__ ws_ml, const float* __restrict__ ws_acc, XT* __restrict__ out,
+    uint32_t heads, uint32_t depth, uint32_t nsplit_single, const int32_t* split_prefix) {
+  const uint32_t head = blockIdx.x, seq = blockIdx.y;
+  uint32_t first, nsplit;
+  if constexpr (RAGGED) {
+    first = (uint32_t)split_prefix[seq];
+    nsplit = (uint32_t)split_prefix[seq + 1] - first;
+  } else {
+    nsplit = nsplit_single;
+    first = seq * nsplit;
+  }
+  if (nsplit == 1) return;  // the decode kernel already wrote the normalised row
+  float m = -INFINITY;
+  for (uint32_t s = 0; s < nsplit; ++s)
+    m = fmaxf(m, ws_ml[((size_t)(first + s) * heads + head) * 2]);
+  float denom = 0.f;
+  for (uint32_t s = 0; s < nsplit; ++s) {
+    const size_t i = ((size_t)(first + s) * heads + head) * 2;
+    denom = fmaf(expf(ws_ml[i] - m), ws_ml[i + 1], denom);
+  }
+  const float inv = 1.0f / denom;
+  for (uint32_t d = threadIdx.x; d < depth; d += blockDim.x) {
+    float total = 0.f;
+    for (uint32_t s = 0; s < nsplit; ++s) {
+      const size_t i = (size_t)(first + s) * heads + head;
+      total = fmaf(expf(ws_ml[i * 2] - m), ws_acc[i * depth + d], total);
+    }
+    st_f32<XT>(out, ((size_t)seq * heads + head) * depth + d, total * inv);
+  }
+}
+
+struct DecodeLaunch {
+  krm_buf q, ins_k, ins_v, slot_k, slot_v, out;
+  float* ws_ml;
+  float* ws_acc;
+  DecodeArgs args;
+  uint32_t grid_x, grid_z;     // splits (or total splits), batch
+  uint32_t combine_seqs;       // sequences the combine kernel covers; 0 = no combine needed
+  uint32_t nsplit_single;
+};
+
+template <typename XT, typename ST, int R, int LPR, bool RAGGED>
+int32_t launch_decode(krm_ctx* ctx, const DecodeLaunch& L) {
+  attention_decode_kernel<XT, ST, R, LPR, RAGGED>
+      <<<dim3(L.grid_x, L.args.kv_heads, L.grid_z), dim3(kThreads), 0, ctx->stream>>>(
+          ptr<const XT>(L.q), ptr<const XT>(L.ins_k), ptr<const XT>(L.ins_v),
+          ptr<const ST>(L.slot_k), ptr<const ST>(L.slot_v), ptr<XT>(L.out), L.ws_ml, L.ws_acc,
+          L.args);
+  KRM_TRY(launched(ctx, "attention_decode_kernel"));
+  if (L.combine_seqs) {
+    constexpr int D = LPR * RowChunk<ST>::E;
+    attention_combine_kernel<XT, RAGGED>
+        <<<dim3(L.args.heads, L.combine_seqs), dim3(128), 0, ctx->stream>>>(
+            L.ws_ml, L.ws_acc, ptr<XT>(L.out), L.args.heads, D, L.nsplit_single,
+            L.args.split_prefix);
+    KRM_TRY(launched(ctx, "attention_combine_kernel"));
+  }
+  return KRM_OK;
+}
+
+template <typename XT, typename ST, int LPR, bool RAGGED>
+int32_t decode_by_repeat(krm_ctx* ctx, const DecodeLaunch& L, uint32_t repeat) {
+  switch (repeat) {
+    case 1: return launch_decode<XT, ST, 1, LPR, RAGGED>(ctx, L);
+    case 2: return launch_decode<XT, ST, 2, LPR, RAGGED>(ctx, L);
+    case 4: return launch_decode<XT, ST, 4, LPR, RAGGED>(ctx, L);
+    case 8: return launch_decode<XT, ST, 8, LPR, RAGGED>(ctx, L);
+    default: return fail(ctx, KRM_ERR_VALIDATION, "decode attention: H/Hkv = %u", repeat);
+  }
+}
+
+template <typename XT, typename ST, bool RAGGED>
+int32_t decode_by_depth(krm_ctx* ctx, const DecodeLaunch& L, uint32_t repeat, uint32_t lpr) {
+  switch (lpr) {
+    case 4: return decode_by_repeat<XT, ST, 4, RAGGED>(ctx, L, repeat);
+    case 8: return decode_by_repeat<XT, ST, 8, RAGGED>(ctx, L, repeat);
+    case 16: return decode_by_repeat<XT, ST, 16, RAGGED>(ctx, L, repeat);
+    case 32: return decode_by_repeat<XT, ST, 32, RAGGED>(ctx, L, repeat);
+    default: return fail(ctx, KRM_ERR_VALIDATION, "decode attention: %u lanes per row", lpr);
+  }
+}
+
+template <bool RAGGED>
+int32_t decode_dispatch(krm_ctx* ctx, const DecodeLaunch& L, uint32_t repeat, uint32_t lpr,
+                        int32_t io_dtype, int32_t kv_dtype) {
+  if (io_dtype == KRM_F16 && kv_dtype == KRM_F16)
+    return decode_by_depth<__half, __half, RAGGED>(ctx, L, repeat, lpr);
+  if (io_dtype == KRM_F32 && kv_dtype == KRM_F32)
+    return decode_by_depth<float, float, RAGGED>(ctx, L, repeat, lpr);
+  if (io_dtype == KRM_F32 && kv_dtype == KRM_F16)
+    return decode_by_depth<float, __half, RAGGED>(ctx, L, repeat, lpr);
+  return decode_by_depth<__half, float, RAGGED>(ctx, L, repeat, lpr);
+}
+
+// lanes a K/V row of `depth` elements spans with 16-byte pieces; 0 = not covered
+uint32_t decode_lanes_per_row(uint32_t depth, int32_t kv_dtype) {
+  const uint32_t row_bytes = depth * (uint32_t)dtype_bytes(kv_dtype);
+  if (row_bytes % 16) return 0;
+  const uint32_t lpr = row_bytes / 16;
+  return (lpr == 4 || lpr == 8 || lpr == 16 || lpr == 32) ? lpr : 0;
+}
+
+bool decode_repeat_ok(uint32_t repeat) {
+  return repeat == 1 || repeat == 2 || repeat == 4 || repeat == 8;
+}
+
+template <typename XT, typename ST>
+int32_t launch_generic(krm_ctx* ctx, krm_buf q, krm_buf ins_k, krm_buf ins_v, krm_buf slot_k,
+                       krm_buf slot_v, krm_buf out, uint32_t batch, const GenericArgs& a) {
+  attention_generic_kernel<XT, ST>
+      <<<dim3(batch * a.heads, a.chunk_rows), dim3(kThreads), 0, ctx->stream>>>(
+          ptr<const XT>(q), ptr<const XT>(ins_k), ptr<const XT>(ins_v), ptr<const ST>(slot_k),
+          ptr<const ST>(slot_v), ptr<XT>(out), a);
+  return launched(ctx, "attention_generic_kernel");
+}
+
+// smallest split any dtype uses for this head dim (f32 rows span the most lanes)
+uint32_t min_split_columns(uint32_t depth) {
+  uint32_t lpr = decode_lanes_per_row(depth, KRM_F32);
+  if (!lpr) lpr = decode_lanes_per_row(depth, KRM_F16);
+  return lpr ? decode_split_columns(lpr) : 0;
+}
+
+}  // namespace
+
+extern "C" {
+
+int32_t krm_attention_state_workspace(uint32_t batch, uint32_t heads, uint32_t kv_heads,
+                                      uint32_t chunk_rows, uint32_t depth, uint32_t window,
+                                      uint32_t max_past, uint32_t max_query, size_t* bytes) {
+  (void)kv_heads;
+  (void)chunk_rows;
+  (void)max_query;
+  if (!bytes) return fail(nullptr, KRM_ERR_VALIDATION, "krm_attention_state_workspace: NULL");
+  const uint32_t sc = min_split_columns(depth);
+  uint64_t columns = max_past;
+  if (window && columns > window - 1) columns = window - 1;
+  const uint64_t nsplit = sc ? decode_splits(columns, sc) : 1;
+  *bytes = (size_t)batch * heads * nsplit * ((size_t)depth + 2) * sizeof(float) + 256;
+  return KRM_OK;
+}
+
+int32_t krm_attention_state(krm_ctx* ctx, krm_buf q, krm_buf ins_k, krm_buf ins_v,
+                            krm_buf slot_k, krm_buf slot_v, krm_buf out, uint32_t batch,
+                            uint32_t heads, uint32_t kv_heads, uint32_t chunk_rows,
+                            uint32_t depth, uint32_t capacity, uint32_t window,
+                            float half_scale, uint32_t past, uint32_t query, int32_t io_dtype,
+                            int32_t kv_dtype, krm_buf workspace, size_t workspace_bytes) {
+  KRM_TRY(enter(ctx));
+  KRM_REQUIRE(ctx, valid_dtype(io_dtype) && valid_dtype(kv_dtype),
+              "krm_attention_state: io_dtype %d / kv_dtype %d", io_dtype, kv_dtype);
+  KRM_REQUIRE(ctx,
+              batch >= 1 && heads >= 1 && kv_heads >= 1 && chunk_rows >= 1 && depth >= 1 &&
+                  capacity >= 1,
+              "krm_attention_state: B / H / Hkv / M / D / C must be positive "
+              "(%u / %u / %u / %u / %u / %u)",
+              batch, heads, kv_heads, chunk_rows, depth, capacity);
+  KRM_REQUIRE(ctx, heads % kv_heads == 0, "krm_attention_state: H = %u is not a multiple of Hkv = %u",
+              heads, kv_heads);
+  KRM_REQUIRE(ctx, window <= capacity, "krm_attention_state: window %u exceeds capacity %u",
+              window, capacity);
+  KRM_REQUIRE(ctx, std::isfinite(half_scale), "krm_attention_state: scale is not finite");
+  KRM_REQUIRE(ctx, depth <= 1024, "krm_attention_state: D = %u exceeds 1024", depth);
+  KRM_REQUIRE(ctx, (uint64_t)batch * heads <= 0x7fffffffull && chunk_rows <= 65535,
+              "krm_attention_state: B*H = %llu or M = %u exceeds the launch grid",
+              (unsigned long long)batch * heads, chunk_rows);
+  if (query < 1 || query > chunk_rows)
+    return fail(ctx, KRM_ERR_EXECUTION, "krm_attention_state: queryLength %u is outside 1..%u",
+                query, chunk_rows);
+  if ((uint64_t)past + query > 0xffffffffull)
+    return fail(ctx, KRM_ERR_EXECUTION,
+                "krm_attention_state: pastLength %u + queryLength %u does not fit in 32 bits",
+                past, query);
+  if (window == 0 && (uint64_t)past + query > capacity)
+    return fail(ctx, KRM_ERR_EXECUTION,
+                "krm_attention_state: pastLength %u + queryLength %u exceeds capacity %u", past,
+                query, capacity);
+  KRM_REQUIRE(ctx, q && ins_k && ins_v && slot_k && slot_v && out,
+              "krm_attention_state: NULL buffer");
+  const size_t io_b = dtype_bytes(io_dtype), kv_b = dtype_bytes(kv_dtype);
+  KRM_REQUIRE(ctx,
+              aligned(q, io_b) && aligned(ins_k, io_b) && aligned(ins_v, io_b) &&
+                  aligned(out, io_b) && aligned(slot_k, kv_b) && aligned(slot_v, kv_b),
+              "krm_attention_state: misaligned buffer");
+
+  const uint32_t repeat = heads / kv_heads;
+  const uint32_t lpr = decode_lanes_per_row(depth, kv_dtype);
+  const bool fast = query == 1 && chunk_rows == 1 && lpr && decode_repeat_ok(repeat) &&
+                    aligned(slot_k, 16) && aligned(slot_v, 16) && batch <= 65535 &&
+                    kv_heads <= 65535;
+  if (fast) {
+    const uint64_t low = window_low(window, past);
+    const uint32_t nsplit = decode_splits((uint64_t)past - low, decode_split_columns(lpr));
+    DecodeLaunch L{};
+    L.q = q; L.ins_k = ins_k; L.ins_v = ins_v; L.slot_k = slot_k; L.slot_v = slot_v; L.out = out;
+    L.args.heads = heads;
+    L.args.kv_heads = kv_heads;
+    L.args.window = window;
+    L.args.past = past;
+    L.args.slot_batch_stride = (uint64_t)kv_heads * capacity * depth;
+    L.args.slot_plane_stride = (uint64_t)capacity * depth;
+    L.args.scale = half_scale;
+    L.args.nseq = batch;
+    L.grid_x = nsplit;
+    L.grid_z = batch;
+    L.nsplit_single = nsplit;
+    if (nsplit > 1) {
+      const size_t ml_floats = (size_t)batch * nsplit * heads * 2;
+      const size_t need = (ml_floats + (size_t)batch * nsplit * heads * depth) * sizeof(float);
+      KRM_REQUIRE(ctx, workspace && aligned(workspace, 16) && workspace_bytes >= need,
+                  "krm_attention_state: workspace of %zu bytes, %zu needed", workspace_bytes,
+                  need);
+      L.ws_ml = ptr<float>(workspace);
+      L.ws_acc = L.ws_ml + ((ml_floats + 3) & ~(size_t)3);
+      KRM_REQUIRE(ctx, workspace_bytes >= (size_t)((char*)(L.ws_acc + (size_t)batch * nsplit *
+                                                           heads * depth) - (char*)L.ws_ml),
+                  "krm_attention_state: workspace of %zu bytes is too small", workspace_bytes);
+      L.combine_seqs = batch;
+    }
+    return decode_dispatch<false>(ctx, L, repeat, lpr, io_dtype, kv_dtype);
+  }
+
+  GenericArgs a{heads, kv_heads, chunk_rows, depth, capacity, window, past, query, half_scale};
+  if (io_dtype == KRM_F32 && kv_dtype == KRM_F32)
+    return launch_generic<float, float>(ctx, q, ins_k, ins_v, slot_k, slot_v, out, batch, a);
+  if (io_dtype == KRM_F16 && kv_dtype == KRM_F16)
+    return launch_generic<__half, __half>(ctx, q, ins_k, ins_v, slot_k, slot_v, out, batch, a);
+  if (io_dtype == KRM_F32 && kv_dtype == KRM_F16)
+    return launch_generic<float, __half>(ctx, q, ins_k, ins_v, slot_k, slot_v, out, batch, a);
+  return launch_generic<__half, float>(ctx, q, ins_k, ins_v, slot_k, slot_v, out, batch, a);
+}
+
+int32_t krm_attention_varlen_workspace(uint32_t nseq, uint32_t heads, uint32_t kv_heads,
+                                       uint32_t depth, uint64_t total_rows, size_t* bytes) {
+  (void)kv_heads;
+  if (!bytes) return fail(nullptr, KRM_ERR_VALIDATION, "krm_attention_varlen_workspace: NULL");
+  const uint32_t sc = min_split_columns(depth);
+  // every sequence rounds its split count up, so at most total/sc + nseq splits
+  const uint64_t splits = sc ? total_rows / sc + nseq : nseq;
+  *bytes = 2 * ((size_t)nseq + 1) * sizeof(int32_t) + 64 +
+           (size_t)splits * heads * ((size_t)depth + 2) * sizeof(float) + 256;
+  return KRM_OK;
+}
+
+int32_t krm_attention_varlen(krm_ctx* ctx, krm_buf q, krm_buf ins_k, krm_buf ins_v,
+                             krm_buf slot_k, krm_buf slot_v, krm_buf out,
+                             const int32_t* cu_seqlens, uint32_t nseq, uint32_t heads,
+                             uint32_t kv_heads, uint32_t depth, uint64_t total_rows,
+                             float half_scale, int32_t io_dtype, int32_t kv_dtype,
+                             krm_buf workspace, size_t workspace_bytes) {
+  KRM_TRY(enter(ctx));
+  KRM_REQUIRE(ctx, valid_dtype(io_dtype) && valid_dtype(kv_dtype),
+              "krm_attention_varlen: io_dtype %d / kv_dtype %d", io_dtype, kv_dtype);
+  KRM_REQUIRE(ctx, nseq >= 1 && heads >= 1 && kv_heads >= 1 && depth >= 1,
+              "krm_attention_varlen: nseq / H / Hkv / D must be positive");
+  KRM_REQUIRE(ctx, heads % kv_heads == 0, "krm_attention_varlen: H = %u is not a multiple of Hkv = %u",
+              heads, kv_heads);
+  KRM_REQUIRE(ctx, std::isfinite(half_scale), "krm_attention_varlen: scale is not finite");
+  KRM_REQUIRE(ctx, cu_seqlens != nullptr, "krm_attention_varlen: cu_seqlens is NULL");
+  KRM_REQUIRE(ctx, total_rows <= 0x7fffffffull, "krm_attention_varlen: total_rows too large");
+  KRM_REQUIRE(ctx, nseq <= 65535 && kv_heads <= 65535, "krm_attention_varlen: grid too large");
+  const uint32_t repeat = heads / kv_heads;
+  const uint32_t lpr = decode_lanes_per_row(depth, kv_dtype);
+  KRM_REQUIRE(ctx, lpr && decode_repeat_ok(repeat),
+              "krm_attention_varlen: D = %u with this slot dtype or H/Hkv = %u is not covered "
+              "by the split-K decode kernel",
+              depth, repeat);
+  KRM_REQUIRE(ctx, q && ins_k && ins_v && slot_k && slot_v && out && workspace,
+              "krm_attention_varlen: NULL buffer");
+  KRM_REQUIRE(ctx, aligned(slot_k, 16) && aligned(slot_v, 16) && aligned(workspace, 16),
+              "krm_attention_varlen: slots and workspace must be 16-byte aligned");
+  KRM_REQUIRE(ctx, cu_seqlens[0] >= 0, "krm_attention_varlen: cu_seqlens[0] is negative");
+
+  // Host-side tables: slot row offsets and the first global split of each sequence.
+  const size_t table_ints = 2 * ((size_t)nseq + 1);
+  KRM_REQUIRE(ctx, table_ints * sizeof(int32_t) <= ctx->pinned_bytes,
+              "krm_attention_varlen: %u sequences exceed the staging table", nseq);
+  // The staging area may still feed the previous call's copy.
+  KRM_TRY(hip_status(ctx, hipStreamSynchronize(ctx->stream), "hipStreamSynchronize"));
+  int32_t* stage = static_cast<int32_t*>(ctx->pinned);
+  int32_t* cu = stage;
+  int32_t* prefix = stage + nseq + 1;
+  const uint32_t sc = decode_split_columns(lpr);
+  uint64_t splits = 0;
+  bool any_split = false;
+  for (uint32_t i = 0; i <= nseq; ++i) {
+    cu[i] = cu_seqlens[i];
+    if (i > 0) {
+      KRM_REQUIRE(ctx, cu_seqlens[i] >= cu_seqlens[i - 1],
+                  "krm_attention_varlen: cu_seqlens is not ascending at %u", i);
+      prefix[i - 1] = (int32_t)splits;
+      const uint32_t ns = decode_splits((uint64_t)(cu_seqlens[i] - cu_seqlens[i - 1]), sc);
+      any_split = any_split || ns > 1;
+      splits += ns;
+    }
+  }
+  prefix[nseq] = (int32_t)splits;
+  KRM_REQUIRE(ctx, (uint64_t)cu_seqlens[nseq] <= total_rows,
+              "krm_attention_varlen: cu_seqlens[%u] = %d exceeds total_rows %llu", nseq,
+              cu_seqlens[nseq], (unsigned long long)total_rows);
+  KRM_REQUIRE(ctx, splits <= 0x7fffffffull, "krm_attention_varlen: too many splits");
+
+  const size_t table_bytes = (table_ints * sizeof(int32_t) + 63) & ~(size_t)63;
+  const size_t ml_floats = ((size_t)splits * heads * 2 + 3) & ~(size_t)3;
+  const size_t need = table_bytes + (ml_floats + (size_t)splits * heads * depth) * sizeof(float);
+  KRM_REQUIRE(ctx, workspace_bytes >= need, "krm_attention_varlen: workspace of %zu bytes, %zu needed",
+              workspace_bytes, need);
+  KRM_TRY(hip_status(ctx,
+                     hipMemcpyAsync(ptr<void>(workspace), stage, table_ints * sizeof(int32_t),
+                                    hipMemcpyHostToDevice, ctx->stream),
+                     "hipMemcpyAsync(tables)"));
+
+  DecodeLaunch L{};
+  L.q = q; L.ins_k = ins_k; L.ins_v = ins_v; L.slot_k = slot_k; L.slot_v = slot_v; L.out = out;
+  L.args.heads = heads;
+  L.args.kv_heads = kv_heads;
+  L.args.window = 0;
+  L.args.past = 0;
+  L.args.slot_batch_stride = 0;
+  L.args.slot_plane_stride = total_rows * depth;
+  L.args.scale = half_scale;
+  L.args.nseq = nseq;
+  L.args.cu_rows = ptr<const int32_t>(workspace);
+  L.args.split_prefix = L.args.cu_rows + nseq + 1;
+  L.ws_ml = ptr<float>(workspace + table_bytes);
+  L.ws_acc = L.ws_ml + ml_floats;
+  L.grid_x = (uint32_t)splits;
+  L.grid_z = 1;
+  L.combine_seqs = any_split ? nseq : 0;
+  L.nsplit_single = 0;
+  return decode_dispatch<true>(ctx, L, repeat, lpr, io_dtype, kv_dtype);
+}
+
+}  // extern "C"

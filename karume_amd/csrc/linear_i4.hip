@@ -1,0 +1,428 @@
+// int4 group-quantised `linear` for gfx950: the dequant kernel (bit-exact gate) and the
+// bandwidth-bound GEMV used for M <= 16 rows of activations.
+//
+// Semantics follow the reference's linear op with i4 weights
+// (packages/runtime/src/kernels/linear.ts:34-64, body packages/runtime/src/kernels/gemm.ts:
+// 1187-1237, dequant packages/runtime/src/kernels/weight-storage.ts:152-187): weights are
+// packed [N, K] with K contiguous, 8 elements per little-endian u32 (element 8w+j at bits
+// 4j), stored u = q + 8, one scale per `group` consecutive K elements of a row.
+//
+// The reference runs M = 1 through a 16x16-tile f32 GEMM with a strictly K-ascending
+// accumulation.  Here a wave owns whole output rows instead: every lane streams 16 bytes
+// (32 codes) of a row per step, accumulates sum((u-8)*x) for its 32 codes in f32, applies the
+// group scale to that partial sum, and the 64 lane sums are added with a fixed DPP tree.  The
+// reduction order therefore differs from the reference's (results agree within a stated
+// tolerance, not bitwise) but depends on (K, group) only — never on M, N or the launch — so a
+// row of x gives the same bits whether it is run alone or in a batch.
+#include "krm_internal.h"
+
+using namespace krm;
+
+namespace {
+
+typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+
+// ------------------------------------------------------------------------------------ dequant
+
+template <typename ST>
+__device__ inline float load_scale(const ST* s, size_t i);
+template <>
+__device__ inline float load_scale<float>(const float* s, size_t i) { return s[i]; }
+template <>
+__device__ inline float load_scale<__half>(const __half* s, size_t i) {
+  return __half2float(s[i]);
+}
+
+// One thread expands one u32 (8 codes).  f32(u - 8) * scale is a single rounded f32 multiply.
+template <typename ST>
+__global__ __launch_bounds__(256) void dequant_i4_kernel(const uint32_t* __restrict__ w,
+                                                         const ST* __restrict__ scales,
+                                                         float* __restrict__ out, size_t words,
+                                                         size_t width, uint32_t group) {
+  const size_t stride = (size_t)gridDim.x * blockDim.x;
+  const size_t groups = width / group;
+  for (size_t wi = blockIdx.x * (size_t)blockDim.x + threadIdx.x; wi < words; wi += stride) {
+    const uint32_t word = w[wi];
+    const size_t i0 = wi * 8;
+    float v[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const size_t i = i0 + j;
+      const size_t row = i / width;
+      const size_t g = (i - row * width) / group;
+      const int code = (int)((word >> (4 * j)) & 0xFu) - 8;
+      v[j] = __fmul_rn((float)code, load_scale<ST>(scales, row * groups + g));
+    }
+    float4* dst = reinterpret_cast<float4*>(out + i0);
+    dst[0] = make_float4(v[0], v[1], v[2], v[3]);
+    dst[1] = make_float4(v[4], v[5], v[6], v[7]);
+  }
+}
+
+// ------------------------------------------------------------------------------------ GEMV
+
+// Sum over the 64 lanes of a wave; every lane returns the total.  Fixed tree: quad swaps,
+// half-row mirror, row mirror (16-lane rows), then the four row sums in ascending order.
+__device__ inline float wave_sum(float v) {
+  int t;
+  t = __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0xB1, 0xf, 0xf, true);
+  v += __builtin_bit_cast(float, t);  // quad_perm [1,0,3,2]
+  t = __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x4E, 0xf, 0xf, true);
+  v += __builtin_bit_cast(float, t);  // quad_perm [2,3,0,1]
+  t = __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x141, 0xf, 0xf, true);
+  v += __builtin_bit_cast(float, t);  // row_half_mirror
+  t = __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x140, 0xf, 0xf, true);
+  v += __builtin_bit_cast(float, t);  // row_mirror
+  const int bits = __builtin_bit_cast(int, v);
+  const float r0 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(bits, 0));
+  const float r1 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(bits, 16));
+  const float r2 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(bits, 32));
+  const float r3 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(bits, 48));
+  return ((r0 + r1) + r2) + r3;
+}
+
+// Eight codes of one u32 as four fp16 pairs holding the exact integers (u - 8):
+// pair i = (code i, code i+4).  1024 + u is built in the fp16 mantissa, then the offset is
+// removed with one packed op; codes in the upper nibble of a byte arrive as 1024 + 16u.
+__device__ inline void codes_to_half2(uint32_t word, half2_t (&q)[4]) {
+  const uint32_t magic = 0x64006400u;  // (1024.0, 1024.0)
+  const half2_t off_lo = {(_Float16)1032.0f, (_Float16)1032.0f};
+  const half2_t sixteenth = {(_Float16)0.0625f, (_Float16)0.0625f};
+  const half2_t off_hi = {(_Float16)-72.0f, (_Float16)-72.0f};
+  const uint32_t upper = word >> 8;
+  q[0] = __builtin_bit_cast(half2_t, (word & 0x000F000Fu) | magic) - off_lo;
+  q[1] = __builtin_bit_cast(half2_t, (word & 0x00F000F0u) | magic) * sixteenth + off_hi;
+  q[2] = __builtin_bit_cast(half2_t, (upper & 0x000F000Fu) | magic) - off_lo;
+  q[3] = __builtin_bit_cast(half2_t, (upper & 0x00F000F0u) | magic) * sixteenth + off_hi;
+}
+
+// Eight consecutive fp16 activations (x0..x7 in four dwords) regrouped to match
+// codes_to_half2: pair i = (x_i, x_{i+4}).
+__device__ inline void pair_activations(const uint4& raw, half2_t (&p)[4]) {
+  p[0] = __builtin_bit_cast(half2_t, __builtin_amdgcn_perm(raw.z, raw.x, 0x05040100u));
+  p[1] = __builtin_bit_cast(half2_t, __builtin_amdgcn_perm(raw.z, raw.x, 0x07060302u));
+  p[2] = __builtin_bit_cast(half2_t, __builtin_amdgcn_perm(raw.w, raw.y, 0x05040100u));
+  p[3] = __builtin_bit_cast(half2_t, __builtin_amdgcn_perm(raw.w, raw.y, 0x07060302u));
+}
+
+template <typename XT>
+struct Acts;  // per-lane activations of one x row for one step (VEC words = VEC*8 elements)
+
+// fp16 activations: exact fp16 products, f32 accumulation through v_dot2_f32_f16.
+template <>
+struct Acts<__half> {
+  template <int VEC>
+  struct Regs {
+    half2_t p[VEC][4];
+  };
+  template <int VEC>
+  __device__ static inline void load(const __half* x, bool active, Regs<VEC>& r) {
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) {
+      uint4 raw = make_uint4(0, 0, 0, 0);
+      if (active) raw = reinterpret_cast<const uint4*>(x)[j];
+      pair_activations(raw, r.p[j]);
+    }
+  }
+  // sum over the lane's VEC*8 codes of (u - 8) * x
+  template <int VEC>
+  __device__ static inline float dot(const uint32_t (&words)[VEC], const Regs<VEC>& r) {
+    float acc = 0.f;
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) {
+      half2_t q[4];
+      codes_to_half2(words[j], q);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) acc = __builtin_amdgcn_fdot2(q[i], r.p[j][i], acc, false);
+    }
+    return acc;
+  }
+};
+
+// f32 activations: f32 products.  sum(u*x) is accumulated with one convert + one fma per
+// code and the offset is removed once per step: sum((u-8)*x) = sum(u*x) - 8*sum(x).
+template <>
+struct Acts<float> {
+  template <int VEC>
+  struct Regs {
+    float v[VEC][8];
+    float sum;
+  };
+  template <int VEC>
+  __device__ static inline void load(const float* x, bool active, Regs<VEC>& r) {
+    float s = 0.f;
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) {
+      float4 a = make_float4(0.f, 0.f, 0.f, 0.f), b = a;
+      if (active) {
+        a = reinterpret_cast<const float4*>(x)[2 * j];
+        b = reinterpret_cast<const float4*>(x)[2 * j + 1];
+      }
+      r.v[j][0] = a.x; r.v[j][1] = a.y; r.v[j][2] = a.z; r.v[j][3] = a.w;
+      r.v[j][4] = b.x; r.v[j][5] = b.y; r.v[j][6] = b.z; r.v[j][7] = b.w;
+      s += ((a.x + a.y) + (a.z + a.w)) + ((b.x + b.y) + (b.z + b.w));
+    }
+    r.sum = s;
+  }
+  template <int VEC>
+  __device__ static inline float dot(const uint32_t (&words)[VEC], const Regs<VEC>& r) {
+    float acc = 0.f;
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) {
+      const uint32_t even = words[j] & 0x0F0F0F0Fu;         // codes 0,2,4,6 one per byte
+      const uint32_t odd = (words[j] >> 4) & 0x0F0F0F0Fu;   // codes 1,3,5,7
+#pragma unroll
+      for (int b = 0; b < 4; ++b) {
+        acc = fmaf((float)((even >> (8 * b)) & 0xFFu), r.v[j][2 * b], acc);
+        acc = fmaf((float)((odd >> (8 * b)) & 0xFFu), r.v[j][2 * b + 1], acc);
+      }
+    }
+    return fmaf(-8.0f, r.sum, acc);
+  }
+};
+
+template <typename T>
+__device__ inline float to_f32(T v);
+template <>
+__device__ inline float to_f32<float>(float v) { return v; }
+template <>
+__device__ inline float to_f32<__half>(__half v) { return __half2float(v); }
+template <typename T>
+__device__ inline T from_f32(float v);
+template <>
+__device__ inline float from_f32<float>(float v) { return v; }
+template <>
+__device__ inline __half from_f32<__half>(float v) { return __float2half_rn(v); }
+
+// One wave = ROWS consecutive output rows over the whole K; a step covers 64 lanes x VEC
+// words (VEC*8 codes per lane, all inside one scale group).  The next step's weight words
+// and scales are requested before the current step is consumed.
+template <typename XT, typename ST, int MB, int ROWS, int VEC>
+__global__ __launch_bounds__(256) void gemv_i4_kernel(
+    const XT* __restrict__ x, const uint32_t* __restrict__ w, const ST* __restrict__ scales,
+    const XT* __restrict__ bias, XT* __restrict__ out, uint32_t m, uint32_t n, uint32_t k,
+    uint32_t group_shift) {
+  constexpr int kLaneElems = VEC * 8;
+  constexpr int kStepElems = kWave * kLaneElems;
+  const int lane = threadIdx.x & (kWave - 1);
+  const int wave = threadIdx.x >> 6;
+  const uint32_t row0 = (blockIdx.x * (blockDim.x >> 6) + wave) * ROWS;
+  if (row0 >= n) return;  // whole wave leaves together
+
+  const uint32_t words_per_row = k >> 3;
+  const uint32_t groups_per_row = k >> group_shift;
+  const uint32_t steps = (k + kStepElems - 1) / kStepElems;
+
+  const uint32_t* wrow[ROWS];
+  const ST* srow[ROWS];
+#pragma unroll
+  for (int r = 0; r < ROWS; ++r) {
+    const uint32_t row = min(row0 + r, n - 1);  // rows past N re-read the last row, unused
+    wrow[r] = w + (size_t)row * words_per_row;
+    srow[r] = scales + (size_t)row * groups_per_row;
+  }
+
+  float acc[ROWS][MB];
+#pragma unroll
+  for (int r = 0; r < ROWS; ++r)
+#pragma unroll
+    for (int b = 0; b < MB; ++b) acc[r][b] = 0.f;
+
+  uint32_t cur_w[ROWS][VEC], nxt_w[ROWS][VEC];
+  float cur_s[ROWS], nxt_s[ROWS];
+
+  auto fetch = [&](uint32_t step, uint32_t (&dst_w)[ROWS][VEC], float (&dst_s)[ROWS]) {
+    const uint32_t k0 = step * kStepElems + lane * kLaneElems;
+    const bool active = k0 < k;
+#pragma unroll
+    for (int r = 0; r < ROWS; ++r) {
+      if (active) {
+        if constexpr (VEC == 4) {
+          const uint4 v = *reinterpret_cast<const uint4*>(wrow[r] + (k0 >> 3));
+          dst_w[r][0] = v.x; dst_w[r][1] = v.y; dst_w[r][2] = v.z; dst_w[r][3] = v.w;
+        } else {
+#pragma unroll
+          for (int j = 0; j < VEC; ++j) dst_w[r][j] = wrow[r][(k0 >> 3) + j];
+        }
+        dst_s[r] = load_scale<ST>(srow[r], k0 >> group_shift);
+      } else {
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) dst_w[r][j] = 0u;
+        dst_s[r] = 0.f;
+      }
+    }
+  };
+
+  fetch(0, cur_w, cur_s);
+  for (uint32_t step = 0; step < steps; ++step) {
+    if (step + 1 < steps) fetch(step + 1, nxt_w, nxt_s);
+    const uint32_t k0 = step * kStepElems + lane * kLaneElems;
+    const bool active = k0 < k;
+#pragma unroll
+    for (int b = 0; b < MB; ++b) {
+      typename Acts<XT>::template Regs<VEC> regs;
+      const uint32_t xrow = min((uint32_t)b, m - 1);  // rows past M re-read the last row, unused
+      Acts<XT>::template load<VEC>(x + (size_t)xrow * k + k0, active, regs);
+#pragma unroll
+      for (int r = 0; r < ROWS; ++r) {
+        const float part = Acts<XT>::template dot<VEC>(cur_w[r], regs);
+        acc[r][b] = fmaf(part, cur_s[r], acc[r][b]);
+      }
+    }
+#pragma unroll
+    for (int r = 0; r < ROWS; ++r) {
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) cur_w[r][j] = nxt_w[r][j];
+      cur_s[r] = nxt_s[r];
+    }
+  }
+
+#pragma unroll
+  for (int r = 0; r < ROWS; ++r) {
+#pragma unroll
+    for (int b = 0; b < MB; ++b) {
+      const float total = wave_sum(acc[r][b]);
+      const uint32_t row = row0 + r;
+      if (lane == (r * MB + b) % kWave && row < n && (uint32_t)b < m) {
+        const float add = bias ? to_f32<XT>(bias[row]) : 0.f;
+        out[(size_t)b * n + row] = from_f32<XT>(total + add);
+      }
+    }
+  }
+}
+
+template <typename XT, typename ST, int MB, int ROWS, int VEC>
+int32_t launch_gemv(krm_ctx* ctx, krm_buf x, krm_buf w, krm_buf scales, krm_buf bias,
+                    krm_buf out, uint32_t m, uint32_t n, uint32_t k, uint32_t group_shift) {
+  const uint32_t rows_per_block = 4 * ROWS;
+  const uint32_t blocks = (n + rows_per_block - 1) / rows_per_block;
+  gemv_i4_kernel<XT, ST, MB, ROWS, VEC><<<dim3(blocks), dim3(256), 0, ctx->stream>>>(
+      ptr<const XT>(x), ptr<const uint32_t>(w), ptr<const ST>(scales), ptr<const XT>(bias),
+      ptr<XT>(out), m, n, k, group_shift);
+  return launched(ctx, "gemv_i4_kernel");
+}
+
+template <typename XT, typename ST, int MB, int VEC>
+int32_t pick_rows(krm_ctx* ctx, krm_buf x, krm_buf w, krm_buf scales, krm_buf bias, krm_buf out,
+                  uint32_t m, uint32_t n, uint32_t k, uint32_t group_shift) {
+  // Rows per wave: more rows amortise the activation fetch, fewer rows give more waves to
+  // hide latency.  The choice never changes a row's reduction order.
+  const uint64_t cus = (uint64_t)ctx->num_cus;
+  if (MB <= 4 && (uint64_t)n >= cus * 4 * 4 * 2)
+    return launch_gemv<XT, ST, MB, 4, VEC>(ctx, x, w, scales, bias, out, m, n, k, group_shift);
+  if ((uint64_t)n >= cus * 4 * 2)
+    return launch_gemv<XT, ST, MB, 2, VEC>(ctx, x, w, scales, bias, out, m, n, k, group_shift);
+  return launch_gemv<XT, ST, MB, 1, VEC>(ctx, x, w, scales, bias, out, m, n, k, group_shift);
+}
+
+template <typename XT, typename ST, int VEC>
+int32_t pick_batch(krm_ctx* ctx, krm_buf x, krm_buf w, krm_buf scales, krm_buf bias, krm_buf out,
+                   uint32_t m, uint32_t n, uint32_t k, uint32_t group_shift) {
+  if (m == 1) return pick_rows<XT, ST, 1, VEC>(ctx, x, w, scales, bias, out, m, n, k, group_shift);
+  if (m == 2) return pick_rows<XT, ST, 2, VEC>(ctx, x, w, scales, bias, out, m, n, k, group_shift);
+  if (m <= 4) return pick_rows<XT, ST, 4, VEC>(ctx, x, w, scales, bias, out, m, n, k, group_shift);
+  if (m <= 8) return pick_rows<XT, ST, 8, VEC>(ctx, x, w, scales, bias, out, m, n, k, group_shift);
+  return pick_rows<XT, ST, 16, VEC>(ctx, x, w, scales, bias, out, m, n, k, group_shift);
+}
+
+template <typename XT, typename ST>
+int32_t pick_vec(krm_ctx* ctx, krm_buf x, krm_buf w, krm_buf scales, krm_buf bias, krm_buf out,
+                 uint32_t m, uint32_t n, uint32_t k, uint32_t group) {
+  uint32_t group_shift = 0;
+  while ((1u << group_shift) < group) ++group_shift;
+  // 16-byte loads need 32 codes per lane inside one group and 16-byte aligned rows.
+  const bool wide = (k % 32 == 0) && (group % 32 == 0) && aligned(w, 16);
+  if (wide) return pick_batch<XT, ST, 4>(ctx, x, w, scales, bias, out, m, n, k, group_shift);
+  return pick_batch<XT, ST, 1>(ctx, x, w, scales, bias, out, m, n, k, group_shift);
+}
+
+}  // namespace
+
+namespace krm {
+
+// Rows M <= 16: the GEMV above.  Declared in gemm_i4.hip's dispatcher too.
+int32_t linear_i4_gemv(krm_ctx* ctx, krm_buf x, krm_buf w, krm_buf scales, krm_buf bias,
+                       krm_buf out, uint32_t m, uint32_t n, uint32_t k, uint32_t group,
+                       int32_t io_dtype, int32_t scale_dtype) {
+  if (io_dtype == KRM_F16) {
+    if (scale_dtype == KRM_F16)
+      return pick_vec<__half, __half>(ctx, x, w, scales, bias, out, m, n, k, group);
+    return pick_vec<__half, float>(ctx, x, w, scales, bias, out, m, n, k, group);
+  }
+  if (scale_dtype == KRM_F16)
+    return pick_vec<float, __half>(ctx, x, w, scales, bias, out, m, n, k, group);
+  return pick_vec<float, float>(ctx, x, w, scales, bias, out, m, n, k, group);
+}
+
+// fp16 MFMA GEMM for M > 16 (gemm_i4.hip).
+int32_t linear_i4_gemm_f16(krm_ctx* ctx, krm_buf x, krm_buf w, krm_buf scales, krm_buf bias,
+                           krm_buf out, uint32_t m, uint32_t n, uint32_t k, uint32_t group,
+                           int32_t io_dtype, int32_t scale_dtype);
+
+}  // namespace krm
+
+extern "C" {
+
+int32_t krm_linear_i4(krm_ctx* ctx, krm_buf x, krm_buf w, krm_buf scales, krm_buf bias,
+                      krm_buf out, uint32_t m, uint32_t n, uint32_t k, uint32_t group,
+                      int32_t io_dtype, int32_t scale_dtype, int32_t compute) {
+  KRM_TRY(enter(ctx));
+  KRM_REQUIRE(ctx, valid_dtype(io_dtype) && valid_dtype(scale_dtype),
+              "krm_linear_i4: io_dtype %d / scale_dtype %d", io_dtype, scale_dtype);
+  KRM_REQUIRE(ctx, compute == KRM_COMPUTE_F32 || compute == KRM_COMPUTE_F16,
+              "krm_linear_i4: compute %d", compute);
+  // Storage rules of the int4 format: group is a power of two >= 16 that divides K.
+  KRM_REQUIRE(ctx, is_pow2(group) && group >= 16,
+              "krm_linear_i4: group_size %u is not a power of two >= 16", group);
+  KRM_REQUIRE(ctx, k >= 1 && k % group == 0,
+              "krm_linear_i4: group_size %u does not divide k = %u", group, k);
+  if (m == 0 || n == 0) return KRM_OK;
+  KRM_REQUIRE(ctx, x && w && scales && out, "krm_linear_i4: NULL buffer");
+  KRM_REQUIRE(ctx, aligned(x, 16) && aligned(out, dtype_bytes(io_dtype)) && aligned(w, 4) &&
+                       aligned(scales, dtype_bytes(scale_dtype)) &&
+                       aligned(bias, dtype_bytes(io_dtype)),
+              "krm_linear_i4: x must be 16-byte aligned, w 4-byte aligned");
+  if (m <= 16)
+    return linear_i4_gemv(ctx, x, w, scales, bias, out, m, n, k, group, io_dtype, scale_dtype);
+  if (compute == KRM_COMPUTE_F16)
+    return linear_i4_gemm_f16(ctx, x, w, scales, bias, out, m, n, k, group, io_dtype,
+                              scale_dtype);
+  // f32 arithmetic for any M: the GEMV over blocks of 16 rows (weights re-read per block).
+  const size_t eb = dtype_bytes(io_dtype);
+  for (uint32_t r = 0; r < m; r += 16) {
+    const uint32_t rows = m - r < 16 ? m - r : 16;
+    KRM_TRY(linear_i4_gemv(ctx, x + (size_t)r * k * eb, w, scales, bias,
+                           out + (size_t)r * n * eb, rows, n, k, group, io_dtype, scale_dtype));
+  }
+  return KRM_OK;
+}
+
+int32_t krm_dequant_i4(krm_ctx* ctx, krm_buf w, krm_buf scales, krm_buf out_f32, uint64_t rows,
+                       uint64_t width, uint32_t group, int32_t scale_dtype) {
+  KRM_TRY(enter(ctx));
+  KRM_REQUIRE(ctx, valid_dtype(scale_dtype), "krm_dequant_i4: scale_dtype %d", scale_dtype);
+  KRM_REQUIRE(ctx, group >= 1 && width >= 1 && width % group == 0,
+              "krm_dequant_i4: group_size %u does not divide the row length %llu", group,
+              (unsigned long long)width);
+  KRM_REQUIRE(ctx, (rows * width) % 8 == 0,
+              "krm_dequant_i4: %llu x %llu codes is not a whole number of 32-bit words",
+              (unsigned long long)rows, (unsigned long long)width);
+  if (rows == 0) return KRM_OK;
+  KRM_REQUIRE(ctx, w && scales && out_f32, "krm_dequant_i4: NULL buffer");
+  KRM_REQUIRE(ctx, aligned(w, 4) && aligned(out_f32, 16) && aligned(scales, dtype_bytes(scale_dtype)),
+              "krm_dequant_i4: w must be 4-byte and out 16-byte aligned");
+  const size_t words = rows * width / 8;
+  size_t blocks = (words + 255) / 256;
+  if (blocks > 65535) blocks = 65535;
+  if (scale_dtype == KRM_F16)
+    dequant_i4_kernel<__half><<<dim3((unsigned)blocks), dim3(256), 0, ctx->stream>>>(
+        ptr<const uint32_t>(w), ptr<const __half>(scales), ptr<float>(out_f32), words, width,
+        group);
+  else
+    dequant_i4_kernel<float><<<dim3((unsigned)blocks), dim3(256), 0, ctx->stream>>>(
+        ptr<const uint32_t>(w), ptr<const float>(scales), ptr<float>(out_f32), words, width,
+        group);
+  return launched(ctx, "dequant_i4_kernel");
+}
+
+}  // extern "C"

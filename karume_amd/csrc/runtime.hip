@@ -1,0 +1,213 @@
+// Context, buffers, events and error plumbing of libkarume_hip.so.
+//
+// Replaces, for the ops this library serves, what the reference does through WebGPU:
+// acquireGpu / GpuContext (packages/runtime/src/gpu/device.ts), createBuffer +
+// queue.writeBuffer + readback (packages/runtime/src/runtime/executor.ts:870-896,1272) and the
+// opt-in timestamp diagnostics (packages/runtime/src/gpu/submit.ts:54-63).
+#include "krm_internal.h"
+
+namespace {
+thread_local char g_error[512] = "";
+}
+
+namespace krm {
+
+int32_t fail(krm_ctx* ctx, int32_t code, const char* fmt, ...) {
+  char* dst = ctx ? ctx->error : g_error;
+  va_list args;
+  va_start(args, fmt);
+  vsnprintf(dst, 512, fmt, args);
+  va_end(args);
+  return code;
+}
+
+int32_t hip_status(krm_ctx* ctx, hipError_t status, const char* what) {
+  if (status == hipSuccess) return KRM_OK;
+  const int32_t code =
+      status == hipErrorOutOfMemory || status == hipErrorMemoryAllocation
+          ? KRM_ERR_OUT_OF_MEMORY
+          : (status == hipErrorInvalidValue || status == hipErrorInvalidDevice ||
+                     status == hipErrorInvalidDevicePointer
+                 ? KRM_ERR_VALIDATION
+                 : KRM_ERR_DEVICE_LOST);
+  return fail(ctx, code, "%s: %s (%s)", what, hipGetErrorString(status),
+              hipGetErrorName(status));
+}
+
+int32_t enter(krm_ctx* ctx) {
+  if (!ctx) return fail(nullptr, KRM_ERR_VALIDATION, "context is NULL");
+  return hip_status(ctx, hipSetDevice(ctx->device), "hipSetDevice");
+}
+
+int32_t launched(krm_ctx* ctx, const char* kernel) {
+  return hip_status(ctx, hipGetLastError(), kernel);
+}
+
+}  // namespace krm
+
+using namespace krm;
+
+extern "C" {
+
+const char* krm_version(void) { return "karume-hip 0.1 gfx950"; }
+
+int32_t krm_ctx_create_on_stream(int32_t device, void* hip_stream, krm_ctx** out) {
+  if (!out) return fail(nullptr, KRM_ERR_VALIDATION, "krm_ctx_create: out is NULL");
+  *out = nullptr;
+  int count = 0;
+  KRM_TRY(hip_status(nullptr, hipGetDeviceCount(&count), "hipGetDeviceCount"));
+  if (device < 0 || device >= count)
+    return fail(nullptr, KRM_ERR_VALIDATION, "krm_ctx_create: device %d of %d", device, count);
+  KRM_TRY(hip_status(nullptr, hipSetDevice(device), "hipSetDevice"));
+  hipDeviceProp_t prop;
+  KRM_TRY(hip_status(nullptr, hipGetDeviceProperties(&prop, device), "hipGetDeviceProperties"));
+  if (strncmp(prop.gcnArchName, "gfx950", 6) != 0)
+    return fail(nullptr, KRM_ERR_VALIDATION,
+                "krm_ctx_create: device %d is %s; this library only carries gfx950 code", device,
+                prop.gcnArchName);
+  krm_ctx* ctx = new krm_ctx();
+  ctx->device = device;
+  ctx->num_cus = prop.multiProcessorCount;
+  ctx->stream = static_cast<hipStream_t>(hip_stream);
+  ctx->owns_stream = false;
+  ctx->pinned_bytes = 1 << 20;
+  hipError_t st = hipHostMalloc(&ctx->pinned, ctx->pinned_bytes, hipHostMallocDefault);
+  if (st != hipSuccess) {
+    delete ctx;
+    return hip_status(nullptr, st, "hipHostMalloc");
+  }
+  *out = ctx;
+  return KRM_OK;
+}
+
+int32_t krm_ctx_create(int32_t device, krm_ctx** out) {
+  KRM_TRY(krm_ctx_create_on_stream(device, nullptr, out));
+  krm_ctx* ctx = *out;
+  // Default priority on purpose: mixed stream priorities are not used anywhere.
+  hipError_t st = hipStreamCreateWithFlags(&ctx->stream, hipStreamNonBlocking);
+  if (st != hipSuccess) {
+    (void)hipHostFree(ctx->pinned);
+    delete ctx;
+    *out = nullptr;
+    return hip_status(nullptr, st, "hipStreamCreateWithFlags");
+  }
+  ctx->owns_stream = true;
+  return KRM_OK;
+}
+
+int32_t krm_ctx_destroy(krm_ctx* ctx) {
+  if (!ctx) return KRM_OK;
+  (void)hipSetDevice(ctx->device);
+  (void)hipStreamSynchronize(ctx->stream);
+  if (ctx->owns_stream) (void)hipStreamDestroy(ctx->stream);
+  if (ctx->pinned) (void)hipHostFree(ctx->pinned);
+  delete ctx;
+  return KRM_OK;
+}
+
+const char* krm_last_error(krm_ctx* ctx) { return ctx ? ctx->error : g_error; }
+
+int32_t krm_sync(krm_ctx* ctx) {
+  KRM_TRY(enter(ctx));
+  return hip_status(ctx, hipStreamSynchronize(ctx->stream), "hipStreamSynchronize");
+}
+
+int32_t krm_buf_alloc(krm_ctx* ctx, size_t bytes, krm_buf* out) {
+  KRM_TRY(enter(ctx));
+  KRM_REQUIRE(ctx, out != nullptr, "krm_buf_alloc: out is NULL");
+  void* p = nullptr;
+  // A zero-byte request still returns a distinct, freeable address.
+  KRM_TRY(hip_status(ctx, hipMalloc(&p, bytes ? bytes : 16), "hipMalloc"));
+  *out = static_cast<krm_buf>(reinterpret_cast<uintptr_t>(p));
+  return KRM_OK;
+}
+
+int32_t krm_buf_free(krm_ctx* ctx, krm_buf buf) {
+  KRM_TRY(enter(ctx));
+  if (!buf) return KRM_OK;
+  // Work queued on the stream may still use the buffer ("flush before destroy").
+  KRM_TRY(hip_status(ctx, hipStreamSynchronize(ctx->stream), "hipStreamSynchronize"));
+  return hip_status(ctx, hipFree(ptr<void>(buf)), "hipFree");
+}
+
+int32_t krm_buf_upload(krm_ctx* ctx, krm_buf dst, size_t dst_offset, const void* host,
+                       size_t bytes) {
+  KRM_TRY(enter(ctx));
+  if (bytes == 0) return KRM_OK;
+  KRM_REQUIRE(ctx, dst != 0 && host != nullptr, "krm_buf_upload: NULL buffer");
+  // The host array is only valid during the call, so the copy completes before returning.
+  KRM_TRY(hip_status(ctx,
+                     hipMemcpyAsync(ptr<char>(dst) + dst_offset, host, bytes,
+                                    hipMemcpyHostToDevice, ctx->stream),
+                     "hipMemcpyAsync(H2D)"));
+  return hip_status(ctx, hipStreamSynchronize(ctx->stream), "hipStreamSynchronize");
+}
+
+int32_t krm_buf_download(krm_ctx* ctx, krm_buf src, size_t src_offset, void* host,
+                         size_t bytes) {
+  KRM_TRY(enter(ctx));
+  if (bytes == 0) return hip_status(ctx, hipStreamSynchronize(ctx->stream), "sync");
+  KRM_REQUIRE(ctx, src != 0 && host != nullptr, "krm_buf_download: NULL buffer");
+  KRM_TRY(hip_status(ctx,
+                     hipMemcpyAsync(host, ptr<char>(src) + src_offset, bytes,
+                                    hipMemcpyDeviceToHost, ctx->stream),
+                     "hipMemcpyAsync(D2H)"));
+  return hip_status(ctx, hipStreamSynchronize(ctx->stream), "hipStreamSynchronize");
+}
+
+__global__ void krm_zero_kernel(uint32_t* __restrict__ dst, size_t words) {
+  size_t i = blockIdx.x * (size_t)blockDim.x + threadIdx.x;
+  const size_t stride = (size_t)gridDim.x * blockDim.x;
+  for (; i < words; i += stride) dst[i] = 0u;
+}
+
+int32_t krm_buf_zero(krm_ctx* ctx, krm_buf dst, size_t dst_offset, size_t bytes) {
+  KRM_TRY(enter(ctx));
+  if (bytes == 0) return KRM_OK;
+  KRM_REQUIRE(ctx, dst != 0, "krm_buf_zero: NULL buffer");
+  KRM_REQUIRE(ctx, (dst + dst_offset) % 4 == 0 && bytes % 4 == 0,
+              "krm_buf_zero: address and size must be multiples of 4 bytes");
+  // A fill kernel rather than a memset node, so the call stays safe under graph capture.
+  const size_t words = bytes / 4;
+  size_t blocks = (words + 255) / 256;
+  if (blocks > 4096) blocks = 4096;
+  krm_zero_kernel<<<dim3((unsigned)blocks), dim3(256), 0, ctx->stream>>>(
+      ptr<uint32_t>(dst + dst_offset), words);
+  return launched(ctx, "krm_zero_kernel");
+}
+
+int32_t krm_event_create(krm_ctx* ctx, krm_event** out) {
+  KRM_TRY(enter(ctx));
+  KRM_REQUIRE(ctx, out != nullptr, "krm_event_create: out is NULL");
+  krm_event* ev = new krm_event();
+  hipError_t st = hipEventCreate(&ev->ev);
+  if (st != hipSuccess) {
+    delete ev;
+    return hip_status(ctx, st, "hipEventCreate");
+  }
+  *out = ev;
+  return KRM_OK;
+}
+
+int32_t krm_event_record(krm_ctx* ctx, krm_event* ev) {
+  KRM_TRY(enter(ctx));
+  KRM_REQUIRE(ctx, ev != nullptr, "krm_event_record: event is NULL");
+  return hip_status(ctx, hipEventRecord(ev->ev, ctx->stream), "hipEventRecord");
+}
+
+int32_t krm_event_elapsed_ms(krm_ctx* ctx, krm_event* start, krm_event* stop, float* ms) {
+  KRM_TRY(enter(ctx));
+  KRM_REQUIRE(ctx, start && stop && ms, "krm_event_elapsed_ms: NULL argument");
+  KRM_TRY(hip_status(ctx, hipEventSynchronize(stop->ev), "hipEventSynchronize"));
+  return hip_status(ctx, hipEventElapsedTime(ms, start->ev, stop->ev), "hipEventElapsedTime");
+}
+
+int32_t krm_event_destroy(krm_ctx* ctx, krm_event* ev) {
+  KRM_TRY(enter(ctx));
+  if (!ev) return KRM_OK;
+  hipError_t st = hipEventDestroy(ev->ev);
+  delete ev;
+  return hip_status(ctx, st, "hipEventDestroy");
+}
+
+}  // extern "C"

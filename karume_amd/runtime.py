@@ -1,0 +1,270 @@
+"""Host-side mirror of the reference's device layer for the ops this backend serves.
+
+``acquire_gpu`` / ``GpuContext`` stand where the reference has ``acquireGpu`` / ``GpuContext``
+(packages/runtime/mod.ts:13-113, packages/runtime/src/gpu/device.ts); the error classes are the
+reference's public ones (packages/runtime/mod.ts:25-35,112).  Everything below is plumbing
+around the C ABI: no arithmetic happens in Python.
+"""
+from __future__ import annotations
+
+import ctypes as C
+from typing import Optional, Sequence, Union
+
+import numpy as np
+
+from . import _ffi
+
+F32 = 0
+F16 = 1
+COMPUTE_F32 = 0
+COMPUTE_F16 = 1
+
+_NP_DTYPE_CODE = {np.dtype(np.float32): F32, np.dtype(np.float16): F16}
+
+
+class KarumeError(RuntimeError):
+    """Base of the errors raised by this backend."""
+
+
+class GpuValidationError(KarumeError):
+    """Shapes, attributes or alignment rejected before launch (status -1)."""
+
+
+class GpuOutOfMemoryError(KarumeError):
+    """Device allocation failed (status -2)."""
+
+
+class GpuDeviceLostError(KarumeError):
+    """The HIP runtime reported a failure; the context should be discarded (status -3)."""
+
+
+class ExecutionError(KarumeError):
+    """A run violated its contract, e.g. pastLength + queryLength > capacity (status -4)."""
+
+
+_ERRORS = {-1: GpuValidationError, -2: GpuOutOfMemoryError, -3: GpuDeviceLostError,
+           -4: ExecutionError}
+
+
+def dtype_code(dtype) -> int:
+    """KRM_F32 / KRM_F16 for a NumPy dtype."""
+    try:
+        return _NP_DTYPE_CODE[np.dtype(dtype)]
+    except KeyError as exc:
+        raise GpuValidationError(f"unsupported element type {dtype}") from exc
+
+
+class DeviceBuffer:
+    """A device allocation (or a borrowed device address) of ``nbytes`` bytes."""
+
+    def __init__(self, ctx: "GpuContext", address: int, nbytes: int, owned: bool):
+        self.ctx = ctx
+        self.address = int(address)
+        self.nbytes = int(nbytes)
+        self._owned = owned
+
+    def __int__(self) -> int:
+        return self.address
+
+    def offset(self, byte_offset: int) -> int:
+        if byte_offset < 0 or byte_offset > self.nbytes:
+            raise GpuValidationError(f"offset {byte_offset} outside a {self.nbytes}-byte buffer")
+        return self.address + byte_offset
+
+    def upload(self, array: np.ndarray, byte_offset: int = 0) -> None:
+        data = np.ascontiguousarray(array)
+        if byte_offset + data.nbytes > self.nbytes:
+            raise GpuValidationError("upload past the end of the buffer")
+        self.ctx._check(self.ctx._lib.krm_buf_upload(
+            self.ctx._handle, self.address, byte_offset, data.ctypes.data, data.nbytes))
+
+    def download(self, dtype, shape: Sequence[int], byte_offset: int = 0) -> np.ndarray:
+        out = np.empty(tuple(shape), dtype=dtype)
+        if byte_offset + out.nbytes > self.nbytes:
+            raise GpuValidationError("download past the end of the buffer")
+        self.ctx._check(self.ctx._lib.krm_buf_download(
+            self.ctx._handle, self.address, byte_offset, out.ctypes.data, out.nbytes))
+        return out
+
+    def zero(self) -> None:
+        self.ctx._check(self.ctx._lib.krm_buf_zero(self.ctx._handle, self.address, 0,
+                                                    self.nbytes - self.nbytes % 4))
+
+    def free(self) -> None:
+        if self._owned and self.address:
+            self.ctx._check(self.ctx._lib.krm_buf_free(self.ctx._handle, self.address))
+        self.address = 0
+        self._owned = False
+
+
+BufferLike = Union[DeviceBuffer, int, None]
+
+
+def _addr(buf: BufferLike) -> int:
+    if buf is None:
+        return 0
+    return int(buf)
+
+
+class GpuEvent:
+    def __init__(self, ctx: "GpuContext"):
+        self.ctx = ctx
+        handle = C.c_void_p()
+        ctx._check(ctx._lib.krm_event_create(ctx._handle, C.byref(handle)))
+        self._handle = handle
+
+    def record(self) -> None:
+        self.ctx._check(self.ctx._lib.krm_event_record(self.ctx._handle, self._handle))
+
+    def elapsed_ms(self, stop: "GpuEvent") -> float:
+        ms = C.c_float()
+        self.ctx._check(self.ctx._lib.krm_event_elapsed_ms(
+            self.ctx._handle, self._handle, stop._handle, C.byref(ms)))
+        return float(ms.value)
+
+    def destroy(self) -> None:
+        if self._handle:
+            self.ctx._lib.krm_event_destroy(self.ctx._handle, self._handle)
+            self._handle = None
+
+
+class GpuContext:
+    """One device + one stream; every op of this backend is queued through it."""
+
+    def __init__(self, device: int = 0, stream: Optional[int] = None):
+        self._lib = _ffi.load()
+        handle = C.c_void_p()
+        if stream is None:
+            status = self._lib.krm_ctx_create(device, C.byref(handle))
+        else:
+            status = self._lib.krm_ctx_create_on_stream(device, C.c_void_p(stream), C.byref(handle))
+        if status != 0:
+            message = self._lib.krm_last_error(None).decode("utf-8", "replace")
+            raise _ERRORS.get(status, KarumeError)(message)
+        self._handle = handle
+        self.device = device
+        self._buffers: list[DeviceBuffer] = []
+
+    # -- lifecycle -------------------------------------------------------------------------
+    def destroy(self) -> None:
+        if self._handle:
+            for buf in self._buffers:
+                buf.free()
+            self._buffers.clear()
+            self._lib.krm_ctx_destroy(self._handle)
+            self._handle = None
+
+    def __enter__(self) -> "GpuContext":
+        return self
+
+    def __exit__(self, *exc) -> None:
+        self.destroy()
+
+    def _check(self, status: int) -> None:
+        if status != 0:
+            message = self._lib.krm_last_error(self._handle).decode("utf-8", "replace")
+            raise _ERRORS.get(status, KarumeError)(message)
+
+    def sync(self) -> None:
+        self._check(self._lib.krm_sync(self._handle))
+
+    def event(self) -> GpuEvent:
+        return GpuEvent(self)
+
+    # -- buffers ---------------------------------------------------------------------------
+    def alloc(self, nbytes: int) -> DeviceBuffer:
+        address = C.c_uint64()
+        self._check(self._lib.krm_buf_alloc(self._handle, nbytes, C.byref(address)))
+        buf = DeviceBuffer(self, address.value, nbytes, owned=True)
+        self._buffers.append(buf)
+        return buf
+
+    def upload(self, array: np.ndarray) -> DeviceBuffer:
+        data = np.ascontiguousarray(array)
+        buf = self.alloc(max(data.nbytes, 16))
+        if data.nbytes:
+            buf.upload(data)
+        return buf
+
+    def zeros(self, nbytes: int) -> DeviceBuffer:
+        buf = self.alloc((nbytes + 3) // 4 * 4)
+        buf.zero()
+        return buf
+
+    def borrow(self, address: int, nbytes: int) -> DeviceBuffer:
+        """Wrap device memory owned by someone else (for example a torch tensor's data_ptr)."""
+        return DeviceBuffer(self, address, nbytes, owned=False)
+
+    # -- ops (argument order = the C ABI's) ---------------------------------------------------
+    def dequant_i4(self, w: BufferLike, scales: BufferLike, out_f32: BufferLike, rows: int,
+                   width: int, group: int, scale_dtype: int = F32) -> None:
+        self._check(self._lib.krm_dequant_i4(self._handle, _addr(w), _addr(scales),
+                                             _addr(out_f32), rows, width, group, scale_dtype))
+
+    def linear_i4(self, x: BufferLike, w: BufferLike, scales: BufferLike, bias: BufferLike,
+                  out: BufferLike, m: int, n: int, k: int, group: int, io_dtype: int = F32,
+                  scale_dtype: int = F32, compute: int = COMPUTE_F32) -> None:
+        self._check(self._lib.krm_linear_i4(self._handle, _addr(x), _addr(w), _addr(scales),
+                                            _addr(bias), _addr(out), m, n, k, group, io_dtype,
+                                            scale_dtype, compute))
+
+    def attention_state_workspace(self, batch: int, heads: int, kv_heads: int, chunk_rows: int,
+                                  depth: int, window: int, max_past: int, max_query: int = 1
+                                  ) -> int:
+        nbytes = C.c_size_t()
+        self._check(self._lib.krm_attention_state_workspace(
+            batch, heads, kv_heads, chunk_rows, depth, window, max_past, max_query,
+            C.byref(nbytes)))
+        return int(nbytes.value)
+
+    def attention_state(self, q: BufferLike, ins_k: BufferLike, ins_v: BufferLike,
+                        slot_k: BufferLike, slot_v: BufferLike, out: BufferLike, *, batch: int,
+                        heads: int, kv_heads: int, chunk_rows: int, depth: int, capacity: int,
+                        window: int, half_scale: float, past: int, query: int,
+                        io_dtype: int = F32, kv_dtype: int = F32,
+                        workspace: BufferLike = None, workspace_bytes: int = 0) -> None:
+        if isinstance(workspace, DeviceBuffer) and not workspace_bytes:
+            workspace_bytes = workspace.nbytes
+        self._check(self._lib.krm_attention_state(
+            self._handle, _addr(q), _addr(ins_k), _addr(ins_v), _addr(slot_k), _addr(slot_v),
+            _addr(out), batch, heads, kv_heads, chunk_rows, depth, capacity, window,
+            float(half_scale), past, query, io_dtype, kv_dtype, _addr(workspace),
+            workspace_bytes))
+
+    def state_append(self, x: BufferLike, slot: BufferLike, *, kv_planes: int, chunk_rows: int,
+                     depth: int, capacity: int, window: int, past: int, query: int,
+                     x_dtype: int = F32, slot_dtype: int = F32) -> None:
+        self._check(self._lib.krm_state_append(
+            self._handle, _addr(x), _addr(slot), kv_planes, chunk_rows, depth, capacity, window,
+            past, query, x_dtype, slot_dtype))
+
+    def attention_varlen_workspace(self, nseq: int, heads: int, kv_heads: int, depth: int,
+                                   total_rows: int) -> int:
+        nbytes = C.c_size_t()
+        self._check(self._lib.krm_attention_varlen_workspace(
+            nseq, heads, kv_heads, depth, total_rows, C.byref(nbytes)))
+        return int(nbytes.value)
+
+    def attention_varlen(self, q: BufferLike, ins_k: BufferLike, ins_v: BufferLike,
+                         slot_k: BufferLike, slot_v: BufferLike, out: BufferLike,
+                         cu_seqlens: Sequence[int], *, heads: int, kv_heads: int, depth: int,
+                         total_rows: int, half_scale: float, io_dtype: int = F32,
+                         kv_dtype: int = F32, workspace: BufferLike = None,
+                         workspace_bytes: int = 0) -> None:
+        cu = np.ascontiguousarray(cu_seqlens, dtype=np.int32)
+        if isinstance(workspace, DeviceBuffer) and not workspace_bytes:
+            workspace_bytes = workspace.nbytes
+        self._check(self._lib.krm_attention_varlen(
+            self._handle, _addr(q), _addr(ins_k), _addr(ins_v), _addr(slot_k), _addr(slot_v),
+            _addr(out), cu.ctypes.data_as(C.POINTER(C.c_int32)), cu.size - 1, heads, kv_heads,
+            depth, total_rows, float(half_scale), io_dtype, kv_dtype, _addr(workspace),
+            workspace_bytes))
+
+
+def acquire_gpu(device: int = 0, stream: Optional[int] = None) -> GpuContext:
+    """Create a context on ``device`` (optionally on an existing hipStream_t handle)."""
+    return GpuContext(device, stream)
+
+
+def version() -> str:
+    return _ffi.load().krm_version().decode()

@@ -1,0 +1,370 @@
+"""GPU parity of states-form attention, state_append and the ragged decode batch (through the
+C ABI) against the CPU oracle."""
+import numpy as np
+import pytest
+
+import helpers
+import karume_amd as ka
+from helpers import PARITY_CASES, StateCase, make_state_inputs, oracle, oracle_state_attention
+
+pytestmark = pytest.mark.gpu
+
+# The reference's own gate for this op: atol 5e-6, rtol 0, outputs O(1)
+# (packages/runtime/tests/gpu_state_attention_test.ts:41-54; its measured worst is 6.6e-7).
+STATE_ATOL = 5e-6
+
+
+def run_attention(ctx, case: StateCase, x: dict, io=np.float32, kv=np.float32, scale=None,
+                  workspace_bytes=None):
+    bufs = {k: ctx.upload(np.ascontiguousarray(v, dtype=io if k in ("q", "ins_k", "ins_v") else kv))
+            for k, v in x.items()}
+    out_elems = case.batch * case.heads * case.chunk_rows * case.depth
+    out = ctx.upload(np.full(out_elems, 123.0, dtype=io))  # every element must be overwritten
+    ws_bytes = ctx.attention_state_workspace(case.batch, case.heads, case.kv_heads,
+                                             case.chunk_rows, case.depth, case.window,
+                                             min(case.past, 1 << 20), case.query)
+    if workspace_bytes is not None:
+        ws_bytes = workspace_bytes
+    ws = ctx.alloc(max(ws_bytes, 16))
+    ctx.attention_state(
+        bufs["q"], bufs["ins_k"], bufs["ins_v"], bufs["slot_k"], bufs["slot_v"], out,
+        half_scale=oracle.half_scale(case.depth) if scale is None else scale,
+        io_dtype=ka.dtype_code(io), kv_dtype=ka.dtype_code(kv), workspace=ws,
+        workspace_bytes=ws_bytes, **case.kwargs())
+    got = out.download(io, (case.batch, case.heads, case.chunk_rows, case.depth))
+    for b in list(bufs.values()) + [out, ws]:
+        b.free()
+    return got
+
+
+@pytest.mark.parametrize("case", PARITY_CASES, ids=lambda c: c.name)
+def test_parity_grid(gpu_ctx, case):
+    """The reference's 17-case grid with poison in every place that must not be read
+    (gpu_state_attention_test.ts:119-347): atol 5e-6 rtol 0, pad rows exact +0."""
+    x = make_state_inputs(case)
+    want = oracle_state_attention(case, x)
+    got = run_attention(gpu_ctx, case, x)
+    ok, fails, max_abs, worst = oracle.allclose(got, want, atol=STATE_ATOL, rtol=0)
+    assert ok, (fails, max_abs, worst)
+    pad = got[:, :, case.query:, :]
+    assert np.all(pad == 0.0) and not np.any(np.signbit(pad))
+
+
+DECODE_CASES = [
+    StateCase("decode r4 D128 P300", 1, 8, 2, 1, 128, 512, 0, 300, 1),
+    StateCase("decode r4 D128 P127 one split", 2, 8, 2, 1, 128, 128, 0, 127, 1),
+    StateCase("decode r4 D128 P128 boundary", 1, 8, 2, 1, 128, 256, 0, 128, 1),
+    StateCase("decode r8 D64 P383", 1, 32, 4, 1, 64, 512, 0, 383, 1),
+    StateCase("decode r1 D64 P0", 1, 4, 4, 1, 64, 16, 0, 0, 1),
+    StateCase("decode r2 D32 B3 P77", 3, 4, 2, 1, 32, 96, 0, 77, 1),
+    StateCase("decode sliding W100 P1000 C128", 1, 8, 2, 1, 128, 128, 100, 1000, 1),
+    StateCase("decode sliding W300 P299", 1, 8, 2, 1, 64, 300, 300, 299, 1),
+    StateCase("decode sliding W256 P5000", 2, 8, 8, 1, 64, 256, 256, 5000, 1),
+]
+
+
+def random_state_inputs(case: StateCase, seed: int, f16_values: bool):
+    rng = np.random.default_rng(seed)
+    b, h, hkv, m, d, c = (case.batch, case.heads, case.kv_heads, case.chunk_rows, case.depth,
+                          case.capacity)
+    x = dict(q=rng.normal(size=(b, h, m, d)), ins_k=rng.normal(size=(b, hkv, m, d)),
+             ins_v=rng.normal(size=(b, hkv, m, d)), slot_k=rng.normal(size=(b, hkv, c, d)),
+             slot_v=rng.normal(size=(b, hkv, c, d)))
+    cast = (lambda a: a.astype(np.float16).astype(np.float32)) if f16_values else \
+        (lambda a: a.astype(np.float32))
+    x = {k: cast(v) for k, v in x.items()}
+    # poison what must not be read: non-resident slot rows
+    base = oracle.state_column_base(case.window, case.past)
+    resident = {col % case.window if case.window else col for col in range(base, case.past)}
+    for row in range(c):
+        if row not in resident:
+            x["slot_k"][:, :, row] = 9.0
+            x["slot_v"][:, :, row] = 400.0
+    return x
+
+
+@pytest.mark.parametrize("case", DECODE_CASES, ids=lambda c: c.name)
+@pytest.mark.parametrize("io,kv", [(np.float32, np.float32), (np.float16, np.float16),
+                                   (np.float32, np.float16)])
+def test_decode_split_k(gpu_ctx, case, io, kv):
+    """The split-K decode path (Q = 1, M = 1) over one or several splits, full and sliding.
+    f32 output: atol 5e-6 rtol 0 (the reference's gate).  fp16 output: the oracle's value
+    rounded to fp16, +-1 fp16 ulp."""
+    x = random_state_inputs(case, seed=case.past + case.depth, f16_values=True)
+    want = oracle_state_attention(case, x)
+    got = run_attention(gpu_ctx, case, x, io=io, kv=kv)
+    if io == np.float32:
+        ok, fails, max_abs, worst = oracle.allclose(got, want, atol=STATE_ATOL, rtol=0)
+        assert ok, (fails, max_abs, worst)
+    else:
+        want16 = want.astype(np.float16)
+        ulp = np.abs(np.nextafter(want16, np.float16(np.inf)).astype(np.float32)
+                     - want16.astype(np.float32))
+        err = np.abs(got.astype(np.float32) - want16.astype(np.float32))
+        assert np.all(err <= ulp), float(np.max(err))
+
+
+def test_config2_decode_attention(gpu_ctx):
+    """BASELINE config 2: B=1, H=32, Hkv=8, D=128, 4095 slot rows + this step's row, fp16."""
+    case = StateCase("config 2", 1, 32, 8, 1, 128, 4096, 0, 4095, 1)
+    x = random_state_inputs(case, seed=2, f16_values=True)
+    want = oracle_state_attention(case, x)
+    got32 = run_attention(gpu_ctx, case, x, io=np.float32, kv=np.float16)
+    ok, fails, max_abs, worst = oracle.allclose(got32, want, atol=STATE_ATOL, rtol=0)
+    assert ok, (fails, max_abs, worst)
+    got16 = run_attention(gpu_ctx, case, x, io=np.float16, kv=np.float16)
+    want16 = want.astype(np.float16).astype(np.float32)
+    assert np.max(np.abs(got16.astype(np.float32) - want16)) <= 2.5e-4  # 1 ulp at |out| < 0.25
+    # identical bits for a larger capacity: the work never depends on C
+    big = StateCase("config 2 C8192", 1, 32, 8, 1, 128, 8192, 0, 4095, 1)
+    xb = {k: v.copy() for k, v in x.items()}
+    for name in ("slot_k", "slot_v"):
+        grown = np.full((1, 8, 8192, 128), 9.0 if name == "slot_k" else 400.0, dtype=np.float32)
+        grown[:, :, :4096] = x[name]
+        xb[name] = grown
+    got_big = run_attention(gpu_ctx, big, xb, io=np.float32, kv=np.float16)
+    assert np.array_equal(got_big.view(np.uint32), got32.view(np.uint32))
+
+
+def test_mutations_would_be_caught(gpu_ctx):
+    """The GPU result sits within tolerance of the faithful oracle and far from every mutated
+    oracle on that mutation's witness case."""
+    witnesses = {
+        oracle.MUT_DROP_LOWER_BOUND: "sliding W4 P10 wrap",
+        oracle.MUT_RING_MOD_CAPACITY: "sliding W4 C8 wrap",
+        oracle.MUT_PAD_ROWS_COMPUTED: "full r2 pad B2 D6",
+        oracle.MUT_IGNORE_KV_REPEAT: "full r2 pad B2 D6",
+        oracle.MUT_SCALE_ONE_SIDE: "full r1 prefill B2",
+        oracle.MUT_OVERFLOW_FORM: "sliding W2 P near u32 max",
+    }
+    for mutation, name in witnesses.items():
+        case = next(c for c in PARITY_CASES if c.name == name)
+        x = make_state_inputs(case)
+        got = run_attention(gpu_ctx, case, x)
+        bad = oracle_state_attention(case, x, mutation=mutation)
+        assert np.max(np.abs(got - bad)) > 1e-3, name
+
+
+def test_attention_rejections(gpu_ctx):
+    buf = gpu_ctx.zeros(1 << 16)
+    base = dict(batch=1, heads=4, kv_heads=2, chunk_rows=2, depth=8, capacity=8, window=0,
+                half_scale=0.5, past=0, query=1)
+    call = lambda **kw: gpu_ctx.attention_state(buf, buf, buf, buf, buf, buf,  # noqa: E731
+                                                **{**base, **kw})
+    with pytest.raises(ka.GpuValidationError):
+        call(heads=3)
+    with pytest.raises(ka.GpuValidationError):
+        call(window=9)
+    with pytest.raises(ka.ExecutionError):  # capacity overflow is rejected before launch
+        call(past=7, query=2)
+    with pytest.raises(ka.ExecutionError):
+        call(query=3)
+    with pytest.raises(ka.ExecutionError):
+        call(query=0)
+    with pytest.raises(ka.GpuValidationError):
+        call(half_scale=float("nan"))
+    # split-K needs a workspace when there is more than one split
+    big = dict(batch=1, heads=8, kv_heads=2, chunk_rows=1, depth=128, capacity=4096, window=0,
+               half_scale=0.3, past=4000, query=1, io_dtype=ka.F16, kv_dtype=ka.F16)
+    huge = gpu_ctx.zeros(2 * 4096 * 128 * 2)
+    with pytest.raises(ka.GpuValidationError):
+        gpu_ctx.attention_state(buf, buf, buf, huge, huge, buf, **big)
+    huge.free()
+    buf.free()
+
+
+# ---------------------------------------------------------------------------- state_append
+
+def run_append(ctx, x, slot, xd=np.float32, sd=np.float32, **spec):
+    dx = ctx.upload(np.ascontiguousarray(x, dtype=xd))
+    ds = ctx.upload(np.ascontiguousarray(slot, dtype=sd))
+    ctx.state_append(dx, ds, x_dtype=ka.dtype_code(xd), slot_dtype=ka.dtype_code(sd), **spec)
+    got = ds.download(sd, np.shape(slot))
+    dx.free()
+    ds.free()
+    return got
+
+
+def test_append_reference_vectors(gpu_ctx):
+    # packages/runtime/tests/kernel_state_attention_test.ts:481-503
+    spec = dict(kv_planes=1, chunk_rows=4, depth=1, capacity=4, window=4)
+    slot = np.array([-1, -2, -3, -4], dtype=np.float32)
+    x = np.array([100, 200, 300, 400], dtype=np.float32)
+    assert run_append(gpu_ctx, x, slot, past=2, query=2, **spec).tolist() == [-1, -2, 100, 200]
+    assert run_append(gpu_ctx, x, slot, past=3, query=3, **spec).tolist() == [200, 300, -3, 100]
+    collide = run_append(gpu_ctx, x, np.array([-1, -2], dtype=np.float32), kv_planes=1,
+                         chunk_rows=4, depth=1, capacity=2, window=2, past=0, query=4)
+    assert collide.tolist() == [300, 400]
+
+
+@pytest.mark.parametrize("window,capacity,past,query,m", [(0, 64, 5, 7, 9), (6, 6, 13, 3, 5),
+                                                          (4, 8, 9, 2, 3), (2, 2, 5, 4, 4),
+                                                          (0, 40, 39, 1, 1)])
+def test_append_matches_oracle_bytes(gpu_ctx, window, capacity, past, query, m):
+    rng = np.random.default_rng(past)
+    planes, d = 6, 16
+    x = rng.normal(size=(planes, m, d)).astype(np.float32)
+    x[:, query:] = 9.0  # pad rows must never reach the slot
+    slot = rng.normal(size=(planes, capacity, d)).astype(np.float32)
+    spec = dict(kv_planes=planes, chunk_rows=m, depth=d, capacity=capacity, window=window,
+                past=past, query=query)
+    want = oracle.state_append(x, slot, **spec)
+    got = run_append(gpu_ctx, x, slot, **spec)
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+    # f32 -> f16 slot: round to nearest even of the same values
+    got16 = run_append(gpu_ctx, x, slot.astype(np.float16), sd=np.float16, **spec)
+    want16 = oracle.state_append(x.astype(np.float16).astype(np.float32),
+                                 slot.astype(np.float16).astype(np.float32), **spec)
+    assert np.array_equal(got16, want16.astype(np.float16))
+
+
+def test_append_rejections(gpu_ctx):
+    buf = gpu_ctx.zeros(4096)
+    spec = dict(kv_planes=1, chunk_rows=2, depth=4, capacity=4, window=0, past=0, query=1)
+    with pytest.raises(ka.ExecutionError):
+        gpu_ctx.state_append(buf, buf, **{**spec, "past": 3, "query": 2})
+    with pytest.raises(ka.ExecutionError):
+        gpu_ctx.state_append(buf, buf, **{**spec, "query": 3})
+    with pytest.raises(ka.GpuValidationError):
+        gpu_ctx.state_append(buf, buf, **{**spec, "window": 5})
+    buf.free()
+
+
+def test_chain_prefill_then_decode_on_device(gpu_ctx):
+    """Prefill -> decode chain with slots that live on the device and start as zeros
+    (packages/runtime/tests/gpu_state_execution_test.ts:152-212,268-350): readers first, then
+    append; equals ONE full-history causal attention in float64."""
+    heads, kv_heads, depth, capacity = 8, 2, 64, 64
+    r = heads // kv_heads
+    rng = np.random.default_rng(77)
+    slot_k = gpu_ctx.zeros(kv_heads * capacity * depth * 4)
+    slot_v = gpu_ctx.zeros(kv_heads * capacity * depth * 4)
+    ws = gpu_ctx.alloc(gpu_ctx.attention_state_workspace(1, heads, kv_heads, 8, depth, 0, capacity))
+    past = 0
+    outs, qs, ks, vs = [], [], [], []
+    for m, query in [(8, 8), (8, 3)] + [(1, 1)] * 20:
+        q = rng.normal(size=(1, heads, m, depth)).astype(np.float32)
+        k = rng.normal(size=(1, kv_heads, m, depth)).astype(np.float32)
+        v = rng.normal(size=(1, kv_heads, m, depth)).astype(np.float32)
+        k[:, :, query:] = 9.0
+        v[:, :, query:] = 400.0
+        dq, dk, dv = gpu_ctx.upload(q), gpu_ctx.upload(k), gpu_ctx.upload(v)
+        out = gpu_ctx.alloc(q.nbytes)
+        gpu_ctx.attention_state(dq, dk, dv, slot_k, slot_v, out, batch=1, heads=heads,
+                                kv_heads=kv_heads, chunk_rows=m, depth=depth, capacity=capacity,
+                                window=0, half_scale=oracle.half_scale(depth), past=past,
+                                query=query, workspace=ws)
+        spec = dict(kv_planes=kv_heads, chunk_rows=m, depth=depth, capacity=capacity, window=0,
+                    past=past, query=query)
+        gpu_ctx.state_append(dk, slot_k, **spec)
+        gpu_ctx.state_append(dv, slot_v, **spec)
+        outs.append(out.download(np.float32, q.shape)[:, :, :query])
+        qs.append(q[:, :, :query])
+        ks.append(k[:, :, :query])
+        vs.append(v[:, :, :query])
+        past += query
+        for b in (dq, dk, dv, out):
+            b.free()
+    cat = lambda parts: np.concatenate(parts, axis=2)  # noqa: E731
+    total = past
+    i = np.arange(total)
+    s = float(oracle.half_scale(depth))
+    want = helpers.dense_attention_f64(cat(qs), np.repeat(cat(ks), r, axis=1),
+                                       np.repeat(cat(vs), r, axis=1), i[None, :] <= i[:, None],
+                                       s * s)
+    assert np.max(np.abs(cat(outs) - want)) <= STATE_ATOL
+    # the slot holds exactly the valid rows; rows past `total` are still the initial zeros
+    got_k = slot_k.download(np.float32, (kv_heads, capacity, depth))
+    assert np.array_equal(got_k[:, :total], cat(ks)[0])
+    assert np.all(got_k[:, total:] == 0.0)
+    for b in (slot_k, slot_v, ws):
+        b.free()
+
+
+# ---------------------------------------------------------------------------- ragged batch
+
+def test_config3_ragged_batch_equals_one_at_a_time(gpu_ctx):
+    """BASELINE config 3: 16 sequences, KV lengths ~ U{128..4096} (seeded), packed with
+    prefix-sum offsets, H=32, Hkv=8, D=128, fp16 KV.  One launch; every sequence is then run
+    alone through krm_attention_state and the bits must agree; a few are checked against the
+    oracle (atol 5e-6 on f32 output)."""
+    rng = np.random.default_rng(3)
+    nseq, heads, kv_heads, depth = 16, 32, 8, 128
+    lengths = rng.integers(128, 4097, size=nseq)
+    cu = np.concatenate([[0], np.cumsum(lengths)]).astype(np.int32)
+    total = int(cu[-1])
+    f16 = lambda a: a.astype(np.float16)  # noqa: E731
+    slot_k = f16(rng.normal(size=(kv_heads, total, depth)))
+    slot_v = f16(rng.normal(size=(kv_heads, total, depth)))
+    q = f16(rng.normal(size=(nseq, heads, depth))).astype(np.float32)
+    ins_k = f16(rng.normal(size=(nseq, kv_heads, depth))).astype(np.float32)
+    ins_v = f16(rng.normal(size=(nseq, kv_heads, depth))).astype(np.float32)
+    half = oracle.half_scale(depth)
+
+    d = {name: gpu_ctx.upload(arr) for name, arr in
+         dict(q=q, ins_k=ins_k, ins_v=ins_v, slot_k=slot_k, slot_v=slot_v).items()}
+    out = gpu_ctx.alloc(q.nbytes)
+    ws = gpu_ctx.alloc(gpu_ctx.attention_varlen_workspace(nseq, heads, kv_heads, depth, total))
+    gpu_ctx.attention_varlen(d["q"], d["ins_k"], d["ins_v"], d["slot_k"], d["slot_v"], out, cu,
+                             heads=heads, kv_heads=kv_heads, depth=depth, total_rows=total,
+                             half_scale=half, io_dtype=ka.F32, kv_dtype=ka.F16, workspace=ws)
+    batched = out.download(np.float32, q.shape)
+    for b in list(d.values()) + [out, ws]:
+        b.free()
+
+    for i in range(nseq):
+        past = int(lengths[i])
+        case = StateCase(f"seq {i}", 1, heads, kv_heads, 1, depth, past + 1, 0, past, 1)
+        sk = np.zeros((1, kv_heads, past + 1, depth), dtype=np.float32)
+        sv = np.zeros_like(sk)
+        sk[0, :, :past] = slot_k[:, cu[i]:cu[i + 1]]
+        sv[0, :, :past] = slot_v[:, cu[i]:cu[i + 1]]
+        x = dict(q=q[i].reshape(1, heads, 1, depth), ins_k=ins_k[i].reshape(1, kv_heads, 1, depth),
+                 ins_v=ins_v[i].reshape(1, kv_heads, 1, depth), slot_k=sk, slot_v=sv)
+        alone = run_attention(gpu_ctx, case, x, io=np.float32, kv=np.float16)
+        assert np.array_equal(alone.reshape(heads, depth).view(np.uint32),
+                              batched[i].view(np.uint32)), i
+        if i % 5 == 0:
+            want = oracle_state_attention(case, x)
+            ok, fails, max_abs, worst = oracle.allclose(alone, want, atol=STATE_ATOL, rtol=0)
+            assert ok, (i, fails, max_abs, worst)
+
+
+def test_varlen_edges(gpu_ctx):
+    """Empty past (a sequence whose only column is its own) and single-split sequences."""
+    heads, kv_heads, depth = 8, 2, 64
+    lengths = np.array([0, 5, 256, 257, 0, 1])
+    cu = np.concatenate([[0], np.cumsum(lengths)]).astype(np.int32)
+    total = int(cu[-1])
+    rng = np.random.default_rng(9)
+    nseq = len(lengths)
+    slot_k = rng.normal(size=(kv_heads, total, depth)).astype(np.float32)
+    slot_v = rng.normal(size=(kv_heads, total, depth)).astype(np.float32)
+    q = rng.normal(size=(nseq, heads, depth)).astype(np.float32)
+    ins_k = rng.normal(size=(nseq, kv_heads, depth)).astype(np.float32)
+    ins_v = rng.normal(size=(nseq, kv_heads, depth)).astype(np.float32)
+    d = {name: gpu_ctx.upload(arr) for name, arr in
+         dict(q=q, ins_k=ins_k, ins_v=ins_v, slot_k=slot_k, slot_v=slot_v).items()}
+    out = gpu_ctx.alloc(q.nbytes)
+    ws = gpu_ctx.alloc(gpu_ctx.attention_varlen_workspace(nseq, heads, kv_heads, depth, total))
+    gpu_ctx.attention_varlen(d["q"], d["ins_k"], d["ins_v"], d["slot_k"], d["slot_v"], out, cu,
+                             heads=heads, kv_heads=kv_heads, depth=depth, total_rows=total,
+                             half_scale=oracle.half_scale(depth), workspace=ws)
+    got = out.download(np.float32, q.shape)
+    for i in range(nseq):
+        past = int(lengths[i])
+        case = StateCase(f"seq {i}", 1, heads, kv_heads, 1, depth, past + 1, 0, past, 1)
+        sk = np.zeros((1, kv_heads, past + 1, depth), dtype=np.float32)
+        sv = np.zeros_like(sk)
+        sk[0, :, :past] = slot_k[:, cu[i]:cu[i + 1]]
+        sv[0, :, :past] = slot_v[:, cu[i]:cu[i + 1]]
+        x = dict(q=q[i].reshape(1, heads, 1, depth), ins_k=ins_k[i].reshape(1, kv_heads, 1, depth),
+                 ins_v=ins_v[i].reshape(1, kv_heads, 1, depth), slot_k=sk, slot_v=sv)
+        want = oracle_state_attention(case, x)
+        assert np.max(np.abs(got[i].reshape(want.shape) - want)) <= STATE_ATOL, i
+    with pytest.raises(ka.GpuValidationError):  # not ascending
+        gpu_ctx.attention_varlen(d["q"], d["ins_k"], d["ins_v"], d["slot_k"], d["slot_v"], out,
+                                 [0, 5, 3], heads=heads, kv_heads=kv_heads, depth=depth,
+                                 total_rows=total, half_scale=0.3, workspace=ws)
+    for b in list(d.values()) + [out, ws]:
+        b.free()

@@ -1,0 +1,175 @@
+"""GPU parity of the int4 dequant kernel and the `linear` op (through the C ABI) against the
+CPU oracle.  Tolerances are written where they are used and follow the reference's rule for
+kernels whose reduction order differs from the oracle's: measure, then add margin
+(docs/decisions/0022-gemm-register-blocking.md:22-24)."""
+import numpy as np
+import pytest
+
+import helpers
+import karume_amd as ka
+from helpers import oracle
+
+pytestmark = pytest.mark.gpu
+
+
+def run_dequant(ctx, packed, scale, rows, width, group):
+    scale = np.ascontiguousarray(scale)
+    w = ctx.upload(packed)
+    s = ctx.upload(scale)
+    out = ctx.alloc(rows * width * 4)
+    ctx.dequant_i4(w, s, out, rows, width, group, ka.dtype_code(scale.dtype))
+    got = out.download(np.float32, (rows, width))
+    for b in (w, s, out):
+        b.free()
+    return got
+
+
+def run_linear(ctx, x, packed, scale, bias, n, k, group, compute=ka.COMPUTE_F32):
+    """x: [m, k] float32 or float16 array (its dtype selects the io dtype)."""
+    x = np.ascontiguousarray(x)
+    scale = np.ascontiguousarray(scale)
+    m = x.shape[0]
+    dx, dw, ds = ctx.upload(x), ctx.upload(packed), ctx.upload(scale)
+    db = ctx.upload(np.ascontiguousarray(bias, dtype=x.dtype)) if bias is not None else None
+    out = ctx.alloc(max(m * n * x.itemsize, 16))
+    ctx.linear_i4(dx, dw, ds, db, out, m, n, k, group, ka.dtype_code(x.dtype),
+                  ka.dtype_code(scale.dtype), compute)
+    got = out.download(x.dtype, (m, n))
+    for b in (dx, dw, ds, out) + ((db,) if db is not None else ()):
+        b.free()
+    return got
+
+
+def test_dequant_bit_exact_all_codes_all_positions(gpu_ctx):
+    """All 16 codes x 8 in-word positions with row x group varying scales: GPU bits == decodeI4
+    bits (packages/runtime/tests/gpu_i4_weights_test.ts:404-459, extended to u = 0)."""
+    rows, width, g = 16, 32, 16
+    q = np.array([(r + c) % 16 - 8 for r in range(rows) for c in range(width)], dtype=np.int8)
+    scale = np.array([[0.1 + 0.017 * r + 0.31 * gi for gi in range(width // g)]
+                      for r in range(rows)], dtype=np.float32)
+    packed = oracle.pack_i4(q)
+    want = oracle.decode_i4(packed, [rows, width], scale, [rows, width // g], g)
+    got = run_dequant(gpu_ctx, packed, scale, rows, width, g)
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+
+
+@pytest.mark.parametrize("scale_dtype", [np.float32, np.float16])
+def test_dequant_bit_exact_random(gpu_ctx, scale_dtype):
+    rng = np.random.default_rng(21)
+    rows, width, g = 67, 384, 128
+    packed, _q, scale = helpers.synthetic_int4(rng, rows, width, g, scale_f16=True)
+    scale = scale.astype(scale_dtype)
+    if scale_dtype == np.float32:  # arbitrary f32 scales: the product rounds, once
+        scale = (scale.astype(np.float32) * np.float32(1.2345678)).astype(np.float32)
+    want = oracle.decode_i4(packed, [rows, width], scale.astype(np.float32),
+                            [rows, width // g], g)
+    got = run_dequant(gpu_ctx, packed, scale, rows, width, g)
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+
+
+@pytest.mark.parametrize("case", helpers.I4_LINEAR_CASES, ids=lambda c: c.name)
+def test_linear_reference_cases_f32(gpu_ctx, case):
+    """The reference's tile-edge shapes (gpu_i4_weights_test.ts:116-145), f32 in/out, f32
+    scales.  |out| reaches ~1e3 here; gate: the reference's default allclose (atol 1e-5,
+    rtol 1e-3) AND a tighter atol 2e-3 / rtol 2e-6 derived from f32 accumulation of ~1e3-sized
+    partial sums (measured worst 2.4e-4)."""
+    x, packed, _q, scale, bias = helpers.make_i4_linear(case)
+    want = oracle.linear_i4(x, packed, scale, bias, case.n, case.k, case.group)
+    got = run_linear(gpu_ctx, x, packed, scale, bias, case.n, case.k, case.group)
+    ok, fails, max_abs, worst = oracle.allclose(got, want, atol=1e-5, rtol=1e-3)
+    assert ok, (fails, max_abs, worst)
+    ok, fails, max_abs, worst = oracle.allclose(got, want, atol=2e-3, rtol=2e-6)
+    assert ok, (fails, max_abs, worst)
+
+
+def test_linear_packed_equals_preexpanded_through_same_kernel(gpu_ctx):
+    """Invariant of gpu_i4_weights_test.ts:262-298 restated for this backend: weights with
+    scale 1 and the same codes must give exactly sum(q * x) — integer arithmetic, bit-exact —
+    and scaling every group by a power of two must scale the output exactly."""
+    rng = np.random.default_rng(2)
+    n, k, g = 40, 256, 32
+    q = rng.integers(-8, 8, size=(n, k), dtype=np.int8)
+    x = rng.integers(-4, 5, size=(3, k)).astype(np.float32)
+    packed = oracle.pack_i4(q)
+    ones = np.ones((n, k // g), dtype=np.float32)
+    got = run_linear(gpu_ctx, x, packed, ones, None, n, k, g)
+    want = (x.astype(np.int64) @ q.astype(np.int64).T).astype(np.float32)
+    assert np.array_equal(got, want)
+    got4 = run_linear(gpu_ctx, x, packed, ones * 0.25, None, n, k, g)
+    assert np.array_equal(got4, want * 0.25)
+
+
+@pytest.mark.parametrize("io", [np.float16, np.float32])
+def test_linear_config0_gemv(gpu_ctx, io):
+    """BASELINE config 0: M=1, K=N=4096, int4 g128, fp16 scales |N(0,0.02)|, x ~ N(0,1) in fp16.
+    f32 output: atol 2e-5 (|out| ~ 5, f32 accumulation; measured worst 4e-6), rtol 0.
+    fp16 output: the oracle's f32 result rounded to fp16, within 1 fp16 ulp."""
+    rng = np.random.default_rng(40960)
+    n = k = 4096
+    g = 128
+    packed, _q, scale = helpers.synthetic_int4(rng, n, k, g)
+    x = rng.normal(size=(1, k)).astype(np.float16)
+    want = oracle.linear_i4(x.astype(np.float32), packed, scale.astype(np.float32),
+                            np.zeros(n, dtype=np.float32), n, k, g)
+    got = run_linear(gpu_ctx, x.astype(io), packed, scale, None, n, k, g)
+    if io == np.float32:
+        ok, fails, max_abs, worst = oracle.allclose(got, want, atol=2e-5, rtol=0)
+        assert ok, (fails, max_abs, worst)
+    else:
+        want16 = want.astype(np.float16)
+        ulp = np.abs(np.nextafter(want16, np.float16(np.inf)).astype(np.float32)
+                     - want16.astype(np.float32))
+        assert np.all(np.abs(got.astype(np.float32) - want16.astype(np.float32)) <= ulp)
+
+
+@pytest.mark.parametrize("io", [np.float16, np.float32])
+def test_linear_batched_rows_equal_single_rows_bitwise(gpu_ctx, io):
+    """BASELINE config 3 (GEMV part): M = 16 in one launch vs the 16 rows one at a time — the
+    per-row reduction order does not depend on M, so the bits agree."""
+    rng = np.random.default_rng(16)
+    n = k = 4096
+    g = 128
+    packed, _q, scale = helpers.synthetic_int4(rng, n, k, g)
+    x = rng.normal(size=(16, k)).astype(np.float16).astype(io)
+    batched = run_linear(gpu_ctx, x, packed, scale, None, n, k, g)
+    for m_sub in (1, 2, 5):
+        part = run_linear(gpu_ctx, x[:m_sub], packed, scale, None, n, k, g)
+        assert np.array_equal(part.view(np.uint8), batched[:m_sub].view(np.uint8)), m_sub
+    single = run_linear(gpu_ctx, x[11:12], packed, scale, None, n, k, g)
+    assert np.array_equal(single.view(np.uint8), batched[11:12].view(np.uint8))
+    want = oracle.linear_i4(x.astype(np.float32), packed, scale.astype(np.float32),
+                            np.zeros(n, dtype=np.float32), n, k, g)
+    tol = 2e-5 if io == np.float32 else 8e-3  # fp16 output: half an ulp at |out| < 16
+    assert np.max(np.abs(batched.astype(np.float32) - want)) <= tol
+
+
+@pytest.mark.parametrize("shape", [(1, 256, 2048, 128), (3, 2048, 5632, 128), (1, 100, 11008, 128),
+                                   (7, 33, 96, 32), (2, 5, 64, 16), (16, 32000, 2048, 128)])
+def test_linear_shapes_of_the_decoder(gpu_ctx, shape):
+    """The GEMV over the layer shapes of the 1.1B decoder (N x K) and ragged edges; f32 io,
+    gate atol 3e-5 rtol 1e-5 against the f64 oracle (measured worst 6e-6)."""
+    m, n, k, g = shape
+    rng = np.random.default_rng(n * 7 + k)
+    packed, _q, scale = helpers.synthetic_int4(rng, n, k, g)
+    x = rng.normal(size=(m, k)).astype(np.float16).astype(np.float32)
+    bias = rng.normal(size=n).astype(np.float32)
+    want = oracle.linear_i4(x, packed, scale.astype(np.float32), bias, n, k, g)
+    got = run_linear(gpu_ctx, x, packed, scale, bias, n, k, g)
+    ok, fails, max_abs, worst = oracle.allclose(got, want, atol=3e-5, rtol=1e-5)
+    assert ok, (fails, max_abs, worst)
+
+
+def test_linear_rejections(gpu_ctx):
+    """Unsupported combinations fail before launch (never approximated)."""
+    buf = gpu_ctx.zeros(4096)
+    with pytest.raises(ka.GpuValidationError):  # group does not divide k
+        gpu_ctx.linear_i4(buf, buf, buf, None, buf, 1, 4, 48, 32)
+    with pytest.raises(ka.GpuValidationError):  # group not a power of two >= 16
+        gpu_ctx.linear_i4(buf, buf, buf, None, buf, 1, 4, 48, 24)
+    with pytest.raises(ka.GpuValidationError):
+        gpu_ctx.linear_i4(buf, buf, buf, None, buf, 1, 4, 64, 8)
+    with pytest.raises(ka.GpuValidationError):  # NULL weights
+        gpu_ctx.linear_i4(buf, None, buf, None, buf, 1, 4, 64, 32)
+    with pytest.raises(ka.GpuValidationError):
+        gpu_ctx.dequant_i4(buf, buf, buf, 2, 8, 3)
+    buf.free()
