@@ -1,0 +1,202 @@
+#!/usr/bin/env python3
+"""Benchmark of the hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+A step is one int4 g128 GEMV at M=1, K=N=4096 (BASELINE config 0: fp16 activations and
+scales, f32 accumulation, fp16 output) through the C ABI.  Steps rotate over enough distinct
+weight buffers (> 512 MiB) that no step finds its weights in the 256 MB Infinity Cache, so
+`value` is an HBM number; the cache-resident figure is reported beside it.  Inputs are
+resident in HBM before the timed region; timing uses HIP events recorded on the stream the
+kernels are launched on.
+
+Prints ONE JSON line.  Extra keys report the other BASELINE configs measured the same way.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
+
+
+def log(msg: str) -> None:
+    print(msg, file=sys.stderr, flush=True)
+
+
+def timed(ctx, fn, steps: int, warmup: int) -> float:
+    """Milliseconds for exactly `steps` calls of fn(i), HIP events on the context's stream."""
+    for i in range(warmup):
+        fn(i)
+    ctx.sync()
+    start, stop = ctx.event(), ctx.event()
+    start.record()
+    for i in range(steps):
+        fn(i)
+    stop.record()
+    ms = start.elapsed_ms(stop)
+    ctx.sync()
+    start.destroy()
+    stop.destroy()
+    return ms
+
+
+def bench_gemv(ctx, ka, rng, steps: int, warmup: int, m: int, n: int, k: int, g: int,
+               copies: int):
+    """Returns (ms_total_rotating, ms_total_resident, algorithmic bytes per call)."""
+    row_bytes = k // 2
+    weights, scales = [], []
+    for _ in range(copies):
+        packed = rng.integers(0, 256, size=n * row_bytes, dtype=np.uint8)  # codes uniform in [-8,7]
+        sc = np.maximum(np.abs(rng.normal(0, 0.02, size=(n, k // g))).astype(np.float16),
+                        np.float16(6.104e-05))
+        weights.append(ctx.upload(packed))
+        scales.append(ctx.upload(sc))
+    x = ctx.upload(rng.normal(size=(m, k)).astype(np.float16))
+    out = ctx.alloc(m * n * 2)
+
+    def step(i: int) -> None:
+        j = i % copies
+        ctx.linear_i4(x, weights[j], scales[j], None, out, m, n, k, g, ka.F16, ka.F16)
+
+    def step_resident(i: int) -> None:
+        ctx.linear_i4(x, weights[0], scales[0], None, out, m, n, k, g, ka.F16, ka.F16)
+
+    ms_rot = timed(ctx, step, steps, warmup)
+    ms_res = timed(ctx, step_resident, steps, warmup)
+    for b in weights + scales + [x, out]:
+        b.free()
+    algo = n * row_bytes + n * (k // g) * 2 + m * k * 2 + m * n * 2
+    return ms_rot, ms_res, algo
+
+
+def bench_attention(ctx, ka, rng, steps: int, warmup: int, copies: int):
+    """BASELINE config 2: B=1, H=32, Hkv=8, D=128, 4095 cached rows + this step's row, fp16."""
+    heads, kv_heads, depth, past, cap = 32, 8, 128, 4095, 4096
+    slots = []
+    for _ in range(copies):
+        sk = rng.normal(size=(kv_heads, cap, depth)).astype(np.float16)
+        sv = rng.normal(size=(kv_heads, cap, depth)).astype(np.float16)
+        slots.append((ctx.upload(sk), ctx.upload(sv)))
+    q = ctx.upload(rng.normal(size=(heads, depth)).astype(np.float16))
+    ik = ctx.upload(rng.normal(size=(kv_heads, depth)).astype(np.float16))
+    iv = ctx.upload(rng.normal(size=(kv_heads, depth)).astype(np.float16))
+    out = ctx.alloc(heads * depth * 2)
+    ws = ctx.alloc(ctx.attention_state_workspace(1, heads, kv_heads, 1, depth, 0, past))
+    half = float(np.float32(np.sqrt(1.0 / np.sqrt(float(depth)))))
+
+    def step(i: int) -> None:
+        sk, sv = slots[i % copies]
+        ctx.attention_state(q, ik, iv, sk, sv, out, batch=1, heads=heads, kv_heads=kv_heads,
+                            chunk_rows=1, depth=depth, capacity=cap, window=0, half_scale=half,
+                            past=past, query=1, io_dtype=ka.F16, kv_dtype=ka.F16, workspace=ws)
+
+    ms = timed(ctx, step, steps, warmup)
+    for pair in slots:
+        pair[0].free()
+        pair[1].free()
+    for b in (q, ik, iv, out, ws):
+        b.free()
+    algo = 2 * kv_heads * (past + 1) * depth * 2 + 2 * heads * depth * 2
+    return ms, algo
+
+
+def cpu_baseline(n: int, k: int, g: int, budget_s: float = 12.0):
+    """The CPU oracle (a port of the reference's decode + linear loops, double accumulation,
+    OpenMP over output rows) timed on the host cores on repetitions of the same GEMV."""
+    from oracle import oracle
+
+    rng = np.random.default_rng(1)
+    packed = rng.integers(0, 256, size=n * k // 2, dtype=np.uint8)
+    scale = np.abs(rng.normal(0, 0.02, size=(n, k // g))).astype(np.float32)
+    x = rng.normal(size=(1, k)).astype(np.float16).astype(np.float32)
+    bias = np.zeros(n, dtype=np.float32)
+    oracle.linear_i4(x, packed, scale, bias, n, k, g)  # warm
+    reps, t0 = 0, time.perf_counter()
+    while time.perf_counter() - t0 < budget_s and reps < 5000:
+        oracle.linear_i4(x, packed, scale, bias, n, k, g)
+        reps += 1
+    dt = time.perf_counter() - t0
+    algo = n * k // 2 + n * (k // g) * 2 + k * 2 + n * 2
+    cores = int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1))
+    return {"value": algo * reps / dt / 1e9, "unit": "GB/s", "cores": cores, "kind": "port",
+            "sample": f"{reps} repetitions of the config-0 GEMV (M=1,K=N=4096) in {dt:.1f} s"}
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=2000)
+    ap.add_argument("--warmup", type=int, default=200)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--only", default="", help="gemv: skip the secondary measurements")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build measures one GPU only (--gpus 1); no multi-GPU figure is "
+              "produced in this run", file=sys.stderr)
+        return 2
+
+    import karume_amd as ka
+
+    ctx = ka.acquire_gpu(int(os.environ.get("LOCAL_RANK", "0")))
+    rng = np.random.default_rng(20261125)
+    m, n, k, g = 1, 4096, 4096, 128
+    copies = 64  # 64 x (8 MiB + 256 KiB) = 528 MiB of weights in rotation
+    log(f"[bench] GEMV M={m} K={k} N={n} g={g}, {copies} weight copies")
+    ms_rot, ms_res, algo = bench_gemv(ctx, ka, rng, args.steps, args.warmup, m, n, k, g, copies)
+    per_call_us = ms_rot * 1e3 / args.steps
+    gbs = algo / (per_call_us * 1e-6) / 1e9
+    gbs_res = algo / (ms_res * 1e3 / args.steps * 1e-6) / 1e9
+    result = {
+        "metric": "q-GEMV HBM GB/s (int4 g128, M=1, K=N=4096)",
+        "value": round(gbs, 1),
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": ms_rot / args.steps,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32",
+        "data": "synthetic",
+        "config": {"workload": "config 0: int4 g128 GEMV M=1 K=4096 N=4096, fp16 x/scales/out, "
+                               "f32 accumulate, 64 rotating weight buffers (528 MiB)"},
+        "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS,
+                     "unit": "GB/s", "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None,
+                     "kernel": "gemv_i4_kernel", "algorithmic_bytes_per_launch": algo,
+                     "us_per_launch": round(per_call_us, 3)},
+        "pct_of_hbm_peak": round(100 * gbs / HBM_PEAK_GBS, 2),
+        "gemv_cache_resident_gbs": round(gbs_res, 1),
+    }
+    if args.only != "gemv":
+        steps2 = max(50, args.steps // 4)
+        log("[bench] GEMV M=16 (config 3)")
+        ms16, _res16, algo16 = bench_gemv(ctx, ka, rng, steps2, max(10, args.warmup // 4), 16, n,
+                                          k, g, copies)
+        result["gemv_m16_gbs"] = round(algo16 / (ms16 / steps2 * 1e-3) / 1e9, 1)
+        result["gemv_m16_us"] = round(ms16 / steps2 * 1e3, 3)
+        log("[bench] decode attention (config 2)")
+        ms_att, algo_att = bench_attention(ctx, ka, rng, steps2, max(10, args.warmup // 4), 20)
+        att_gbs = algo_att / (ms_att / steps2 * 1e-3) / 1e9
+        result["attention_decode_gbs"] = round(att_gbs, 1)
+        result["attention_decode_us"] = round(ms_att / steps2 * 1e3, 3)
+        result["attention_decode_pct_of_hbm_peak"] = round(100 * att_gbs / HBM_PEAK_GBS, 2)
+    ctx.destroy()
+    if not args.no_cpu_baseline:
+        log("[bench] CPU baseline (oracle port on the host cores)")
+        result["cpu_baseline"] = cpu_baseline(n, k, g)
+    print(json.dumps(result), flush=True)
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())
