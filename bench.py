@@ -32,20 +32,31 @@ def log(msg: str) -> None:
     print(msg, file=sys.stderr, flush=True)
 
 
-def timed(ctx, fn, steps: int, warmup: int) -> float:
-    """Milliseconds for exactly `steps` calls of fn(i), HIP events on the context's stream."""
-    for i in range(warmup):
-        fn(i)
+def timed(ctx, fn, steps: int, warmup: int, period: int = 64) -> float:
+    """Milliseconds for exactly `steps` calls of fn(i), HIP events on the context's stream.
+
+    The calls are recorded once (`period` consecutive steps = one graph) and replayed, the way
+    a decode loop replays its recorded token step, so the host's launch cost is not what is
+    measured; a remainder of steps % period is issued as plain calls."""
+    with ctx.record() as rec:
+        for i in range(period):
+            fn(i)
+    graph = rec.graph
+    for _ in range(max(1, warmup // period)):
+        graph.launch()
     ctx.sync()
     start, stop = ctx.event(), ctx.event()
     start.record()
-    for i in range(steps):
+    for _ in range(steps // period):
+        graph.launch()
+    for i in range(steps % period):
         fn(i)
     stop.record()
     ms = start.elapsed_ms(stop)
     ctx.sync()
     start.destroy()
     stop.destroy()
+    graph.destroy()
     return ms
 
 
@@ -70,8 +81,8 @@ def bench_gemv(ctx, ka, rng, steps: int, warmup: int, m: int, n: int, k: int, g:
     def step_resident(i: int) -> None:
         ctx.linear_i4(x, weights[0], scales[0], None, out, m, n, k, g, ka.F16, ka.F16)
 
-    ms_rot = timed(ctx, step, steps, warmup)
-    ms_res = timed(ctx, step_resident, steps, warmup)
+    ms_rot = timed(ctx, step, steps, warmup, copies)
+    ms_res = timed(ctx, step_resident, steps, warmup, copies)
     for b in weights + scales + [x, out]:
         b.free()
     algo = n * row_bytes + n * (k // g) * 2 + m * k * 2 + m * n * 2
@@ -99,7 +110,7 @@ def bench_attention(ctx, ka, rng, steps: int, warmup: int, copies: int):
                             chunk_rows=1, depth=depth, capacity=cap, window=0, half_scale=half,
                             past=past, query=1, io_dtype=ka.F16, kv_dtype=ka.F16, workspace=ws)
 
-    ms = timed(ctx, step, steps, warmup)
+    ms = timed(ctx, step, steps, warmup, copies)
     for pair in slots:
         pair[0].free()
         pair[1].free()

@@ -89,6 +89,18 @@ int32_t krm_event_record(krm_ctx* ctx, krm_event* ev);
 int32_t krm_event_elapsed_ms(krm_ctx* ctx, krm_event* start, krm_event* stop, float* ms);
 int32_t krm_event_destroy(krm_ctx* ctx, krm_event* ev);
 
+/* ---- recorded launch sequences (the reference bakes a step's dispatch recipes once and
+ *      replays them: executeBakedPlan, packages/runtime/src/runtime/recipe.ts:357-394) ------
+ * Between krm_graph_begin and krm_graph_end the op entry points record instead of running
+ * (HIP stream capture); krm_graph_launch replays the recorded sequence on the context's
+ * stream with the pointers and scalars it was recorded with.  Calls that must wait for the
+ * device (upload, download, free, sync, krm_attention_varlen) are rejected while recording. */
+typedef struct krm_graph krm_graph;
+int32_t krm_graph_begin(krm_ctx* ctx);
+int32_t krm_graph_end(krm_ctx* ctx, krm_graph** out);
+int32_t krm_graph_launch(krm_ctx* ctx, krm_graph* graph);
+int32_t krm_graph_destroy(krm_ctx* ctx, krm_graph* graph);
+
 /* ---- int4 storage (packages/runtime/src/format/i4.ts:63-118,
  *      packages/runtime/src/kernels/weight-storage.ts:152-187) ------------------------------
  * Expands packed int4 `w` ([rows, width] elements, 2 per byte, element 2j = low nibble,

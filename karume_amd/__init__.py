@@ -7,12 +7,12 @@ the host-side mirror of the reference's interface for those ops.
 """
 from .format_i4 import I4Error, check_int4, group_scale_shape, pack_int4
 from .runtime import (COMPUTE_F16, COMPUTE_F32, F16, F32, DeviceBuffer, ExecutionError,
-                      GpuContext, GpuDeviceLostError, GpuEvent, GpuOutOfMemoryError,
+                      GpuContext, GpuDeviceLostError, GpuEvent, GpuGraph, GpuOutOfMemoryError,
                       GpuValidationError, KarumeError, acquire_gpu, dtype_code, version)
 
 __all__ = [
     "I4Error", "check_int4", "group_scale_shape", "pack_int4",
     "COMPUTE_F16", "COMPUTE_F32", "F16", "F32", "DeviceBuffer", "ExecutionError", "GpuContext",
-    "GpuDeviceLostError", "GpuEvent", "GpuOutOfMemoryError", "GpuValidationError", "KarumeError",
+    "GpuDeviceLostError", "GpuEvent", "GpuGraph", "GpuOutOfMemoryError", "GpuValidationError", "KarumeError",
     "acquire_gpu", "dtype_code", "version",
 ]

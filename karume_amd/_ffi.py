@@ -35,6 +35,10 @@ PROTOTYPES = {
     "krm_event_record": (i32, [c_ctx, c_evt]),
     "krm_event_elapsed_ms": (i32, [c_ctx, c_evt, c_evt, C.POINTER(C.c_float)]),
     "krm_event_destroy": (i32, [c_ctx, c_evt]),
+    "krm_graph_begin": (i32, [c_ctx]),
+    "krm_graph_end": (i32, [c_ctx, C.POINTER(C.c_void_p)]),
+    "krm_graph_launch": (i32, [c_ctx, C.c_void_p]),
+    "krm_graph_destroy": (i32, [c_ctx, C.c_void_p]),
     "krm_dequant_i4": (i32, [c_ctx, c_buf, c_buf, c_buf, u64, u64, u32, i32]),
     "krm_linear_i4": (i32, [c_ctx, c_buf, c_buf, c_buf, c_buf, c_buf, u32, u32, u32, u32, i32,
                             i32, i32]),

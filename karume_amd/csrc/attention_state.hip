@@ -218,6 +218,7 @@ struct DecodeArgs {
   uint32_t nseq;             // ragged batch: sequences; single: batch
   const int32_t* cu_rows;    // ragged batch: [nseq+1] first slot row of each sequence
   const int32_t* split_prefix;  // ragged batch: [nseq+1] first global split of each sequence
+  uint32_t* tickets;         // [nseq * kv_heads] arrival counters, zero between launches
 };
 
 __host__ __device__ inline uint32_t decode_split_columns(uint32_t lanes_per_row) {
@@ -228,13 +229,30 @@ __host__ __device__ inline uint32_t decode_splits(uint64_t slot_columns, uint32_
   return n ? (uint32_t)n : 1u;
 }
 
+constexpr float kLog2e = 1.4426950408889634f;
+
+// Device-scope store / load of one float: written through to (read from) memory that every
+// XCD sees, without touching the rest of the cache.
+__device__ inline void publish(float* p, float v) {
+  __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ inline float observe(const float* p) {
+  return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+constexpr int kMergeChunk = 64;  // split partials merged per pass
+
 // Workgroup = (split, kv head, batch | -): 256 threads = G groups of LPR lanes; a group owns
-// one K/V row per iteration, a lane 16 bytes of it.
+// one K/V row per iteration, a lane 16 bytes of it.  Scores are kept in the base-2 domain
+// (q carries scale^2 * log2 e) so the exponentials are single v_exp_f32 instructions.
+// With several splits, every workgroup stores its (max, sum, weighted V) partial; the one
+// that arrives last at the (sequence, kv head) counter merges all partials of its r heads in
+// ascending split order — the result does not depend on which workgroup that is.
 template <typename XT, typename ST, int R, int LPR, bool RAGGED>
-__global__ __launch_bounds__(kThreads) void attention_decode_kernel(
+__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 2)))
+void attention_decode_kernel(
     const XT* __restrict__ q, const XT* __restrict__ ins_k, const XT* __restrict__ ins_v,
     const ST* __restrict__ slot_k, const ST* __restrict__ slot_v, XT* __restrict__ out,
-    float* __restrict__ ws_ml, float* __restrict__ ws_acc, DecodeArgs a) {
+    float* ws_ml, float* ws_acc, DecodeArgs a) {
   constexpr int E = RowChunk<ST>::E;
   constexpr int D = LPR * E;
   constexpr int G = kThreads / LPR;
@@ -242,6 +260,8 @@ __global__ __launch_bounds__(kThreads) void attention_decode_kernel(
   __shared__ float s_max[kWaves][R];
   __shared__ float s_sum[kWaves][R];
   __shared__ float s_acc[kWaves][R][D];
+  __shared__ float s_ml[R][kMergeChunk][2];
+  __shared__ uint32_t s_ticket;
 
   const int tid = threadIdx.x;
   const int sub = tid % LPR;   // which 16 bytes of the row
@@ -268,8 +288,7 @@ __global__ __launch_bounds__(kThreads) void attention_decode_kernel(
     seq = blockIdx.z;
     past = a.past;
     row_base = 0;
-    const uint64_t low = window_low(a.window, past);
-    nsplit = decode_splits(past - low, kDecodeIter * G);
+    nsplit = decode_splits(past - window_low(a.window, past), kDecodeIter * G);
     split = blockIdx.x;
     first_split = seq * nsplit;
   }
@@ -307,11 +326,12 @@ __global__ __launch_bounds__(kThreads) void attention_decode_kernel(
   const bool own = last && group == 0;  // the lanes that also take this step's own column
   float kx[E], vx[E];
   {
+    // read by every lane (the address is valid for all of them), used by `own` lanes only
     const size_t ins_base = ((size_t)seq * a.kv_heads + hk) * D + sub * E;
 #pragma unroll
     for (int e = 0; e < E; ++e) {
-      kx[e] = own ? ld_f32<XT>(ins_k, ins_base + e) : 0.f;
-      vx[e] = own ? ld_f32<XT>(ins_v, ins_base + e) : 0.f;
+      kx[e] = ld_f32<XT>(ins_k, ins_base + e);
+      vx[e] = ld_f32<XT>(ins_v, ins_base + e);
     }
   }
   float qf[R][E];
@@ -319,10 +339,11 @@ __global__ __launch_bounds__(kThreads) void attention_decode_kernel(
   for (int h = 0; h < R; ++h) {
     const size_t q_base = ((size_t)seq * a.heads + (size_t)hk * R + h) * D + sub * E;
 #pragma unroll
-    for (int e = 0; e < E; ++e) qf[h][e] = (ld_f32<XT>(q, q_base + e) * a.scale) * a.scale;
+    for (int e = 0; e < E; ++e)
+      qf[h][e] = ((ld_f32<XT>(q, q_base + e) * a.scale) * a.scale) * kLog2e;
   }
 
-  // scores
+  // scores (base-2 domain)
   float sc[kDecodeIter + 1][R];
 #pragma unroll
   for (int it = 0; it < kDecodeIter; ++it) {
@@ -382,11 +403,12 @@ __global__ __launch_bounds__(kThreads) void attention_decode_kernel(
       RowChunk<ST>::unpack(vraw[it < kDecodeIter ? it : 0], vf);
     } else {
 #pragma unroll
-      for (int e = 0; e < E; ++e) vf[e] = vx[e];
+      for (int e = 0; e < E; ++e) vf[e] = own ? vx[e] : 0.f;  // 0 * NaN must not leak
     }
 #pragma unroll
     for (int h = 0; h < R; ++h) {
-      const float p = expf(sc[it][h] - mx[h]);  // exp(-inf) = 0 for columns outside the split
+      // 2^(-inf) = 0 for columns outside the split
+      const float p = __builtin_amdgcn_exp2f(sc[it][h] - mx[h]);
       sum[h] += p;
 #pragma unroll
       for (int e = 0; e < E; ++e) acc[h][e] = fmaf(p, vf[e], acc[h][e]);
@@ -414,60 +436,117 @@ __global__ __launch_bounds__(kThreads) void attention_decode_kernel(
     const int h = o / D, d = o - h * D;
     float total = s_acc[0][h][d];
     float l = s_sum[0][h];
+    float m = s_max[0][h];
 #pragma unroll
     for (int w = 1; w < kWaves; ++w) {
       total += s_acc[w][h][d];
       l += s_sum[w][h];
+      m = fmaxf(m, s_max[w][h]);
     }
     const uint32_t head = hk * R + h;
     if (nsplit == 1) {
       st_f32<XT>(out, ((size_t)seq * a.heads + head) * D + d, total / l);
     } else {
       const size_t slot_index = (size_t)gsplit * a.heads + head;
-      ws_acc[slot_index * D + d] = total;
+      publish(&ws_acc[slot_index * D + d], total);
       if (d == 0) {
-        float m = s_max[0][h];
-#pragma unroll
-        for (int w = 1; w < kWaves; ++w) m = fmaxf(m, s_max[w][h]);
-        ws_ml[slot_index * 2] = m;
-        ws_ml[slot_index * 2 + 1] = l;
+        publish(&ws_ml[slot_index * 2], m);
+        publish(&ws_ml[slot_index * 2 + 1], l);
       }
     }
   }
-}
+  if (nsplit == 1) return;
 
-// Merge of the split partials of one (sequence, head), in ascending split order.
-template <typename XT, bool RAGGED>
-__global__ __launch_bounds__(128) void attention_combine_kernel(
-    const float* __restrict__ ws_ml, const float* __restrict__ ws_acc, XT* __restrict__ out,
-    uint32_t heads, uint32_t depth, uint32_t nsplit_single, const int32_t* split_prefix) {
-  const uint32_t head = blockIdx.x, seq = blockIdx.y;
-  uint32_t first, nsplit;
-  if constexpr (RAGGED) {
-    first = (uint32_t)split_prefix[seq];
-    nsplit = (uint32_t)split_prefix[seq + 1] - first;
-  } else {
-    nsplit = nsplit_single;
-    first = seq * nsplit;
+  // Arrival: the partial was written through to memory (device-scope stores); once every
+  // thread's stores have completed, take a ticket.  The last arrival merges, reading the
+  // partials with device-scope loads.  No cache-wide write-back or invalidate is involved.
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+  __syncthreads();
+  if (tid == 0)
+    s_ticket = __hip_atomic_fetch_add(&a.tickets[seq * a.kv_heads + hk], 1u, __ATOMIC_RELAXED,
+                                      __HIP_MEMORY_SCOPE_AGENT);
+  __syncthreads();
+  if (s_ticket + 1 != nsplit) return;
+
+  // Merge nsplit partials of each of the R heads, kMergeChunk at a time, ascending order.
+  // Weights are prepared in LDS so the partial rows can be requested eight at a time.
+  constexpr int kOuts = (R * D + kThreads - 1) / kThreads;
+  float run_m[R], run_l[R];
+  float run_o[kOuts];
+#pragma unroll
+  for (int h = 0; h < R; ++h) {
+    run_m[h] = -INFINITY;
+    run_l[h] = 0.f;
   }
-  if (nsplit == 1) return;  // the decode kernel already wrote the normalised row
-  float m = -INFINITY;
-  for (uint32_t s = 0; s < nsplit; ++s)
-    m = fmaxf(m, ws_ml[((size_t)(first + s) * heads + head) * 2]);
-  float denom = 0.f;
-  for (uint32_t s = 0; s < nsplit; ++s) {
-    const size_t i = ((size_t)(first + s) * heads + head) * 2;
-    denom = fmaf(expf(ws_ml[i] - m), ws_ml[i + 1], denom);
-  }
-  const float inv = 1.0f / denom;
-  for (uint32_t d = threadIdx.x; d < depth; d += blockDim.x) {
-    float total = 0.f;
-    for (uint32_t s = 0; s < nsplit; ++s) {
-      const size_t i = (size_t)(first + s) * heads + head;
-      total = fmaf(expf(ws_ml[i * 2] - m), ws_acc[i * depth + d], total);
+#pragma unroll
+  for (int i = 0; i < kOuts; ++i) run_o[i] = 0.f;
+  for (uint32_t s0 = 0; s0 < nsplit; s0 += kMergeChunk) {
+    const uint32_t cnt = nsplit - s0 < (uint32_t)kMergeChunk ? nsplit - s0 : (uint32_t)kMergeChunk;
+    __syncthreads();
+    for (uint32_t i = tid; i < R * cnt; i += kThreads) {
+      const uint32_t h = i / cnt, s = i - h * cnt;
+      const size_t slot_index = (size_t)(first_split + s0 + s) * a.heads + hk * R + h;
+      s_ml[h][s][0] = observe(&ws_ml[slot_index * 2]);
+      s_ml[h][s][1] = observe(&ws_ml[slot_index * 2 + 1]);
     }
-    st_f32<XT>(out, ((size_t)seq * heads + head) * depth + d, total * inv);
+    __syncthreads();
+    float keep[R];
+#pragma unroll
+    for (int h = 0; h < R; ++h) {  // every thread tracks every head (uniform work)
+      float m = run_m[h];
+      for (uint32_t s = 0; s < cnt; ++s) m = fmaxf(m, s_ml[h][s][0]);
+      keep[h] = __builtin_amdgcn_exp2f(run_m[h] - m);  // 0 on the first pass
+      float l = run_l[h] * keep[h];
+      for (uint32_t s = 0; s < cnt; ++s)
+        l = fmaf(__builtin_amdgcn_exp2f(s_ml[h][s][0] - m), s_ml[h][s][1], l);
+      run_m[h] = m;
+      run_l[h] = l;
+    }
+    __syncthreads();
+    for (uint32_t i = tid; i < R * cnt; i += kThreads) {  // max -> weight, in place
+      const uint32_t h = i / cnt, s = i - h * cnt;
+      float m = run_m[0];
+#pragma unroll
+      for (int hh = 1; hh < R; ++hh) m = (h == (uint32_t)hh) ? run_m[hh] : m;
+      s_ml[h][s][0] = __builtin_amdgcn_exp2f(s_ml[h][s][0] - m);
+    }
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < kOuts; ++i) {
+      const int o = tid + i * kThreads;
+      if (o >= R * D) break;
+      const int h = o / D, d = o - h * D;
+      float k_h = keep[0];
+#pragma unroll
+      for (int hh = 1; hh < R; ++hh) k_h = (h == hh) ? keep[hh] : k_h;
+      float total = run_o[i] * k_h;
+      const float* src = ws_acc + ((size_t)(first_split + s0) * a.heads + hk * R + h) * D + d;
+      const size_t stride = (size_t)a.heads * D;
+      for (uint32_t s = 0; s < cnt; s += 8) {
+        float v[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j)
+          v[j] = observe(&src[(size_t)(s + j < cnt ? s + j : s) * stride]);
+#pragma unroll
+        for (int j = 0; j < 8; ++j)
+          if (s + j < cnt) total = fmaf(s_ml[h][s + j][0], v[j], total);
+      }
+      run_o[i] = total;
+    }
   }
+#pragma unroll
+  for (int i = 0; i < kOuts; ++i) {
+    const int o = tid + i * kThreads;
+    if (o >= R * D) break;
+    const int h = o / D, d = o - h * D;
+    float l_h = run_l[0];
+#pragma unroll
+    for (int hh = 1; hh < R; ++hh) l_h = (h == hh) ? run_l[hh] : l_h;
+    st_f32<XT>(out, ((size_t)seq * a.heads + hk * R + h) * D + d, run_o[i] / l_h);
+  }
+  if (tid == 0)  // ready for the next launch
+    __hip_atomic_store(&a.tickets[seq * a.kv_heads + hk], 0u, __ATOMIC_RELAXED,
+                       __HIP_MEMORY_SCOPE_AGENT);
 }
 
 struct DecodeLaunch {
@@ -476,8 +555,6 @@ struct DecodeLaunch {
   float* ws_acc;
   DecodeArgs args;
   uint32_t grid_x, grid_z;     // splits (or total splits), batch
-  uint32_t combine_seqs;       // sequences the combine kernel covers; 0 = no combine needed
-  uint32_t nsplit_single;
 };
 
 template <typename XT, typename ST, int R, int LPR, bool RAGGED>
@@ -487,16 +564,7 @@ int32_t launch_decode(krm_ctx* ctx, const DecodeLaunch& L) {
           ptr<const XT>(L.q), ptr<const XT>(L.ins_k), ptr<const XT>(L.ins_v),
           ptr<const ST>(L.slot_k), ptr<const ST>(L.slot_v), ptr<XT>(L.out), L.ws_ml, L.ws_acc,
           L.args);
-  KRM_TRY(launched(ctx, "attention_decode_kernel"));
-  if (L.combine_seqs) {
-    constexpr int D = LPR * RowChunk<ST>::E;
-    attention_combine_kernel<XT, RAGGED>
-        <<<dim3(L.args.heads, L.combine_seqs), dim3(128), 0, ctx->stream>>>(
-            L.ws_ml, L.ws_acc, ptr<XT>(L.out), L.args.heads, D, L.nsplit_single,
-            L.args.split_prefix);
-    KRM_TRY(launched(ctx, "attention_combine_kernel"));
-  }
-  return KRM_OK;
+  return launched(ctx, "attention_decode_kernel");
 }
 
 template <typename XT, typename ST, int LPR, bool RAGGED>
@@ -628,7 +696,7 @@ int32_t krm_attention_state(krm_ctx* ctx, krm_buf q, krm_buf ins_k, krm_buf ins_
   const uint32_t lpr = decode_lanes_per_row(depth, kv_dtype);
   const bool fast = query == 1 && chunk_rows == 1 && lpr && decode_repeat_ok(repeat) &&
                     aligned(slot_k, 16) && aligned(slot_v, 16) && batch <= 65535 &&
-                    kv_heads <= 65535;
+                    kv_heads <= 65535 && (uint64_t)batch * kv_heads <= kTicketSlots;
   if (fast) {
     const uint64_t low = window_low(window, past);
     const uint32_t nsplit = decode_splits((uint64_t)past - low, decode_split_columns(lpr));
@@ -644,7 +712,7 @@ int32_t krm_attention_state(krm_ctx* ctx, krm_buf q, krm_buf ins_k, krm_buf ins_
     L.args.nseq = batch;
     L.grid_x = nsplit;
     L.grid_z = batch;
-    L.nsplit_single = nsplit;
+    L.args.tickets = ctx->tickets;
     if (nsplit > 1) {
       const size_t ml_floats = (size_t)batch * nsplit * heads * 2;
       const size_t need = (ml_floats + (size_t)batch * nsplit * heads * depth) * sizeof(float);
@@ -656,7 +724,6 @@ int32_t krm_attention_state(krm_ctx* ctx, krm_buf q, krm_buf ins_k, krm_buf ins_
       KRM_REQUIRE(ctx, workspace_bytes >= (size_t)((char*)(L.ws_acc + (size_t)batch * nsplit *
                                                            heads * depth) - (char*)L.ws_ml),
                   "krm_attention_state: workspace of %zu bytes is too small", workspace_bytes);
-      L.combine_seqs = batch;
     }
     return decode_dispatch<false>(ctx, L, repeat, lpr, io_dtype, kv_dtype);
   }
@@ -699,7 +766,9 @@ int32_t krm_attention_varlen(krm_ctx* ctx, krm_buf q, krm_buf ins_k, krm_buf ins
   KRM_REQUIRE(ctx, std::isfinite(half_scale), "krm_attention_varlen: scale is not finite");
   KRM_REQUIRE(ctx, cu_seqlens != nullptr, "krm_attention_varlen: cu_seqlens is NULL");
   KRM_REQUIRE(ctx, total_rows <= 0x7fffffffull, "krm_attention_varlen: total_rows too large");
-  KRM_REQUIRE(ctx, nseq <= 65535 && kv_heads <= 65535, "krm_attention_varlen: grid too large");
+  KRM_REQUIRE(ctx, kv_heads <= 65535 && (uint64_t)nseq * kv_heads <= kTicketSlots,
+              "krm_attention_varlen: nseq * Hkv = %llu exceeds %u", (unsigned long long)nseq * kv_heads,
+              kTicketSlots);
   const uint32_t repeat = heads / kv_heads;
   const uint32_t lpr = decode_lanes_per_row(depth, kv_dtype);
   KRM_REQUIRE(ctx, lpr && decode_repeat_ok(repeat),
@@ -716,6 +785,7 @@ int32_t krm_attention_varlen(krm_ctx* ctx, krm_buf q, krm_buf ins_k, krm_buf ins
   const size_t table_ints = 2 * ((size_t)nseq + 1);
   KRM_REQUIRE(ctx, table_ints * sizeof(int32_t) <= ctx->pinned_bytes,
               "krm_attention_varlen: %u sequences exceed the staging table", nseq);
+  KRM_TRY(not_recording(ctx, "krm_attention_varlen"));
   // The staging area may still feed the previous call's copy.
   KRM_TRY(hip_status(ctx, hipStreamSynchronize(ctx->stream), "hipStreamSynchronize"));
   int32_t* stage = static_cast<int32_t*>(ctx->pinned);
@@ -723,7 +793,6 @@ int32_t krm_attention_varlen(krm_ctx* ctx, krm_buf q, krm_buf ins_k, krm_buf ins
   int32_t* prefix = stage + nseq + 1;
   const uint32_t sc = decode_split_columns(lpr);
   uint64_t splits = 0;
-  bool any_split = false;
   for (uint32_t i = 0; i <= nseq; ++i) {
     cu[i] = cu_seqlens[i];
     if (i > 0) {
@@ -731,7 +800,6 @@ int32_t krm_attention_varlen(krm_ctx* ctx, krm_buf q, krm_buf ins_k, krm_buf ins
                   "krm_attention_varlen: cu_seqlens is not ascending at %u", i);
       prefix[i - 1] = (int32_t)splits;
       const uint32_t ns = decode_splits((uint64_t)(cu_seqlens[i] - cu_seqlens[i - 1]), sc);
-      any_split = any_split || ns > 1;
       splits += ns;
     }
   }
@@ -767,8 +835,7 @@ int32_t krm_attention_varlen(krm_ctx* ctx, krm_buf q, krm_buf ins_k, krm_buf ins
   L.ws_acc = L.ws_ml + ml_floats;
   L.grid_x = (uint32_t)splits;
   L.grid_z = 1;
-  L.combine_seqs = any_split ? nseq : 0;
-  L.nsplit_single = 0;
+  L.args.tickets = ctx->tickets;
   return decode_dispatch<true>(ctx, L, repeat, lpr, io_dtype, kv_dtype);
 }
 

@@ -19,6 +19,10 @@ struct krm_ctx {
   // Host staging for small per-call tables (pinned, allocated once at context creation).
   void* pinned = nullptr;
   size_t pinned_bytes = 0;
+  // Arrival counters of the split-K attention (device memory, zeroed at creation; the last
+  // workgroup of every (sequence, kv head) puts its counter back to zero).
+  uint32_t* tickets = nullptr;
+  bool recording = false;  // between krm_graph_begin and krm_graph_end
   char error[512] = {0};
 };
 
@@ -26,9 +30,15 @@ struct krm_event {
   hipEvent_t ev;
 };
 
+struct krm_graph {
+  hipGraph_t graph = nullptr;
+  hipGraphExec_t exec = nullptr;
+};
+
 namespace krm {
 
 constexpr int kWave = 64;
+constexpr uint32_t kTicketSlots = 1u << 16;
 
 // Records the message on the context (or on the context-less slot) and returns `code`.
 int32_t fail(krm_ctx* ctx, int32_t code, const char* fmt, ...);
@@ -38,6 +48,9 @@ int32_t hip_status(krm_ctx* ctx, hipError_t status, const char* what);
 
 // Makes the context's device current on the calling thread (calls may arrive on any thread).
 int32_t enter(krm_ctx* ctx);
+
+// Rejects calls that have to wait for the device while a launch sequence is being recorded.
+int32_t not_recording(krm_ctx* ctx, const char* what);
 
 // Error check of the launch that was just queued.
 int32_t launched(krm_ctx* ctx, const char* kernel);

@@ -119,8 +119,9 @@ struct Acts<__half> {
   __device__ static inline void load(const __half* x, bool active, Regs<VEC>& r) {
 #pragma unroll
     for (int j = 0; j < VEC; ++j) {
-      uint4 raw = make_uint4(0, 0, 0, 0);
-      if (active) raw = reinterpret_cast<const uint4*>(x)[j];
+      uint4 raw = reinterpret_cast<const uint4*>(x)[j];
+      const uint32_t keep = active ? 0xFFFFFFFFu : 0u;  // bit mask: no control flow
+      raw.x &= keep; raw.y &= keep; raw.z &= keep; raw.w &= keep;
       pair_activations(raw, r.p[j]);
     }
   }
@@ -153,11 +154,13 @@ struct Acts<float> {
     float s = 0.f;
 #pragma unroll
     for (int j = 0; j < VEC; ++j) {
-      float4 a = make_float4(0.f, 0.f, 0.f, 0.f), b = a;
-      if (active) {
-        a = reinterpret_cast<const float4*>(x)[2 * j];
-        b = reinterpret_cast<const float4*>(x)[2 * j + 1];
-      }
+      uint4 ua = reinterpret_cast<const uint4*>(x)[2 * j];
+      uint4 ub = reinterpret_cast<const uint4*>(x)[2 * j + 1];
+      const uint32_t keep = active ? 0xFFFFFFFFu : 0u;  // bit mask: no control flow
+      const float4 a = make_float4(__uint_as_float(ua.x & keep), __uint_as_float(ua.y & keep),
+                                   __uint_as_float(ua.z & keep), __uint_as_float(ua.w & keep));
+      const float4 b = make_float4(__uint_as_float(ub.x & keep), __uint_as_float(ub.y & keep),
+                                   __uint_as_float(ub.z & keep), __uint_as_float(ub.w & keep));
       r.v[j][0] = a.x; r.v[j][1] = a.y; r.v[j][2] = a.z; r.v[j][3] = a.w;
       r.v[j][4] = b.x; r.v[j][5] = b.y; r.v[j][6] = b.z; r.v[j][7] = b.w;
       s += ((a.x + a.y) + (a.z + a.w)) + ((b.x + b.y) + (b.z + b.w));
@@ -195,15 +198,21 @@ template <>
 __device__ inline __half from_f32<__half>(float v) { return __float2half_rn(v); }
 
 // One wave = ROWS consecutive output rows over the whole K; a step covers 64 lanes x VEC
-// words (VEC*8 codes per lane, all inside one scale group).  The next step's weight words
-// and scales are requested before the current step is consumed.
-template <typename XT, typename ST, int MB, int ROWS, int VEC>
-__global__ __launch_bounds__(256) void gemv_i4_kernel(
+// words (VEC*8 codes per lane, all inside one scale group).
+//  NSTEP > 0: K fits in NSTEP steps; every weight word, scale and (for MB == 1) activation of
+//             the wave is requested before anything is consumed, so one memory round trip
+//             covers the whole kernel.
+//  NSTEP == 0: any K; the next step's weights, scales and activations are requested before
+//             the current step is consumed.
+// Both forms add the per-step partial sums in ascending step order, so they agree bitwise.
+template <typename XT, typename ST, int MB, int ROWS, int VEC, int NSTEP>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 4))) void gemv_i4_kernel(
     const XT* __restrict__ x, const uint32_t* __restrict__ w, const ST* __restrict__ scales,
     const XT* __restrict__ bias, XT* __restrict__ out, uint32_t m, uint32_t n, uint32_t k,
     uint32_t group_shift) {
   constexpr int kLaneElems = VEC * 8;
   constexpr int kStepElems = kWave * kLaneElems;
+  using Regs = typename Acts<XT>::template Regs<VEC>;
   const int lane = threadIdx.x & (kWave - 1);
   const int wave = threadIdx.x >> 6;
   const uint32_t row0 = (blockIdx.x * (blockDim.x >> 6) + wave) * ROWS;
@@ -211,7 +220,6 @@ __global__ __launch_bounds__(256) void gemv_i4_kernel(
 
   const uint32_t words_per_row = k >> 3;
   const uint32_t groups_per_row = k >> group_shift;
-  const uint32_t steps = (k + kStepElems - 1) / kStepElems;
 
   const uint32_t* wrow[ROWS];
   const ST* srow[ROWS];
@@ -228,52 +236,91 @@ __global__ __launch_bounds__(256) void gemv_i4_kernel(
 #pragma unroll
     for (int b = 0; b < MB; ++b) acc[r][b] = 0.f;
 
-  uint32_t cur_w[ROWS][VEC], nxt_w[ROWS][VEC];
-  float cur_s[ROWS], nxt_s[ROWS];
-
+  // Lanes past the end of K (last step of a K that is not a multiple of the step) read the
+  // row's first words instead and get zero activations and a zero scale, so every load is
+  // unconditional and all of them can be in flight together.
   auto fetch = [&](uint32_t step, uint32_t (&dst_w)[ROWS][VEC], float (&dst_s)[ROWS]) {
     const uint32_t k0 = step * kStepElems + lane * kLaneElems;
     const bool active = k0 < k;
+    const uint32_t kc = active ? k0 : 0u;
 #pragma unroll
     for (int r = 0; r < ROWS; ++r) {
-      if (active) {
-        if constexpr (VEC == 4) {
-          const uint4 v = *reinterpret_cast<const uint4*>(wrow[r] + (k0 >> 3));
-          dst_w[r][0] = v.x; dst_w[r][1] = v.y; dst_w[r][2] = v.z; dst_w[r][3] = v.w;
-        } else {
-#pragma unroll
-          for (int j = 0; j < VEC; ++j) dst_w[r][j] = wrow[r][(k0 >> 3) + j];
-        }
-        dst_s[r] = load_scale<ST>(srow[r], k0 >> group_shift);
+      if constexpr (VEC == 4) {
+        const uint4 v = *reinterpret_cast<const uint4*>(wrow[r] + (kc >> 3));
+        dst_w[r][0] = v.x; dst_w[r][1] = v.y; dst_w[r][2] = v.z; dst_w[r][3] = v.w;
       } else {
 #pragma unroll
-        for (int j = 0; j < VEC; ++j) dst_w[r][j] = 0u;
-        dst_s[r] = 0.f;
+        for (int j = 0; j < VEC; ++j) dst_w[r][j] = wrow[r][(kc >> 3) + j];
       }
+      const float sv = load_scale<ST>(srow[r], kc >> group_shift);
+      dst_s[r] = active ? sv : 0.f;
+    }
+  };
+  auto fetch_x = [&](uint32_t step, int b, Regs& regs) {
+    const uint32_t k0 = step * kStepElems + lane * kLaneElems;
+    const uint32_t xrow = min((uint32_t)b, m - 1);  // rows past M re-read the last row, unused
+    Acts<XT>::template load<VEC>(x + (size_t)xrow * k + (k0 < k ? k0 : 0u), k0 < k, regs);
+  };
+  auto consume = [&](const uint32_t (&cw)[ROWS][VEC], const float (&cs)[ROWS], int b,
+                     const Regs& regs) {
+#pragma unroll
+    for (int r = 0; r < ROWS; ++r) {
+      const float part = Acts<XT>::template dot<VEC>(cw[r], regs);
+      acc[r][b] = fmaf(part, cs[r], acc[r][b]);
     }
   };
 
-  fetch(0, cur_w, cur_s);
-  for (uint32_t step = 0; step < steps; ++step) {
-    if (step + 1 < steps) fetch(step + 1, nxt_w, nxt_s);
-    const uint32_t k0 = step * kStepElems + lane * kLaneElems;
-    const bool active = k0 < k;
+  if constexpr (NSTEP > 0) {
+    uint32_t all_w[NSTEP][ROWS][VEC];
+    float all_s[NSTEP][ROWS];
 #pragma unroll
-    for (int b = 0; b < MB; ++b) {
-      typename Acts<XT>::template Regs<VEC> regs;
-      const uint32_t xrow = min((uint32_t)b, m - 1);  // rows past M re-read the last row, unused
-      Acts<XT>::template load<VEC>(x + (size_t)xrow * k + k0, active, regs);
+    for (int step = 0; step < NSTEP; ++step) fetch(step, all_w[step], all_s[step]);
+    if constexpr (MB == 1) {
+      Regs regs[NSTEP];
 #pragma unroll
-      for (int r = 0; r < ROWS; ++r) {
-        const float part = Acts<XT>::template dot<VEC>(cur_w[r], regs);
-        acc[r][b] = fmaf(part, cur_s[r], acc[r][b]);
+      for (int step = 0; step < NSTEP; ++step) fetch_x(step, 0, regs[step]);
+#pragma unroll
+      for (int step = 0; step < NSTEP; ++step) consume(all_w[step], all_s[step], 0, regs[step]);
+    } else {
+#pragma unroll
+      for (int step = 0; step < NSTEP; ++step) {
+#pragma unroll
+        for (int b = 0; b < MB; ++b) {
+          Regs regs;
+          fetch_x(step, b, regs);
+          consume(all_w[step], all_s[step], b, regs);
+        }
       }
     }
+  } else {
+    const uint32_t steps = (k + kStepElems - 1) / kStepElems;
+    uint32_t cur_w[ROWS][VEC], nxt_w[ROWS][VEC];
+    float cur_s[ROWS], nxt_s[ROWS];
+    Regs cur_x, nxt_x;  // MB == 1 only: activations travel with the weights
+    fetch(0, cur_w, cur_s);
+    if constexpr (MB == 1) fetch_x(0, 0, cur_x);
+    for (uint32_t step = 0; step < steps; ++step) {
+      if (step + 1 < steps) {
+        fetch(step + 1, nxt_w, nxt_s);
+        if constexpr (MB == 1) fetch_x(step + 1, 0, nxt_x);
+      }
+      if constexpr (MB == 1) {
+        consume(cur_w, cur_s, 0, cur_x);
+        cur_x = nxt_x;
+      } else {
 #pragma unroll
-    for (int r = 0; r < ROWS; ++r) {
+        for (int b = 0; b < MB; ++b) {
+          Regs regs;
+          fetch_x(step, b, regs);
+          consume(cur_w, cur_s, b, regs);
+        }
+      }
 #pragma unroll
-      for (int j = 0; j < VEC; ++j) cur_w[r][j] = nxt_w[r][j];
-      cur_s[r] = nxt_s[r];
+      for (int r = 0; r < ROWS; ++r) {
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) cur_w[r][j] = nxt_w[r][j];
+        cur_s[r] = nxt_s[r];
+      }
     }
   }
 
@@ -291,28 +338,42 @@ __global__ __launch_bounds__(256) void gemv_i4_kernel(
   }
 }
 
-template <typename XT, typename ST, int MB, int ROWS, int VEC>
+template <typename XT, typename ST, int MB, int ROWS, int VEC, int NSTEP>
 int32_t launch_gemv(krm_ctx* ctx, krm_buf x, krm_buf w, krm_buf scales, krm_buf bias,
                     krm_buf out, uint32_t m, uint32_t n, uint32_t k, uint32_t group_shift) {
   const uint32_t rows_per_block = 4 * ROWS;
   const uint32_t blocks = (n + rows_per_block - 1) / rows_per_block;
-  gemv_i4_kernel<XT, ST, MB, ROWS, VEC><<<dim3(blocks), dim3(256), 0, ctx->stream>>>(
+  gemv_i4_kernel<XT, ST, MB, ROWS, VEC, NSTEP><<<dim3(blocks), dim3(256), 0, ctx->stream>>>(
       ptr<const XT>(x), ptr<const uint32_t>(w), ptr<const ST>(scales), ptr<const XT>(bias),
       ptr<XT>(out), m, n, k, group_shift);
   return launched(ctx, "gemv_i4_kernel");
 }
 
+template <typename XT, typename ST, int MB, int ROWS, int VEC>
+int32_t pick_steps(krm_ctx* ctx, krm_buf x, krm_buf w, krm_buf scales, krm_buf bias, krm_buf out,
+                   uint32_t m, uint32_t n, uint32_t k, uint32_t group_shift) {
+  // Rows short enough to hold in registers are requested whole (VEC == 4: 2048 codes a step).
+  if constexpr (VEC == 4 && MB == 1) {
+    const uint32_t steps = (k + 2047) / 2048;
+    if (steps == 1)
+      return launch_gemv<XT, ST, MB, ROWS, VEC, 1>(ctx, x, w, scales, bias, out, m, n, k, group_shift);
+    if (steps == 2)
+      return launch_gemv<XT, ST, MB, ROWS, VEC, 2>(ctx, x, w, scales, bias, out, m, n, k, group_shift);
+    if (steps == 3 && ROWS <= 2)
+      return launch_gemv<XT, ST, MB, ROWS, VEC, 3>(ctx, x, w, scales, bias, out, m, n, k, group_shift);
+  }
+  return launch_gemv<XT, ST, MB, ROWS, VEC, 0>(ctx, x, w, scales, bias, out, m, n, k, group_shift);
+}
+
 template <typename XT, typename ST, int MB, int VEC>
 int32_t pick_rows(krm_ctx* ctx, krm_buf x, krm_buf w, krm_buf scales, krm_buf bias, krm_buf out,
                   uint32_t m, uint32_t n, uint32_t k, uint32_t group_shift) {
-  // Rows per wave: more rows amortise the activation fetch, fewer rows give more waves to
-  // hide latency.  The choice never changes a row's reduction order.
+  // Rows per wave: two rows share one fetch of the activations; one row per wave keeps more
+  // waves in flight when N is small.  The choice never changes a row's reduction order.
   const uint64_t cus = (uint64_t)ctx->num_cus;
-  if (MB <= 4 && (uint64_t)n >= cus * 4 * 4 * 2)
-    return launch_gemv<XT, ST, MB, 4, VEC>(ctx, x, w, scales, bias, out, m, n, k, group_shift);
   if ((uint64_t)n >= cus * 4 * 2)
-    return launch_gemv<XT, ST, MB, 2, VEC>(ctx, x, w, scales, bias, out, m, n, k, group_shift);
-  return launch_gemv<XT, ST, MB, 1, VEC>(ctx, x, w, scales, bias, out, m, n, k, group_shift);
+    return pick_steps<XT, ST, MB, 2, VEC>(ctx, x, w, scales, bias, out, m, n, k, group_shift);
+  return pick_steps<XT, ST, MB, 1, VEC>(ctx, x, w, scales, bias, out, m, n, k, group_shift);
 }
 
 template <typename XT, typename ST, int VEC>

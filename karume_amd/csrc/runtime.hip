@@ -39,6 +39,13 @@ int32_t enter(krm_ctx* ctx) {
   return hip_status(ctx, hipSetDevice(ctx->device), "hipSetDevice");
 }
 
+int32_t not_recording(krm_ctx* ctx, const char* what) {
+  if (ctx->recording)
+    return fail(ctx, KRM_ERR_VALIDATION, "%s cannot be called while a graph is being recorded",
+                what);
+  return KRM_OK;
+}
+
 int32_t launched(krm_ctx* ctx, const char* kernel) {
   return hip_status(ctx, hipGetLastError(), kernel);
 }
@@ -76,6 +83,15 @@ int32_t krm_ctx_create_on_stream(int32_t device, void* hip_stream, krm_ctx** out
     delete ctx;
     return hip_status(nullptr, st, "hipHostMalloc");
   }
+  st = hipMalloc(reinterpret_cast<void**>(&ctx->tickets), kTicketSlots * sizeof(uint32_t));
+  if (st == hipSuccess) st = hipMemset(ctx->tickets, 0, kTicketSlots * sizeof(uint32_t));
+  if (st == hipSuccess) st = hipDeviceSynchronize();
+  if (st != hipSuccess) {
+    if (ctx->tickets) (void)hipFree(ctx->tickets);
+    (void)hipHostFree(ctx->pinned);
+    delete ctx;
+    return hip_status(nullptr, st, "hipMalloc(tickets)");
+  }
   *out = ctx;
   return KRM_OK;
 }
@@ -86,6 +102,7 @@ int32_t krm_ctx_create(int32_t device, krm_ctx** out) {
   // Default priority on purpose: mixed stream priorities are not used anywhere.
   hipError_t st = hipStreamCreateWithFlags(&ctx->stream, hipStreamNonBlocking);
   if (st != hipSuccess) {
+    (void)hipFree(ctx->tickets);
     (void)hipHostFree(ctx->pinned);
     delete ctx;
     *out = nullptr;
@@ -101,6 +118,7 @@ int32_t krm_ctx_destroy(krm_ctx* ctx) {
   (void)hipStreamSynchronize(ctx->stream);
   if (ctx->owns_stream) (void)hipStreamDestroy(ctx->stream);
   if (ctx->pinned) (void)hipHostFree(ctx->pinned);
+  if (ctx->tickets) (void)hipFree(ctx->tickets);
   delete ctx;
   return KRM_OK;
 }
@@ -109,6 +127,7 @@ const char* krm_last_error(krm_ctx* ctx) { return ctx ? ctx->error : g_error; }
 
 int32_t krm_sync(krm_ctx* ctx) {
   KRM_TRY(enter(ctx));
+  KRM_TRY(not_recording(ctx, "krm_sync"));
   return hip_status(ctx, hipStreamSynchronize(ctx->stream), "hipStreamSynchronize");
 }
 
@@ -125,6 +144,7 @@ int32_t krm_buf_alloc(krm_ctx* ctx, size_t bytes, krm_buf* out) {
 int32_t krm_buf_free(krm_ctx* ctx, krm_buf buf) {
   KRM_TRY(enter(ctx));
   if (!buf) return KRM_OK;
+  KRM_TRY(not_recording(ctx, "krm_buf_free"));
   // Work queued on the stream may still use the buffer ("flush before destroy").
   KRM_TRY(hip_status(ctx, hipStreamSynchronize(ctx->stream), "hipStreamSynchronize"));
   return hip_status(ctx, hipFree(ptr<void>(buf)), "hipFree");
@@ -133,6 +153,7 @@ int32_t krm_buf_free(krm_ctx* ctx, krm_buf buf) {
 int32_t krm_buf_upload(krm_ctx* ctx, krm_buf dst, size_t dst_offset, const void* host,
                        size_t bytes) {
   KRM_TRY(enter(ctx));
+  KRM_TRY(not_recording(ctx, "krm_buf_upload"));
   if (bytes == 0) return KRM_OK;
   KRM_REQUIRE(ctx, dst != 0 && host != nullptr, "krm_buf_upload: NULL buffer");
   // The host array is only valid during the call, so the copy completes before returning.
@@ -146,6 +167,7 @@ int32_t krm_buf_upload(krm_ctx* ctx, krm_buf dst, size_t dst_offset, const void*
 int32_t krm_buf_download(krm_ctx* ctx, krm_buf src, size_t src_offset, void* host,
                          size_t bytes) {
   KRM_TRY(enter(ctx));
+  KRM_TRY(not_recording(ctx, "krm_buf_download"));
   if (bytes == 0) return hip_status(ctx, hipStreamSynchronize(ctx->stream), "sync");
   KRM_REQUIRE(ctx, src != 0 && host != nullptr, "krm_buf_download: NULL buffer");
   KRM_TRY(hip_status(ctx,
@@ -174,6 +196,49 @@ int32_t krm_buf_zero(krm_ctx* ctx, krm_buf dst, size_t dst_offset, size_t bytes)
   krm_zero_kernel<<<dim3((unsigned)blocks), dim3(256), 0, ctx->stream>>>(
       ptr<uint32_t>(dst + dst_offset), words);
   return launched(ctx, "krm_zero_kernel");
+}
+
+int32_t krm_graph_begin(krm_ctx* ctx) {
+  KRM_TRY(enter(ctx));
+  KRM_TRY(not_recording(ctx, "krm_graph_begin"));
+  KRM_TRY(hip_status(ctx, hipStreamBeginCapture(ctx->stream, hipStreamCaptureModeThreadLocal),
+                     "hipStreamBeginCapture"));
+  ctx->recording = true;
+  return KRM_OK;
+}
+
+int32_t krm_graph_end(krm_ctx* ctx, krm_graph** out) {
+  KRM_TRY(enter(ctx));
+  KRM_REQUIRE(ctx, out != nullptr, "krm_graph_end: out is NULL");
+  KRM_REQUIRE(ctx, ctx->recording, "krm_graph_end: no recording in progress");
+  ctx->recording = false;
+  krm_graph* g = new krm_graph();
+  hipError_t st = hipStreamEndCapture(ctx->stream, &g->graph);
+  if (st == hipSuccess) st = hipGraphInstantiate(&g->exec, g->graph, nullptr, nullptr, 0);
+  if (st != hipSuccess) {
+    if (g->graph) (void)hipGraphDestroy(g->graph);
+    delete g;
+    return hip_status(ctx, st, "hipStreamEndCapture/hipGraphInstantiate");
+  }
+  *out = g;
+  return KRM_OK;
+}
+
+int32_t krm_graph_launch(krm_ctx* ctx, krm_graph* graph) {
+  KRM_TRY(enter(ctx));
+  KRM_TRY(not_recording(ctx, "krm_graph_launch"));
+  KRM_REQUIRE(ctx, graph && graph->exec, "krm_graph_launch: graph is NULL");
+  return hip_status(ctx, hipGraphLaunch(graph->exec, ctx->stream), "hipGraphLaunch");
+}
+
+int32_t krm_graph_destroy(krm_ctx* ctx, krm_graph* graph) {
+  KRM_TRY(enter(ctx));
+  if (!graph) return KRM_OK;
+  (void)hipStreamSynchronize(ctx->stream);
+  if (graph->exec) (void)hipGraphExecDestroy(graph->exec);
+  if (graph->graph) (void)hipGraphDestroy(graph->graph);
+  delete graph;
+  return KRM_OK;
 }
 
 int32_t krm_event_create(krm_ctx* ctx, krm_event** out) {

@@ -128,6 +128,41 @@ class GpuEvent:
             self._handle = None
 
 
+class GpuGraph:
+    """A recorded launch sequence (see GpuContext.record)."""
+
+    def __init__(self, ctx: "GpuContext", handle):
+        self.ctx = ctx
+        self._handle = handle
+
+    def launch(self) -> None:
+        self.ctx._check(self.ctx._lib.krm_graph_launch(self.ctx._handle, self._handle))
+
+    def destroy(self) -> None:
+        if self._handle:
+            self.ctx._lib.krm_graph_destroy(self.ctx._handle, self._handle)
+            self._handle = None
+
+
+class _Recording:
+    def __init__(self, ctx: "GpuContext"):
+        self.ctx = ctx
+        self.graph: Optional[GpuGraph] = None
+
+    def __enter__(self) -> "_Recording":
+        self.ctx._check(self.ctx._lib.krm_graph_begin(self.ctx._handle))
+        return self
+
+    def __exit__(self, exc_type, exc, tb) -> None:
+        handle = C.c_void_p()
+        status = self.ctx._lib.krm_graph_end(self.ctx._handle, C.byref(handle))
+        if exc_type is None:
+            self.ctx._check(status)
+            self.graph = GpuGraph(self.ctx, handle)
+        elif status == 0:
+            self.ctx._lib.krm_graph_destroy(self.ctx._handle, handle)
+
+
 class GpuContext:
     """One device + one stream; every op of this backend is queued through it."""
 
@@ -170,6 +205,10 @@ class GpuContext:
 
     def event(self) -> GpuEvent:
         return GpuEvent(self)
+
+    def record(self) -> _Recording:
+        """``with ctx.record() as rec: ...ops...`` then ``rec.graph.launch()`` replays them."""
+        return _Recording(self)
 
     # -- buffers ---------------------------------------------------------------------------
     def alloc(self, nbytes: int) -> DeviceBuffer:
