@@ -120,6 +120,29 @@ def bench_attention(ctx, ka, rng, steps: int, warmup: int, copies: int):
     return ms, algo
 
 
+def bench_gemm(ctx, ka, rng, steps: int, warmup: int, m: int, n: int, k: int, g: int):
+    """BASELINE config 1: prefill GEMM on the matrix cores, fp16 activations and output."""
+    copies = 4
+    weights, scales = [], []
+    for _ in range(copies):
+        weights.append(ctx.upload(rng.integers(0, 256, size=n * k // 2, dtype=np.uint8)))
+        scales.append(ctx.upload(np.maximum(
+            np.abs(rng.normal(0, 0.02, size=(n, k // g))).astype(np.float16),
+            np.float16(6.104e-05))))
+    x = ctx.upload(rng.normal(size=(m, k)).astype(np.float16))
+    out = ctx.alloc(m * n * 2)
+
+    def step(i: int) -> None:
+        j = i % copies
+        ctx.linear_i4(x, weights[j], scales[j], None, out, m, n, k, g, ka.F16, ka.F16,
+                      ka.COMPUTE_F16)
+
+    ms = timed(ctx, step, steps, warmup, copies)
+    for b in weights + scales + [x, out]:
+        b.free()
+    return ms / steps, 2.0 * m * n * k
+
+
 def cpu_baseline(n: int, k: int, g: int, budget_s: float = 12.0):
     """The CPU oracle (a port of the reference's decode + linear loops, double accumulation,
     OpenMP over output rows) timed on the host cores on repetitions of the same GEMV."""
@@ -201,6 +224,13 @@ def main() -> int:
         result["attention_decode_gbs"] = round(att_gbs, 1)
         result["attention_decode_us"] = round(ms_att / steps2 * 1e3, 3)
         result["attention_decode_pct_of_hbm_peak"] = round(100 * att_gbs / HBM_PEAK_GBS, 2)
+        for name, (gn, gk) in {"up": (11008, 4096), "down": (4096, 11008)}.items():
+            log(f"[bench] prefill GEMM M=512 K={gk} N={gn} (config 1, {name}-projection)")
+            ms_g, flops = bench_gemm(ctx, ka, rng, 40, 8, 512, gn, gk, g)
+            result[f"gemm_{name}_tflops"] = round(flops / (ms_g * 1e-3) / 1e12, 1)
+            result[f"gemm_{name}_us"] = round(ms_g * 1e3, 2)
+            result[f"gemm_{name}_pct_of_f16_mfma_peak"] = round(
+                100 * flops / (ms_g * 1e-3) / 2.5e15, 2)
     ctx.destroy()
     if not args.no_cpu_baseline:
         log("[bench] CPU baseline (oracle port on the host cores)")

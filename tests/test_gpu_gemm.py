@@ -1,0 +1,114 @@
+"""GPU parity of the fp16 MFMA GEMM path of `linear` (M > 16, KRM_COMPUTE_F16) against the CPU
+oracle.
+
+Numerics of this path (stated in the kernel): x is rounded to fp16 (exact when it already is),
+each weight is dequantised to fp16 as fp16((u-8) * scale) — one fp16 rounding, relative error
+<= 2^-11 — and products are accumulated in f32.  With K terms of typical size t the error of an
+output behaves like sqrt(K) * t * 2^-11 / sqrt(3); the tests scale their tolerance with the
+RMS of the oracle's output:  |got - want| <= 2e-3 * rms(want) + 1e-3 * |want|  (measured worst
+case about a third of that).  When every scale is a power of two the dequantised weights are
+exact and the gate tightens to f32-accumulation level (atol 3e-5 * rms, measured ~5e-6).
+"""
+import numpy as np
+import pytest
+
+import helpers
+import karume_amd as ka
+from helpers import oracle
+from test_gpu_linear import run_linear
+
+pytestmark = pytest.mark.gpu
+
+
+def sampled_oracle(x, packed, scale, bias, n, k, g, cols):
+    """Oracle output restricted to a sample of output columns (weight rows)."""
+    rows = packed.reshape(n, k // 2)[cols]
+    return oracle.linear_i4(x, rows.reshape(-1), scale[cols], bias[cols], len(cols), k, g)
+
+
+def check(got, want, exact_weights=False):
+    rms = float(np.sqrt(np.mean(want.astype(np.float64) ** 2)))
+    err = np.abs(got.astype(np.float64) - want)
+    if exact_weights:
+        bound = 3e-5 * rms + 1e-6 * np.abs(want)
+    else:
+        bound = 2e-3 * rms + 1e-3 * np.abs(want)
+    worst = float(np.max(err / bound))
+    assert worst <= 1.0, (worst, float(err.max()), rms)
+    return worst
+
+
+@pytest.mark.parametrize("m,n,k,g", [(512, 11008, 4096, 128), (512, 4096, 11008, 128)])
+@pytest.mark.parametrize("io", [np.float16, np.float32])
+def test_config1_prefill_gemm(gpu_ctx, m, n, k, g, io):
+    """BASELINE config 1 at full size (up- and down-projection); 192 sampled output columns
+    are checked against the f64 oracle, all rows."""
+    rng = np.random.default_rng(n + k)
+    packed, _q, scale = helpers.synthetic_int4(rng, n, k, g)
+    x = rng.normal(size=(m, k)).astype(np.float16)
+    bias = rng.normal(size=n).astype(np.float16)
+    got = run_linear(gpu_ctx, x.astype(io), packed, scale, bias, n, k, g, compute=ka.COMPUTE_F16)
+    cols = np.sort(rng.choice(n, size=192, replace=False))
+    cols[:3] = [0, 1, 63]
+    cols[-3:] = [n - 65, n - 2, n - 1]
+    cols = np.unique(cols)
+    want = sampled_oracle(x.astype(np.float32), packed, scale.astype(np.float32),
+                          bias.astype(np.float32), n, k, g, cols)
+    got_cols = got[:, cols].astype(np.float32)
+    if io == np.float16:  # add the output rounding to the budget: half an fp16 ulp of |want|
+        rms = float(np.sqrt(np.mean(want.astype(np.float64) ** 2)))
+        err = np.abs(got_cols - want)
+        bound = 2e-3 * rms + 1.5e-3 * np.abs(want) + 1e-3
+        assert np.all(err <= bound), float(np.max(err / bound))
+    else:
+        check(got_cols, want)
+
+
+@pytest.mark.parametrize("shape", [(17, 64, 64, 16), (65, 68, 48, 16), (130, 200, 96, 32),
+                                   (100, 129, 320, 64), (300, 1000, 2048, 128),
+                                   (64, 256, 512, 128), (33, 8, 128, 128)])
+def test_gemm_edges_exact_weights(gpu_ctx, shape):
+    """Tile edges in M, N and K (K not a multiple of the 64-code stage, N not a multiple of
+    the tile) with power-of-two scales: dequantised weights are exact in fp16, x is fp16, so
+    only the f32 accumulation order differs from the oracle."""
+    m, n, k, g = shape
+    rng = np.random.default_rng(m * 1000 + n)
+    q = rng.integers(-8, 8, size=(n, k), dtype=np.int8)
+    scale = (2.0 ** rng.integers(-8, -3, size=(n, k // g))).astype(np.float32)
+    packed = oracle.pack_i4(q)
+    x = rng.normal(size=(m, k)).astype(np.float16).astype(np.float32)
+    bias = rng.normal(size=n).astype(np.float32)
+    want = oracle.linear_i4(x, packed, scale, bias, n, k, g)
+    got = run_linear(gpu_ctx, x, packed, scale, bias, n, k, g, compute=ka.COMPUTE_F16)
+    check(got, want, exact_weights=True)
+    got_h = run_linear(gpu_ctx, x.astype(np.float16), packed, scale.astype(np.float16),
+                       bias.astype(np.float16), n, k, g, compute=ka.COMPUTE_F16)
+    want_h = oracle.linear_i4(x, packed, scale, bias.astype(np.float16).astype(np.float32), n, k,
+                              g)
+    assert np.max(np.abs(got_h.astype(np.float32) - want_h)
+                  - 1e-3 * np.abs(want_h)) <= 2e-3  # fp16 output rounding
+
+
+def test_gemm_reference_cases(gpu_ctx):
+    """The reference's tile-edge shapes with its own generators (M = 65 and 17 take the MFMA
+    path with KRM_COMPUTE_F16); arbitrary f32 scales, f32 x that is not fp16-representable."""
+    for case in helpers.I4_LINEAR_CASES[:2]:
+        x, packed, _q, scale, bias = helpers.make_i4_linear(case)
+        want = oracle.linear_i4(x, packed, scale, bias, case.n, case.k, case.group)
+        got = run_linear(gpu_ctx, x, packed, scale, bias, case.n, case.k, case.group,
+                         compute=ka.COMPUTE_F16)
+        check(got, want)
+
+
+def test_gemm_f32_mode_stays_on_f32_arithmetic(gpu_ctx):
+    """KRM_COMPUTE_F32 with M > 16 keeps f32 products and accumulation (the GEMV over row
+    blocks): same gate as the GEMV tests (atol 3e-5, rtol 1e-5), far tighter than fp16."""
+    rng = np.random.default_rng(5)
+    m, n, k, g = 40, 512, 1024, 128
+    packed, _q, scale = helpers.synthetic_int4(rng, n, k, g)
+    x = rng.normal(size=(m, k)).astype(np.float32)  # not fp16-representable
+    bias = rng.normal(size=n).astype(np.float32)
+    want = oracle.linear_i4(x, packed, scale.astype(np.float32), bias, n, k, g)
+    got = run_linear(gpu_ctx, x, packed, scale, bias, n, k, g, compute=ka.COMPUTE_F32)
+    ok, fails, max_abs, worst = oracle.allclose(got, want, atol=3e-5, rtol=1e-5)
+    assert ok, (fails, max_abs, worst)
