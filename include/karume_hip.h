@@ -167,6 +167,41 @@ int32_t krm_state_append(krm_ctx* ctx, krm_buf x, krm_buf slot, uint32_t kv_plan
                          uint32_t window, uint32_t past, uint32_t query, int32_t x_dtype,
                          int32_t slot_dtype);
 
+/* ---- run-time lengths on the device ---------------------------------------------------------
+ * The reference carries (pastLength, queryLength) in an 8-byte uniform owned by the generation
+ * context and rewritten every run, so that a baked plan can be replayed
+ * (packages/runtime/src/kernels/state-attention.ts:190-193,
+ * packages/runtime/src/runtime/generation-context.ts:559-591).  `lengths` below is the same
+ * idea: 16 bytes of device memory {u32 past, u32 query, u32 fault, u32 reserved}.  The
+ * `_lengths` forms of attention and append read past/query from it on the device, which lets
+ * a recorded decode step (krm_graph_*) be replayed while the sequence grows.  A step whose
+ * lengths break the run contract (query outside 1..M, past + query > C on a full slot) writes
+ * nothing and raises `fault`; krm_lengths_advance then leaves `past` unchanged. */
+int32_t krm_lengths_set(krm_ctx* ctx, krm_buf lengths, uint32_t past, uint32_t query);
+/* past += query (only when no fault is raised). */
+int32_t krm_lengths_advance(krm_ctx* ctx, krm_buf lengths);
+/* positions[i] = past + i for i < rows (the decode graph's position_ids input). */
+int32_t krm_lengths_positions(krm_ctx* ctx, krm_buf lengths, krm_buf positions_i32,
+                              uint32_t rows);
+/* history[lengths.reserved++] = token[0] (when in range): keeps the tokens of a replayed
+ * greedy loop on the device until the host reads them in one go, instead of one read-back per
+ * step (packages/models/src/generation/greedy.ts:245-252 reads back every step). */
+int32_t krm_lengths_log_token(krm_ctx* ctx, krm_buf lengths, krm_buf token_i32,
+                              krm_buf history_i32, uint32_t history_len);
+/* krm_attention_state with device lengths; `max_past` sizes the launch and the workspace. */
+int32_t krm_attention_state_lengths(krm_ctx* ctx, krm_buf q, krm_buf ins_k, krm_buf ins_v,
+                                    krm_buf slot_k, krm_buf slot_v, krm_buf out, uint32_t batch,
+                                    uint32_t heads, uint32_t kv_heads, uint32_t chunk_rows,
+                                    uint32_t depth, uint32_t capacity, uint32_t window,
+                                    float half_scale, krm_buf lengths, uint32_t max_past,
+                                    int32_t io_dtype, int32_t kv_dtype, krm_buf workspace,
+                                    size_t workspace_bytes);
+/* krm_state_append with device lengths. */
+int32_t krm_state_append_lengths(krm_ctx* ctx, krm_buf x, krm_buf slot, uint32_t kv_planes,
+                                 uint32_t chunk_rows, uint32_t depth, uint32_t capacity,
+                                 uint32_t window, krm_buf lengths, int32_t x_dtype,
+                                 int32_t slot_dtype);
+
 /* ---- ragged decode batch (no counterpart in the reference, which runs one sequence at a
  *      time: docs/decisions/0066-generation-context-state-slots.md:130-135) -----------------
  * `nseq` sequences, one query row each, packed along the slot's row axis:
@@ -188,6 +223,43 @@ int32_t krm_attention_varlen(krm_ctx* ctx, krm_buf q, krm_buf ins_k, krm_buf ins
                              uint32_t kv_heads, uint32_t depth, uint64_t total_rows,
                              float half_scale, int32_t io_dtype, int32_t kv_dtype,
                              krm_buf workspace, size_t workspace_bytes);
+
+/* ---- decoder-layer glue ops (f32 arithmetic; activations f32 or fp16) ------------------------
+ * The ops a Llama-style layer runs around the linears and the attention in the decode graph
+ * (tools/export-recipes/minicpm5/export_decode.py:14-35).  Each one follows the reference
+ * kernel of the same name. */
+
+/* out[r, i] = x[r, i] * rsqrt(mean_i(x[r]^2) + eps) * weight[i]; weight is f32.
+ * packages/runtime/src/kernels/rms-norm.ts:35-91 */
+int32_t krm_rms_norm(krm_ctx* ctx, krm_buf x, krm_buf weight_f32, krm_buf out, uint32_t rows,
+                     uint32_t dim, float eps, int32_t io_dtype);
+/* Half-split RoPE: out = x*cos[pos] + rotate_half(x)*sin[pos] with cos/sin rows [table_rows, D]
+ * (f32) looked up by positions[row] (i32, device); both products are rounded before the add
+ * (packages/runtime/src/kernels/rope.ts:5-20,52-80).  x is [rows, heads, D]; out is
+ * [heads, rows, D] when to_head_major != 0 (what the attention reads), else [rows, heads, D].
+ * A position outside the table yields NaN (the reference's out-of-range gather does too). */
+int32_t krm_rope_half(krm_ctx* ctx, krm_buf x, krm_buf positions_i32, krm_buf cos_table_f32,
+                      krm_buf sin_table_f32, krm_buf out, uint32_t rows, uint32_t heads,
+                      uint32_t head_dim, uint32_t table_rows, int32_t to_head_major,
+                      int32_t io_dtype);
+/* [a, b, d] -> [b, a, d] (the reshape + permute between linears and attention). */
+int32_t krm_transpose_01(krm_ctx* ctx, krm_buf x, krm_buf out, uint32_t a, uint32_t b, uint32_t d,
+                         int32_t io_dtype);
+/* out = (gate * sigmoid(gate)) * up, the sigmoid and both products rounded to f32 in turn
+ * (packages/runtime/src/kernels/silu.ts:47-93). */
+int32_t krm_silu_mul(krm_ctx* ctx, krm_buf gate, krm_buf up, krm_buf out, uint64_t count,
+                     int32_t io_dtype);
+/* out = a + b (packages/runtime/src/codegen/elementwise.ts). */
+int32_t krm_add(krm_ctx* ctx, krm_buf a, krm_buf b, krm_buf out, uint64_t count,
+                int32_t io_dtype);
+/* out[r, :] = table[index[r], :]; an index outside [0, vocab) fills the row with NaN, it is
+ * never clamped (packages/runtime/src/kernels/embedding.ts:1-43). */
+int32_t krm_embedding(krm_ctx* ctx, krm_buf table, krm_buf index_i32, krm_buf out, uint32_t rows,
+                      uint32_t vocab, uint32_t hidden, int32_t table_dtype, int32_t out_dtype);
+/* out[r] = argmax_i x[r, i]: ties -> smallest index, NaN is the maximum, all -inf -> 0
+ * (packages/runtime/src/kernels/argmax.ts:16-34). */
+int32_t krm_argmax(krm_ctx* ctx, krm_buf x, krm_buf out_i32, uint32_t rows, uint32_t dim,
+                   int32_t io_dtype);
 
 #ifdef __cplusplus
 }

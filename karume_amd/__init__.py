@@ -10,7 +10,12 @@ from .runtime import (COMPUTE_F16, COMPUTE_F32, F16, F32, DeviceBuffer, Executio
                       GpuContext, GpuDeviceLostError, GpuEvent, GpuGraph, GpuOutOfMemoryError,
                       GpuValidationError, KarumeError, acquire_gpu, dtype_code, version)
 
+from .generation import (GenerationContext, GenerationContextError, PrefillChunk,
+                         generate_greedy, plan_prefill_chunks)
+
 __all__ = [
+    "GenerationContext", "GenerationContextError", "PrefillChunk", "generate_greedy",
+    "plan_prefill_chunks",
     "I4Error", "check_int4", "group_scale_shape", "pack_int4",
     "COMPUTE_F16", "COMPUTE_F32", "F16", "F32", "DeviceBuffer", "ExecutionError", "GpuContext",
     "GpuDeviceLostError", "GpuEvent", "GpuGraph", "GpuOutOfMemoryError", "GpuValidationError", "KarumeError",

@@ -52,6 +52,23 @@ PROTOTYPES = {
     "krm_attention_varlen": (i32, [c_ctx, c_buf, c_buf, c_buf, c_buf, c_buf, c_buf,
                                    C.POINTER(i32), u32, u32, u32, u32, u64, C.c_float, i32, i32,
                                    c_buf, size_t]),
+    "krm_lengths_set": (i32, [c_ctx, c_buf, u32, u32]),
+    "krm_lengths_advance": (i32, [c_ctx, c_buf]),
+    "krm_lengths_positions": (i32, [c_ctx, c_buf, c_buf, u32]),
+    "krm_lengths_log_token": (i32, [c_ctx, c_buf, c_buf, c_buf, u32]),
+    "krm_attention_state_lengths": (i32, [c_ctx, c_buf, c_buf, c_buf, c_buf, c_buf, c_buf, u32,
+                                          u32, u32, u32, u32, u32, u32, C.c_float, c_buf, u32,
+                                          i32, i32, c_buf, size_t]),
+    "krm_state_append_lengths": (i32, [c_ctx, c_buf, c_buf, u32, u32, u32, u32, u32, c_buf, i32,
+                                       i32]),
+    "krm_rms_norm": (i32, [c_ctx, c_buf, c_buf, c_buf, u32, u32, C.c_float, i32]),
+    "krm_rope_half": (i32, [c_ctx, c_buf, c_buf, c_buf, c_buf, c_buf, u32, u32, u32, u32, i32,
+                            i32]),
+    "krm_transpose_01": (i32, [c_ctx, c_buf, c_buf, u32, u32, u32, i32]),
+    "krm_silu_mul": (i32, [c_ctx, c_buf, c_buf, c_buf, u64, i32]),
+    "krm_add": (i32, [c_ctx, c_buf, c_buf, c_buf, u64, i32]),
+    "krm_embedding": (i32, [c_ctx, c_buf, c_buf, c_buf, u32, u32, u32, i32, i32]),
+    "krm_argmax": (i32, [c_ctx, c_buf, c_buf, u32, u32, i32]),
 }
 
 _lib = None

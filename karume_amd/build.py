@@ -23,7 +23,7 @@ HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = [
     "-O3", "-std=c++17", "-fPIC", "--offload-arch=gfx950",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
-    "-fno-fast-math", "-Wall", "-Wno-unused-function", "-Wno-unknown-warning-option",
+    "-fno-fast-math", "-ffp-contract=off", "-Wall", "-Wno-unused-function", "-Wno-unknown-warning-option",
 ]
 
 

@@ -50,7 +50,24 @@ __host__ __device__ inline uint64_t window_low(uint32_t window, uint64_t limit) 
 struct GenericArgs {
   uint32_t heads, kv_heads, chunk_rows, depth, capacity, window, past, query;
   float scale;
+  uint32_t* lengths;  // device {past, query, fault} overriding past / query when not null
 };
+
+// Run-time lengths read on the device (the reference carries them in a uniform buffer the
+// generation context rewrites every run, packages/runtime/src/kernels/state-attention.ts:
+// 190-193).  The host checks of the scalar form are repeated here; a violation raises the
+// fault word instead of touching memory.
+__device__ inline bool device_lengths(uint32_t* lengths, uint32_t chunk_rows, uint32_t capacity,
+                                      uint32_t window, uint32_t& past, uint32_t& query) {
+  if (!lengths) return true;
+  past = lengths[0];
+  query = lengths[1];
+  const bool ok = query >= 1 && query <= chunk_rows &&
+                  (uint64_t)past + query <= 0xffffffffull &&
+                  (window != 0 || (uint64_t)past + query <= capacity);
+  if (!ok && threadIdx.x == 0) lengths[2] = 1u;
+  return ok;
+}
 
 // One workgroup per (plane z = b*H + h, row).  Columns are walked 256 at a time: a thread
 // scores one column (serial dot over D), the block folds the chunk into the running
@@ -70,6 +87,7 @@ __global__ __launch_bounds__(kThreads) void attention_generic_kernel(
   const uint32_t tid = threadIdx.x;
   const uint32_t D = a.depth;
   const size_t q_base = ((size_t)z * a.chunk_rows + row) * D;
+  if (!device_lengths(a.lengths, a.chunk_rows, a.capacity, a.window, a.past, a.query)) return;
 
   if (row >= a.query) {  // pad row: exact zeros, nothing is read
     for (uint32_t d = tid; d < D; d += kThreads) st_f32<XT>(out, q_base + d, 0.0f);
@@ -219,6 +237,8 @@ struct DecodeArgs {
   const int32_t* cu_rows;    // ragged batch: [nseq+1] first slot row of each sequence
   const int32_t* split_prefix;  // ragged batch: [nseq+1] first global split of each sequence
   uint32_t* tickets;         // [nseq * kv_heads] arrival counters, zero between launches
+  uint32_t* lengths;         // single sequence: device {past, query, fault} or null
+  uint32_t capacity;         // single sequence: slot rows (checked against device lengths)
 };
 
 __host__ __device__ inline uint32_t decode_split_columns(uint32_t lanes_per_row) {
@@ -286,10 +306,13 @@ void attention_decode_kernel(
     past = (uint64_t)a.cu_rows[seq + 1] - row_base;
   } else {
     seq = blockIdx.z;
-    past = a.past;
+    uint32_t p32 = a.past, q32 = 1;
+    if (!device_lengths(a.lengths, 1, a.capacity, a.window, p32, q32)) return;
+    past = p32;
     row_base = 0;
     nsplit = decode_splits(past - window_low(a.window, past), kDecodeIter * G);
     split = blockIdx.x;
+    if (split >= nsplit) return;  // the grid is sized for the longest past it may see
     first_split = seq * nsplit;
   }
   const uint64_t low = window_low(a.window, past);  // limit of row 0 is `past`
@@ -649,13 +672,18 @@ int32_t krm_attention_state_workspace(uint32_t batch, uint32_t heads, uint32_t k
   return KRM_OK;
 }
 
-int32_t krm_attention_state(krm_ctx* ctx, krm_buf q, krm_buf ins_k, krm_buf ins_v,
-                            krm_buf slot_k, krm_buf slot_v, krm_buf out, uint32_t batch,
-                            uint32_t heads, uint32_t kv_heads, uint32_t chunk_rows,
-                            uint32_t depth, uint32_t capacity, uint32_t window,
-                            float half_scale, uint32_t past, uint32_t query, int32_t io_dtype,
-                            int32_t kv_dtype, krm_buf workspace, size_t workspace_bytes) {
+// `lengths` == 0: past / query are this run's values.  Otherwise they are read on the device
+// and `past` is the largest pastLength the launch has to be sized for.
+static int32_t attention_state_impl(krm_ctx* ctx, krm_buf q, krm_buf ins_k, krm_buf ins_v,
+                                    krm_buf slot_k, krm_buf slot_v, krm_buf out, uint32_t batch,
+                                    uint32_t heads, uint32_t kv_heads, uint32_t chunk_rows,
+                                    uint32_t depth, uint32_t capacity, uint32_t window,
+                                    float half_scale, uint32_t past, uint32_t query,
+                                    krm_buf lengths, int32_t io_dtype, int32_t kv_dtype,
+                                    krm_buf workspace, size_t workspace_bytes) {
   KRM_TRY(enter(ctx));
+  const bool dyn = lengths != 0;
+  KRM_REQUIRE(ctx, aligned(lengths, 4), "krm_attention_state: misaligned lengths buffer");
   KRM_REQUIRE(ctx, valid_dtype(io_dtype) && valid_dtype(kv_dtype),
               "krm_attention_state: io_dtype %d / kv_dtype %d", io_dtype, kv_dtype);
   KRM_REQUIRE(ctx,
@@ -673,14 +701,14 @@ int32_t krm_attention_state(krm_ctx* ctx, krm_buf q, krm_buf ins_k, krm_buf ins_
   KRM_REQUIRE(ctx, (uint64_t)batch * heads <= 0x7fffffffull && chunk_rows <= 65535,
               "krm_attention_state: B*H = %llu or M = %u exceeds the launch grid",
               (unsigned long long)batch * heads, chunk_rows);
-  if (query < 1 || query > chunk_rows)
+  if (!dyn && (query < 1 || query > chunk_rows))
     return fail(ctx, KRM_ERR_EXECUTION, "krm_attention_state: queryLength %u is outside 1..%u",
                 query, chunk_rows);
-  if ((uint64_t)past + query > 0xffffffffull)
+  if (!dyn && (uint64_t)past + query > 0xffffffffull)
     return fail(ctx, KRM_ERR_EXECUTION,
                 "krm_attention_state: pastLength %u + queryLength %u does not fit in 32 bits",
                 past, query);
-  if (window == 0 && (uint64_t)past + query > capacity)
+  if (!dyn && window == 0 && (uint64_t)past + query > capacity)
     return fail(ctx, KRM_ERR_EXECUTION,
                 "krm_attention_state: pastLength %u + queryLength %u exceeds capacity %u", past,
                 query, capacity);
@@ -694,7 +722,7 @@ int32_t krm_attention_state(krm_ctx* ctx, krm_buf q, krm_buf ins_k, krm_buf ins_
 
   const uint32_t repeat = heads / kv_heads;
   const uint32_t lpr = decode_lanes_per_row(depth, kv_dtype);
-  const bool fast = query == 1 && chunk_rows == 1 && lpr && decode_repeat_ok(repeat) &&
+  const bool fast = (dyn || query == 1) && chunk_rows == 1 && lpr && decode_repeat_ok(repeat) &&
                     aligned(slot_k, 16) && aligned(slot_v, 16) && batch <= 65535 &&
                     kv_heads <= 65535 && (uint64_t)batch * kv_heads <= kTicketSlots;
   if (fast) {
@@ -713,6 +741,8 @@ int32_t krm_attention_state(krm_ctx* ctx, krm_buf q, krm_buf ins_k, krm_buf ins_
     L.grid_x = nsplit;
     L.grid_z = batch;
     L.args.tickets = ctx->tickets;
+    L.args.lengths = ptr<uint32_t>(lengths);
+    L.args.capacity = capacity;
     if (nsplit > 1) {
       const size_t ml_floats = (size_t)batch * nsplit * heads * 2;
       const size_t need = (ml_floats + (size_t)batch * nsplit * heads * depth) * sizeof(float);
@@ -728,7 +758,8 @@ int32_t krm_attention_state(krm_ctx* ctx, krm_buf q, krm_buf ins_k, krm_buf ins_
     return decode_dispatch<false>(ctx, L, repeat, lpr, io_dtype, kv_dtype);
   }
 
-  GenericArgs a{heads, kv_heads, chunk_rows, depth, capacity, window, past, query, half_scale};
+  GenericArgs a{heads, kv_heads, chunk_rows, depth, capacity, window, past, query, half_scale,
+                ptr<uint32_t>(lengths)};
   if (io_dtype == KRM_F32 && kv_dtype == KRM_F32)
     return launch_generic<float, float>(ctx, q, ins_k, ins_v, slot_k, slot_v, out, batch, a);
   if (io_dtype == KRM_F16 && kv_dtype == KRM_F16)
@@ -736,6 +767,30 @@ int32_t krm_attention_state(krm_ctx* ctx, krm_buf q, krm_buf ins_k, krm_buf ins_
   if (io_dtype == KRM_F32 && kv_dtype == KRM_F16)
     return launch_generic<float, __half>(ctx, q, ins_k, ins_v, slot_k, slot_v, out, batch, a);
   return launch_generic<__half, float>(ctx, q, ins_k, ins_v, slot_k, slot_v, out, batch, a);
+}
+
+int32_t krm_attention_state(krm_ctx* ctx, krm_buf q, krm_buf ins_k, krm_buf ins_v,
+                            krm_buf slot_k, krm_buf slot_v, krm_buf out, uint32_t batch,
+                            uint32_t heads, uint32_t kv_heads, uint32_t chunk_rows,
+                            uint32_t depth, uint32_t capacity, uint32_t window,
+                            float half_scale, uint32_t past, uint32_t query, int32_t io_dtype,
+                            int32_t kv_dtype, krm_buf workspace, size_t workspace_bytes) {
+  return attention_state_impl(ctx, q, ins_k, ins_v, slot_k, slot_v, out, batch, heads, kv_heads,
+                              chunk_rows, depth, capacity, window, half_scale, past, query, 0,
+                              io_dtype, kv_dtype, workspace, workspace_bytes);
+}
+
+int32_t krm_attention_state_lengths(krm_ctx* ctx, krm_buf q, krm_buf ins_k, krm_buf ins_v,
+                                    krm_buf slot_k, krm_buf slot_v, krm_buf out, uint32_t batch,
+                                    uint32_t heads, uint32_t kv_heads, uint32_t chunk_rows,
+                                    uint32_t depth, uint32_t capacity, uint32_t window,
+                                    float half_scale, krm_buf lengths, uint32_t max_past,
+                                    int32_t io_dtype, int32_t kv_dtype, krm_buf workspace,
+                                    size_t workspace_bytes) {
+  if (!lengths) return fail(ctx, KRM_ERR_VALIDATION, "krm_attention_state_lengths: NULL lengths");
+  return attention_state_impl(ctx, q, ins_k, ins_v, slot_k, slot_v, out, batch, heads, kv_heads,
+                              chunk_rows, depth, capacity, window, half_scale, max_past,
+                              chunk_rows, lengths, io_dtype, kv_dtype, workspace, workspace_bytes);
 }
 
 int32_t krm_attention_varlen_workspace(uint32_t nseq, uint32_t heads, uint32_t kv_heads,

@@ -1,0 +1,354 @@
+// The small ops a Llama-style decoder layer runs between the linears and the attention:
+// rms_norm, half-split RoPE with a position table, SiLU-gate, residual add, embedding gather,
+// argmax and the [rows, heads, D] <-> [heads, rows, D] transposition.  Each follows the
+// reference kernel of the same name (cited per kernel); activations may be f32 or fp16,
+// arithmetic is f32.
+#include "krm_internal.h"
+
+#include <cmath>
+
+using namespace krm;
+
+namespace {
+
+constexpr int kThreads = 256;
+
+template <typename T>
+__device__ inline float ld(const T* p, size_t i);
+template <>
+__device__ inline float ld<float>(const float* p, size_t i) { return p[i]; }
+template <>
+__device__ inline float ld<__half>(const __half* p, size_t i) { return __half2float(p[i]); }
+template <typename T>
+__device__ inline void st(T* p, size_t i, float v);
+template <>
+__device__ inline void st<float>(float* p, size_t i, float v) { p[i] = v; }
+template <>
+__device__ inline void st<__half>(__half* p, size_t i, float v) { p[i] = __float2half_rn(v); }
+
+__device__ inline float block_sum(float v, float* scratch) {
+  for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, kWave);
+  const int wave = threadIdx.x >> 6;
+  if ((threadIdx.x & 63) == 0) scratch[wave] = v;
+  __syncthreads();
+  float total = 0.f;
+  for (int w = 0; w < kThreads / kWave; ++w) total += scratch[w];
+  __syncthreads();
+  return total;
+}
+
+// rms_norm: out = x * rsqrt(mean(x^2) + eps) * weight, one workgroup per row.
+// packages/runtime/src/kernels/rms-norm.ts:35-91 (no mean subtraction; weight is f32).
+template <typename XT>
+__global__ __launch_bounds__(kThreads) void rms_norm_kernel(const XT* __restrict__ x,
+                                                           const float* __restrict__ weight,
+                                                           XT* __restrict__ out, uint32_t dim,
+                                                           float eps) {
+  __shared__ float scratch[kThreads / kWave];
+  const size_t base = (size_t)blockIdx.x * dim;
+  float squares = 0.f;
+  for (uint32_t i = threadIdx.x; i < dim; i += kThreads) {
+    const float v = ld<XT>(x, base + i);
+    squares = fmaf(v, v, squares);
+  }
+  const float total = block_sum(squares, scratch);
+  const float inv = 1.0f / sqrtf(total / (float)dim + eps);
+  for (uint32_t i = threadIdx.x; i < dim; i += kThreads)
+    st<XT>(out, base + i, ld<XT>(x, base + i) * inv * weight[i]);
+}
+
+// Half-split RoPE with the cos / sin rows looked up by absolute position:
+//   out = x*cos[pos] + rotate_half(x)*sin[pos],  rotate_half(x) = cat(-x[D/2:], x[:D/2]).
+// Both products are rounded before the add, as in the reference's fused kernel
+// (packages/runtime/src/kernels/rope.ts:5-20,52-80); the table lookup is the decode graph's
+// embedding(position_ids, table) (tools/export-recipes/minicpm5/export_decode.py:24-35).
+// `x` is [rows, heads, D] (the layout a linear writes); `out` is [heads, rows, D] (the layout
+// the attention reads) when to_head_major is set, otherwise the same layout as `x`.
+template <typename XT>
+__global__ __launch_bounds__(kThreads) void rope_kernel(
+    const XT* __restrict__ x, const int32_t* __restrict__ positions,
+    const float* __restrict__ cos_table, const float* __restrict__ sin_table,
+    XT* __restrict__ out, uint32_t rows, uint32_t heads, uint32_t head_dim,
+    uint32_t table_rows, uint32_t to_head_major) {
+  const size_t total = (size_t)rows * heads * head_dim;
+  const uint32_t half = head_dim / 2;
+  const size_t stride = (size_t)gridDim.x * blockDim.x;
+  for (size_t i = blockIdx.x * (size_t)blockDim.x + threadIdx.x; i < total; i += stride) {
+    const uint32_t d = (uint32_t)(i % head_dim);
+    const size_t rest = i / head_dim;
+    const uint32_t head = (uint32_t)(rest % heads);
+    const uint32_t row = (uint32_t)(rest / heads);
+    const int32_t pos = positions[row];
+    const size_t row_base = i - d;
+    float value;
+    if (pos < 0 || (uint32_t)pos >= table_rows) {
+      value = NAN;  // a position outside the table must not look like a valid rotation
+    } else {
+      const float self = ld<XT>(x, i);
+      const float other = d < half ? -ld<XT>(x, row_base + d + half) : ld<XT>(x, row_base + d - half);
+      const size_t t = (size_t)pos * head_dim + d;
+      const float direct = __fmul_rn(self, cos_table[t]);
+      const float cross = __fmul_rn(other, sin_table[t]);
+      value = __fadd_rn(direct, cross);
+    }
+    const size_t dst = to_head_major ? ((size_t)head * rows + row) * head_dim + d : i;
+    st<XT>(out, dst, value);
+  }
+}
+
+// [a, b, d] -> [b, a, d]
+template <typename XT>
+__global__ __launch_bounds__(kThreads) void transpose_kernel(const XT* __restrict__ x,
+                                                            XT* __restrict__ out, uint32_t a,
+                                                            uint32_t b, uint32_t d) {
+  const size_t total = (size_t)a * b * d;
+  const size_t stride = (size_t)gridDim.x * blockDim.x;
+  for (size_t i = blockIdx.x * (size_t)blockDim.x + threadIdx.x; i < total; i += stride) {
+    const uint32_t e = (uint32_t)(i % d);
+    const size_t rest = i / d;
+    const uint32_t bi = (uint32_t)(rest % b);
+    const uint32_t ai = (uint32_t)(rest / b);
+    out[((size_t)bi * a + ai) * d + e] = x[i];
+  }
+}
+
+// silu(gate) * up with the reference's roundings: s = sigmoid_stable(gate) is rounded, then
+// gate*s, then *up (packages/runtime/src/kernels/silu.ts:47-93,
+// packages/runtime/src/codegen/elementwise.ts:187-190).
+__device__ inline float sigmoid_stable(float v) {
+  const float t = expf(-fabsf(v));
+  return v < 0.f ? t / (1.0f + t) : 1.0f / (1.0f + t);
+}
+template <typename XT>
+__global__ __launch_bounds__(kThreads) void silu_mul_kernel(const XT* __restrict__ gate,
+                                                           const XT* __restrict__ up,
+                                                           XT* __restrict__ out, size_t count) {
+  const size_t stride = (size_t)gridDim.x * blockDim.x;
+  for (size_t i = blockIdx.x * (size_t)blockDim.x + threadIdx.x; i < count; i += stride) {
+    const float g = ld<XT>(gate, i);
+    const float act = __fmul_rn(g, sigmoid_stable(g));
+    st<XT>(out, i, __fmul_rn(act, ld<XT>(up, i)));
+  }
+}
+
+// elementwise add (the residual connections).  packages/runtime/src/codegen/elementwise.ts
+template <typename XT>
+__global__ __launch_bounds__(kThreads) void add_kernel(const XT* __restrict__ a,
+                                                      const XT* __restrict__ b,
+                                                      XT* __restrict__ out, size_t count) {
+  const size_t stride = (size_t)gridDim.x * blockDim.x;
+  for (size_t i = blockIdx.x * (size_t)blockDim.x + threadIdx.x; i < count; i += stride)
+    st<XT>(out, i, __fadd_rn(ld<XT>(a, i), ld<XT>(b, i)));
+}
+
+// embedding row gather; an index outside [0, vocab) writes NaN to that row, it is never
+// clamped (packages/runtime/src/kernels/embedding.ts:1-43).
+template <typename WT, typename XT>
+__global__ __launch_bounds__(kThreads) void embedding_kernel(const WT* __restrict__ table,
+                                                            const int32_t* __restrict__ index,
+                                                            XT* __restrict__ out, uint32_t rows,
+                                                            uint32_t vocab, uint32_t hidden) {
+  const size_t total = (size_t)rows * hidden;
+  const size_t stride = (size_t)gridDim.x * blockDim.x;
+  for (size_t i = blockIdx.x * (size_t)blockDim.x + threadIdx.x; i < total; i += stride) {
+    const uint32_t col = (uint32_t)(i % hidden);
+    const int32_t pick = index[i / hidden];
+    const float v = (pick < 0 || (uint32_t)pick >= vocab) ? NAN
+                                                          : ld<WT>(table, (size_t)pick * hidden + col);
+    st<XT>(out, i, v);
+  }
+}
+
+// argmax over the last dim: ties -> smallest index, NaN counts as the maximum, a row of -inf
+// gives 0 (packages/runtime/src/kernels/argmax.ts:16-34).  (value, index) pairs are ordered
+// lexicographically (value descending, index ascending), so the tree shape does not matter.
+__device__ inline bool beats(float va, uint32_t ia, float vb, uint32_t ib) {
+  const bool na = va != va, nb = vb != vb;
+  if (na != nb) return na;
+  if (!na && va != vb) return va > vb;
+  return ia < ib;
+}
+template <typename XT>
+__global__ __launch_bounds__(kThreads) void argmax_kernel(const XT* __restrict__ x,
+                                                         int32_t* __restrict__ out, uint32_t dim) {
+  __shared__ float s_val[kThreads / kWave];
+  __shared__ uint32_t s_idx[kThreads / kWave];
+  const size_t base = (size_t)blockIdx.x * dim;
+  float best = -INFINITY;
+  uint32_t at = dim;  // sentinel: any real element beats it on the index comparison
+  for (uint32_t i = threadIdx.x; i < dim; i += kThreads) {
+    const float v = ld<XT>(x, base + i);
+    if (beats(v, i, best, at)) {
+      best = v;
+      at = i;
+    }
+  }
+  for (int off = 32; off > 0; off >>= 1) {
+    const float ov = __shfl_xor(best, off, kWave);
+    const uint32_t oi = (uint32_t)__shfl_xor((int)at, off, kWave);
+    if (beats(ov, oi, best, at)) {
+      best = ov;
+      at = oi;
+    }
+  }
+  if ((threadIdx.x & 63) == 0) {
+    s_val[threadIdx.x >> 6] = best;
+    s_idx[threadIdx.x >> 6] = at;
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    for (int w = 1; w < kThreads / kWave; ++w)
+      if (beats(s_val[w], s_idx[w], best, at)) {
+        best = s_val[w];
+        at = s_idx[w];
+      }
+    out[blockIdx.x] = (int32_t)at;
+  }
+}
+
+inline unsigned grid_for(size_t total) {
+  size_t blocks = (total + kThreads - 1) / kThreads;
+  if (blocks > 4096) blocks = 4096;
+  return (unsigned)(blocks ? blocks : 1);
+}
+
+}  // namespace
+
+#define KRM_IO_DISPATCH(io_dtype, CALL_F32, CALL_F16) \
+  do {                                                \
+    if ((io_dtype) == KRM_F32) {                      \
+      CALL_F32;                                       \
+    } else {                                          \
+      CALL_F16;                                       \
+    }                                                 \
+  } while (0)
+
+extern "C" {
+
+int32_t krm_rms_norm(krm_ctx* ctx, krm_buf x, krm_buf weight_f32, krm_buf out, uint32_t rows,
+                     uint32_t dim, float eps, int32_t io_dtype) {
+  KRM_TRY(enter(ctx));
+  KRM_REQUIRE(ctx, valid_dtype(io_dtype), "krm_rms_norm: io_dtype %d", io_dtype);
+  KRM_REQUIRE(ctx, dim >= 1 && std::isfinite(eps), "krm_rms_norm: dim %u / eps", dim);
+  if (rows == 0) return KRM_OK;
+  KRM_REQUIRE(ctx, x && weight_f32 && out, "krm_rms_norm: NULL buffer");
+  KRM_IO_DISPATCH(io_dtype,
+                  (rms_norm_kernel<float><<<dim3(rows), dim3(kThreads), 0, ctx->stream>>>(
+                      ptr<const float>(x), ptr<const float>(weight_f32), ptr<float>(out), dim, eps)),
+                  (rms_norm_kernel<__half><<<dim3(rows), dim3(kThreads), 0, ctx->stream>>>(
+                      ptr<const __half>(x), ptr<const float>(weight_f32), ptr<__half>(out), dim,
+                      eps)));
+  return launched(ctx, "rms_norm_kernel");
+}
+
+int32_t krm_rope_half(krm_ctx* ctx, krm_buf x, krm_buf positions_i32, krm_buf cos_table_f32,
+                      krm_buf sin_table_f32, krm_buf out, uint32_t rows, uint32_t heads,
+                      uint32_t head_dim, uint32_t table_rows, int32_t to_head_major,
+                      int32_t io_dtype) {
+  KRM_TRY(enter(ctx));
+  KRM_REQUIRE(ctx, valid_dtype(io_dtype), "krm_rope_half: io_dtype %d", io_dtype);
+  KRM_REQUIRE(ctx, head_dim >= 2 && head_dim % 2 == 0, "krm_rope_half: head_dim %u is odd",
+              head_dim);
+  if (rows == 0 || heads == 0) return KRM_OK;
+  KRM_REQUIRE(ctx, x && positions_i32 && cos_table_f32 && sin_table_f32 && out,
+              "krm_rope_half: NULL buffer");
+  KRM_REQUIRE(ctx, !(to_head_major && x == out && rows > 1 && heads > 1),
+              "krm_rope_half: the transposing form cannot run in place");
+  const size_t total = (size_t)rows * heads * head_dim;
+  KRM_IO_DISPATCH(io_dtype,
+                  (rope_kernel<float><<<dim3(grid_for(total)), dim3(kThreads), 0, ctx->stream>>>(
+                      ptr<const float>(x), ptr<const int32_t>(positions_i32),
+                      ptr<const float>(cos_table_f32), ptr<const float>(sin_table_f32),
+                      ptr<float>(out), rows, heads, head_dim, table_rows, (uint32_t)to_head_major)),
+                  (rope_kernel<__half><<<dim3(grid_for(total)), dim3(kThreads), 0, ctx->stream>>>(
+                      ptr<const __half>(x), ptr<const int32_t>(positions_i32),
+                      ptr<const float>(cos_table_f32), ptr<const float>(sin_table_f32),
+                      ptr<__half>(out), rows, heads, head_dim, table_rows,
+                      (uint32_t)to_head_major)));
+  return launched(ctx, "rope_kernel");
+}
+
+int32_t krm_transpose_01(krm_ctx* ctx, krm_buf x, krm_buf out, uint32_t a, uint32_t b, uint32_t d,
+                         int32_t io_dtype) {
+  KRM_TRY(enter(ctx));
+  KRM_REQUIRE(ctx, valid_dtype(io_dtype), "krm_transpose_01: io_dtype %d", io_dtype);
+  const size_t total = (size_t)a * b * d;
+  if (total == 0) return KRM_OK;
+  KRM_REQUIRE(ctx, x && out && x != out, "krm_transpose_01: NULL or aliased buffer");
+  KRM_IO_DISPATCH(io_dtype,
+                  (transpose_kernel<float><<<dim3(grid_for(total)), dim3(kThreads), 0, ctx->stream>>>(
+                      ptr<const float>(x), ptr<float>(out), a, b, d)),
+                  (transpose_kernel<__half><<<dim3(grid_for(total)), dim3(kThreads), 0, ctx->stream>>>(
+                      ptr<const __half>(x), ptr<__half>(out), a, b, d)));
+  return launched(ctx, "transpose_kernel");
+}
+
+int32_t krm_silu_mul(krm_ctx* ctx, krm_buf gate, krm_buf up, krm_buf out, uint64_t count,
+                     int32_t io_dtype) {
+  KRM_TRY(enter(ctx));
+  KRM_REQUIRE(ctx, valid_dtype(io_dtype), "krm_silu_mul: io_dtype %d", io_dtype);
+  if (count == 0) return KRM_OK;
+  KRM_REQUIRE(ctx, gate && up && out, "krm_silu_mul: NULL buffer");
+  KRM_IO_DISPATCH(io_dtype,
+                  (silu_mul_kernel<float><<<dim3(grid_for(count)), dim3(kThreads), 0, ctx->stream>>>(
+                      ptr<const float>(gate), ptr<const float>(up), ptr<float>(out), count)),
+                  (silu_mul_kernel<__half><<<dim3(grid_for(count)), dim3(kThreads), 0, ctx->stream>>>(
+                      ptr<const __half>(gate), ptr<const __half>(up), ptr<__half>(out), count)));
+  return launched(ctx, "silu_mul_kernel");
+}
+
+int32_t krm_add(krm_ctx* ctx, krm_buf a, krm_buf b, krm_buf out, uint64_t count,
+                int32_t io_dtype) {
+  KRM_TRY(enter(ctx));
+  KRM_REQUIRE(ctx, valid_dtype(io_dtype), "krm_add: io_dtype %d", io_dtype);
+  if (count == 0) return KRM_OK;
+  KRM_REQUIRE(ctx, a && b && out, "krm_add: NULL buffer");
+  KRM_IO_DISPATCH(io_dtype,
+                  (add_kernel<float><<<dim3(grid_for(count)), dim3(kThreads), 0, ctx->stream>>>(
+                      ptr<const float>(a), ptr<const float>(b), ptr<float>(out), count)),
+                  (add_kernel<__half><<<dim3(grid_for(count)), dim3(kThreads), 0, ctx->stream>>>(
+                      ptr<const __half>(a), ptr<const __half>(b), ptr<__half>(out), count)));
+  return launched(ctx, "add_kernel");
+}
+
+int32_t krm_embedding(krm_ctx* ctx, krm_buf table, krm_buf index_i32, krm_buf out, uint32_t rows,
+                      uint32_t vocab, uint32_t hidden, int32_t table_dtype, int32_t out_dtype) {
+  KRM_TRY(enter(ctx));
+  KRM_REQUIRE(ctx, valid_dtype(table_dtype) && valid_dtype(out_dtype),
+              "krm_embedding: table_dtype %d / out_dtype %d", table_dtype, out_dtype);
+  KRM_REQUIRE(ctx, vocab >= 1 && hidden >= 1, "krm_embedding: vocab %u / hidden %u", vocab, hidden);
+  if (rows == 0) return KRM_OK;
+  KRM_REQUIRE(ctx, table && index_i32 && out, "krm_embedding: NULL buffer");
+  const size_t total = (size_t)rows * hidden;
+  const dim3 grid(grid_for(total)), block(kThreads);
+  if (table_dtype == KRM_F16 && out_dtype == KRM_F16)
+    embedding_kernel<__half, __half><<<grid, block, 0, ctx->stream>>>(
+        ptr<const __half>(table), ptr<const int32_t>(index_i32), ptr<__half>(out), rows, vocab, hidden);
+  else if (table_dtype == KRM_F16)
+    embedding_kernel<__half, float><<<grid, block, 0, ctx->stream>>>(
+        ptr<const __half>(table), ptr<const int32_t>(index_i32), ptr<float>(out), rows, vocab, hidden);
+  else if (out_dtype == KRM_F16)
+    embedding_kernel<float, __half><<<grid, block, 0, ctx->stream>>>(
+        ptr<const float>(table), ptr<const int32_t>(index_i32), ptr<__half>(out), rows, vocab, hidden);
+  else
+    embedding_kernel<float, float><<<grid, block, 0, ctx->stream>>>(
+        ptr<const float>(table), ptr<const int32_t>(index_i32), ptr<float>(out), rows, vocab, hidden);
+  return launched(ctx, "embedding_kernel");
+}
+
+int32_t krm_argmax(krm_ctx* ctx, krm_buf x, krm_buf out_i32, uint32_t rows, uint32_t dim,
+                   int32_t io_dtype) {
+  KRM_TRY(enter(ctx));
+  KRM_REQUIRE(ctx, valid_dtype(io_dtype), "krm_argmax: io_dtype %d", io_dtype);
+  KRM_REQUIRE(ctx, dim >= 1, "krm_argmax: the reduced dimension is empty");
+  if (rows == 0) return KRM_OK;
+  KRM_REQUIRE(ctx, x && out_i32, "krm_argmax: NULL buffer");
+  KRM_IO_DISPATCH(io_dtype,
+                  (argmax_kernel<float><<<dim3(rows), dim3(kThreads), 0, ctx->stream>>>(
+                      ptr<const float>(x), ptr<int32_t>(out_i32), dim)),
+                  (argmax_kernel<__half><<<dim3(rows), dim3(kThreads), 0, ctx->stream>>>(
+                      ptr<const __half>(x), ptr<int32_t>(out_i32), dim)));
+  return launched(ctx, "argmax_kernel");
+}
+
+}  // extern "C"

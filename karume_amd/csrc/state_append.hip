@@ -31,7 +31,19 @@ __device__ inline void store_from_f32<__half>(__half* p, size_t i, float v) {
 template <typename XT, typename ST>
 __global__ __launch_bounds__(256) void state_append_kernel(
     const XT* __restrict__ x, ST* __restrict__ slot, uint32_t kv_planes, uint32_t chunk_rows,
-    uint32_t depth, uint32_t capacity, uint32_t window, uint32_t past, uint32_t query) {
+    uint32_t depth, uint32_t capacity, uint32_t window, uint32_t past, uint32_t query,
+    uint32_t* lengths) {
+  if (lengths) {  // run-time lengths read on the device; same checks as the scalar form
+    past = lengths[0];
+    query = lengths[1];
+    const bool ok = query >= 1 && query <= chunk_rows &&
+                    (uint64_t)past + query <= 0xffffffffull &&
+                    (window != 0 || (uint64_t)past + query <= capacity);
+    if (!ok) {
+      if (blockIdx.x == 0 && threadIdx.x == 0) lengths[2] = 1u;
+      return;
+    }
+  }
   const uint64_t total = (uint64_t)kv_planes * query * depth;
   const uint64_t stride = (uint64_t)gridDim.x * blockDim.x;
   for (uint64_t i = blockIdx.x * (uint64_t)blockDim.x + threadIdx.x; i < total; i += stride) {
@@ -53,25 +65,26 @@ __global__ __launch_bounds__(256) void state_append_kernel(
 template <typename XT, typename ST>
 int32_t launch(krm_ctx* ctx, krm_buf x, krm_buf slot, uint32_t kv_planes, uint32_t chunk_rows,
                uint32_t depth, uint32_t capacity, uint32_t window, uint32_t past,
-               uint32_t query) {
+               uint32_t query, krm_buf lengths) {
   const uint64_t total = (uint64_t)kv_planes * query * depth;
   uint64_t blocks = (total + 255) / 256;
   if (blocks > 8192) blocks = 8192;
   state_append_kernel<XT, ST><<<dim3((unsigned)blocks), dim3(256), 0, ctx->stream>>>(
       ptr<const XT>(x), ptr<ST>(slot), kv_planes, chunk_rows, depth, capacity, window, past,
-      query);
+      query, ptr<uint32_t>(lengths));
   return launched(ctx, "state_append_kernel");
 }
 
 }  // namespace
 
-extern "C" {
-
-int32_t krm_state_append(krm_ctx* ctx, krm_buf x, krm_buf slot, uint32_t kv_planes,
-                         uint32_t chunk_rows, uint32_t depth, uint32_t capacity,
-                         uint32_t window, uint32_t past, uint32_t query, int32_t x_dtype,
-                         int32_t slot_dtype) {
+// `lengths` == 0: past / query are this run's values; otherwise they are read on the device
+// and `query` only sizes the launch (the chunk's physical rows).
+static int32_t state_append_impl(krm_ctx* ctx, krm_buf x, krm_buf slot, uint32_t kv_planes,
+                                 uint32_t chunk_rows, uint32_t depth, uint32_t capacity,
+                                 uint32_t window, uint32_t past, uint32_t query, krm_buf lengths,
+                                 int32_t x_dtype, int32_t slot_dtype) {
   KRM_TRY(enter(ctx));
+  const bool dyn = lengths != 0;
   KRM_REQUIRE(ctx, valid_dtype(x_dtype) && valid_dtype(slot_dtype),
               "krm_state_append: x_dtype %d / slot_dtype %d", x_dtype, slot_dtype);
   KRM_REQUIRE(ctx, kv_planes >= 1 && chunk_rows >= 1 && depth >= 1 && capacity >= 1,
@@ -80,10 +93,10 @@ int32_t krm_state_append(krm_ctx* ctx, krm_buf x, krm_buf slot, uint32_t kv_plan
               kv_planes, chunk_rows, depth, capacity);
   KRM_REQUIRE(ctx, window <= capacity, "krm_state_append: window %u exceeds capacity %u", window,
               capacity);
-  if (query < 1 || query > chunk_rows)
+  if (!dyn && (query < 1 || query > chunk_rows))
     return fail(ctx, KRM_ERR_EXECUTION, "krm_state_append: queryLength %u is outside 1..%u", query,
                 chunk_rows);
-  if (window == 0 && (uint64_t)past + query > capacity)
+  if (!dyn && window == 0 && (uint64_t)past + query > capacity)
     return fail(ctx, KRM_ERR_EXECUTION,
                 "krm_state_append: pastLength %u + queryLength %u exceeds capacity %u", past,
                 query, capacity);
@@ -92,15 +105,98 @@ int32_t krm_state_append(krm_ctx* ctx, krm_buf x, krm_buf slot, uint32_t kv_plan
               "krm_state_append: misaligned buffer");
   if (x_dtype == KRM_F32 && slot_dtype == KRM_F32)
     return launch<float, float>(ctx, x, slot, kv_planes, chunk_rows, depth, capacity, window,
-                                past, query);
+                                past, query, lengths);
   if (x_dtype == KRM_F32 && slot_dtype == KRM_F16)
     return launch<float, __half>(ctx, x, slot, kv_planes, chunk_rows, depth, capacity, window,
-                                 past, query);
+                                 past, query, lengths);
   if (x_dtype == KRM_F16 && slot_dtype == KRM_F16)
     return launch<__half, __half>(ctx, x, slot, kv_planes, chunk_rows, depth, capacity, window,
-                                  past, query);
+                                  past, query, lengths);
   return launch<__half, float>(ctx, x, slot, kv_planes, chunk_rows, depth, capacity, window, past,
-                               query);
+                               query, lengths);
+}
+
+// Run-time lengths {past, query, fault} kept in device memory so a recorded step can be
+// replayed while the sequence grows (the reference keeps them in an 8-byte uniform owned by
+// the generation context, packages/runtime/src/runtime/generation-context.ts:559-566).
+__global__ void lengths_set_kernel(uint32_t* lengths, uint32_t past, uint32_t query) {
+  lengths[0] = past;
+  lengths[1] = query;
+  lengths[2] = 0u;
+  lengths[3] = 0u;
+}
+__global__ void lengths_advance_kernel(uint32_t* lengths) {
+  // P advances by Q only when the step ran clean (generation-context.ts:576-591)
+  if (lengths[2] == 0u) lengths[0] += lengths[1];
+}
+__global__ void lengths_positions_kernel(const uint32_t* lengths, int32_t* positions,
+                                         uint32_t rows) {
+  const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < rows) positions[i] = (int32_t)(lengths[0] + i);
+}
+
+__global__ void lengths_log_token_kernel(uint32_t* lengths, const int32_t* token,
+                                         int32_t* history, uint32_t history_len) {
+  const uint32_t at = lengths[3];
+  if (at < history_len) history[at] = token[0];
+  lengths[3] = at + 1;
+}
+
+extern "C" {
+
+int32_t krm_lengths_log_token(krm_ctx* ctx, krm_buf lengths, krm_buf token_i32,
+                              krm_buf history_i32, uint32_t history_len) {
+  KRM_TRY(enter(ctx));
+  KRM_REQUIRE(ctx, lengths && token_i32 && history_i32 && lengths % 4 == 0 &&
+                       token_i32 % 4 == 0 && history_i32 % 4 == 0,
+              "krm_lengths_log_token: bad buffer");
+  lengths_log_token_kernel<<<dim3(1), dim3(1), 0, ctx->stream>>>(
+      ptr<uint32_t>(lengths), ptr<const int32_t>(token_i32), ptr<int32_t>(history_i32),
+      history_len);
+  return launched(ctx, "lengths_log_token_kernel");
+}
+
+int32_t krm_state_append(krm_ctx* ctx, krm_buf x, krm_buf slot, uint32_t kv_planes,
+                         uint32_t chunk_rows, uint32_t depth, uint32_t capacity,
+                         uint32_t window, uint32_t past, uint32_t query, int32_t x_dtype,
+                         int32_t slot_dtype) {
+  return state_append_impl(ctx, x, slot, kv_planes, chunk_rows, depth, capacity, window, past,
+                           query, 0, x_dtype, slot_dtype);
+}
+
+int32_t krm_state_append_lengths(krm_ctx* ctx, krm_buf x, krm_buf slot, uint32_t kv_planes,
+                                 uint32_t chunk_rows, uint32_t depth, uint32_t capacity,
+                                 uint32_t window, krm_buf lengths, int32_t x_dtype,
+                                 int32_t slot_dtype) {
+  if (!lengths || lengths % 4)
+    return fail(ctx, KRM_ERR_VALIDATION, "krm_state_append_lengths: bad lengths buffer");
+  return state_append_impl(ctx, x, slot, kv_planes, chunk_rows, depth, capacity, window, 0,
+                           chunk_rows, lengths, x_dtype, slot_dtype);
+}
+
+int32_t krm_lengths_set(krm_ctx* ctx, krm_buf lengths, uint32_t past, uint32_t query) {
+  KRM_TRY(enter(ctx));
+  KRM_REQUIRE(ctx, lengths && lengths % 4 == 0, "krm_lengths_set: bad lengths buffer");
+  lengths_set_kernel<<<dim3(1), dim3(1), 0, ctx->stream>>>(ptr<uint32_t>(lengths), past, query);
+  return launched(ctx, "lengths_set_kernel");
+}
+
+int32_t krm_lengths_advance(krm_ctx* ctx, krm_buf lengths) {
+  KRM_TRY(enter(ctx));
+  KRM_REQUIRE(ctx, lengths && lengths % 4 == 0, "krm_lengths_advance: bad lengths buffer");
+  lengths_advance_kernel<<<dim3(1), dim3(1), 0, ctx->stream>>>(ptr<uint32_t>(lengths));
+  return launched(ctx, "lengths_advance_kernel");
+}
+
+int32_t krm_lengths_positions(krm_ctx* ctx, krm_buf lengths, krm_buf positions_i32,
+                              uint32_t rows) {
+  KRM_TRY(enter(ctx));
+  KRM_REQUIRE(ctx, lengths && positions_i32 && lengths % 4 == 0 && positions_i32 % 4 == 0,
+              "krm_lengths_positions: bad buffer");
+  if (rows == 0) return KRM_OK;
+  lengths_positions_kernel<<<dim3((rows + 63) / 64), dim3(64), 0, ctx->stream>>>(
+      ptr<const uint32_t>(lengths), ptr<int32_t>(positions_i32), rows);
+  return launched(ctx, "lengths_positions_kernel");
 }
 
 }  // extern "C"

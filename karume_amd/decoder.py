@@ -1,0 +1,310 @@
+"""A Llama-style int4 decoder driven through the C ABI — the decode graph the reference exports
+(tools/export-recipes/minicpm5/export_decode.py:14-35), op for op:
+
+    embedding -> per layer [ rms_norm -> q/k/v linear -> rope(q, k) -> attention(states)
+                             -> state_append(k), state_append(v) -> o linear -> add
+                             -> rms_norm -> gate/up linear -> silu*mul -> down linear -> add ]
+              -> rms_norm(last valid row) -> lm_head linear -> argmax
+
+``run`` has the shape of the reference's ``Session.run`` for that graph (ids and positions of
+the chunk in, argmax token of the last valid row out; the context's lengths advance on success
+and the context is poisoned on failure).  ``decode_tokens`` replays one recorded decode step
+with the lengths, the positions and the fed-back token all living on the device, so the greedy
+loop needs no per-step read-back.
+
+Every tensor operation is a call into libkarume_hip.so; this module only sequences them.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import Dict, List, Optional
+
+import numpy as np
+
+from .format_i4 import pack_int4
+from .generation import GenerationContext
+from .runtime import (COMPUTE_F16, COMPUTE_F32, F16, F32, DeviceBuffer, ExecutionError,
+                      GpuContext, KarumeError)
+
+
+@dataclass(frozen=True)
+class LlamaConfig:
+    layers: int = 22
+    d_model: int = 2048
+    ffn: int = 5632
+    heads: int = 32
+    kv_heads: int = 4
+    head_dim: int = 64
+    vocab: int = 32000
+    group_size: int = 128
+    rms_eps: float = 1e-5
+    rope_base: float = 10000.0
+    max_position: int = 512
+
+    @property
+    def half_scale(self) -> float:
+        return float(np.float32(np.sqrt(1.0 / np.sqrt(float(self.head_dim)))))
+
+
+@dataclass
+class Int4Linear:
+    """Host copy of one quantised linear: packed [N, K/2] bytes and [N, K/g] scales."""
+    n: int
+    k: int
+    packed: np.ndarray
+    scales: np.ndarray  # float16
+
+
+@dataclass
+class DecoderWeights:
+    config: LlamaConfig
+    embedding: np.ndarray                      # [vocab, d_model] float16
+    layers: List[Dict[str, object]] = field(default_factory=list)
+    final_norm: np.ndarray = None              # [d_model] float32
+    lm_head: Int4Linear = None
+    rope_cos: np.ndarray = None                # [max_position, head_dim] float32
+    rope_sin: np.ndarray = None
+
+
+def rope_tables(config: LlamaConfig):
+    """cos / sin rows for positions 0..max_position-1, half-split convention (the two halves of
+    a row repeat the same angles), computed in float64 and stored as float32."""
+    half = config.head_dim // 2
+    inv_freq = 1.0 / (config.rope_base ** (np.arange(half, dtype=np.float64) / half))
+    angles = np.arange(config.max_position, dtype=np.float64)[:, None] * inv_freq[None, :]
+    angles = np.concatenate([angles, angles], axis=1)
+    return np.cos(angles).astype(np.float32), np.sin(angles).astype(np.float32)
+
+
+def random_weights(config: LlamaConfig, seed: int = 0) -> DecoderWeights:
+    """Random-init weights of the benchmark's shape: int4 codes uniform in [-8, 7], fp16 scales
+    |N(0, 0.02)|, fp16 embeddings N(0, 0.02), norm weights 1."""
+    rng = np.random.default_rng(seed)
+
+    def lin(n: int, k: int) -> Int4Linear:
+        packed = rng.integers(0, 256, size=(n, k // 2), dtype=np.uint8)
+        scales = np.maximum(np.abs(rng.normal(0, 0.02, size=(n, k // config.group_size)))
+                            .astype(np.float16), np.float16(6.104e-05))
+        return Int4Linear(n, k, packed, scales)
+
+    d, kv = config.d_model, config.kv_heads * config.head_dim
+    w = DecoderWeights(config, rng.normal(0, 0.02, size=(config.vocab, d)).astype(np.float16))
+    for _ in range(config.layers):
+        w.layers.append({
+            "attn_norm": np.ones(d, dtype=np.float32), "ffn_norm": np.ones(d, dtype=np.float32),
+            "q": lin(config.heads * config.head_dim, d), "k": lin(kv, d), "v": lin(kv, d),
+            "o": lin(d, config.heads * config.head_dim),
+            "gate": lin(config.ffn, d), "up": lin(config.ffn, d), "down": lin(d, config.ffn),
+        })
+    w.final_norm = np.ones(d, dtype=np.float32)
+    w.lm_head = lin(config.vocab, d)
+    w.rope_cos, w.rope_sin = rope_tables(config)
+    return w
+
+
+class _DeviceLinear:
+    def __init__(self, gpu: GpuContext, lin: Int4Linear):
+        self.n, self.k = lin.n, lin.k
+        self.w = gpu.upload(lin.packed)
+        self.s = gpu.upload(lin.scales)
+
+
+class LlamaDecoderSession:
+    """Weights resident on the device + scratch activations for chunks of up to chunk_length
+    rows.  io dtype selects f32 (the reference's semantic dtype) or fp16 activations; kv dtype
+    the state-slot storage."""
+
+    def __init__(self, gpu: GpuContext, weights: DecoderWeights, *, io_dtype: int = F32,
+                 kv_dtype: int = F32, chunk_length: int = 128,
+                 prefill_compute: int = COMPUTE_F32):
+        self.gpu = gpu
+        self.config = c = weights.config
+        self.io_dtype, self.kv_dtype = io_dtype, kv_dtype
+        self.io_np = np.float16 if io_dtype == F16 else np.float32
+        self.eb = 2 if io_dtype == F16 else 4
+        self.kv_eb = 2 if kv_dtype == F16 else 4
+        self.chunk_length = chunk_length
+        self.prefill_compute = prefill_compute
+        self.embedding = gpu.upload(weights.embedding)
+        self.layers = []
+        for lw in weights.layers:
+            self.layers.append({
+                "attn_norm": gpu.upload(lw["attn_norm"]), "ffn_norm": gpu.upload(lw["ffn_norm"]),
+                **{name: _DeviceLinear(gpu, lw[name])
+                   for name in ("q", "k", "v", "o", "gate", "up", "down")},
+            })
+        self.final_norm = gpu.upload(weights.final_norm)
+        self.lm_head = _DeviceLinear(gpu, weights.lm_head)
+        self.rope_cos = gpu.upload(weights.rope_cos)
+        self.rope_sin = gpu.upload(weights.rope_sin)
+        m, d = chunk_length, c.d_model
+        hd, kvd = c.heads * c.head_dim, c.kv_heads * c.head_dim
+        eb = self.eb
+        a = gpu.alloc
+        self.buf = {
+            "ids": a(m * 4), "pos": a(m * 4), "h": a(m * d * eb), "xn": a(m * d * eb),
+            "q": a(m * hd * eb), "k": a(m * kvd * eb), "v": a(m * kvd * eb),
+            "qr": a(m * hd * eb), "kr": a(m * kvd * eb), "vt": a(m * kvd * eb),
+            "att": a(m * hd * eb), "att2": a(m * hd * eb), "o": a(m * d * eb),
+            "g": a(m * c.ffn * eb), "u": a(m * c.ffn * eb), "act": a(m * c.ffn * eb),
+            "dn": a(m * d * eb), "logits": a(c.vocab * eb), "token": a(16),
+        }
+        self.workspace: Optional[DeviceBuffer] = None
+        self.logits_shape = (1, c.vocab)
+
+    # -- GreedySession surface ---------------------------------------------------------------
+    def create_generation_context(self, *, capacity: int, chunk_length: int) -> GenerationContext:
+        if chunk_length != self.chunk_length:
+            raise ExecutionError(f"chunkLength {chunk_length} differs from the session's "
+                                 f"{self.chunk_length}")
+        c = self.config
+        ctx = GenerationContext(self.gpu, layers=c.layers, kv_planes=c.kv_heads,
+                                depth=c.head_dim, capacity=capacity, chunk_length=chunk_length,
+                                kv_itemsize=self.kv_eb)
+        need = self.gpu.attention_state_workspace(1, c.heads, c.kv_heads, 1, c.head_dim, 0,
+                                                  capacity)
+        if self.workspace is None or self.workspace.nbytes < need:
+            if self.workspace is not None:
+                self.workspace.free()
+            self.workspace = self.gpu.alloc(need)
+        return ctx
+
+    def run(self, input_ids: np.ndarray, position_ids: np.ndarray, last_row: int, *,
+            context: GenerationContext, query_length: int, want_logits: bool = False):
+        ids = np.ascontiguousarray(input_ids, dtype=np.int32)
+        pos = np.ascontiguousarray(position_ids, dtype=np.int32)
+        if ids.ndim != 2 or ids.shape[0] != 1 or pos.shape != ids.shape:
+            raise ExecutionError(f"ids {list(ids.shape)} / positions {list(pos.shape)} are not "
+                                 "[1, M]")
+        m = ids.shape[1]
+        past = context.begin_run(m, query_length)
+        if not 0 <= last_row < query_length:
+            raise ExecutionError(f"last_row {last_row} is outside the {query_length} valid rows")
+        try:
+            self.buf["ids"].upload(ids)
+            self.buf["pos"].upload(pos)
+            self._forward(context, m, past, query_length, last_row, lengths=None)
+            token = self.buf["token"].download(np.int32, (1, 1, 1))
+            logits = (self.buf["logits"].download(self.io_np, self.logits_shape)
+                      if want_logits else None)
+        except KarumeError:
+            context.poison()  # a state write may already have happened: no rollback
+            raise
+        context.advance(past, query_length)
+        return (token, logits) if want_logits else token
+
+    # -- one chunk ---------------------------------------------------------------------------
+    def _linear(self, x, lin: _DeviceLinear, out, m: int) -> None:
+        compute = self.prefill_compute if m > 16 else COMPUTE_F32
+        self.gpu.linear_i4(x, lin.w, lin.s, None, out, m, lin.n, lin.k, self.config.group_size,
+                           self.io_dtype, F16, compute)
+
+    def _forward(self, context: GenerationContext, m: int, past: int, query: int, last_row: int,
+                 lengths: Optional[DeviceBuffer], ids: Optional[DeviceBuffer] = None) -> None:
+        g, c, b, io = self.gpu, self.config, self.buf, self.io_dtype
+        d = c.d_model
+        g.embedding(self.embedding, ids if ids is not None else b["ids"], b["h"], m, c.vocab, d,
+                    F16, io)
+        for li, lw in enumerate(self.layers):
+            g.rms_norm(b["h"], lw["attn_norm"], b["xn"], m, d, c.rms_eps, io)
+            self._linear(b["xn"], lw["q"], b["q"], m)
+            self._linear(b["xn"], lw["k"], b["k"], m)
+            self._linear(b["xn"], lw["v"], b["v"], m)
+            g.rope_half(b["q"], b["pos"], self.rope_cos, self.rope_sin, b["qr"], m, c.heads,
+                        c.head_dim, c.max_position, True, io)
+            g.rope_half(b["k"], b["pos"], self.rope_cos, self.rope_sin, b["kr"], m, c.kv_heads,
+                        c.head_dim, c.max_position, True, io)
+            if m > 1:
+                g.transpose_01(b["v"], b["vt"], m, c.kv_heads, c.head_dim, io)
+                vt = b["vt"]
+            else:
+                vt = b["v"]
+            spec = dict(chunk_rows=m, depth=c.head_dim, capacity=context.capacity,
+                        window=context.window)
+            if lengths is None:
+                g.attention_state(b["qr"], b["kr"], vt, context.slots_k[li], context.slots_v[li],
+                                  b["att"], batch=1, heads=c.heads, kv_heads=c.kv_heads,
+                                  half_scale=c.half_scale, past=past, query=query, io_dtype=io,
+                                  kv_dtype=self.kv_dtype, workspace=self.workspace, **spec)
+                # readers first, then the appends (docs/ir-v1.md:345-348)
+                g.state_append(b["kr"], context.slots_k[li], kv_planes=c.kv_heads, past=past,
+                               query=query, x_dtype=io, slot_dtype=self.kv_dtype, **spec)
+                g.state_append(vt, context.slots_v[li], kv_planes=c.kv_heads, past=past,
+                               query=query, x_dtype=io, slot_dtype=self.kv_dtype, **spec)
+            else:
+                g.attention_state_lengths(b["qr"], b["kr"], vt, context.slots_k[li],
+                                          context.slots_v[li], b["att"], batch=1, heads=c.heads,
+                                          kv_heads=c.kv_heads, half_scale=c.half_scale,
+                                          lengths=lengths, max_past=context.capacity - 1,
+                                          io_dtype=io, kv_dtype=self.kv_dtype,
+                                          workspace=self.workspace, **spec)
+                g.state_append_lengths(b["kr"], context.slots_k[li], kv_planes=c.kv_heads,
+                                       lengths=lengths, x_dtype=io, slot_dtype=self.kv_dtype,
+                                       **spec)
+                g.state_append_lengths(vt, context.slots_v[li], kv_planes=c.kv_heads,
+                                       lengths=lengths, x_dtype=io, slot_dtype=self.kv_dtype,
+                                       **spec)
+            if m > 1:
+                g.transpose_01(b["att"], b["att2"], c.heads, m, c.head_dim, io)
+                att = b["att2"]
+            else:
+                att = b["att"]
+            self._linear(att, lw["o"], b["o"], m)
+            g.add(b["h"], b["o"], b["h"], m * d, io)
+            g.rms_norm(b["h"], lw["ffn_norm"], b["xn"], m, d, c.rms_eps, io)
+            self._linear(b["xn"], lw["gate"], b["g"], m)
+            self._linear(b["xn"], lw["up"], b["u"], m)
+            g.silu_mul(b["g"], b["u"], b["act"], m * c.ffn, io)
+            self._linear(b["act"], lw["down"], b["dn"], m)
+            g.add(b["h"], b["dn"], b["h"], m * d, io)
+        # token-only exit: the head runs on the last valid row only
+        row = b["h"].offset(last_row * d * self.eb)
+        g.rms_norm(row, self.final_norm, b["xn"], 1, d, c.rms_eps, io)
+        self._linear(b["xn"], self.lm_head, b["logits"], 1)
+        g.argmax(b["logits"], b["token"], 1, c.vocab, io)
+
+    # -- replayed decode ---------------------------------------------------------------------
+    def decode_tokens(self, context: GenerationContext, first_token: int, count: int
+                      ) -> List[int]:
+        """Feed `first_token` at position context.past and generate `count` more tokens, one
+        recorded decode step replayed `count` times; lengths, positions and the fed-back token
+        stay on the device and the tokens are read back once at the end."""
+        if count < 1:
+            return []
+        if context.window == 0 and context.past + count > context.capacity:
+            raise ExecutionError(f"pastLength {context.past} + {count} steps exceeds capacity "
+                                 f"{context.capacity}")
+        if context.past + count > self.config.max_position:
+            raise ExecutionError("the decode would run past the RoPE table")
+        g, b = self.gpu, self.buf
+        context.begin_run(1, 1)
+        history = g.zeros(count * 4)
+        graph = None
+        try:
+            # the token buffer doubles as the id input: argmax writes it, the next replay's
+            # embedding reads it
+            b["token"].upload(np.array([first_token, 0, 0, 0], dtype=np.int32))
+            g.lengths_set(context.lengths, context.past, 1)
+            with g.record() as rec:
+                g.lengths_positions(context.lengths, b["pos"], 1)
+                self._forward(context, 1, 0, 1, 0, lengths=context.lengths, ids=b["token"])
+                g.lengths_log_token(context.lengths, b["token"], history, count)
+                g.lengths_advance(context.lengths)
+            graph = rec.graph
+            for _ in range(count):
+                graph.launch()
+            state = context.lengths.download(np.uint32, (4,))
+            tokens = history.download(np.int32, (count,))
+        except KarumeError:
+            context.poison()
+            raise
+        finally:
+            if graph is not None:
+                graph.destroy()
+            history.free()
+        if state[2] != 0:
+            context.poison()
+            raise ExecutionError("a decode step violated the run contract on the device "
+                                 "(pastLength + queryLength exceeded the capacity)")
+        context.past = int(state[0])
+        return [int(t) for t in tokens]

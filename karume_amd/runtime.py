@@ -93,6 +93,7 @@ class DeviceBuffer:
     def free(self) -> None:
         if self._owned and self.address:
             self.ctx._check(self.ctx._lib.krm_buf_free(self.ctx._handle, self.address))
+            self.ctx._buffers.discard(self)
         self.address = 0
         self._owned = False
 
@@ -178,12 +179,12 @@ class GpuContext:
             raise _ERRORS.get(status, KarumeError)(message)
         self._handle = handle
         self.device = device
-        self._buffers: list[DeviceBuffer] = []
+        self._buffers: set[DeviceBuffer] = set()
 
     # -- lifecycle -------------------------------------------------------------------------
     def destroy(self) -> None:
         if self._handle:
-            for buf in self._buffers:
+            for buf in list(self._buffers):
                 buf.free()
             self._buffers.clear()
             self._lib.krm_ctx_destroy(self._handle)
@@ -215,7 +216,7 @@ class GpuContext:
         address = C.c_uint64()
         self._check(self._lib.krm_buf_alloc(self._handle, nbytes, C.byref(address)))
         buf = DeviceBuffer(self, address.value, nbytes, owned=True)
-        self._buffers.append(buf)
+        self._buffers.add(buf)
         return buf
 
     def upload(self, array: np.ndarray) -> DeviceBuffer:
@@ -298,6 +299,84 @@ class GpuContext:
             _addr(out), cu.ctypes.data_as(C.POINTER(C.c_int32)), cu.size - 1, heads, kv_heads,
             depth, total_rows, float(half_scale), io_dtype, kv_dtype, _addr(workspace),
             workspace_bytes))
+
+
+    # -- run-time lengths on the device ----------------------------------------------------------
+    def lengths_set(self, lengths: BufferLike, past: int, query: int) -> None:
+        self._check(self._lib.krm_lengths_set(self._handle, _addr(lengths), past, query))
+
+    def lengths_advance(self, lengths: BufferLike) -> None:
+        self._check(self._lib.krm_lengths_advance(self._handle, _addr(lengths)))
+
+    def lengths_positions(self, lengths: BufferLike, positions: BufferLike, rows: int) -> None:
+        self._check(self._lib.krm_lengths_positions(self._handle, _addr(lengths),
+                                                    _addr(positions), rows))
+
+    def lengths_log_token(self, lengths: BufferLike, token: BufferLike, history: BufferLike,
+                          history_len: int) -> None:
+        self._check(self._lib.krm_lengths_log_token(self._handle, _addr(lengths), _addr(token),
+                                                    _addr(history), history_len))
+
+    def attention_state_lengths(self, q: BufferLike, ins_k: BufferLike, ins_v: BufferLike,
+                                slot_k: BufferLike, slot_v: BufferLike, out: BufferLike, *,
+                                batch: int, heads: int, kv_heads: int, chunk_rows: int,
+                                depth: int, capacity: int, window: int, half_scale: float,
+                                lengths: BufferLike, max_past: int, io_dtype: int = F32,
+                                kv_dtype: int = F32, workspace: BufferLike = None,
+                                workspace_bytes: int = 0) -> None:
+        if isinstance(workspace, DeviceBuffer) and not workspace_bytes:
+            workspace_bytes = workspace.nbytes
+        self._check(self._lib.krm_attention_state_lengths(
+            self._handle, _addr(q), _addr(ins_k), _addr(ins_v), _addr(slot_k), _addr(slot_v),
+            _addr(out), batch, heads, kv_heads, chunk_rows, depth, capacity, window,
+            float(half_scale), _addr(lengths), max_past, io_dtype, kv_dtype, _addr(workspace),
+            workspace_bytes))
+
+    def state_append_lengths(self, x: BufferLike, slot: BufferLike, *, kv_planes: int,
+                             chunk_rows: int, depth: int, capacity: int, window: int,
+                             lengths: BufferLike, x_dtype: int = F32, slot_dtype: int = F32
+                             ) -> None:
+        self._check(self._lib.krm_state_append_lengths(
+            self._handle, _addr(x), _addr(slot), kv_planes, chunk_rows, depth, capacity, window,
+            _addr(lengths), x_dtype, slot_dtype))
+
+    # -- decoder glue ops -----------------------------------------------------------------------
+    def rms_norm(self, x: BufferLike, weight_f32: BufferLike, out: BufferLike, rows: int,
+                 dim: int, eps: float, io_dtype: int = F32) -> None:
+        self._check(self._lib.krm_rms_norm(self._handle, _addr(x), _addr(weight_f32), _addr(out),
+                                           rows, dim, float(eps), io_dtype))
+
+    def rope_half(self, x: BufferLike, positions: BufferLike, cos_table: BufferLike,
+                  sin_table: BufferLike, out: BufferLike, rows: int, heads: int, head_dim: int,
+                  table_rows: int, to_head_major: bool = False, io_dtype: int = F32) -> None:
+        self._check(self._lib.krm_rope_half(
+            self._handle, _addr(x), _addr(positions), _addr(cos_table), _addr(sin_table),
+            _addr(out), rows, heads, head_dim, table_rows, int(to_head_major), io_dtype))
+
+    def transpose_01(self, x: BufferLike, out: BufferLike, a: int, b: int, d: int,
+                     io_dtype: int = F32) -> None:
+        self._check(self._lib.krm_transpose_01(self._handle, _addr(x), _addr(out), a, b, d,
+                                               io_dtype))
+
+    def silu_mul(self, gate: BufferLike, up: BufferLike, out: BufferLike, count: int,
+                 io_dtype: int = F32) -> None:
+        self._check(self._lib.krm_silu_mul(self._handle, _addr(gate), _addr(up), _addr(out),
+                                           count, io_dtype))
+
+    def add(self, a: BufferLike, b: BufferLike, out: BufferLike, count: int,
+            io_dtype: int = F32) -> None:
+        self._check(self._lib.krm_add(self._handle, _addr(a), _addr(b), _addr(out), count,
+                                      io_dtype))
+
+    def embedding(self, table: BufferLike, index: BufferLike, out: BufferLike, rows: int,
+                  vocab: int, hidden: int, table_dtype: int = F32, out_dtype: int = F32) -> None:
+        self._check(self._lib.krm_embedding(self._handle, _addr(table), _addr(index), _addr(out),
+                                            rows, vocab, hidden, table_dtype, out_dtype))
+
+    def argmax(self, x: BufferLike, out_i32: BufferLike, rows: int, dim: int,
+               io_dtype: int = F32) -> None:
+        self._check(self._lib.krm_argmax(self._handle, _addr(x), _addr(out_i32), rows, dim,
+                                         io_dtype))
 
 
 def acquire_gpu(device: int = 0, stream: Optional[int] = None) -> GpuContext:

@@ -212,3 +212,42 @@ def synthetic_int4(rng: np.random.Generator, n: int, k: int, group: int, scale_f
     else:
         scale = np.maximum(scale, F32_TINY)
     return oracle.pack_i4(q), q, scale
+
+
+# ---------------------------------------------------------------------------- decoder oracle
+
+def oracle_decoder_logits(weights, ids) -> np.ndarray:
+    """Full re-forward WITHOUT a KV cache over the whole id sequence (the way the reference
+    derives its greedy goldens, tools/export-recipes/_shared/decode_series.py:51-73): every op
+    is the CPU oracle's; attention is one causal pass (P = 0, Q = M = T).  Returns logits [T, V]
+    in float32."""
+    c = weights.config
+    ids = np.asarray(ids, dtype=np.int32)
+    t = ids.size
+    g = c.group_size
+
+    def lin(x, l):
+        return oracle.linear_i4(x, l.packed.reshape(-1), l.scales.astype(np.float32),
+                                np.zeros(l.n, dtype=np.float32), l.n, l.k, g)
+
+    h = oracle.embedding(weights.embedding.astype(np.float32), ids)          # [T, d]
+    cos, sin = weights.rope_cos[:t], weights.rope_sin[:t]
+    for lw in weights.layers:
+        xn = oracle.rms_norm(h, lw["attn_norm"], c.rms_eps)
+        q = lin(xn, lw["q"]).reshape(t, c.heads, c.head_dim).transpose(1, 0, 2)
+        k = lin(xn, lw["k"]).reshape(t, c.kv_heads, c.head_dim).transpose(1, 0, 2)
+        v = lin(xn, lw["v"]).reshape(t, c.kv_heads, c.head_dim).transpose(1, 0, 2)
+        q = oracle.rope_half(q[None], cos, sin)
+        k = oracle.rope_half(k[None], cos, sin)
+        zeros = np.zeros((1, c.kv_heads, t, c.head_dim), dtype=np.float32)
+        att = oracle.state_attention(q, k, np.ascontiguousarray(v[None]), zeros, zeros, batch=1,
+                                     heads=c.heads, kv_heads=c.kv_heads, chunk_rows=t,
+                                     depth=c.head_dim, capacity=t, window=0, past=0, query=t,
+                                     scale=np.float32(c.half_scale))
+        att = att[0].transpose(1, 0, 2).reshape(t, c.heads * c.head_dim)
+        h = (h + lin(att, lw["o"])).astype(np.float32)
+        xn = oracle.rms_norm(h, lw["ffn_norm"], c.rms_eps)
+        act = oracle.silu_mul(lin(xn, lw["gate"]), lin(xn, lw["up"]))
+        h = (h + lin(act, lw["down"])).astype(np.float32)
+    xn = oracle.rms_norm(h, weights.final_norm, c.rms_eps)
+    return lin(xn, weights.lm_head)
