@@ -26,6 +26,10 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
+# HBM bytes per config-0 GEMV launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled
+# by an 8 MiB copy kernel's readings (profiles/gemv_i4_config0_pmc_traffic.txt).
+GEMV_PMC_TRAFFIC_BYTES = 8_803_900
+USE_GRAPHS = True       # --no-graph: plain launches (rocprofv3's kernel trace crashes on graph launches)
 
 
 def log(msg: str) -> None:
@@ -38,6 +42,20 @@ def timed(ctx, fn, steps: int, warmup: int, period: int = 64) -> float:
     The calls are recorded once (`period` consecutive steps = one graph) and replayed, the way
     a decode loop replays its recorded token step, so the host's launch cost is not what is
     measured; a remainder of steps % period is issued as plain calls."""
+    if not USE_GRAPHS:
+        for i in range(warmup):
+            fn(i)
+        ctx.sync()
+        start, stop = ctx.event(), ctx.event()
+        start.record()
+        for i in range(steps):
+            fn(i)
+        stop.record()
+        ms = start.elapsed_ms(stop)
+        ctx.sync()
+        start.destroy()
+        stop.destroy()
+        return ms
     with ctx.record() as rec:
         for i in range(period):
             fn(i)
@@ -143,6 +161,61 @@ def bench_gemm(ctx, ka, rng, steps: int, warmup: int, m: int, n: int, k: int, g:
     return ms / steps, 2.0 * m * n * k
 
 
+def bench_model(ctx, ka, io_dtype, kv_dtype, prompt_len: int = 128, new_tokens: int = 256):
+    """BASELINE config 4: random-init 1.1B-shape int4 decoder, 128-token random prompt, 256
+    greedy decode steps, batch 1.  The decode steps replay one recorded step (lengths and the
+    fed-back token stay on the device); timing covers the replays only, then prefill + decode."""
+    from karume_amd.decoder import LlamaConfig, LlamaDecoderSession, random_weights
+    from karume_amd.generation import plan_prefill_chunks
+
+    config = LlamaConfig()
+    t0 = time.perf_counter()
+    weights = random_weights(config, seed=4)
+    session = LlamaDecoderSession(ctx, weights, io_dtype=io_dtype, kv_dtype=kv_dtype,
+                                  chunk_length=prompt_len, prefill_compute=ka.COMPUTE_F16)
+    log(f"[bench]   weights generated and uploaded in {time.perf_counter() - t0:.1f} s")
+    rng = np.random.default_rng(44)
+    prompt = rng.integers(0, config.vocab, size=prompt_len).astype(np.int32)
+    times = []
+    for _ in range(2):  # first pass warms up
+        gen = session.create_generation_context(capacity=config.max_position,
+                                                chunk_length=prompt_len)
+        ctx.sync()
+        t_start = time.perf_counter()
+        token = None
+        for chunk in plan_prefill_chunks(prompt_len, prompt_len):
+            n = chunk.query_length
+            ids = np.zeros((1, prompt_len), dtype=np.int32)
+            pos = np.zeros((1, prompt_len), dtype=np.int32)
+            ids[0, :n] = prompt[chunk.position:chunk.position + n]
+            pos[0, :n] = np.arange(chunk.position, chunk.position + n)
+            token = session.run(ids, pos, n - 1, context=gen, query_length=n)
+        t_prefill = time.perf_counter()
+        if USE_GRAPHS:
+            tokens = session.decode_tokens(gen, int(token[0, 0, 0]), new_tokens - 1)
+        else:  # one run (and one read-back) per token
+            tokens, tok = [], int(token[0, 0, 0])
+            for i in range(new_tokens - 1):
+                tok = int(session.run(np.array([[tok]], dtype=np.int32),
+                                      np.array([[prompt_len + i]], dtype=np.int32), 0,
+                                      context=gen, query_length=1)[0, 0, 0])
+                tokens.append(tok)
+        t_end = time.perf_counter()
+        times.append((t_prefill - t_start, t_end - t_prefill))
+        gen.dispose()
+    prefill_s, decode_s = times[-1]
+    bytes_per_token = 517_210_112 + 16_162_816  # int4 weights + fp16 scales read per token
+    return {
+        "decode_tokens_per_s": round((new_tokens - 1) / decode_s, 1),
+        "decode_ms_per_token": round(decode_s / (new_tokens - 1) * 1e3, 4),
+        "prefill_ms": round(prefill_s * 1e3, 2),
+        "end_to_end_tokens_per_s": round(new_tokens / (prefill_s + decode_s), 1),
+        "weight_gbs": round(bytes_per_token * (new_tokens - 1) / decode_s / 1e9, 1),
+        "pct_of_hbm_peak": round(100 * bytes_per_token * (new_tokens - 1) / decode_s / 8e12, 2),
+        "first_tokens": [int(t) for t in tokens[:8]],
+    }
+
+
 def cpu_baseline(n: int, k: int, g: int, budget_s: float = 12.0):
     """The CPU oracle (a port of the reference's decode + linear loops, double accumulation,
     OpenMP over output rows) timed on the host cores on repetitions of the same GEMV."""
@@ -171,7 +244,9 @@ def main() -> int:
     ap.add_argument("--steps", type=int, default=2000)
     ap.add_argument("--warmup", type=int, default=200)
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--only", default="", help="gemv: skip the secondary measurements")
+    ap.add_argument("--no-graph", action="store_true",
+                    help="issue plain launches instead of replaying recorded graphs")
+    ap.add_argument("--only", default="", help="gemv | model: run only that part besides the headline GEMV")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build measures one GPU only (--gpus 1); no multi-GPU figure is "
@@ -180,6 +255,8 @@ def main() -> int:
 
     import karume_amd as ka
 
+    global USE_GRAPHS
+    USE_GRAPHS = not args.no_graph
     ctx = ka.acquire_gpu(int(os.environ.get("LOCAL_RANK", "0")))
     rng = np.random.default_rng(20261125)
     m, n, k, g = 1, 4096, 4096, 128
@@ -202,16 +279,24 @@ def main() -> int:
         "vs_baseline": None,
         "dtype": "f32",
         "data": "synthetic",
+        "launch_mode": "hipGraph replay" if USE_GRAPHS else "plain launches",
         "config": {"workload": "config 0: int4 g128 GEMV M=1 K=4096 N=4096, fp16 x/scales/out, "
                                "f32 accumulate, 64 rotating weight buffers (528 MiB)"},
         "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS,
-                     "unit": "GB/s", "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None,
+                     "unit": "GB/s", "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": GEMV_PMC_TRAFFIC_BYTES,
                      "kernel": "gemv_i4_kernel", "algorithmic_bytes_per_launch": algo,
                      "us_per_launch": round(per_call_us, 3)},
         "pct_of_hbm_peak": round(100 * gbs / HBM_PEAK_GBS, 2),
         "gemv_cache_resident_gbs": round(gbs_res, 1),
     }
-    if args.only != "gemv":
+    if args.only == "traffic":
+        # For `rocprofv3 --pmc FETCH_SIZE` / `--pmc WRITE_SIZE`: a plain 8 MiB copy (known
+        # traffic: 8 MiB read + 8 MiB written) beside the GEMV, a few launches of each.
+        src, dst = ctx.alloc(8 << 20), ctx.alloc(8 << 20)
+        for _ in range(8):
+            ctx.copy(dst, src, 8 << 20)
+        ctx.sync()
+    if args.only == "":
         steps2 = max(50, args.steps // 4)
         log("[bench] GEMV M=16 (config 3)")
         ms16, _res16, algo16 = bench_gemv(ctx, ka, rng, steps2, max(10, args.warmup // 4), 16, n,
@@ -231,6 +316,15 @@ def main() -> int:
             result[f"gemm_{name}_us"] = round(ms_g * 1e3, 2)
             result[f"gemm_{name}_pct_of_f16_mfma_peak"] = round(
                 100 * flops / (ms_g * 1e-3) / 2.5e15, 2)
+    if args.only in ("", "model"):
+        # f32 activations: with this random init (|N(0,0.02)| scales on uniform codes) the
+        # residual stream passes 65504 after a few layers, so fp16 activations are not usable
+        # for config 4; the KV state may still be kept in fp16.
+        for label, (io_d, kv_d) in {"f32": (ka.F32, ka.F32), "f32_kv16": (ka.F32, ka.F16)}.items():
+            log(f"[bench] 1.1B-shape int4 decoder, 128-token prompt + 256 greedy steps "
+                f"(config 4, {label})")
+            result[f"model_decode_{label}"] = bench_model(ctx, ka, io_d, kv_d)
+        result["decode_tokens_per_s"] = result["model_decode_f32"]["decode_tokens_per_s"]
     ctx.destroy()
     if not args.no_cpu_baseline:
         log("[bench] CPU baseline (oracle port on the host cores)")

@@ -82,6 +82,9 @@ int32_t krm_buf_download(krm_ctx* ctx, krm_buf src, size_t src_offset, void* hos
  * (packages/runtime/tests/gpu_state_execution_test.ts:159-164). */
 int32_t krm_buf_zero(krm_ctx* ctx, krm_buf dst, size_t dst_offset, size_t bytes);
 
+/* Device-to-device copy on the context's stream (copyBufferToBuffer); 16-byte granularity. */
+int32_t krm_buf_copy(krm_ctx* ctx, krm_buf dst, krm_buf src, size_t bytes);
+
 /* ---- timing (timestamp-query diagnostics, packages/runtime/src/gpu/submit.ts:54-63) ------ */
 int32_t krm_event_create(krm_ctx* ctx, krm_event** out);
 int32_t krm_event_record(krm_ctx* ctx, krm_event* ev);

@@ -31,6 +31,7 @@ PROTOTYPES = {
     "krm_buf_upload": (i32, [c_ctx, c_buf, size_t, C.c_void_p, size_t]),
     "krm_buf_download": (i32, [c_ctx, c_buf, size_t, C.c_void_p, size_t]),
     "krm_buf_zero": (i32, [c_ctx, c_buf, size_t, size_t]),
+    "krm_buf_copy": (i32, [c_ctx, c_buf, c_buf, size_t]),
     "krm_event_create": (i32, [c_ctx, C.POINTER(c_evt)]),
     "krm_event_record": (i32, [c_ctx, c_evt]),
     "krm_event_elapsed_ms": (i32, [c_ctx, c_evt, c_evt, C.POINTER(C.c_float)]),

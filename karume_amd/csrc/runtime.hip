@@ -198,6 +198,27 @@ int32_t krm_buf_zero(krm_ctx* ctx, krm_buf dst, size_t dst_offset, size_t bytes)
   return launched(ctx, "krm_zero_kernel");
 }
 
+__global__ void krm_copy_kernel(uint4* __restrict__ dst, const uint4* __restrict__ src,
+                                size_t pieces) {
+  size_t i = blockIdx.x * (size_t)blockDim.x + threadIdx.x;
+  const size_t stride = (size_t)gridDim.x * blockDim.x;
+  for (; i < pieces; i += stride) dst[i] = src[i];
+}
+
+int32_t krm_buf_copy(krm_ctx* ctx, krm_buf dst, krm_buf src, size_t bytes) {
+  KRM_TRY(enter(ctx));
+  if (bytes == 0) return KRM_OK;
+  KRM_REQUIRE(ctx, dst && src, "krm_buf_copy: NULL buffer");
+  KRM_REQUIRE(ctx, dst % 16 == 0 && src % 16 == 0 && bytes % 16 == 0,
+              "krm_buf_copy: addresses and size must be multiples of 16 bytes");
+  const size_t pieces = bytes / 16;
+  size_t blocks = (pieces + 255) / 256;
+  if (blocks > 8192) blocks = 8192;
+  krm_copy_kernel<<<dim3((unsigned)blocks), dim3(256), 0, ctx->stream>>>(
+      ptr<uint4>(dst), ptr<const uint4>(src), pieces);
+  return launched(ctx, "krm_copy_kernel");
+}
+
 int32_t krm_graph_begin(krm_ctx* ctx) {
   KRM_TRY(enter(ctx));
   KRM_TRY(not_recording(ctx, "krm_graph_begin"));

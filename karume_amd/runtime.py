@@ -231,6 +231,9 @@ class GpuContext:
         buf.zero()
         return buf
 
+    def copy(self, dst: BufferLike, src: BufferLike, nbytes: int) -> None:
+        self._check(self._lib.krm_buf_copy(self._handle, _addr(dst), _addr(src), nbytes))
+
     def borrow(self, address: int, nbytes: int) -> DeviceBuffer:
         """Wrap device memory owned by someone else (for example a torch tensor's data_ptr)."""
         return DeviceBuffer(self, address, nbytes, owned=False)
