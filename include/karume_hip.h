@@ -129,6 +129,21 @@ int32_t krm_linear_i4(krm_ctx* ctx, krm_buf x, krm_buf w, krm_buf scales, krm_bu
                       krm_buf out, uint32_t m, uint32_t n, uint32_t k, uint32_t group,
                       int32_t io_dtype, int32_t scale_dtype, int32_t compute);
 
+/* Decode-step fusion of the same op (m <= 16): what the reference's peephole fusion pass does
+ * at the recipe level (packages/runtime/src/runtime/fusion.ts), done here inside the GEMV:
+ *   norm_weight_f32 != 0 : x is first rms-normalised,  x' = x * rsqrt(mean(x^2) + eps) * weight
+ *                          (krm_rms_norm folded in; the normalised row is not rounded in between)
+ *   residual != 0        : out = linear(...) + residual        ([m, n_out], io_dtype)
+ *   KRM_EPILOGUE_SILU_PAIRS : weight rows are interleaved (2i, 2i+1) = (gate_i, up_i) and
+ *                          out[m, i] = silu(gate_i) * up_i with n_out = n / 2 (krm_silu_mul folded in)
+ * Each output row still depends on its own x row only. */
+#define KRM_EPILOGUE_NONE 0
+#define KRM_EPILOGUE_SILU_PAIRS 1
+int32_t krm_linear_i4_fused(krm_ctx* ctx, krm_buf x, krm_buf norm_weight_f32, float norm_eps,
+                            krm_buf w, krm_buf scales, krm_buf bias, krm_buf residual,
+                            krm_buf out, uint32_t m, uint32_t n, uint32_t k, uint32_t group,
+                            int32_t io_dtype, int32_t scale_dtype, int32_t epilogue);
+
 /* ---- states-form attention (Params 10 words + Lengths{past,query} + bindings:
  *      packages/runtime/src/kernels/state-attention.ts:169-180,190-193,284-294,476-487;
  *      builder packages/runtime/src/runtime/recipe-builder.ts:1856-2002;

@@ -16,6 +16,8 @@
 // row of x gives the same bits whether it is run alone or in a batch.
 #include "krm_internal.h"
 
+#include <cmath>
+
 using namespace krm;
 
 namespace {
@@ -115,13 +117,32 @@ struct Acts<__half> {
   struct Regs {
     half2_t p[VEC][4];
   };
+  // `g` (optional): rms_norm weights of the same 8*VEC positions; the lane then carries
+  // fp16(x * g) and adds its x^2 to `squares`.
   template <int VEC>
-  __device__ static inline void load(const __half* x, bool active, Regs<VEC>& r) {
+  __device__ static inline void load(const __half* x, const float* g, bool active, Regs<VEC>& r,
+                                     float& squares) {
 #pragma unroll
     for (int j = 0; j < VEC; ++j) {
       uint4 raw = reinterpret_cast<const uint4*>(x)[j];
       const uint32_t keep = active ? 0xFFFFFFFFu : 0u;  // bit mask: no control flow
       raw.x &= keep; raw.y &= keep; raw.z &= keep; raw.w &= keep;
+      if (g) {
+        const float4 ga = reinterpret_cast<const float4*>(g)[2 * j];
+        const float4 gb = reinterpret_cast<const float4*>(g)[2 * j + 1];
+        const float gw[8] = {ga.x, ga.y, ga.z, ga.w, gb.x, gb.y, gb.z, gb.w};
+        uint32_t words[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const half2_t h = __builtin_bit_cast(half2_t, words[i]);
+          const float lo = (float)h.x, hi = (float)h.y;
+          squares = fmaf(lo, lo, squares);
+          squares = fmaf(hi, hi, squares);
+          const half2_t scaled = {(_Float16)(lo * gw[2 * i]), (_Float16)(hi * gw[2 * i + 1])};
+          words[i] = __builtin_bit_cast(uint32_t, scaled);
+        }
+        raw = make_uint4(words[0], words[1], words[2], words[3]);
+      }
       pair_activations(raw, r.p[j]);
     }
   }
@@ -150,17 +171,28 @@ struct Acts<float> {
     float sum;
   };
   template <int VEC>
-  __device__ static inline void load(const float* x, bool active, Regs<VEC>& r) {
+  __device__ static inline void load(const float* x, const float* g, bool active, Regs<VEC>& r,
+                                     float& squares) {
     float s = 0.f;
 #pragma unroll
     for (int j = 0; j < VEC; ++j) {
       uint4 ua = reinterpret_cast<const uint4*>(x)[2 * j];
       uint4 ub = reinterpret_cast<const uint4*>(x)[2 * j + 1];
       const uint32_t keep = active ? 0xFFFFFFFFu : 0u;  // bit mask: no control flow
-      const float4 a = make_float4(__uint_as_float(ua.x & keep), __uint_as_float(ua.y & keep),
-                                   __uint_as_float(ua.z & keep), __uint_as_float(ua.w & keep));
-      const float4 b = make_float4(__uint_as_float(ub.x & keep), __uint_as_float(ub.y & keep),
-                                   __uint_as_float(ub.z & keep), __uint_as_float(ub.w & keep));
+      float4 a = make_float4(__uint_as_float(ua.x & keep), __uint_as_float(ua.y & keep),
+                             __uint_as_float(ua.z & keep), __uint_as_float(ua.w & keep));
+      float4 b = make_float4(__uint_as_float(ub.x & keep), __uint_as_float(ub.y & keep),
+                             __uint_as_float(ub.z & keep), __uint_as_float(ub.w & keep));
+      if (g) {
+        const float4 ga = reinterpret_cast<const float4*>(g)[2 * j];
+        const float4 gb = reinterpret_cast<const float4*>(g)[2 * j + 1];
+        squares = fmaf(a.x, a.x, squares); squares = fmaf(a.y, a.y, squares);
+        squares = fmaf(a.z, a.z, squares); squares = fmaf(a.w, a.w, squares);
+        squares = fmaf(b.x, b.x, squares); squares = fmaf(b.y, b.y, squares);
+        squares = fmaf(b.z, b.z, squares); squares = fmaf(b.w, b.w, squares);
+        a = make_float4(a.x * ga.x, a.y * ga.y, a.z * ga.z, a.w * ga.w);
+        b = make_float4(b.x * gb.x, b.y * gb.y, b.z * gb.z, b.w * gb.w);
+      }
       r.v[j][0] = a.x; r.v[j][1] = a.y; r.v[j][2] = a.z; r.v[j][3] = a.w;
       r.v[j][4] = b.x; r.v[j][5] = b.y; r.v[j][6] = b.z; r.v[j][7] = b.w;
       s += ((a.x + a.y) + (a.z + a.w)) + ((b.x + b.y) + (b.z + b.w));
@@ -197,6 +229,14 @@ __device__ inline float from_f32<float>(float v) { return v; }
 template <>
 __device__ inline __half from_f32<__half>(float v) { return __float2half_rn(v); }
 
+// Optional work fused around the dot products (all null / 0 = the plain linear op).
+struct GemvFusion {
+  const float* norm_weight;  // [K] rms_norm weight applied to x before the product
+  float norm_eps;
+  const void* residual;      // [M, N_out] added to the result (same element type as out)
+  uint32_t pair_silu;        // rows (2i, 2i+1) = (gate_i, up_i): out[., i] = silu(gate) * up
+};
+
 // One wave = ROWS consecutive output rows over the whole K; a step covers 64 lanes x VEC
 // words (VEC*8 codes per lane, all inside one scale group).
 //  NSTEP > 0: K fits in NSTEP steps; every weight word, scale and (for MB == 1) activation of
@@ -209,7 +249,7 @@ template <typename XT, typename ST, int MB, int ROWS, int VEC, int NSTEP>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 4))) void gemv_i4_kernel(
     const XT* __restrict__ x, const uint32_t* __restrict__ w, const ST* __restrict__ scales,
     const XT* __restrict__ bias, XT* __restrict__ out, uint32_t m, uint32_t n, uint32_t k,
-    uint32_t group_shift) {
+    uint32_t group_shift, GemvFusion fuse) {
   constexpr int kLaneElems = VEC * 8;
   constexpr int kStepElems = kWave * kLaneElems;
   using Regs = typename Acts<XT>::template Regs<VEC>;
@@ -231,10 +271,13 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 4))) voi
   }
 
   float acc[ROWS][MB];
+  float squares[MB];  // sum of x^2 over the lane's share of K (fused rms_norm only)
 #pragma unroll
-  for (int r = 0; r < ROWS; ++r)
+  for (int b = 0; b < MB; ++b) {
+    squares[b] = 0.f;
 #pragma unroll
-    for (int b = 0; b < MB; ++b) acc[r][b] = 0.f;
+    for (int r = 0; r < ROWS; ++r) acc[r][b] = 0.f;
+  }
 
   // Lanes past the end of K (last step of a K that is not a multiple of the step) read the
   // row's first words instead and get zero activations and a zero scale, so every load is
@@ -259,7 +302,10 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 4))) voi
   auto fetch_x = [&](uint32_t step, int b, Regs& regs) {
     const uint32_t k0 = step * kStepElems + lane * kLaneElems;
     const uint32_t xrow = min((uint32_t)b, m - 1);  // rows past M re-read the last row, unused
-    Acts<XT>::template load<VEC>(x + (size_t)xrow * k + (k0 < k ? k0 : 0u), k0 < k, regs);
+    const uint32_t kc = k0 < k ? k0 : 0u;
+    Acts<XT>::template load<VEC>(x + (size_t)xrow * k + kc,
+                                 fuse.norm_weight ? fuse.norm_weight + kc : nullptr, k0 < k, regs,
+                                 squares[b]);
   };
   auto consume = [&](const uint32_t (&cw)[ROWS][VEC], const float (&cs)[ROWS], int b,
                      const Regs& regs) {
@@ -324,15 +370,46 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 4))) voi
     }
   }
 
+  // fused rms_norm: every wave has seen the whole row of x, so 1/sqrt(mean(x^2)+eps) is a
+  // wave reduction; it scales the finished dot product (the norm weight already multiplied x).
+  float inv[MB];
+#pragma unroll
+  for (int b = 0; b < MB; ++b)
+    inv[b] = fuse.norm_weight ? 1.0f / sqrtf(wave_sum(squares[b]) / (float)k + fuse.norm_eps)
+                              : 1.0f;
+  const XT* residual = static_cast<const XT*>(fuse.residual);
+  if constexpr (ROWS == 2) {
+    if (fuse.pair_silu) {
+      // rows (2i, 2i+1) hold (gate_i, up_i): out[., i] = silu(gate) * up, n/2 outputs per row
+      const uint32_t half_n = n >> 1, col = row0 >> 1;
+#pragma unroll
+      for (int b = 0; b < MB; ++b) {
+        float gate = wave_sum(acc[0][b]) * inv[b], up = wave_sum(acc[1][b]) * inv[b];
+        if (lane == b % kWave && row0 + 1 < n && (uint32_t)b < m) {
+          if (bias) {
+            gate += to_f32<XT>(bias[row0]);
+            up += to_f32<XT>(bias[row0 + 1]);
+          }
+          const float t = expf(-fabsf(gate));
+          const float sig = gate < 0.f ? t / (1.0f + t) : 1.0f / (1.0f + t);
+          float value = __fmul_rn(__fmul_rn(gate, sig), up);
+          if (residual) value += to_f32<XT>(residual[(size_t)b * half_n + col]);
+          out[(size_t)b * half_n + col] = from_f32<XT>(value);
+        }
+      }
+      return;
+    }
+  }
 #pragma unroll
   for (int r = 0; r < ROWS; ++r) {
 #pragma unroll
     for (int b = 0; b < MB; ++b) {
-      const float total = wave_sum(acc[r][b]);
+      const float total = wave_sum(acc[r][b]) * inv[b];
       const uint32_t row = row0 + r;
       if (lane == (r * MB + b) % kWave && row < n && (uint32_t)b < m) {
-        const float add = bias ? to_f32<XT>(bias[row]) : 0.f;
-        out[(size_t)b * n + row] = from_f32<XT>(total + add);
+        float value = total + (bias ? to_f32<XT>(bias[row]) : 0.f);
+        if (residual) value += to_f32<XT>(residual[(size_t)b * n + row]);
+        out[(size_t)b * n + row] = from_f32<XT>(value);
       }
     }
   }
@@ -340,61 +417,65 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 4))) voi
 
 template <typename XT, typename ST, int MB, int ROWS, int VEC, int NSTEP>
 int32_t launch_gemv(krm_ctx* ctx, krm_buf x, krm_buf w, krm_buf scales, krm_buf bias,
-                    krm_buf out, uint32_t m, uint32_t n, uint32_t k, uint32_t group_shift) {
+                    krm_buf out, uint32_t m, uint32_t n, uint32_t k, uint32_t group_shift,
+                    const GemvFusion& fuse = GemvFusion{}) {
   const uint32_t rows_per_block = 4 * ROWS;
   const uint32_t blocks = (n + rows_per_block - 1) / rows_per_block;
   gemv_i4_kernel<XT, ST, MB, ROWS, VEC, NSTEP><<<dim3(blocks), dim3(256), 0, ctx->stream>>>(
       ptr<const XT>(x), ptr<const uint32_t>(w), ptr<const ST>(scales), ptr<const XT>(bias),
-      ptr<XT>(out), m, n, k, group_shift);
+      ptr<XT>(out), m, n, k, group_shift, fuse);
   return launched(ctx, "gemv_i4_kernel");
 }
 
 template <typename XT, typename ST, int MB, int ROWS, int VEC>
 int32_t pick_steps(krm_ctx* ctx, krm_buf x, krm_buf w, krm_buf scales, krm_buf bias, krm_buf out,
-                   uint32_t m, uint32_t n, uint32_t k, uint32_t group_shift) {
+                   uint32_t m, uint32_t n, uint32_t k, uint32_t group_shift,
+                   const GemvFusion& fuse) {
   // Rows short enough to hold in registers are requested whole (VEC == 4: 2048 codes a step).
   if constexpr (VEC == 4 && MB == 1) {
     const uint32_t steps = (k + 2047) / 2048;
     if (steps == 1)
-      return launch_gemv<XT, ST, MB, ROWS, VEC, 1>(ctx, x, w, scales, bias, out, m, n, k, group_shift);
+      return launch_gemv<XT, ST, MB, ROWS, VEC, 1>(ctx, x, w, scales, bias, out, m, n, k, group_shift, fuse);
     if (steps == 2)
-      return launch_gemv<XT, ST, MB, ROWS, VEC, 2>(ctx, x, w, scales, bias, out, m, n, k, group_shift);
+      return launch_gemv<XT, ST, MB, ROWS, VEC, 2>(ctx, x, w, scales, bias, out, m, n, k, group_shift, fuse);
     if (steps == 3 && ROWS <= 2)
-      return launch_gemv<XT, ST, MB, ROWS, VEC, 3>(ctx, x, w, scales, bias, out, m, n, k, group_shift);
+      return launch_gemv<XT, ST, MB, ROWS, VEC, 3>(ctx, x, w, scales, bias, out, m, n, k, group_shift, fuse);
   }
-  return launch_gemv<XT, ST, MB, ROWS, VEC, 0>(ctx, x, w, scales, bias, out, m, n, k, group_shift);
+  return launch_gemv<XT, ST, MB, ROWS, VEC, 0>(ctx, x, w, scales, bias, out, m, n, k, group_shift, fuse);
 }
 
 template <typename XT, typename ST, int MB, int VEC>
 int32_t pick_rows(krm_ctx* ctx, krm_buf x, krm_buf w, krm_buf scales, krm_buf bias, krm_buf out,
-                  uint32_t m, uint32_t n, uint32_t k, uint32_t group_shift) {
+                  uint32_t m, uint32_t n, uint32_t k, uint32_t group_shift,
+                  const GemvFusion& fuse) {
   // Rows per wave: two rows share one fetch of the activations; one row per wave keeps more
   // waves in flight when N is small.  The choice never changes a row's reduction order.
   const uint64_t cus = (uint64_t)ctx->num_cus;
-  if ((uint64_t)n >= cus * 4 * 2)
-    return pick_steps<XT, ST, MB, 2, VEC>(ctx, x, w, scales, bias, out, m, n, k, group_shift);
-  return pick_steps<XT, ST, MB, 1, VEC>(ctx, x, w, scales, bias, out, m, n, k, group_shift);
+  if (fuse.pair_silu || (uint64_t)n >= cus * 4 * 2)
+    return pick_steps<XT, ST, MB, 2, VEC>(ctx, x, w, scales, bias, out, m, n, k, group_shift, fuse);
+  return pick_steps<XT, ST, MB, 1, VEC>(ctx, x, w, scales, bias, out, m, n, k, group_shift, fuse);
 }
 
 template <typename XT, typename ST, int VEC>
 int32_t pick_batch(krm_ctx* ctx, krm_buf x, krm_buf w, krm_buf scales, krm_buf bias, krm_buf out,
-                   uint32_t m, uint32_t n, uint32_t k, uint32_t group_shift) {
-  if (m == 1) return pick_rows<XT, ST, 1, VEC>(ctx, x, w, scales, bias, out, m, n, k, group_shift);
-  if (m == 2) return pick_rows<XT, ST, 2, VEC>(ctx, x, w, scales, bias, out, m, n, k, group_shift);
-  if (m <= 4) return pick_rows<XT, ST, 4, VEC>(ctx, x, w, scales, bias, out, m, n, k, group_shift);
-  if (m <= 8) return pick_rows<XT, ST, 8, VEC>(ctx, x, w, scales, bias, out, m, n, k, group_shift);
-  return pick_rows<XT, ST, 16, VEC>(ctx, x, w, scales, bias, out, m, n, k, group_shift);
+                   uint32_t m, uint32_t n, uint32_t k, uint32_t group_shift,
+                   const GemvFusion& fuse) {
+  if (m == 1) return pick_rows<XT, ST, 1, VEC>(ctx, x, w, scales, bias, out, m, n, k, group_shift, fuse);
+  if (m == 2) return pick_rows<XT, ST, 2, VEC>(ctx, x, w, scales, bias, out, m, n, k, group_shift, fuse);
+  if (m <= 4) return pick_rows<XT, ST, 4, VEC>(ctx, x, w, scales, bias, out, m, n, k, group_shift, fuse);
+  if (m <= 8) return pick_rows<XT, ST, 8, VEC>(ctx, x, w, scales, bias, out, m, n, k, group_shift, fuse);
+  return pick_rows<XT, ST, 16, VEC>(ctx, x, w, scales, bias, out, m, n, k, group_shift, fuse);
 }
 
 template <typename XT, typename ST>
 int32_t pick_vec(krm_ctx* ctx, krm_buf x, krm_buf w, krm_buf scales, krm_buf bias, krm_buf out,
-                 uint32_t m, uint32_t n, uint32_t k, uint32_t group) {
+                 uint32_t m, uint32_t n, uint32_t k, uint32_t group, const GemvFusion& fuse) {
   uint32_t group_shift = 0;
   while ((1u << group_shift) < group) ++group_shift;
   // 16-byte loads need 32 codes per lane inside one group and 16-byte aligned rows.
   const bool wide = (k % 32 == 0) && (group % 32 == 0) && aligned(w, 16);
-  if (wide) return pick_batch<XT, ST, 4>(ctx, x, w, scales, bias, out, m, n, k, group_shift);
-  return pick_batch<XT, ST, 1>(ctx, x, w, scales, bias, out, m, n, k, group_shift);
+  if (wide) return pick_batch<XT, ST, 4>(ctx, x, w, scales, bias, out, m, n, k, group_shift, fuse);
+  return pick_batch<XT, ST, 1>(ctx, x, w, scales, bias, out, m, n, k, group_shift, fuse);
 }
 
 }  // namespace
@@ -402,17 +483,24 @@ int32_t pick_vec(krm_ctx* ctx, krm_buf x, krm_buf w, krm_buf scales, krm_buf bia
 namespace krm {
 
 // Rows M <= 16: the GEMV above.  Declared in gemm_i4.hip's dispatcher too.
+static int32_t gemv_dispatch(krm_ctx* ctx, krm_buf x, krm_buf w, krm_buf scales, krm_buf bias,
+                             krm_buf out, uint32_t m, uint32_t n, uint32_t k, uint32_t group,
+                             int32_t io_dtype, int32_t scale_dtype, const GemvFusion& fuse) {
+  if (io_dtype == KRM_F16) {
+    if (scale_dtype == KRM_F16)
+      return pick_vec<__half, __half>(ctx, x, w, scales, bias, out, m, n, k, group, fuse);
+    return pick_vec<__half, float>(ctx, x, w, scales, bias, out, m, n, k, group, fuse);
+  }
+  if (scale_dtype == KRM_F16)
+    return pick_vec<float, __half>(ctx, x, w, scales, bias, out, m, n, k, group, fuse);
+  return pick_vec<float, float>(ctx, x, w, scales, bias, out, m, n, k, group, fuse);
+}
+
 int32_t linear_i4_gemv(krm_ctx* ctx, krm_buf x, krm_buf w, krm_buf scales, krm_buf bias,
                        krm_buf out, uint32_t m, uint32_t n, uint32_t k, uint32_t group,
                        int32_t io_dtype, int32_t scale_dtype) {
-  if (io_dtype == KRM_F16) {
-    if (scale_dtype == KRM_F16)
-      return pick_vec<__half, __half>(ctx, x, w, scales, bias, out, m, n, k, group);
-    return pick_vec<__half, float>(ctx, x, w, scales, bias, out, m, n, k, group);
-  }
-  if (scale_dtype == KRM_F16)
-    return pick_vec<float, __half>(ctx, x, w, scales, bias, out, m, n, k, group);
-  return pick_vec<float, float>(ctx, x, w, scales, bias, out, m, n, k, group);
+  return gemv_dispatch(ctx, x, w, scales, bias, out, m, n, k, group, io_dtype, scale_dtype,
+                       GemvFusion{});
 }
 
 // fp16 MFMA GEMM for M > 16 (gemm_i4.hip).
@@ -456,6 +544,40 @@ int32_t krm_linear_i4(krm_ctx* ctx, krm_buf x, krm_buf w, krm_buf scales, krm_bu
                            out + (size_t)r * n * eb, rows, n, k, group, io_dtype, scale_dtype));
   }
   return KRM_OK;
+}
+
+int32_t krm_linear_i4_fused(krm_ctx* ctx, krm_buf x, krm_buf norm_weight_f32, float norm_eps,
+                            krm_buf w, krm_buf scales, krm_buf bias, krm_buf residual,
+                            krm_buf out, uint32_t m, uint32_t n, uint32_t k, uint32_t group,
+                            int32_t io_dtype, int32_t scale_dtype, int32_t epilogue) {
+  KRM_TRY(enter(ctx));
+  KRM_REQUIRE(ctx, valid_dtype(io_dtype) && valid_dtype(scale_dtype),
+              "krm_linear_i4_fused: io_dtype %d / scale_dtype %d", io_dtype, scale_dtype);
+  KRM_REQUIRE(ctx, epilogue == KRM_EPILOGUE_NONE || epilogue == KRM_EPILOGUE_SILU_PAIRS,
+              "krm_linear_i4_fused: epilogue %d", epilogue);
+  KRM_REQUIRE(ctx, is_pow2(group) && group >= 16 && k >= 1 && k % group == 0,
+              "krm_linear_i4_fused: group_size %u must be a power of two >= 16 dividing k = %u",
+              group, k);
+  KRM_REQUIRE(ctx, m >= 1 && m <= 16,
+              "krm_linear_i4_fused: m = %u; the fused form covers 1..16 rows (use the separate ops "
+              "for prefill chunks)", m);
+  KRM_REQUIRE(ctx, epilogue != KRM_EPILOGUE_SILU_PAIRS || n % 2 == 0,
+              "krm_linear_i4_fused: the gate/up epilogue needs an even n, got %u", n);
+  KRM_REQUIRE(ctx, !norm_weight_f32 || std::isfinite(norm_eps), "krm_linear_i4_fused: eps");
+  if (n == 0) return KRM_OK;
+  KRM_REQUIRE(ctx, x && w && scales && out, "krm_linear_i4_fused: NULL buffer");
+  KRM_REQUIRE(ctx, aligned(x, 16) && aligned(norm_weight_f32, 16) && aligned(w, 4) &&
+                       aligned(out, dtype_bytes(io_dtype)) &&
+                       aligned(residual, dtype_bytes(io_dtype)) &&
+                       aligned(bias, dtype_bytes(io_dtype)) &&
+                       aligned(scales, dtype_bytes(scale_dtype)),
+              "krm_linear_i4_fused: x and norm weight must be 16-byte aligned, w 4-byte aligned");
+  GemvFusion fuse{};
+  fuse.norm_weight = ptr<const float>(norm_weight_f32);
+  fuse.norm_eps = norm_eps;
+  fuse.residual = ptr<const void>(residual);
+  fuse.pair_silu = epilogue == KRM_EPILOGUE_SILU_PAIRS ? 1u : 0u;
+  return gemv_dispatch(ctx, x, w, scales, bias, out, m, n, k, group, io_dtype, scale_dtype, fuse);
 }
 
 int32_t krm_dequant_i4(krm_ctx* ctx, krm_buf w, krm_buf scales, krm_buf out_f32, uint64_t rows,

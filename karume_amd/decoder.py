@@ -109,6 +109,22 @@ class _DeviceLinear:
         self.s = gpu.upload(lin.scales)
 
 
+def _stack_rows(*lins: Int4Linear) -> Int4Linear:
+    """[a; b; ...] along the output rows (one launch for q, k and v)."""
+    return Int4Linear(sum(l.n for l in lins), lins[0].k,
+                      np.concatenate([l.packed for l in lins], axis=0),
+                      np.concatenate([l.scales for l in lins], axis=0))
+
+
+def _interleave_rows(a: Int4Linear, b: Int4Linear) -> Int4Linear:
+    """Rows (2i, 2i+1) = (a_i, b_i): the layout of the fused gate/up epilogue."""
+    packed = np.empty((a.n * 2, a.packed.shape[1]), dtype=np.uint8)
+    packed[0::2], packed[1::2] = a.packed, b.packed
+    scales = np.empty((a.n * 2, a.scales.shape[1]), dtype=a.scales.dtype)
+    scales[0::2], scales[1::2] = a.scales, b.scales
+    return Int4Linear(a.n * 2, a.k, packed, scales)
+
+
 class LlamaDecoderSession:
     """Weights resident on the device + scratch activations for chunks of up to chunk_length
     rows.  io dtype selects f32 (the reference's semantic dtype) or fp16 activations; kv dtype
@@ -116,7 +132,7 @@ class LlamaDecoderSession:
 
     def __init__(self, gpu: GpuContext, weights: DecoderWeights, *, io_dtype: int = F32,
                  kv_dtype: int = F32, chunk_length: int = 128,
-                 prefill_compute: int = COMPUTE_F32):
+                 prefill_compute: int = COMPUTE_F32, fuse_decode: bool = True):
         self.gpu = gpu
         self.config = c = weights.config
         self.io_dtype, self.kv_dtype = io_dtype, kv_dtype
@@ -125,14 +141,21 @@ class LlamaDecoderSession:
         self.kv_eb = 2 if kv_dtype == F16 else 4
         self.chunk_length = chunk_length
         self.prefill_compute = prefill_compute
+        # One-row steps use the fused launches: rms_norm + [q;k;v], o + residual,
+        # rms_norm + interleaved gate/up + silu*mul, down + residual.
+        self.fuse_decode = fuse_decode
         self.embedding = gpu.upload(weights.embedding)
         self.layers = []
         for lw in weights.layers:
-            self.layers.append({
+            entry = {
                 "attn_norm": gpu.upload(lw["attn_norm"]), "ffn_norm": gpu.upload(lw["ffn_norm"]),
                 **{name: _DeviceLinear(gpu, lw[name])
                    for name in ("q", "k", "v", "o", "gate", "up", "down")},
-            })
+            }
+            if fuse_decode:
+                entry["qkv"] = _DeviceLinear(gpu, _stack_rows(lw["q"], lw["k"], lw["v"]))
+                entry["gate_up"] = _DeviceLinear(gpu, _interleave_rows(lw["gate"], lw["up"]))
+            self.layers.append(entry)
         self.final_norm = gpu.upload(weights.final_norm)
         self.lm_head = _DeviceLinear(gpu, weights.lm_head)
         self.rope_cos = gpu.upload(weights.rope_cos)
@@ -148,6 +171,7 @@ class LlamaDecoderSession:
             "att": a(m * hd * eb), "att2": a(m * hd * eb), "o": a(m * d * eb),
             "g": a(m * c.ffn * eb), "u": a(m * c.ffn * eb), "act": a(m * c.ffn * eb),
             "dn": a(m * d * eb), "logits": a(c.vocab * eb), "token": a(16),
+            "qkv": a((hd + 2 * kvd) * eb), "qkr": a((hd + kvd) * eb),
         }
         self.workspace: Optional[DeviceBuffer] = None
         self.logits_shape = (1, c.vocab)
@@ -205,6 +229,9 @@ class LlamaDecoderSession:
         d = c.d_model
         g.embedding(self.embedding, ids if ids is not None else b["ids"], b["h"], m, c.vocab, d,
                     F16, io)
+        if m == 1 and self.fuse_decode:
+            self._forward_fused_row(context, past, lengths)
+            return
         for li, lw in enumerate(self.layers):
             g.rms_norm(b["h"], lw["attn_norm"], b["xn"], m, d, c.rms_eps, io)
             self._linear(b["xn"], lw["q"], b["q"], m)
@@ -261,6 +288,56 @@ class LlamaDecoderSession:
         row = b["h"].offset(last_row * d * self.eb)
         g.rms_norm(row, self.final_norm, b["xn"], 1, d, c.rms_eps, io)
         self._linear(b["xn"], self.lm_head, b["logits"], 1)
+        g.argmax(b["logits"], b["token"], 1, c.vocab, io)
+
+    def _fused(self, x, lin: _DeviceLinear, out, **kw) -> None:
+        self.gpu.linear_i4_fused(x, lin.w, lin.s, out, 1, lin.n, lin.k, self.config.group_size,
+                                 io_dtype=self.io_dtype, scale_dtype=F16, **kw)
+
+    def _forward_fused_row(self, context: GenerationContext, past: int,
+                           lengths: Optional[DeviceBuffer]) -> None:
+        """One decode row (M = Q = 1), 8 launches per layer instead of 16."""
+        from .runtime import EPILOGUE_SILU_PAIRS
+        g, c, b, io, eb = self.gpu, self.config, self.buf, self.io_dtype, self.eb
+        hd, kvd = c.heads * c.head_dim, c.kv_heads * c.head_dim
+        q_r, k_r = b["qkr"], b["qkr"].offset(hd * eb)
+        v_row = b["qkv"].offset((hd + kvd) * eb)
+        spec = dict(chunk_rows=1, depth=c.head_dim, capacity=context.capacity,
+                    window=context.window)
+        for li, lw in enumerate(self.layers):
+            self._fused(b["h"], lw["qkv"], b["qkv"], norm_weight=lw["attn_norm"],
+                        norm_eps=c.rms_eps)
+            # q and k heads are contiguous in the [q;k;v] row: one rope launch over H + Hkv heads
+            g.rope_half(b["qkv"], b["pos"], self.rope_cos, self.rope_sin, b["qkr"], 1,
+                        c.heads + c.kv_heads, c.head_dim, c.max_position, True, io)
+            if lengths is None:
+                g.attention_state(q_r, k_r, v_row, context.slots_k[li], context.slots_v[li],
+                                  b["att"], batch=1, heads=c.heads, kv_heads=c.kv_heads,
+                                  half_scale=c.half_scale, past=past, query=1, io_dtype=io,
+                                  kv_dtype=self.kv_dtype, workspace=self.workspace, **spec)
+                g.state_append(k_r, context.slots_k[li], kv_planes=c.kv_heads, past=past, query=1,
+                               x_dtype=io, slot_dtype=self.kv_dtype, **spec)
+                g.state_append(v_row, context.slots_v[li], kv_planes=c.kv_heads, past=past,
+                               query=1, x_dtype=io, slot_dtype=self.kv_dtype, **spec)
+            else:
+                g.attention_state_lengths(q_r, k_r, v_row, context.slots_k[li],
+                                          context.slots_v[li], b["att"], batch=1, heads=c.heads,
+                                          kv_heads=c.kv_heads, half_scale=c.half_scale,
+                                          lengths=lengths, max_past=context.capacity - 1,
+                                          io_dtype=io, kv_dtype=self.kv_dtype,
+                                          workspace=self.workspace, **spec)
+                g.state_append_lengths(k_r, context.slots_k[li], kv_planes=c.kv_heads,
+                                       lengths=lengths, x_dtype=io, slot_dtype=self.kv_dtype,
+                                       **spec)
+                g.state_append_lengths(v_row, context.slots_v[li], kv_planes=c.kv_heads,
+                                       lengths=lengths, x_dtype=io, slot_dtype=self.kv_dtype,
+                                       **spec)
+            self._fused(b["att"], lw["o"], b["h"], residual=b["h"])
+            self._fused(b["h"], lw["gate_up"], b["act"], norm_weight=lw["ffn_norm"],
+                        norm_eps=c.rms_eps, epilogue=EPILOGUE_SILU_PAIRS)
+            self._fused(b["act"], lw["down"], b["h"], residual=b["h"])
+        self._fused(b["h"], self.lm_head, b["logits"], norm_weight=self.final_norm,
+                    norm_eps=c.rms_eps)
         g.argmax(b["logits"], b["token"], 1, c.vocab, io)
 
     # -- replayed decode ---------------------------------------------------------------------

@@ -18,6 +18,8 @@ F32 = 0
 F16 = 1
 COMPUTE_F32 = 0
 COMPUTE_F16 = 1
+EPILOGUE_NONE = 0
+EPILOGUE_SILU_PAIRS = 1
 
 _NP_DTYPE_CODE = {np.dtype(np.float32): F32, np.dtype(np.float16): F16}
 
@@ -250,6 +252,16 @@ class GpuContext:
         self._check(self._lib.krm_linear_i4(self._handle, _addr(x), _addr(w), _addr(scales),
                                             _addr(bias), _addr(out), m, n, k, group, io_dtype,
                                             scale_dtype, compute))
+
+    def linear_i4_fused(self, x: BufferLike, w: BufferLike, scales: BufferLike, out: BufferLike,
+                        m: int, n: int, k: int, group: int, *, norm_weight: BufferLike = None,
+                        norm_eps: float = 0.0, bias: BufferLike = None,
+                        residual: BufferLike = None, io_dtype: int = F32, scale_dtype: int = F32,
+                        epilogue: int = EPILOGUE_NONE) -> None:
+        self._check(self._lib.krm_linear_i4_fused(
+            self._handle, _addr(x), _addr(norm_weight), float(norm_eps), _addr(w), _addr(scales),
+            _addr(bias), _addr(residual), _addr(out), m, n, k, group, io_dtype, scale_dtype,
+            epilogue))
 
     def attention_state_workspace(self, batch: int, heads: int, kv_heads: int, chunk_rows: int,
                                   depth: int, window: int, max_past: int, max_query: int = 1

@@ -186,6 +186,27 @@ def test_greedy_loop_and_replayed_decode_agree(gpu_ctx):
         seq.append(stepwise[step])
 
 
+def test_fused_and_separate_decode_launches_agree(gpu_ctx):
+    """The fused one-row step (8 launches per layer) and the op-by-op step (16 launches) give
+    logits within 1e-4 of each other and the same tokens on a teacher-forced sequence."""
+    weights = random_weights(SMALL, seed=7)
+    ids = np.random.default_rng(2).integers(0, SMALL.vocab, size=14).astype(np.int32)
+    outs = []
+    for fuse in (True, False):
+        session = LlamaDecoderSession(gpu_ctx, weights, chunk_length=8, fuse_decode=fuse)
+        ctx = session.create_generation_context(capacity=32, chunk_length=8)
+        rows = []
+        for pos in range(14):
+            _tok, logits = session.run(ids[pos:pos + 1][None], np.array([[pos]], dtype=np.int32),
+                                       0, context=ctx, query_length=1, want_logits=True)
+            rows.append(logits[0].copy())
+        outs.append(np.stack(rows))
+        ctx.dispose()
+    assert np.max(np.abs(outs[0] - outs[1])) <= 1e-4
+    want = helpers.oracle_decoder_logits(weights, ids)
+    assert np.max(np.abs(outs[0] - want)) <= 2e-4
+
+
 def test_context_capacity_and_poison(gpu_ctx):
     """Capacity overflow is rejected before launch and leaves the context usable; a context is
     unusable after dispose (packages/runtime/tests/gpu_state_execution_test.ts:670-712)."""

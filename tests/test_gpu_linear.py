@@ -173,3 +173,51 @@ def test_linear_rejections(gpu_ctx):
     with pytest.raises(ka.GpuValidationError):
         gpu_ctx.dequant_i4(buf, buf, buf, 2, 8, 3)
     buf.free()
+
+
+def test_linear_fused_decode_forms(gpu_ctx):
+    """krm_linear_i4_fused: rms_norm folded in front, residual and silu(gate)*up folded behind,
+    against the oracle's op chain rms_norm -> linear -> (+ residual | silu*mul).  f32 io: atol
+    3e-5 rtol 2e-5 (the normalised row is not rounded between the ops here, so the result sits
+    slightly closer to the f64 chain than the unfused launches do)."""
+    rng = np.random.default_rng(8)
+    for m, n, k, g in [(1, 2560, 2048, 128), (3, 512, 1024, 128), (1, 64, 256, 32), (2, 40, 96, 16)]:
+        packed, _q, scale = helpers.synthetic_int4(rng, n, k, g)
+        x = (rng.normal(size=(m, k)) * 5).astype(np.float32)
+        gamma = rng.normal(size=k).astype(np.float32)
+        res = rng.normal(size=(m, n)).astype(np.float32)
+        sf = scale.astype(np.float32)
+        zeros = np.zeros(n, dtype=np.float32)
+        xn = oracle.rms_norm(x, gamma, 1e-5)
+        lin = oracle.linear_i4(xn, packed, sf, zeros, n, k, g)
+        bufs = [gpu_ctx.upload(a) for a in (x, packed, scale, gamma, res)]
+        dx, dw, ds, dg, dr = bufs
+        out = gpu_ctx.alloc(m * n * 4)
+        # norm + linear + residual
+        gpu_ctx.linear_i4_fused(dx, dw, ds, out, m, n, k, g, norm_weight=dg, norm_eps=1e-5,
+                                residual=dr, scale_dtype=ka.F16)
+        got = out.download(np.float32, (m, n))
+        ok, fails, max_abs, worst = oracle.allclose(got, lin + res, atol=3e-5, rtol=2e-5)
+        assert ok, (m, n, k, fails, max_abs, worst)
+        # in place on the residual buffer
+        gpu_ctx.linear_i4_fused(dx, dw, ds, dr, m, n, k, g, residual=dr, scale_dtype=ka.F16)
+        plain = oracle.linear_i4(x, packed, sf, zeros, n, k, g)
+        ok, fails, max_abs, worst = oracle.allclose(dr.download(np.float32, (m, n)), plain + res,
+                                                    atol=2e-4, rtol=2e-5)
+        assert ok, (fails, max_abs, worst)
+        # norm + interleaved gate/up + silu*mul
+        gpu_ctx.linear_i4_fused(dx, dw, ds, out, m, n, k, g, norm_weight=dg, norm_eps=1e-5,
+                                scale_dtype=ka.F16, epilogue=ka.EPILOGUE_SILU_PAIRS)
+        got = out.download(np.float32, (m, n // 2))
+        want = oracle.silu_mul(lin[:, 0::2], lin[:, 1::2])
+        ok, fails, max_abs, worst = oracle.allclose(got, want, atol=3e-5, rtol=5e-5)
+        assert ok, (fails, max_abs, worst)
+        for b in bufs + [out]:
+            b.free()
+    buf = gpu_ctx.zeros(1 << 16)
+    with pytest.raises(ka.GpuValidationError):  # prefill chunks use the separate ops
+        gpu_ctx.linear_i4_fused(buf, buf, buf, buf, 17, 64, 128, 128)
+    with pytest.raises(ka.GpuValidationError):
+        gpu_ctx.linear_i4_fused(buf, buf, buf, buf, 1, 63, 128, 128,
+                                epilogue=ka.EPILOGUE_SILU_PAIRS)
+    buf.free()
