@@ -241,12 +241,21 @@ struct DecodeArgs {
   uint32_t capacity;         // single sequence: slot rows (checked against device lengths)
 };
 
+// Columns are walked in chunks of kDecodeIter * G rows (G = 256 / lanes-per-row groups, each
+// owning one row per iteration).  Short pasts (<= kSingleSplitChunks chunks) stay in ONE split
+// that loops over its chunks — no partials, no merge; longer ones get one chunk per split.
+// The rule is a pure function of the number of past columns and the chunk size, so a sequence
+// is partitioned the same way alone and inside a ragged batch.
+constexpr uint32_t kSingleSplitChunks = 4;
 __host__ __device__ inline uint32_t decode_split_columns(uint32_t lanes_per_row) {
   return kDecodeIter * (kThreads / lanes_per_row);
 }
-__host__ __device__ inline uint32_t decode_splits(uint64_t slot_columns, uint32_t split_columns) {
-  const uint64_t n = (slot_columns + split_columns - 1) / split_columns;
-  return n ? (uint32_t)n : 1u;
+__host__ __device__ inline uint32_t decode_chunks(uint64_t slot_columns, uint32_t chunk_columns) {
+  return (uint32_t)((slot_columns + chunk_columns - 1) / chunk_columns);
+}
+__host__ __device__ inline uint32_t decode_splits(uint64_t slot_columns, uint32_t chunk_columns) {
+  const uint32_t chunks = decode_chunks(slot_columns, chunk_columns);
+  return chunks <= kSingleSplitChunks ? 1u : chunks;
 }
 
 constexpr float kLog2e = 1.4426950408889634f;
@@ -259,14 +268,16 @@ __device__ inline void publish(float* p, float v) {
 __device__ inline float observe(const float* p) {
   return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
-constexpr int kMergeChunk = 64;  // split partials merged per pass
+constexpr int kMergeChunk = 32;  // split partials merged per pass (all requested at once)
 
 // Workgroup = (split, kv head, batch | -): 256 threads = G groups of LPR lanes; a group owns
-// one K/V row per iteration, a lane 16 bytes of it.  Scores are kept in the base-2 domain
-// (q carries scale^2 * log2 e) so the exponentials are single v_exp_f32 instructions.
-// With several splits, every workgroup stores its (max, sum, weighted V) partial; the one
-// that arrives last at the (sequence, kv head) counter merges all partials of its r heads in
-// ascending split order — the result does not depend on which workgroup that is.
+// one K/V row per iteration, a lane 16 bytes of it.  Every group keeps its own running
+// (max, sum, weighted V) over the rows it sees — no workgroup barrier inside the column walk —
+// and the G group states are merged once at the end, in ascending group order.  Scores live
+// in the base-2 domain (q carries scale^2 * log2 e), so exponentials are single v_exp_f32.
+// With several splits every workgroup publishes its merged partial; the one that arrives last
+// at the (sequence, kv head) counter merges the partials of its r heads in ascending split
+// order — the result does not depend on which workgroup that is.
 template <typename XT, typename ST, int R, int LPR, bool RAGGED>
 __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 2)))
 void attention_decode_kernel(
@@ -276,17 +287,18 @@ void attention_decode_kernel(
   constexpr int E = RowChunk<ST>::E;
   constexpr int D = LPR * E;
   constexpr int G = kThreads / LPR;
-  constexpr int kWaves = kThreads / kWave;
-  __shared__ float s_max[kWaves][R];
-  __shared__ float s_sum[kWaves][R];
-  __shared__ float s_acc[kWaves][R][D];
-  __shared__ float s_ml[R][kMergeChunk][2];
+  constexpr int kChunkCols = kDecodeIter * G;
+  constexpr int kOuts = (R * D + kThreads - 1) / kThreads;
+  __shared__ float s_m[G][R];
+  __shared__ float s_l[G][R];
+  __shared__ float s_acc[G][R][D];
+  __shared__ float s_w[R][kMergeChunk];
+  __shared__ float s_wl[R][kMergeChunk];
   __shared__ uint32_t s_ticket;
 
   const int tid = threadIdx.x;
   const int sub = tid % LPR;   // which 16 bytes of the row
   const int group = tid / LPR;
-  const int wave = tid >> 6;
   const uint32_t hk = blockIdx.y;
 
   uint32_t seq, split, nsplit, first_split;
@@ -310,46 +322,25 @@ void attention_decode_kernel(
     if (!device_lengths(a.lengths, 1, a.capacity, a.window, p32, q32)) return;
     past = p32;
     row_base = 0;
-    nsplit = decode_splits(past - window_low(a.window, past), kDecodeIter * G);
+    nsplit = decode_splits(past - window_low(a.window, past), kChunkCols);
     split = blockIdx.x;
     if (split >= nsplit) return;  // the grid is sized for the longest past it may see
     first_split = seq * nsplit;
   }
   const uint64_t low = window_low(a.window, past);  // limit of row 0 is `past`
-  const uint64_t c_begin = low + (uint64_t)split * (kDecodeIter * G);
-  const uint64_t c_end = (c_begin + kDecodeIter * G < past) ? c_begin + kDecodeIter * G : past;
+  const uint32_t total_chunks = decode_chunks(past - low, kChunkCols);
+  const uint32_t my_chunks = nsplit == 1 ? total_chunks : 1u;
+  const uint64_t c_first = low + (uint64_t)split * kChunkCols;
   const bool last = split + 1 == nsplit;
 
   const size_t slot_base = (size_t)seq * a.slot_batch_stride + (size_t)hk * a.slot_plane_stride;
   const ST* kslot = slot_k + slot_base;
   const ST* vslot = slot_v + slot_base;
 
-  // requests first: K rows, V rows, this step's row (last split only)
-  uint4 kraw[kDecodeIter], vraw[kDecodeIter];
-  bool valid[kDecodeIter];
-#pragma unroll
-  for (int it = 0; it < kDecodeIter; ++it) {
-    const uint64_t col = c_begin + (uint64_t)it * G + group;
-    valid[it] = col < c_end;
-    kraw[it] = make_uint4(0, 0, 0, 0);
-    if (valid[it]) {
-      const uint64_t prow = row_base + (a.window ? col % a.window : col);
-      kraw[it] = *reinterpret_cast<const uint4*>(kslot + prow * D + sub * E);
-    }
-  }
-#pragma unroll
-  for (int it = 0; it < kDecodeIter; ++it) {
-    const uint64_t col = c_begin + (uint64_t)it * G + group;
-    vraw[it] = make_uint4(0, 0, 0, 0);
-    if (valid[it]) {
-      const uint64_t prow = row_base + (a.window ? col % a.window : col);
-      vraw[it] = *reinterpret_cast<const uint4*>(vslot + prow * D + sub * E);
-    }
-  }
+  // this step's own row and the query heads (valid addresses for every lane)
   const bool own = last && group == 0;  // the lanes that also take this step's own column
   float kx[E], vx[E];
   {
-    // read by every lane (the address is valid for all of them), used by `own` lanes only
     const size_t ins_base = ((size_t)seq * a.kv_heads + hk) * D + sub * E;
 #pragma unroll
     for (int e = 0; e < E; ++e) {
@@ -366,111 +357,138 @@ void attention_decode_kernel(
       qf[h][e] = ((ld_f32<XT>(q, q_base + e) * a.scale) * a.scale) * kLog2e;
   }
 
-  // scores (base-2 domain)
-  float sc[kDecodeIter + 1][R];
+  float run_m[R], run_l[R], acc[R][E];
 #pragma unroll
-  for (int it = 0; it < kDecodeIter; ++it) {
-    float kf[E];
-    RowChunk<ST>::unpack(kraw[it], kf);
+  for (int h = 0; h < R; ++h) {
+    run_m[h] = -INFINITY;
+    run_l[h] = 0.f;
+#pragma unroll
+    for (int e = 0; e < E; ++e) acc[h][e] = 0.f;
+  }
+
+  for (uint32_t chunk = 0; chunk < my_chunks; ++chunk) {
+    const uint64_t c_begin = c_first + (uint64_t)chunk * kChunkCols;
+    const uint64_t c_end = (c_begin + kChunkCols < past) ? c_begin + kChunkCols : past;
+    // requests first: every K row, then every V row of the chunk
+    uint4 kraw[kDecodeIter], vraw[kDecodeIter];
+    bool valid[kDecodeIter];
+#pragma unroll
+    for (int it = 0; it < kDecodeIter; ++it) {
+      const uint64_t col = c_begin + (uint64_t)it * G + group;
+      valid[it] = col < c_end;
+      kraw[it] = make_uint4(0, 0, 0, 0);
+      if (valid[it]) {
+        const uint64_t prow = row_base + (a.window ? col % a.window : col);
+        kraw[it] = *reinterpret_cast<const uint4*>(kslot + prow * D + sub * E);
+      }
+    }
+#pragma unroll
+    for (int it = 0; it < kDecodeIter; ++it) {
+      const uint64_t col = c_begin + (uint64_t)it * G + group;
+      vraw[it] = make_uint4(0, 0, 0, 0);
+      if (valid[it]) {
+        const uint64_t prow = row_base + (a.window ? col % a.window : col);
+        vraw[it] = *reinterpret_cast<const uint4*>(vslot + prow * D + sub * E);
+      }
+    }
+    float sc[kDecodeIter][R];
+    float cm[R];
+#pragma unroll
+    for (int h = 0; h < R; ++h) cm[h] = -INFINITY;
+#pragma unroll
+    for (int it = 0; it < kDecodeIter; ++it) {
+      float kf[E];
+      RowChunk<ST>::unpack(kraw[it], kf);
+#pragma unroll
+      for (int h = 0; h < R; ++h) {
+        float part = 0.f;
+#pragma unroll
+        for (int e = 0; e < E; ++e) part = fmaf(qf[h][e], kf[e], part);
+        part = group_sum<LPR>(part);
+        sc[it][h] = valid[it] ? part : -INFINITY;
+        cm[h] = fmaxf(cm[h], sc[it][h]);
+      }
+    }
+    float keep[R], ref[R];
 #pragma unroll
     for (int h = 0; h < R; ++h) {
-      float part = 0.f;
+      const float m_new = fmaxf(run_m[h], cm[h]);
+      ref[h] = m_new == -INFINITY ? 0.f : m_new;      // nothing seen yet: 2^(-inf - 0) = 0
+      keep[h] = __builtin_amdgcn_exp2f(run_m[h] - ref[h]);
+      run_m[h] = m_new;
+      run_l[h] *= keep[h];
 #pragma unroll
-      for (int e = 0; e < E; ++e) part = fmaf(qf[h][e], kf[e], part);
-      part = group_sum<LPR>(part);
-      sc[it][h] = valid[it] ? part : -INFINITY;
+      for (int e = 0; e < E; ++e) acc[h][e] *= keep[h];
+    }
+#pragma unroll
+    for (int it = 0; it < kDecodeIter; ++it) {
+      float vf[E];
+      RowChunk<ST>::unpack(vraw[it], vf);
+#pragma unroll
+      for (int h = 0; h < R; ++h) {
+        const float p = __builtin_amdgcn_exp2f(sc[it][h] - ref[h]);  // 0 outside the chunk
+        run_l[h] += p;
+#pragma unroll
+        for (int e = 0; e < E; ++e) acc[h][e] = fmaf(p, vf[e], acc[h][e]);
+      }
     }
   }
+  // this step's own column: one more row for group 0 of the last split
 #pragma unroll
   for (int h = 0; h < R; ++h) {
     float part = 0.f;
 #pragma unroll
     for (int e = 0; e < E; ++e) part = fmaf(qf[h][e], kx[e], part);
     part = group_sum<LPR>(part);
-    sc[kDecodeIter][h] = own ? part : -INFINITY;
+    const float s_own = own ? part : -INFINITY;
+    const float m_new = fmaxf(run_m[h], s_own);
+    const float ref = m_new == -INFINITY ? 0.f : m_new;
+    const float keep = __builtin_amdgcn_exp2f(run_m[h] - ref);
+    const float p = __builtin_amdgcn_exp2f(s_own - ref);
+    run_m[h] = m_new;
+    run_l[h] = run_l[h] * keep + p;
+#pragma unroll
+    for (int e = 0; e < E; ++e)
+      acc[h][e] = fmaf(p, own ? vx[e] : 0.f, acc[h][e] * keep);  // 0 * NaN must not leak
   }
 
-  // block max per head
-  float mx[R];
-#pragma unroll
-  for (int h = 0; h < R; ++h) {
-    float m = sc[0][h];
-#pragma unroll
-    for (int it = 1; it <= kDecodeIter; ++it) m = fmaxf(m, sc[it][h]);
-#pragma unroll
-    for (int off = LPR; off < kWave; off <<= 1) m = fmaxf(m, __shfl_xor(m, off, kWave));
-    if ((tid & (kWave - 1)) == 0) s_max[wave][h] = m;
-  }
-  __syncthreads();
-#pragma unroll
-  for (int h = 0; h < R; ++h) {
-    float m = s_max[0][h];
-#pragma unroll
-    for (int w = 1; w < kWaves; ++w) m = fmaxf(m, s_max[w][h]);
-    mx[h] = m;  // finite: a split always holds at least one column
-  }
-
-  // weights, their sum, and the weighted V rows
-  float acc[R][E];
-  float sum[R];
-#pragma unroll
-  for (int h = 0; h < R; ++h) {
-    sum[h] = 0.f;
-#pragma unroll
-    for (int e = 0; e < E; ++e) acc[h][e] = 0.f;
-  }
-#pragma unroll
-  for (int it = 0; it <= kDecodeIter; ++it) {
-    float vf[E];
-    if (it < kDecodeIter) {
-      RowChunk<ST>::unpack(vraw[it < kDecodeIter ? it : 0], vf);
-    } else {
-#pragma unroll
-      for (int e = 0; e < E; ++e) vf[e] = own ? vx[e] : 0.f;  // 0 * NaN must not leak
-    }
-#pragma unroll
-    for (int h = 0; h < R; ++h) {
-      // 2^(-inf) = 0 for columns outside the split
-      const float p = __builtin_amdgcn_exp2f(sc[it][h] - mx[h]);
-      sum[h] += p;
-#pragma unroll
-      for (int e = 0; e < E; ++e) acc[h][e] = fmaf(p, vf[e], acc[h][e]);
-    }
-  }
-  // fold the groups of a wave (lanes with equal `sub`), then the waves through LDS
+  // merge of the G group states, ascending group order
 #pragma unroll
   for (int h = 0; h < R; ++h) {
 #pragma unroll
-    for (int off = LPR; off < kWave; off <<= 1) {
-      sum[h] += __shfl_xor(sum[h], off, kWave);
-#pragma unroll
-      for (int e = 0; e < E; ++e) acc[h][e] += __shfl_xor(acc[h][e], off, kWave);
-    }
-    if ((tid & (kWave - 1)) < LPR) {
-#pragma unroll
-      for (int e = 0; e < E; ++e) s_acc[wave][h][sub * E + e] = acc[h][e];
-      if (sub == 0) s_sum[wave][h] = sum[h];
+    for (int e = 0; e < E; ++e) s_acc[group][h][sub * E + e] = acc[h][e];
+    if (sub == 0) {
+      s_m[group][h] = run_m[h];
+      s_l[group][h] = run_l[h];
     }
   }
   __syncthreads();
-
   const uint32_t gsplit = first_split + split;
-  for (int o = tid; o < R * D; o += kThreads) {
-    const int h = o / D, d = o - h * D;
-    float total = s_acc[0][h][d];
-    float l = s_sum[0][h];
-    float m = s_max[0][h];
+  float part_o[kOuts], part_l[kOuts], part_m[kOuts];
 #pragma unroll
-    for (int w = 1; w < kWaves; ++w) {
-      total += s_acc[w][h][d];
-      l += s_sum[w][h];
-      m = fmaxf(m, s_max[w][h]);
+  for (int i = 0; i < kOuts; ++i) {
+    const int o = tid + i * kThreads;
+    part_o[i] = part_l[i] = 0.f;
+    part_m[i] = -INFINITY;
+    if (o >= R * D) continue;
+    const int h = o / D, d = o - h * D;
+    float m = s_m[0][h];
+#pragma unroll
+    for (int g = 1; g < G; ++g) m = fmaxf(m, s_m[g][h]);  // finite: the split holds a column
+    float total = 0.f, l = 0.f;
+#pragma unroll
+    for (int g = 0; g < G; ++g) {
+      const float wgt = __builtin_amdgcn_exp2f(s_m[g][h] - m);
+      total = fmaf(wgt, s_acc[g][h][d], total);
+      l = fmaf(wgt, s_l[g][h], l);
     }
-    const uint32_t head = hk * R + h;
+    part_o[i] = total;
+    part_l[i] = l;
+    part_m[i] = m;
     if (nsplit == 1) {
-      st_f32<XT>(out, ((size_t)seq * a.heads + head) * D + d, total / l);
+      st_f32<XT>(out, ((size_t)seq * a.heads + hk * R + h) * D + d, total / l);
     } else {
-      const size_t slot_index = (size_t)gsplit * a.heads + head;
+      const size_t slot_index = (size_t)gsplit * a.heads + hk * R + h;
       publish(&ws_acc[slot_index * D + d], total);
       if (d == 0) {
         publish(&ws_ml[slot_index * 2], m);
@@ -491,70 +509,70 @@ void attention_decode_kernel(
   __syncthreads();
   if (s_ticket + 1 != nsplit) return;
 
-  // Merge nsplit partials of each of the R heads, kMergeChunk at a time, ascending order.
-  // Weights are prepared in LDS so the partial rows can be requested eight at a time.
-  constexpr int kOuts = (R * D + kThreads - 1) / kThreads;
-  float run_m[R], run_l[R];
-  float run_o[kOuts];
+  // Merge nsplit partials of each of the R heads, kMergeChunk at a time, ascending order; the
+  // partial rows of a pass are all requested before any is used.
+  float tot_m[R], tot_l[R];
+  float tot_o[kOuts];
 #pragma unroll
   for (int h = 0; h < R; ++h) {
-    run_m[h] = -INFINITY;
-    run_l[h] = 0.f;
+    tot_m[h] = -INFINITY;
+    tot_l[h] = 0.f;
   }
 #pragma unroll
-  for (int i = 0; i < kOuts; ++i) run_o[i] = 0.f;
+  for (int i = 0; i < kOuts; ++i) tot_o[i] = 0.f;
   for (uint32_t s0 = 0; s0 < nsplit; s0 += kMergeChunk) {
     const uint32_t cnt = nsplit - s0 < (uint32_t)kMergeChunk ? nsplit - s0 : (uint32_t)kMergeChunk;
+    // the weighted rows first (long latency), the small (max, sum) pairs next
+    float rows[kOuts][kMergeChunk];
+#pragma unroll
+    for (int i = 0; i < kOuts; ++i) {
+      const int o = tid + i * kThreads;
+      const int oo = o < R * D ? o : 0;
+      const int h = oo / D, d = oo - h * D;
+      const float* src = ws_acc + ((size_t)(first_split + s0) * a.heads + hk * R + h) * D + d;
+      const size_t stride = (size_t)a.heads * D;
+#pragma unroll
+      for (int j = 0; j < kMergeChunk; ++j)
+        rows[i][j] = observe(&src[(size_t)((uint32_t)j < cnt ? j : 0) * stride]);
+    }
     __syncthreads();
-    for (uint32_t i = tid; i < R * cnt; i += kThreads) {
-      const uint32_t h = i / cnt, s = i - h * cnt;
-      const size_t slot_index = (size_t)(first_split + s0 + s) * a.heads + hk * R + h;
-      s_ml[h][s][0] = observe(&ws_ml[slot_index * 2]);
-      s_ml[h][s][1] = observe(&ws_ml[slot_index * 2 + 1]);
+    for (uint32_t i = tid; i < R * kMergeChunk; i += kThreads) {
+      const uint32_t h = i / kMergeChunk, s = i - h * kMergeChunk;
+      const size_t slot_index = (size_t)(first_split + s0 + (s < cnt ? s : 0)) * a.heads + hk * R + h;
+      s_w[h][s] = s < cnt ? observe(&ws_ml[slot_index * 2]) : -INFINITY;
+      s_wl[h][s] = s < cnt ? observe(&ws_ml[slot_index * 2 + 1]) : 0.f;
     }
     __syncthreads();
     float keep[R];
 #pragma unroll
     for (int h = 0; h < R; ++h) {  // every thread tracks every head (uniform work)
-      float m = run_m[h];
-      for (uint32_t s = 0; s < cnt; ++s) m = fmaxf(m, s_ml[h][s][0]);
-      keep[h] = __builtin_amdgcn_exp2f(run_m[h] - m);  // 0 on the first pass
-      float l = run_l[h] * keep[h];
-      for (uint32_t s = 0; s < cnt; ++s)
-        l = fmaf(__builtin_amdgcn_exp2f(s_ml[h][s][0] - m), s_ml[h][s][1], l);
-      run_m[h] = m;
-      run_l[h] = l;
-    }
-    __syncthreads();
-    for (uint32_t i = tid; i < R * cnt; i += kThreads) {  // max -> weight, in place
-      const uint32_t h = i / cnt, s = i - h * cnt;
-      float m = run_m[0];
+      float m = tot_m[h];
 #pragma unroll
-      for (int hh = 1; hh < R; ++hh) m = (h == (uint32_t)hh) ? run_m[hh] : m;
-      s_ml[h][s][0] = __builtin_amdgcn_exp2f(s_ml[h][s][0] - m);
+      for (int j = 0; j < kMergeChunk; ++j) m = fmaxf(m, s_w[h][j]);
+      keep[h] = __builtin_amdgcn_exp2f(tot_m[h] - m);  // 0 on the first pass
+      float l = tot_l[h] * keep[h];
+#pragma unroll
+      for (int j = 0; j < kMergeChunk; ++j)
+        l = fmaf(__builtin_amdgcn_exp2f(s_w[h][j] - m), s_wl[h][j], l);
+      tot_m[h] = m;
+      tot_l[h] = l;
     }
-    __syncthreads();
 #pragma unroll
     for (int i = 0; i < kOuts; ++i) {
       const int o = tid + i * kThreads;
-      if (o >= R * D) break;
-      const int h = o / D, d = o - h * D;
-      float k_h = keep[0];
+      const int oo = o < R * D ? o : 0;
+      const int h = oo / D;
+      float k_h = keep[0], m_h = tot_m[0];
 #pragma unroll
-      for (int hh = 1; hh < R; ++hh) k_h = (h == hh) ? keep[hh] : k_h;
-      float total = run_o[i] * k_h;
-      const float* src = ws_acc + ((size_t)(first_split + s0) * a.heads + hk * R + h) * D + d;
-      const size_t stride = (size_t)a.heads * D;
-      for (uint32_t s = 0; s < cnt; s += 8) {
-        float v[8];
-#pragma unroll
-        for (int j = 0; j < 8; ++j)
-          v[j] = observe(&src[(size_t)(s + j < cnt ? s + j : s) * stride]);
-#pragma unroll
-        for (int j = 0; j < 8; ++j)
-          if (s + j < cnt) total = fmaf(s_ml[h][s + j][0], v[j], total);
+      for (int hh = 1; hh < R; ++hh) {
+        k_h = (h == hh) ? keep[hh] : k_h;
+        m_h = (h == hh) ? tot_m[hh] : m_h;
       }
-      run_o[i] = total;
+      float total = tot_o[i] * k_h;
+#pragma unroll
+      for (int j = 0; j < kMergeChunk; ++j)
+        total = fmaf(__builtin_amdgcn_exp2f(s_w[h][j] - m_h), rows[i][j], total);
+      tot_o[i] = total;
     }
   }
 #pragma unroll
@@ -562,10 +580,10 @@ void attention_decode_kernel(
     const int o = tid + i * kThreads;
     if (o >= R * D) break;
     const int h = o / D, d = o - h * D;
-    float l_h = run_l[0];
+    float l_h = tot_l[0];
 #pragma unroll
-    for (int hh = 1; hh < R; ++hh) l_h = (h == hh) ? run_l[hh] : l_h;
-    st_f32<XT>(out, ((size_t)seq * a.heads + hk * R + h) * D + d, run_o[i] / l_h);
+    for (int hh = 1; hh < R; ++hh) l_h = (h == hh) ? tot_l[hh] : l_h;
+    st_f32<XT>(out, ((size_t)seq * a.heads + hk * R + h) * D + d, tot_o[i] / l_h);
   }
   if (tid == 0)  // ready for the next launch
     __hip_atomic_store(&a.tickets[seq * a.kv_heads + hk], 0u, __ATOMIC_RELAXED,

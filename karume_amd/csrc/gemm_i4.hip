@@ -52,10 +52,10 @@ __device__ inline uint4 dequant_word(uint32_t word, _Float16 scale) {
   const uint32_t upper = word >> 8;
   const half2_t q0 = (__builtin_bit_cast(half2_t, (word & 0x000F000Fu) | magic) - off_lo) * s2;
   const half2_t q1 =
-      (__builtin_bit_cast(half2_t, (word & 0x00F000F0u) | magic) * sixteenth + off_hi) * s2;
+      (__builtin_elementwise_fma(__builtin_bit_cast(half2_t, (word & 0x00F000F0u) | magic), sixteenth, off_hi)) * s2;
   const half2_t q2 = (__builtin_bit_cast(half2_t, (upper & 0x000F000Fu) | magic) - off_lo) * s2;
   const half2_t q3 =
-      (__builtin_bit_cast(half2_t, (upper & 0x00F000F0u) | magic) * sixteenth + off_hi) * s2;
+      (__builtin_elementwise_fma(__builtin_bit_cast(half2_t, (upper & 0x00F000F0u) | magic), sixteenth, off_hi)) * s2;
   return make_uint4(__builtin_bit_cast(uint32_t, q0), __builtin_bit_cast(uint32_t, q1),
                     __builtin_bit_cast(uint32_t, q2), __builtin_bit_cast(uint32_t, q3));
 }

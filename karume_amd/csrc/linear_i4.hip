@@ -93,9 +93,9 @@ __device__ inline void codes_to_half2(uint32_t word, half2_t (&q)[4]) {
   const half2_t off_hi = {(_Float16)-72.0f, (_Float16)-72.0f};
   const uint32_t upper = word >> 8;
   q[0] = __builtin_bit_cast(half2_t, (word & 0x000F000Fu) | magic) - off_lo;
-  q[1] = __builtin_bit_cast(half2_t, (word & 0x00F000F0u) | magic) * sixteenth + off_hi;
+  q[1] = __builtin_elementwise_fma(__builtin_bit_cast(half2_t, (word & 0x00F000F0u) | magic), sixteenth, off_hi);
   q[2] = __builtin_bit_cast(half2_t, (upper & 0x000F000Fu) | magic) - off_lo;
-  q[3] = __builtin_bit_cast(half2_t, (upper & 0x00F000F0u) | magic) * sixteenth + off_hi;
+  q[3] = __builtin_elementwise_fma(__builtin_bit_cast(half2_t, (upper & 0x00F000F0u) | magic), sixteenth, off_hi);
 }
 
 // Eight consecutive fp16 activations (x0..x7 in four dwords) regrouped to match
@@ -119,7 +119,7 @@ struct Acts<__half> {
   };
   // `g` (optional): rms_norm weights of the same 8*VEC positions; the lane then carries
   // fp16(x * g) and adds its x^2 to `squares`.
-  template <int VEC>
+  template <int VEC, bool NORM>
   __device__ static inline void load(const __half* x, const float* g, bool active, Regs<VEC>& r,
                                      float& squares) {
 #pragma unroll
@@ -127,7 +127,7 @@ struct Acts<__half> {
       uint4 raw = reinterpret_cast<const uint4*>(x)[j];
       const uint32_t keep = active ? 0xFFFFFFFFu : 0u;  // bit mask: no control flow
       raw.x &= keep; raw.y &= keep; raw.z &= keep; raw.w &= keep;
-      if (g) {
+      if constexpr (NORM) {
         const float4 ga = reinterpret_cast<const float4*>(g)[2 * j];
         const float4 gb = reinterpret_cast<const float4*>(g)[2 * j + 1];
         const float gw[8] = {ga.x, ga.y, ga.z, ga.w, gb.x, gb.y, gb.z, gb.w};
@@ -170,7 +170,7 @@ struct Acts<float> {
     float v[VEC][8];
     float sum;
   };
-  template <int VEC>
+  template <int VEC, bool NORM>
   __device__ static inline void load(const float* x, const float* g, bool active, Regs<VEC>& r,
                                      float& squares) {
     float s = 0.f;
@@ -183,7 +183,7 @@ struct Acts<float> {
                              __uint_as_float(ua.z & keep), __uint_as_float(ua.w & keep));
       float4 b = make_float4(__uint_as_float(ub.x & keep), __uint_as_float(ub.y & keep),
                              __uint_as_float(ub.z & keep), __uint_as_float(ub.w & keep));
-      if (g) {
+      if constexpr (NORM) {
         const float4 ga = reinterpret_cast<const float4*>(g)[2 * j];
         const float4 gb = reinterpret_cast<const float4*>(g)[2 * j + 1];
         squares = fmaf(a.x, a.x, squares); squares = fmaf(a.y, a.y, squares);
@@ -245,7 +245,7 @@ struct GemvFusion {
 //  NSTEP == 0: any K; the next step's weights, scales and activations are requested before
 //             the current step is consumed.
 // Both forms add the per-step partial sums in ascending step order, so they agree bitwise.
-template <typename XT, typename ST, int MB, int ROWS, int VEC, int NSTEP>
+template <typename XT, typename ST, int MB, int ROWS, int VEC, int NSTEP, bool NORM>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 4))) void gemv_i4_kernel(
     const XT* __restrict__ x, const uint32_t* __restrict__ w, const ST* __restrict__ scales,
     const XT* __restrict__ bias, XT* __restrict__ out, uint32_t m, uint32_t n, uint32_t k,
@@ -303,9 +303,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 4))) voi
     const uint32_t k0 = step * kStepElems + lane * kLaneElems;
     const uint32_t xrow = min((uint32_t)b, m - 1);  // rows past M re-read the last row, unused
     const uint32_t kc = k0 < k ? k0 : 0u;
-    Acts<XT>::template load<VEC>(x + (size_t)xrow * k + kc,
-                                 fuse.norm_weight ? fuse.norm_weight + kc : nullptr, k0 < k, regs,
-                                 squares[b]);
+    Acts<XT>::template load<VEC, NORM>(x + (size_t)xrow * k + kc, fuse.norm_weight + kc, k0 < k,
+                                       regs, squares[b]);
   };
   auto consume = [&](const uint32_t (&cw)[ROWS][VEC], const float (&cs)[ROWS], int b,
                      const Regs& regs) {
@@ -375,8 +374,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 4))) voi
   float inv[MB];
 #pragma unroll
   for (int b = 0; b < MB; ++b)
-    inv[b] = fuse.norm_weight ? 1.0f / sqrtf(wave_sum(squares[b]) / (float)k + fuse.norm_eps)
-                              : 1.0f;
+    inv[b] = NORM ? 1.0f / sqrtf(wave_sum(squares[b]) / (float)k + fuse.norm_eps) : 1.0f;
   const XT* residual = static_cast<const XT*>(fuse.residual);
   if constexpr (ROWS == 2) {
     if (fuse.pair_silu) {
@@ -421,9 +419,14 @@ int32_t launch_gemv(krm_ctx* ctx, krm_buf x, krm_buf w, krm_buf scales, krm_buf 
                     const GemvFusion& fuse = GemvFusion{}) {
   const uint32_t rows_per_block = 4 * ROWS;
   const uint32_t blocks = (n + rows_per_block - 1) / rows_per_block;
-  gemv_i4_kernel<XT, ST, MB, ROWS, VEC, NSTEP><<<dim3(blocks), dim3(256), 0, ctx->stream>>>(
-      ptr<const XT>(x), ptr<const uint32_t>(w), ptr<const ST>(scales), ptr<const XT>(bias),
-      ptr<XT>(out), m, n, k, group_shift, fuse);
+  if (fuse.norm_weight)
+    gemv_i4_kernel<XT, ST, MB, ROWS, VEC, NSTEP, true><<<dim3(blocks), dim3(256), 0, ctx->stream>>>(
+        ptr<const XT>(x), ptr<const uint32_t>(w), ptr<const ST>(scales), ptr<const XT>(bias),
+        ptr<XT>(out), m, n, k, group_shift, fuse);
+  else
+    gemv_i4_kernel<XT, ST, MB, ROWS, VEC, NSTEP, false><<<dim3(blocks), dim3(256), 0, ctx->stream>>>(
+        ptr<const XT>(x), ptr<const uint32_t>(w), ptr<const ST>(scales), ptr<const XT>(bias),
+        ptr<XT>(out), m, n, k, group_shift, fuse);
   return launched(ctx, "gemv_i4_kernel");
 }
 
