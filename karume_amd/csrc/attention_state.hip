@@ -228,6 +228,8 @@ struct RowChunk<float> {
 
 struct DecodeArgs {
   uint32_t heads, kv_heads;
+  uint32_t repeat;           // query heads per kv head (H / Hkv)
+  uint32_t head_groups;      // workgroups one kv head's query heads are spread over
   uint32_t window;           // 0 = full context
   uint32_t past;             // single sequence: P.  ragged batch: unused
   uint64_t slot_batch_stride;  // elements between batches of the slot (0 for a ragged batch)
@@ -299,7 +301,8 @@ void attention_decode_kernel(
   const int tid = threadIdx.x;
   const int sub = tid % LPR;   // which 16 bytes of the row
   const int group = tid / LPR;
-  const uint32_t hk = blockIdx.y;
+  const uint32_t hk = blockIdx.y / a.head_groups;
+  const uint32_t head0 = hk * a.repeat + (blockIdx.y - hk * a.head_groups) * R;  // first head
 
   uint32_t seq, split, nsplit, first_split;
   uint64_t past, row_base;
@@ -351,7 +354,7 @@ void attention_decode_kernel(
   float qf[R][E];
 #pragma unroll
   for (int h = 0; h < R; ++h) {
-    const size_t q_base = ((size_t)seq * a.heads + (size_t)hk * R + h) * D + sub * E;
+    const size_t q_base = ((size_t)seq * a.heads + head0 + h) * D + sub * E;
 #pragma unroll
     for (int e = 0; e < E; ++e)
       qf[h][e] = ((ld_f32<XT>(q, q_base + e) * a.scale) * a.scale) * kLog2e;
@@ -486,9 +489,9 @@ void attention_decode_kernel(
     part_l[i] = l;
     part_m[i] = m;
     if (nsplit == 1) {
-      st_f32<XT>(out, ((size_t)seq * a.heads + hk * R + h) * D + d, total / l);
+      st_f32<XT>(out, ((size_t)seq * a.heads + head0 + h) * D + d, total / l);
     } else {
-      const size_t slot_index = (size_t)gsplit * a.heads + hk * R + h;
+      const size_t slot_index = (size_t)gsplit * a.heads + head0 + h;
       publish(&ws_acc[slot_index * D + d], total);
       if (d == 0) {
         publish(&ws_ml[slot_index * 2], m);
@@ -504,8 +507,8 @@ void attention_decode_kernel(
   __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
   __syncthreads();
   if (tid == 0)
-    s_ticket = __hip_atomic_fetch_add(&a.tickets[seq * a.kv_heads + hk], 1u, __ATOMIC_RELAXED,
-                                      __HIP_MEMORY_SCOPE_AGENT);
+    s_ticket = __hip_atomic_fetch_add(&a.tickets[seq * gridDim.y + blockIdx.y], 1u,
+                                      __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   __syncthreads();
   if (s_ticket + 1 != nsplit) return;
 
@@ -529,7 +532,7 @@ void attention_decode_kernel(
       const int o = tid + i * kThreads;
       const int oo = o < R * D ? o : 0;
       const int h = oo / D, d = oo - h * D;
-      const float* src = ws_acc + ((size_t)(first_split + s0) * a.heads + hk * R + h) * D + d;
+      const float* src = ws_acc + ((size_t)(first_split + s0) * a.heads + head0 + h) * D + d;
       const size_t stride = (size_t)a.heads * D;
 #pragma unroll
       for (int j = 0; j < kMergeChunk; ++j)
@@ -538,7 +541,7 @@ void attention_decode_kernel(
     __syncthreads();
     for (uint32_t i = tid; i < R * kMergeChunk; i += kThreads) {
       const uint32_t h = i / kMergeChunk, s = i - h * kMergeChunk;
-      const size_t slot_index = (size_t)(first_split + s0 + (s < cnt ? s : 0)) * a.heads + hk * R + h;
+      const size_t slot_index = (size_t)(first_split + s0 + (s < cnt ? s : 0)) * a.heads + head0 + h;
       s_w[h][s] = s < cnt ? observe(&ws_ml[slot_index * 2]) : -INFINITY;
       s_wl[h][s] = s < cnt ? observe(&ws_ml[slot_index * 2 + 1]) : 0.f;
     }
@@ -583,10 +586,10 @@ void attention_decode_kernel(
     float l_h = tot_l[0];
 #pragma unroll
     for (int hh = 1; hh < R; ++hh) l_h = (h == hh) ? tot_l[hh] : l_h;
-    st_f32<XT>(out, ((size_t)seq * a.heads + hk * R + h) * D + d, tot_o[i] / l_h);
+    st_f32<XT>(out, ((size_t)seq * a.heads + head0 + h) * D + d, tot_o[i] / l_h);
   }
   if (tid == 0)  // ready for the next launch
-    __hip_atomic_store(&a.tickets[seq * a.kv_heads + hk], 0u, __ATOMIC_RELAXED,
+    __hip_atomic_store(&a.tickets[seq * gridDim.y + blockIdx.y], 0u, __ATOMIC_RELAXED,
                        __HIP_MEMORY_SCOPE_AGENT);
 }
 
@@ -601,45 +604,64 @@ struct DecodeLaunch {
 template <typename XT, typename ST, int R, int LPR, bool RAGGED>
 int32_t launch_decode(krm_ctx* ctx, const DecodeLaunch& L) {
   attention_decode_kernel<XT, ST, R, LPR, RAGGED>
-      <<<dim3(L.grid_x, L.args.kv_heads, L.grid_z), dim3(kThreads), 0, ctx->stream>>>(
+      <<<dim3(L.grid_x, L.args.kv_heads * L.args.head_groups, L.grid_z), dim3(kThreads), 0,
+         ctx->stream>>>(
           ptr<const XT>(L.q), ptr<const XT>(L.ins_k), ptr<const XT>(L.ins_v),
           ptr<const ST>(L.slot_k), ptr<const ST>(L.slot_v), ptr<XT>(L.out), L.ws_ml, L.ws_acc,
           L.args);
   return launched(ctx, "attention_decode_kernel");
 }
 
+// `per_block` = query heads one workgroup carries (a divisor of H / Hkv).  A head's result
+// does not depend on it: every head keeps its own running state and its own merge.
 template <typename XT, typename ST, int LPR, bool RAGGED>
-int32_t decode_by_repeat(krm_ctx* ctx, const DecodeLaunch& L, uint32_t repeat) {
-  switch (repeat) {
+int32_t decode_by_repeat(krm_ctx* ctx, const DecodeLaunch& L, uint32_t per_block) {
+  switch (per_block) {
     case 1: return launch_decode<XT, ST, 1, LPR, RAGGED>(ctx, L);
     case 2: return launch_decode<XT, ST, 2, LPR, RAGGED>(ctx, L);
     case 4: return launch_decode<XT, ST, 4, LPR, RAGGED>(ctx, L);
     case 8: return launch_decode<XT, ST, 8, LPR, RAGGED>(ctx, L);
-    default: return fail(ctx, KRM_ERR_VALIDATION, "decode attention: H/Hkv = %u", repeat);
+    default: return fail(ctx, KRM_ERR_VALIDATION, "decode attention: %u heads per block", per_block);
   }
 }
 
 template <typename XT, typename ST, bool RAGGED>
-int32_t decode_by_depth(krm_ctx* ctx, const DecodeLaunch& L, uint32_t repeat, uint32_t lpr) {
+int32_t decode_by_depth(krm_ctx* ctx, const DecodeLaunch& L, uint32_t per_block, uint32_t lpr) {
   switch (lpr) {
-    case 4: return decode_by_repeat<XT, ST, 4, RAGGED>(ctx, L, repeat);
-    case 8: return decode_by_repeat<XT, ST, 8, RAGGED>(ctx, L, repeat);
-    case 16: return decode_by_repeat<XT, ST, 16, RAGGED>(ctx, L, repeat);
-    case 32: return decode_by_repeat<XT, ST, 32, RAGGED>(ctx, L, repeat);
+    case 4: return decode_by_repeat<XT, ST, 4, RAGGED>(ctx, L, per_block);
+    case 8: return decode_by_repeat<XT, ST, 8, RAGGED>(ctx, L, per_block);
+    case 16: return decode_by_repeat<XT, ST, 16, RAGGED>(ctx, L, per_block);
+    case 32: return decode_by_repeat<XT, ST, 32, RAGGED>(ctx, L, per_block);
     default: return fail(ctx, KRM_ERR_VALIDATION, "decode attention: %u lanes per row", lpr);
   }
 }
 
+// Few (split, kv head) pairs leave most of the chip idle while each workgroup walks its
+// columns once per query head; the query heads of a kv head are then spread over several
+// workgroups (each re-reads the K/V rows, which the L2 serves) until the grid covers the CUs.
 template <bool RAGGED>
-int32_t decode_dispatch(krm_ctx* ctx, const DecodeLaunch& L, uint32_t repeat, uint32_t lpr,
+int32_t decode_dispatch(krm_ctx* ctx, DecodeLaunch& L, uint32_t repeat, uint32_t lpr,
                         int32_t io_dtype, int32_t kv_dtype) {
+  uint32_t per_block = repeat;
+  uint64_t blocks = (uint64_t)L.grid_x * L.grid_z * L.args.kv_heads;
+  while (per_block > 1 && blocks < 2ull * (uint64_t)ctx->num_cus) {
+    per_block >>= 1;
+    blocks <<= 1;
+  }
+  L.args.repeat = repeat;
+  L.args.head_groups = repeat / per_block;
+  if ((uint64_t)L.args.kv_heads * L.args.head_groups > 65535 ||
+      (uint64_t)L.args.nseq * L.args.kv_heads * L.args.head_groups > kTicketSlots)
+    return fail(ctx, KRM_ERR_VALIDATION, "decode attention: B * H = %llu exceeds %u",
+                (unsigned long long)L.args.nseq * L.args.kv_heads * L.args.head_groups,
+                kTicketSlots);
   if (io_dtype == KRM_F16 && kv_dtype == KRM_F16)
-    return decode_by_depth<__half, __half, RAGGED>(ctx, L, repeat, lpr);
+    return decode_by_depth<__half, __half, RAGGED>(ctx, L, per_block, lpr);
   if (io_dtype == KRM_F32 && kv_dtype == KRM_F32)
-    return decode_by_depth<float, float, RAGGED>(ctx, L, repeat, lpr);
+    return decode_by_depth<float, float, RAGGED>(ctx, L, per_block, lpr);
   if (io_dtype == KRM_F32 && kv_dtype == KRM_F16)
-    return decode_by_depth<float, __half, RAGGED>(ctx, L, repeat, lpr);
-  return decode_by_depth<__half, float, RAGGED>(ctx, L, repeat, lpr);
+    return decode_by_depth<float, __half, RAGGED>(ctx, L, per_block, lpr);
+  return decode_by_depth<__half, float, RAGGED>(ctx, L, per_block, lpr);
 }
 
 // lanes a K/V row of `depth` elements spans with 16-byte pieces; 0 = not covered
@@ -742,7 +764,7 @@ static int32_t attention_state_impl(krm_ctx* ctx, krm_buf q, krm_buf ins_k, krm_
   const uint32_t lpr = decode_lanes_per_row(depth, kv_dtype);
   const bool fast = (dyn || query == 1) && chunk_rows == 1 && lpr && decode_repeat_ok(repeat) &&
                     aligned(slot_k, 16) && aligned(slot_v, 16) && batch <= 65535 &&
-                    kv_heads <= 65535 && (uint64_t)batch * kv_heads <= kTicketSlots;
+                    heads <= 65535 && (uint64_t)batch * heads <= kTicketSlots;
   if (fast) {
     const uint64_t low = window_low(window, past);
     const uint32_t nsplit = decode_splits((uint64_t)past - low, decode_split_columns(lpr));
@@ -839,8 +861,8 @@ int32_t krm_attention_varlen(krm_ctx* ctx, krm_buf q, krm_buf ins_k, krm_buf ins
   KRM_REQUIRE(ctx, std::isfinite(half_scale), "krm_attention_varlen: scale is not finite");
   KRM_REQUIRE(ctx, cu_seqlens != nullptr, "krm_attention_varlen: cu_seqlens is NULL");
   KRM_REQUIRE(ctx, total_rows <= 0x7fffffffull, "krm_attention_varlen: total_rows too large");
-  KRM_REQUIRE(ctx, kv_heads <= 65535 && (uint64_t)nseq * kv_heads <= kTicketSlots,
-              "krm_attention_varlen: nseq * Hkv = %llu exceeds %u", (unsigned long long)nseq * kv_heads,
+  KRM_REQUIRE(ctx, heads <= 65535 && (uint64_t)nseq * heads <= kTicketSlots,
+              "krm_attention_varlen: nseq * H = %llu exceeds %u", (unsigned long long)nseq * heads,
               kTicketSlots);
   const uint32_t repeat = heads / kv_heads;
   const uint32_t lpr = decode_lanes_per_row(depth, kv_dtype);

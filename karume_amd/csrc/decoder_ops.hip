@@ -168,19 +168,31 @@ __device__ inline bool beats(float va, uint32_t ia, float vb, uint32_t ib) {
   if (!na && va != vb) return va > vb;
   return ia < ib;
 }
+constexpr int kArgmaxThreads = 1024;
+constexpr int kArgmaxUnroll = 4;  // independent loads in flight per thread
 template <typename XT>
-__global__ __launch_bounds__(kThreads) void argmax_kernel(const XT* __restrict__ x,
-                                                         int32_t* __restrict__ out, uint32_t dim) {
-  __shared__ float s_val[kThreads / kWave];
-  __shared__ uint32_t s_idx[kThreads / kWave];
+__global__ __launch_bounds__(kArgmaxThreads) void argmax_kernel(const XT* __restrict__ x,
+                                                               int32_t* __restrict__ out,
+                                                               uint32_t dim) {
+  __shared__ float s_val[kArgmaxThreads / kWave];
+  __shared__ uint32_t s_idx[kArgmaxThreads / kWave];
   const size_t base = (size_t)blockIdx.x * dim;
   float best = -INFINITY;
   uint32_t at = dim;  // sentinel: any real element beats it on the index comparison
-  for (uint32_t i = threadIdx.x; i < dim; i += kThreads) {
-    const float v = ld<XT>(x, base + i);
-    if (beats(v, i, best, at)) {
-      best = v;
-      at = i;
+  for (uint32_t i0 = threadIdx.x; i0 < dim; i0 += kArgmaxThreads * kArgmaxUnroll) {
+    float v[kArgmaxUnroll];
+#pragma unroll
+    for (int u = 0; u < kArgmaxUnroll; ++u) {
+      const uint32_t i = i0 + u * kArgmaxThreads;
+      v[u] = ld<XT>(x, base + (i < dim ? i : i0));  // past the end: re-read, never wins (index)
+    }
+#pragma unroll
+    for (int u = 0; u < kArgmaxUnroll; ++u) {
+      const uint32_t i = i0 + u * kArgmaxThreads;
+      if (i < dim && beats(v[u], i, best, at)) {
+        best = v[u];
+        at = i;
+      }
     }
   }
   for (int off = 32; off > 0; off >>= 1) {
@@ -197,7 +209,7 @@ __global__ __launch_bounds__(kThreads) void argmax_kernel(const XT* __restrict__
   }
   __syncthreads();
   if (threadIdx.x == 0) {
-    for (int w = 1; w < kThreads / kWave; ++w)
+    for (int w = 1; w < kArgmaxThreads / kWave; ++w)
       if (beats(s_val[w], s_idx[w], best, at)) {
         best = s_val[w];
         at = s_idx[w];
@@ -344,9 +356,9 @@ int32_t krm_argmax(krm_ctx* ctx, krm_buf x, krm_buf out_i32, uint32_t rows, uint
   if (rows == 0) return KRM_OK;
   KRM_REQUIRE(ctx, x && out_i32, "krm_argmax: NULL buffer");
   KRM_IO_DISPATCH(io_dtype,
-                  (argmax_kernel<float><<<dim3(rows), dim3(kThreads), 0, ctx->stream>>>(
+                  (argmax_kernel<float><<<dim3(rows), dim3(kArgmaxThreads), 0, ctx->stream>>>(
                       ptr<const float>(x), ptr<int32_t>(out_i32), dim)),
-                  (argmax_kernel<__half><<<dim3(rows), dim3(kThreads), 0, ctx->stream>>>(
+                  (argmax_kernel<__half><<<dim3(rows), dim3(kArgmaxThreads), 0, ctx->stream>>>(
                       ptr<const __half>(x), ptr<int32_t>(out_i32), dim)));
   return launched(ctx, "argmax_kernel");
 }

@@ -86,16 +86,26 @@ __device__ inline float wave_sum(float v) {
 // Eight codes of one u32 as four fp16 pairs holding the exact integers (u - 8):
 // pair i = (code i, code i+4).  1024 + u is built in the fp16 mantissa, then the offset is
 // removed with one packed op; codes in the upper nibble of a byte arrive as 1024 + 16u.
+// (a & mask) | bits in one VALU op: the compiler splits it in two when both constants are
+// literals, because this ISA's three-operand encodings take no literal.
+__device__ inline uint32_t and_or(uint32_t a, uint32_t mask, uint32_t bits) {
+  uint32_t d;
+  asm("v_and_or_b32 %0, %1, %2, %3" : "=v"(d) : "v"(a), "s"(mask), "v"(bits));
+  return d;
+}
+
 __device__ inline void codes_to_half2(uint32_t word, half2_t (&q)[4]) {
   const uint32_t magic = 0x64006400u;  // (1024.0, 1024.0)
   const half2_t off_lo = {(_Float16)1032.0f, (_Float16)1032.0f};
   const half2_t sixteenth = {(_Float16)0.0625f, (_Float16)0.0625f};
   const half2_t off_hi = {(_Float16)-72.0f, (_Float16)-72.0f};
   const uint32_t upper = word >> 8;
-  q[0] = __builtin_bit_cast(half2_t, (word & 0x000F000Fu) | magic) - off_lo;
-  q[1] = __builtin_elementwise_fma(__builtin_bit_cast(half2_t, (word & 0x00F000F0u) | magic), sixteenth, off_hi);
-  q[2] = __builtin_bit_cast(half2_t, (upper & 0x000F000Fu) | magic) - off_lo;
-  q[3] = __builtin_elementwise_fma(__builtin_bit_cast(half2_t, (upper & 0x00F000F0u) | magic), sixteenth, off_hi);
+  q[0] = __builtin_bit_cast(half2_t, and_or(word, 0x000F000Fu, magic)) - off_lo;
+  q[1] = __builtin_elementwise_fma(__builtin_bit_cast(half2_t, and_or(word, 0x00F000F0u, magic)),
+                                   sixteenth, off_hi);
+  q[2] = __builtin_bit_cast(half2_t, and_or(upper, 0x000F000Fu, magic)) - off_lo;
+  q[3] = __builtin_elementwise_fma(__builtin_bit_cast(half2_t, and_or(upper, 0x00F000F0u, magic)),
+                                   sixteenth, off_hi);
 }
 
 // Eight consecutive fp16 activations (x0..x7 in four dwords) regrouped to match
@@ -125,9 +135,9 @@ struct Acts<__half> {
 #pragma unroll
     for (int j = 0; j < VEC; ++j) {
       uint4 raw = reinterpret_cast<const uint4*>(x)[j];
-      const uint32_t keep = active ? 0xFFFFFFFFu : 0u;  // bit mask: no control flow
-      raw.x &= keep; raw.y &= keep; raw.z &= keep; raw.w &= keep;
       if constexpr (NORM) {
+        const uint32_t keep = active ? 0xFFFFFFFFu : 0u;  // x^2 of a lane past K must be 0
+        raw.x &= keep; raw.y &= keep; raw.z &= keep; raw.w &= keep;
         const float4 ga = reinterpret_cast<const float4*>(g)[2 * j];
         const float4 gb = reinterpret_cast<const float4*>(g)[2 * j + 1];
         const float gw[8] = {ga.x, ga.y, ga.z, ga.w, gb.x, gb.y, gb.z, gb.w};
@@ -178,7 +188,7 @@ struct Acts<float> {
     for (int j = 0; j < VEC; ++j) {
       uint4 ua = reinterpret_cast<const uint4*>(x)[2 * j];
       uint4 ub = reinterpret_cast<const uint4*>(x)[2 * j + 1];
-      const uint32_t keep = active ? 0xFFFFFFFFu : 0u;  // bit mask: no control flow
+      const uint32_t keep = (!NORM || active) ? 0xFFFFFFFFu : 0u;  // x^2 past K must be 0
       float4 a = make_float4(__uint_as_float(ua.x & keep), __uint_as_float(ua.y & keep),
                              __uint_as_float(ua.z & keep), __uint_as_float(ua.w & keep));
       float4 b = make_float4(__uint_as_float(ub.x & keep), __uint_as_float(ub.y & keep),
@@ -280,8 +290,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 4))) voi
   }
 
   // Lanes past the end of K (last step of a K that is not a multiple of the step) read the
-  // row's first words instead and get zero activations and a zero scale, so every load is
-  // unconditional and all of them can be in flight together.
+  // row's first words and activations instead and their partial sum is dropped, so every load
+  // is unconditional and all of them can be in flight together.
   auto fetch = [&](uint32_t step, uint32_t (&dst_w)[ROWS][VEC], float (&dst_s)[ROWS]) {
     const uint32_t k0 = step * kStepElems + lane * kLaneElems;
     const bool active = k0 < k;
@@ -295,8 +305,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 4))) voi
 #pragma unroll
         for (int j = 0; j < VEC; ++j) dst_w[r][j] = wrow[r][(kc >> 3) + j];
       }
-      const float sv = load_scale<ST>(srow[r], kc >> group_shift);
-      dst_s[r] = active ? sv : 0.f;
+      dst_s[r] = load_scale<ST>(srow[r], kc >> group_shift);
     }
   };
   auto fetch_x = [&](uint32_t step, int b, Regs& regs) {
@@ -306,12 +315,14 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 4))) voi
     Acts<XT>::template load<VEC, NORM>(x + (size_t)xrow * k + kc, fuse.norm_weight + kc, k0 < k,
                                        regs, squares[b]);
   };
-  auto consume = [&](const uint32_t (&cw)[ROWS][VEC], const float (&cs)[ROWS], int b,
-                     const Regs& regs) {
+  auto consume = [&](uint32_t step, const uint32_t (&cw)[ROWS][VEC], const float (&cs)[ROWS],
+                     int b, const Regs& regs) {
+    // bit mask, not a select: a select lets the compiler move the dot product behind a branch
+    const uint32_t keep = step * kStepElems + lane * kLaneElems < k ? 0xFFFFFFFFu : 0u;
 #pragma unroll
     for (int r = 0; r < ROWS; ++r) {
       const float part = Acts<XT>::template dot<VEC>(cw[r], regs);
-      acc[r][b] = fmaf(part, cs[r], acc[r][b]);
+      acc[r][b] += __uint_as_float(__float_as_uint(part * cs[r]) & keep);
     }
   };
 
@@ -325,7 +336,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 4))) voi
 #pragma unroll
       for (int step = 0; step < NSTEP; ++step) fetch_x(step, 0, regs[step]);
 #pragma unroll
-      for (int step = 0; step < NSTEP; ++step) consume(all_w[step], all_s[step], 0, regs[step]);
+      for (int step = 0; step < NSTEP; ++step) consume(step, all_w[step], all_s[step], 0, regs[step]);
     } else {
 #pragma unroll
       for (int step = 0; step < NSTEP; ++step) {
@@ -333,7 +344,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 4))) voi
         for (int b = 0; b < MB; ++b) {
           Regs regs;
           fetch_x(step, b, regs);
-          consume(all_w[step], all_s[step], b, regs);
+          consume(step, all_w[step], all_s[step], b, regs);
         }
       }
     }
@@ -350,14 +361,14 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 4))) voi
         if constexpr (MB == 1) fetch_x(step + 1, 0, nxt_x);
       }
       if constexpr (MB == 1) {
-        consume(cur_w, cur_s, 0, cur_x);
+        consume(step, cur_w, cur_s, 0, cur_x);
         cur_x = nxt_x;
       } else {
 #pragma unroll
         for (int b = 0; b < MB; ++b) {
           Regs regs;
           fetch_x(step, b, regs);
-          consume(cur_w, cur_s, b, regs);
+          consume(step, cur_w, cur_s, b, regs);
         }
       }
 #pragma unroll
