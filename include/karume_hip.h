@@ -260,6 +260,21 @@ int32_t krm_rope_half(krm_ctx* ctx, krm_buf x, krm_buf positions_i32, krm_buf co
                       krm_buf sin_table_f32, krm_buf out, uint32_t rows, uint32_t heads,
                       uint32_t head_dim, uint32_t table_rows, int32_t to_head_major,
                       int32_t io_dtype);
+/* One decode row in one launch: RoPE (as krm_rope_half) of the H + Hkv leading heads of the
+ * [q; k; v] row `qkv` ([H + 2*Hkv, D], what a fused qkv linear writes) into qk_out
+ * ([H + Hkv, D]), plus the state_append (as krm_state_append with M = Q = 1) of the roped k row
+ * into slot_k and of the v row into slot_v.  `lengths` == 0: `past` is this run's pastLength;
+ * otherwise it is read on the device (and a violated run contract sets the fault word and
+ * appends nothing).  May be issued BEFORE the attention of the same step: a one-row step's
+ * attention never reads the slot row this writes.
+ * Fuses packages/runtime/src/kernels/rope.ts:5-20,52-80 and
+ * packages/runtime/src/kernels/state-append.ts:47-96. */
+int32_t krm_decode_rope_append(krm_ctx* ctx, krm_buf qkv, krm_buf positions_i32,
+                               krm_buf cos_table_f32, krm_buf sin_table_f32, krm_buf qk_out,
+                               krm_buf slot_k, krm_buf slot_v, uint32_t heads, uint32_t kv_heads,
+                               uint32_t depth, uint32_t table_rows, uint32_t capacity,
+                               uint32_t window, uint32_t past, krm_buf lengths, int32_t io_dtype,
+                               int32_t kv_dtype);
 /* [a, b, d] -> [b, a, d] (the reshape + permute between linears and attention). */
 int32_t krm_transpose_01(krm_ctx* ctx, krm_buf x, krm_buf out, uint32_t a, uint32_t b, uint32_t d,
                          int32_t io_dtype);

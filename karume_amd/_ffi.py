@@ -67,6 +67,8 @@ PROTOTYPES = {
     "krm_rms_norm": (i32, [c_ctx, c_buf, c_buf, c_buf, u32, u32, C.c_float, i32]),
     "krm_rope_half": (i32, [c_ctx, c_buf, c_buf, c_buf, c_buf, c_buf, u32, u32, u32, u32, i32,
                             i32]),
+    "krm_decode_rope_append": (i32, [c_ctx, c_buf, c_buf, c_buf, c_buf, c_buf, c_buf, c_buf, u32,
+                                     u32, u32, u32, u32, u32, u32, c_buf, i32, i32]),
     "krm_transpose_01": (i32, [c_ctx, c_buf, c_buf, u32, u32, u32, i32]),
     "krm_silu_mul": (i32, [c_ctx, c_buf, c_buf, c_buf, u64, i32]),
     "krm_add": (i32, [c_ctx, c_buf, c_buf, c_buf, u64, i32]),

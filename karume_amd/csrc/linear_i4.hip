@@ -171,19 +171,17 @@ struct Acts<__half> {
   }
 };
 
-// f32 activations: f32 products.  sum(u*x) is accumulated with one convert + one fma per
-// code and the offset is removed once per step: sum((u-8)*x) = sum(u*x) - 8*sum(x).
+// f32 activations: f32 products.  The codes become exact fp16 integers (u - 8) as above and
+// each one feeds a mixed-precision fma (fp16 * f32 + f32, the product is exact in f32).
 template <>
 struct Acts<float> {
   template <int VEC>
   struct Regs {
     float v[VEC][8];
-    float sum;
   };
   template <int VEC, bool NORM>
   __device__ static inline void load(const float* x, const float* g, bool active, Regs<VEC>& r,
                                      float& squares) {
-    float s = 0.f;
 #pragma unroll
     for (int j = 0; j < VEC; ++j) {
       uint4 ua = reinterpret_cast<const uint4*>(x)[2 * j];
@@ -205,24 +203,22 @@ struct Acts<float> {
       }
       r.v[j][0] = a.x; r.v[j][1] = a.y; r.v[j][2] = a.z; r.v[j][3] = a.w;
       r.v[j][4] = b.x; r.v[j][5] = b.y; r.v[j][6] = b.z; r.v[j][7] = b.w;
-      s += ((a.x + a.y) + (a.z + a.w)) + ((b.x + b.y) + (b.z + b.w));
     }
-    r.sum = s;
   }
   template <int VEC>
   __device__ static inline float dot(const uint32_t (&words)[VEC], const Regs<VEC>& r) {
     float acc = 0.f;
 #pragma unroll
     for (int j = 0; j < VEC; ++j) {
-      const uint32_t even = words[j] & 0x0F0F0F0Fu;         // codes 0,2,4,6 one per byte
-      const uint32_t odd = (words[j] >> 4) & 0x0F0F0F0Fu;   // codes 1,3,5,7
+      half2_t q[4];  // pair i = codes (i, i + 4)
+      codes_to_half2(words[j], q);
 #pragma unroll
-      for (int b = 0; b < 4; ++b) {
-        acc = fmaf((float)((even >> (8 * b)) & 0xFFu), r.v[j][2 * b], acc);
-        acc = fmaf((float)((odd >> (8 * b)) & 0xFFu), r.v[j][2 * b + 1], acc);
+      for (int i = 0; i < 4; ++i) {
+        acc = fmaf((float)q[i].x, r.v[j][i], acc);
+        acc = fmaf((float)q[i].y, r.v[j][i + 4], acc);
       }
     }
-    return fmaf(-8.0f, r.sum, acc);
+    return acc;
   }
 };
 

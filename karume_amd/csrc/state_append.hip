@@ -62,6 +62,63 @@ __global__ __launch_bounds__(256) void state_append_kernel(
   }
 }
 
+
+// One decode row ([q; k; v] as a fused qkv linear writes it): half-split RoPE of the q and k
+// heads (same roundings as rope_kernel: two rounded products, then the add;
+// packages/runtime/src/kernels/rope.ts:5-20,52-80) and the state_append of the roped k row and
+// the v row (packages/runtime/src/kernels/state-append.ts:47-96) in one launch.  Appending
+// before the attention of the same step is safe for a one-row step: the attention reads slot
+// columns c < past only, and the row written is column `past` (full context) or the physical
+// row of column past - window, which has just left the window (ring).
+template <typename XT, typename ST>
+__global__ __launch_bounds__(256) void decode_rope_append_kernel(
+    const XT* __restrict__ qkv, const int32_t* __restrict__ positions,
+    const float* __restrict__ cos_table, const float* __restrict__ sin_table,
+    XT* __restrict__ qk_out, ST* __restrict__ slot_k, ST* __restrict__ slot_v, uint32_t heads,
+    uint32_t kv_heads, uint32_t depth, uint32_t table_rows, uint32_t capacity, uint32_t window,
+    uint32_t past, uint32_t* lengths) {
+  bool append = true;
+  if (lengths) {
+    past = lengths[0];
+    const uint32_t query = lengths[1];
+    append = query == 1 && (uint64_t)past + 1 <= 0xffffffffull &&
+             (window != 0 || (uint64_t)past + 1 <= capacity);
+    if (!append && blockIdx.x == 0 && threadIdx.x == 0) lengths[2] = 1u;
+  }
+  const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
+  const uint32_t total = (heads + 2 * kv_heads) * depth;
+  if (i >= total) return;
+  const uint32_t head = i / depth, d = i - head * depth;
+  const uint64_t prow = window ? (uint64_t)past % window : (uint64_t)past;
+  if (head >= heads + kv_heads) {  // v: copy into the slot
+    if (append) {
+      const uint32_t plane = head - heads - kv_heads;
+      store_from_f32<ST>(slot_v, ((size_t)plane * capacity + prow) * depth + d,
+                         load_as_f32<XT>(qkv, i));
+    }
+    return;
+  }
+  const int32_t pos = positions[0];
+  const uint32_t half = depth / 2;
+  float value;
+  if (pos < 0 || (uint32_t)pos >= table_rows) {
+    value = NAN;
+  } else {
+    const float self = load_as_f32<XT>(qkv, i);
+    const float other = d < half ? -load_as_f32<XT>(qkv, i + half) : load_as_f32<XT>(qkv, i - half);
+    const size_t t = (size_t)pos * depth + d;
+    const float direct = __fmul_rn(self, cos_table[t]);
+    const float cross = __fmul_rn(other, sin_table[t]);
+    value = __fadd_rn(direct, cross);
+  }
+  store_from_f32<XT>(qk_out, i, value);
+  if (head >= heads && append) {
+    // the slot holds what a separate state_append would copy from the stored (rounded) k row
+    const float stored = sizeof(XT) == 2 ? __half2float(__float2half_rn(value)) : value;
+    store_from_f32<ST>(slot_k, ((size_t)(head - heads) * capacity + prow) * depth + d, stored);
+  }
+}
+
 template <typename XT, typename ST>
 int32_t launch(krm_ctx* ctx, krm_buf x, krm_buf slot, uint32_t kv_planes, uint32_t chunk_rows,
                uint32_t depth, uint32_t capacity, uint32_t window, uint32_t past,
@@ -114,6 +171,62 @@ static int32_t state_append_impl(krm_ctx* ctx, krm_buf x, krm_buf slot, uint32_t
                                   past, query, lengths);
   return launch<__half, float>(ctx, x, slot, kv_planes, chunk_rows, depth, capacity, window, past,
                                query, lengths);
+}
+
+template <typename XT, typename ST>
+static int32_t launch_rope_append(krm_ctx* ctx, krm_buf qkv, krm_buf positions, krm_buf cos_table,
+                                  krm_buf sin_table, krm_buf qk_out, krm_buf slot_k,
+                                  krm_buf slot_v, uint32_t heads, uint32_t kv_heads,
+                                  uint32_t depth, uint32_t table_rows, uint32_t capacity,
+                                  uint32_t window, uint32_t past, krm_buf lengths) {
+  const uint32_t total = (heads + 2 * kv_heads) * depth;
+  decode_rope_append_kernel<XT, ST><<<dim3((total + 255) / 256), dim3(256), 0, ctx->stream>>>(
+      ptr<const XT>(qkv), ptr<const int32_t>(positions), ptr<const float>(cos_table),
+      ptr<const float>(sin_table), ptr<XT>(qk_out), ptr<ST>(slot_k), ptr<ST>(slot_v), heads,
+      kv_heads, depth, table_rows, capacity, window, past, ptr<uint32_t>(lengths));
+  return launched(ctx, "decode_rope_append_kernel");
+}
+
+extern "C" int32_t krm_decode_rope_append(krm_ctx* ctx, krm_buf qkv, krm_buf positions_i32,
+                                          krm_buf cos_table_f32, krm_buf sin_table_f32,
+                                          krm_buf qk_out, krm_buf slot_k, krm_buf slot_v,
+                                          uint32_t heads, uint32_t kv_heads, uint32_t depth,
+                                          uint32_t table_rows, uint32_t capacity, uint32_t window,
+                                          uint32_t past, krm_buf lengths, int32_t io_dtype,
+                                          int32_t kv_dtype) {
+  KRM_TRY(enter(ctx));
+  KRM_REQUIRE(ctx, valid_dtype(io_dtype) && valid_dtype(kv_dtype),
+              "krm_decode_rope_append: io_dtype %d / kv_dtype %d", io_dtype, kv_dtype);
+  KRM_REQUIRE(ctx, heads >= 1 && kv_heads >= 1 && depth >= 2 && depth % 2 == 0 && capacity >= 1 &&
+                       table_rows >= 1,
+              "krm_decode_rope_append: H / Hkv / D / C / table rows (%u / %u / %u / %u / %u)",
+              heads, kv_heads, depth, capacity, table_rows);
+  KRM_REQUIRE(ctx, ((uint64_t)heads + 2ull * kv_heads) * depth <= 0x7fffffffull,
+              "krm_decode_rope_append: the row is too long");
+  KRM_REQUIRE(ctx, window <= capacity, "krm_decode_rope_append: window %u exceeds capacity %u",
+              window, capacity);
+  if (!lengths && window == 0 && (uint64_t)past + 1 > capacity)
+    return fail(ctx, KRM_ERR_EXECUTION,
+                "krm_decode_rope_append: pastLength %u + queryLength 1 exceeds capacity %u", past,
+                capacity);
+  KRM_REQUIRE(ctx, qkv && positions_i32 && cos_table_f32 && sin_table_f32 && qk_out && slot_k &&
+                       slot_v,
+              "krm_decode_rope_append: NULL buffer");
+  const size_t io_b = dtype_bytes(io_dtype), kv_b = dtype_bytes(kv_dtype);
+  KRM_REQUIRE(ctx,
+              aligned(qkv, io_b) && aligned(qk_out, io_b) && aligned(slot_k, kv_b) &&
+                  aligned(slot_v, kv_b) && aligned(positions_i32, 4) &&
+                  aligned(cos_table_f32, 4) && aligned(sin_table_f32, 4) && aligned(lengths, 4),
+              "krm_decode_rope_append: misaligned buffer");
+#define KRM_ROPE_APPEND(XT, ST)                                                              \
+  return launch_rope_append<XT, ST>(ctx, qkv, positions_i32, cos_table_f32, sin_table_f32,   \
+                                    qk_out, slot_k, slot_v, heads, kv_heads, depth,          \
+                                    table_rows, capacity, window, past, lengths)
+  if (io_dtype == KRM_F32 && kv_dtype == KRM_F32) KRM_ROPE_APPEND(float, float);
+  if (io_dtype == KRM_F32 && kv_dtype == KRM_F16) KRM_ROPE_APPEND(float, __half);
+  if (io_dtype == KRM_F16 && kv_dtype == KRM_F16) KRM_ROPE_APPEND(__half, __half);
+  KRM_ROPE_APPEND(__half, float);
+#undef KRM_ROPE_APPEND
 }
 
 // Run-time lengths {past, query, fault} kept in device memory so a recorded step can be

@@ -296,7 +296,7 @@ class LlamaDecoderSession:
 
     def _forward_fused_row(self, context: GenerationContext, past: int,
                            lengths: Optional[DeviceBuffer]) -> None:
-        """One decode row (M = Q = 1), 8 launches per layer instead of 16."""
+        """One decode row (M = Q = 1), 6 launches per layer instead of 16."""
         from .runtime import EPILOGUE_SILU_PAIRS
         g, c, b, io, eb = self.gpu, self.config, self.buf, self.io_dtype, self.eb
         hd, kvd = c.heads * c.head_dim, c.kv_heads * c.head_dim
@@ -307,18 +307,19 @@ class LlamaDecoderSession:
         for li, lw in enumerate(self.layers):
             self._fused(b["h"], lw["qkv"], b["qkv"], norm_weight=lw["attn_norm"],
                         norm_eps=c.rms_eps)
-            # q and k heads are contiguous in the [q;k;v] row: one rope launch over H + Hkv heads
-            g.rope_half(b["qkv"], b["pos"], self.rope_cos, self.rope_sin, b["qkr"], 1,
-                        c.heads + c.kv_heads, c.head_dim, c.max_position, True, io)
+            # rope of the q and k heads and both appends in one launch; a one-row step's
+            # attention never reads the slot row this writes, so it may go first
+            g.decode_rope_append(b["qkv"], b["pos"], self.rope_cos, self.rope_sin, b["qkr"],
+                                 context.slots_k[li], context.slots_v[li], heads=c.heads,
+                                 kv_heads=c.kv_heads, depth=c.head_dim,
+                                 table_rows=c.max_position, capacity=context.capacity,
+                                 window=context.window, past=past, lengths=lengths, io_dtype=io,
+                                 kv_dtype=self.kv_dtype)
             if lengths is None:
                 g.attention_state(q_r, k_r, v_row, context.slots_k[li], context.slots_v[li],
                                   b["att"], batch=1, heads=c.heads, kv_heads=c.kv_heads,
                                   half_scale=c.half_scale, past=past, query=1, io_dtype=io,
                                   kv_dtype=self.kv_dtype, workspace=self.workspace, **spec)
-                g.state_append(k_r, context.slots_k[li], kv_planes=c.kv_heads, past=past, query=1,
-                               x_dtype=io, slot_dtype=self.kv_dtype, **spec)
-                g.state_append(v_row, context.slots_v[li], kv_planes=c.kv_heads, past=past,
-                               query=1, x_dtype=io, slot_dtype=self.kv_dtype, **spec)
             else:
                 g.attention_state_lengths(q_r, k_r, v_row, context.slots_k[li],
                                           context.slots_v[li], b["att"], batch=1, heads=c.heads,
@@ -326,12 +327,6 @@ class LlamaDecoderSession:
                                           lengths=lengths, max_past=context.capacity - 1,
                                           io_dtype=io, kv_dtype=self.kv_dtype,
                                           workspace=self.workspace, **spec)
-                g.state_append_lengths(k_r, context.slots_k[li], kv_planes=c.kv_heads,
-                                       lengths=lengths, x_dtype=io, slot_dtype=self.kv_dtype,
-                                       **spec)
-                g.state_append_lengths(v_row, context.slots_v[li], kv_planes=c.kv_heads,
-                                       lengths=lengths, x_dtype=io, slot_dtype=self.kv_dtype,
-                                       **spec)
             self._fused(b["att"], lw["o"], b["h"], residual=b["h"])
             self._fused(b["h"], lw["gate_up"], b["act"], norm_weight=lw["ffn_norm"],
                         norm_eps=c.rms_eps, epilogue=EPILOGUE_SILU_PAIRS)

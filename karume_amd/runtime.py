@@ -368,6 +368,19 @@ class GpuContext:
             self._handle, _addr(x), _addr(positions), _addr(cos_table), _addr(sin_table),
             _addr(out), rows, heads, head_dim, table_rows, int(to_head_major), io_dtype))
 
+    def decode_rope_append(self, qkv: BufferLike, positions: BufferLike, cos_table: BufferLike,
+                           sin_table: BufferLike, qk_out: BufferLike, slot_k: BufferLike,
+                           slot_v: BufferLike, *, heads: int, kv_heads: int, depth: int,
+                           table_rows: int, capacity: int, window: int = 0, past: int = 0,
+                           lengths: Optional[BufferLike] = None, io_dtype: int = F32,
+                           kv_dtype: int = F32) -> None:
+        """RoPE of the q and k heads of one [q; k; v] row + state_append of k and v."""
+        self._check(self._lib.krm_decode_rope_append(
+            self._handle, _addr(qkv), _addr(positions), _addr(cos_table), _addr(sin_table),
+            _addr(qk_out), _addr(slot_k), _addr(slot_v), heads, kv_heads, depth, table_rows,
+            capacity, window, past, _addr(lengths) if lengths is not None else 0, io_dtype,
+            kv_dtype))
+
     def transpose_01(self, x: BufferLike, out: BufferLike, a: int, b: int, d: int,
                      io_dtype: int = F32) -> None:
         self._check(self._lib.krm_transpose_01(self._handle, _addr(x), _addr(out), a, b, d,

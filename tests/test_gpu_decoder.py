@@ -84,6 +84,69 @@ def test_rope_silu_add_embedding_argmax(gpu_ctx):
     assert got.tolist() == [300, 2, 0, 999, int(oracle.argmax(rows_x[4:5])[0, 0])]
 
 
+@pytest.mark.parametrize("io,kv", [(ka.F32, ka.F32), (ka.F32, ka.F16), (ka.F16, ka.F16)])
+@pytest.mark.parametrize("window,past", [(0, 5), (4, 9), (0, 0)])
+def test_decode_rope_append_equals_rope_then_appends(gpu_ctx, io, kv, window, past):
+    """The one-launch decode row is bit-identical to krm_rope_half + two krm_state_append,
+    with a host past and with device lengths; a violated contract appends nothing."""
+    rng = np.random.default_rng(7 + past)
+    heads, kv_heads, d, table, cap = 6, 2, 16, 32, 12
+    io_np = np.float32 if io == ka.F32 else np.float16
+    kv_np = np.float32 if kv == ka.F32 else np.float16
+    qkv = rng.normal(size=(heads + 2 * kv_heads, d)).astype(io_np)
+    ang = rng.normal(size=(table, d))
+    cos, sin = np.cos(ang).astype(np.float32), np.sin(ang).astype(np.float32)
+    pos = np.array([past], dtype=np.int32)
+    slot0_k = rng.normal(size=(kv_heads, cap, d)).astype(kv_np)
+    slot0_v = rng.normal(size=(kv_heads, cap, d)).astype(kv_np)
+    dq, dp, dc, ds = map(gpu_ctx.upload, (qkv, pos, cos, sin))
+
+    # separate launches
+    ref_qk = gpu_ctx.alloc((heads + kv_heads) * d * qkv.itemsize)
+    ref_k, ref_v = gpu_ctx.upload(slot0_k), gpu_ctx.upload(slot0_v)
+    gpu_ctx.rope_half(dq, dp, dc, ds, ref_qk, 1, heads + kv_heads, d, table, True, io)
+    spec = dict(kv_planes=kv_heads, chunk_rows=1, depth=d, capacity=cap, window=window,
+                x_dtype=io, slot_dtype=kv)
+    gpu_ctx.state_append(ref_qk.offset(heads * d * qkv.itemsize), ref_k, past=past, query=1, **spec)
+    gpu_ctx.state_append(dq.offset((heads + kv_heads) * d * qkv.itemsize), ref_v, past=past,
+                         query=1, **spec)
+    want_qk = ref_qk.download(io_np, (heads + kv_heads, d))
+    want_k, want_v = ref_k.download(kv_np, slot0_k.shape), ref_v.download(kv_np, slot0_v.shape)
+    row = past % window if window else past
+    assert not np.array_equal(want_k[:, row], slot0_k[:, row])
+
+    lengths = gpu_ctx.zeros(16)
+    for dyn in (False, True):
+        got_qk = gpu_ctx.zeros((heads + kv_heads) * d * qkv.itemsize)
+        got_k, got_v = gpu_ctx.upload(slot0_k), gpu_ctx.upload(slot0_v)
+        if dyn:
+            gpu_ctx.lengths_set(lengths, past, 1)
+        gpu_ctx.decode_rope_append(dq, dp, dc, ds, got_qk, got_k, got_v, heads=heads,
+                                   kv_heads=kv_heads, depth=d, table_rows=table, capacity=cap,
+                                   window=window, past=0 if dyn else past,
+                                   lengths=lengths if dyn else None, io_dtype=io, kv_dtype=kv)
+        assert got_qk.download(io_np, want_qk.shape).tobytes() == want_qk.tobytes()
+        assert got_k.download(kv_np, want_k.shape).tobytes() == want_k.tobytes()
+        assert got_v.download(kv_np, want_v.shape).tobytes() == want_v.tobytes()
+    assert lengths.download(np.uint32, (4,))[2] == 0
+
+    if window == 0:
+        # past = capacity: the host form refuses, the device form raises the fault word and
+        # leaves both slots untouched
+        with pytest.raises(ka.ExecutionError):
+            gpu_ctx.decode_rope_append(dq, dp, dc, ds, got_qk, got_k, got_v, heads=heads,
+                                       kv_heads=kv_heads, depth=d, table_rows=table,
+                                       capacity=cap, past=cap, io_dtype=io, kv_dtype=kv)
+        clean_k, clean_v = gpu_ctx.upload(slot0_k), gpu_ctx.upload(slot0_v)
+        gpu_ctx.lengths_set(lengths, cap, 1)
+        gpu_ctx.decode_rope_append(dq, dp, dc, ds, got_qk, clean_k, clean_v, heads=heads,
+                                   kv_heads=kv_heads, depth=d, table_rows=table, capacity=cap,
+                                   lengths=lengths, io_dtype=io, kv_dtype=kv)
+        assert lengths.download(np.uint32, (4,))[2] == 1
+        assert clean_k.download(kv_np, slot0_k.shape).tobytes() == slot0_k.tobytes()
+        assert clean_v.download(kv_np, slot0_v.shape).tobytes() == slot0_v.tobytes()
+
+
 def test_transpose(gpu_ctx):
     x = np.arange(3 * 5 * 4, dtype=np.float32).reshape(3, 5, 4)
     dx = gpu_ctx.upload(x)
