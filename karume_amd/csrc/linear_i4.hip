@@ -251,6 +251,15 @@ struct GemvFusion {
 //  NSTEP == 0: any K; the next step's weights, scales and activations are requested before
 //             the current step is consumed.
 // Both forms add the per-step partial sums in ascending step order, so they agree bitwise.
+//  Shared activations (one row of f32 x, NSTEP > 0): every wave of the workgroup needs the
+//  same x, which for f32 is four times the bytes of the two weight rows it meets; wave s
+//  prepares step s once (norm weight applied) and parks it in LDS for the others, after all
+//  weight requests are out.
+template <typename XT, int MB, int NSTEP>
+constexpr bool share_x_in_lds() {
+  return sizeof(XT) == 4 && MB == 1 && NSTEP > 0 && NSTEP <= 4;
+}
+
 template <typename XT, typename ST, int MB, int ROWS, int VEC, int NSTEP, bool NORM>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 4))) void gemv_i4_kernel(
     const XT* __restrict__ x, const uint32_t* __restrict__ w, const ST* __restrict__ scales,
@@ -261,8 +270,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 4))) voi
   using Regs = typename Acts<XT>::template Regs<VEC>;
   const int lane = threadIdx.x & (kWave - 1);
   const int wave = threadIdx.x >> 6;
+  constexpr bool XLDS = share_x_in_lds<XT, MB, NSTEP>();
   const uint32_t row0 = (blockIdx.x * (blockDim.x >> 6) + wave) * ROWS;
-  if (row0 >= n) return;  // whole wave leaves together
+  if (!XLDS && row0 >= n) return;  // whole wave leaves together (XLDS: it still stages x)
 
   const uint32_t words_per_row = k >> 3;
   const uint32_t groups_per_row = k >> group_shift;
@@ -277,6 +287,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 4))) voi
   }
 
   float acc[ROWS][MB];
+  float shared_squares = 0.f;  // XLDS: sum of x^2 over the whole row
   float squares[MB];  // sum of x^2 over the lane's share of K (fused rms_norm only)
 #pragma unroll
   for (int b = 0; b < MB; ++b) {
@@ -327,7 +338,41 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 4))) voi
     float all_s[NSTEP][ROWS];
 #pragma unroll
     for (int step = 0; step < NSTEP; ++step) fetch(step, all_w[step], all_s[step]);
-    if constexpr (MB == 1) {
+    if constexpr (XLDS) {
+      // 16-byte units, unit u of lane l at [(step * kUnits + u) * 64 + l]: conflict-free
+      constexpr int kUnits = sizeof(Regs) / 16;
+      static_assert(sizeof(Regs) % 16 == 0, "activation registers are whole 16-byte units");
+      __shared__ uint4 s_x[NSTEP * kUnits * kWave];
+      __shared__ float s_squares[NSTEP];
+      if (wave < NSTEP) {
+        Regs regs;
+        fetch_x(wave, 0, regs);
+        uint4 units[kUnits];
+        __builtin_memcpy(units, &regs, sizeof(Regs));
+#pragma unroll
+        for (int u = 0; u < kUnits; ++u) s_x[(wave * kUnits + u) * kWave + lane] = units[u];
+        if constexpr (NORM) {
+          const float total = wave_sum(squares[0]);
+          if (lane == 0) s_squares[wave] = total;
+        }
+      }
+      __syncthreads();
+      if constexpr (NORM) {
+        float total = 0.f;
+#pragma unroll
+        for (int step = 0; step < NSTEP; ++step) total += s_squares[step];
+        shared_squares = total;
+      }
+#pragma unroll
+      for (int step = 0; step < NSTEP; ++step) {
+        uint4 units[kUnits];
+#pragma unroll
+        for (int u = 0; u < kUnits; ++u) units[u] = s_x[(step * kUnits + u) * kWave + lane];
+        Regs regs;
+        __builtin_memcpy(&regs, units, sizeof(Regs));
+        consume(step, all_w[step], all_s[step], 0, regs);
+      }
+    } else if constexpr (MB == 1) {
       Regs regs[NSTEP];
 #pragma unroll
       for (int step = 0; step < NSTEP; ++step) fetch_x(step, 0, regs[step]);
@@ -381,7 +426,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 4))) voi
   float inv[MB];
 #pragma unroll
   for (int b = 0; b < MB; ++b)
-    inv[b] = NORM ? 1.0f / sqrtf(wave_sum(squares[b]) / (float)k + fuse.norm_eps) : 1.0f;
+    inv[b] = NORM ? 1.0f / sqrtf((XLDS ? shared_squares : wave_sum(squares[b])) / (float)k +
+                                 fuse.norm_eps)
+                  : 1.0f;
   const XT* residual = static_cast<const XT*>(fuse.residual);
   if constexpr (ROWS == 2) {
     if (fuse.pair_silu) {
