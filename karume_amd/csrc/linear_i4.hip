@@ -430,23 +430,28 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 4))) voi
                                  fuse.norm_eps)
                   : 1.0f;
   const XT* residual = static_cast<const XT*>(fuse.residual);
-  if constexpr (ROWS == 2) {
+  if constexpr (ROWS % 2 == 0) {
     if (fuse.pair_silu) {
       // rows (2i, 2i+1) hold (gate_i, up_i): out[., i] = silu(gate) * up, n/2 outputs per row
-      const uint32_t half_n = n >> 1, col = row0 >> 1;
+      const uint32_t half_n = n >> 1;
 #pragma unroll
-      for (int b = 0; b < MB; ++b) {
-        float gate = wave_sum(acc[0][b]) * inv[b], up = wave_sum(acc[1][b]) * inv[b];
-        if (lane == b % kWave && row0 + 1 < n && (uint32_t)b < m) {
-          if (bias) {
-            gate += to_f32<XT>(bias[row0]);
-            up += to_f32<XT>(bias[row0 + 1]);
+      for (int p = 0; p < ROWS / 2; ++p) {
+        const uint32_t row = row0 + 2 * p, col = row >> 1;
+#pragma unroll
+        for (int b = 0; b < MB; ++b) {
+          float gate = wave_sum(acc[2 * p][b]) * inv[b];
+          float up = wave_sum(acc[2 * p + 1][b]) * inv[b];
+          if (lane == (p * MB + b) % kWave && row + 1 < n && (uint32_t)b < m) {
+            if (bias) {
+              gate += to_f32<XT>(bias[row]);
+              up += to_f32<XT>(bias[row + 1]);
+            }
+            const float t = expf(-fabsf(gate));
+            const float sig = gate < 0.f ? t / (1.0f + t) : 1.0f / (1.0f + t);
+            float value = __fmul_rn(__fmul_rn(gate, sig), up);
+            if (residual) value += to_f32<XT>(residual[(size_t)b * half_n + col]);
+            out[(size_t)b * half_n + col] = from_f32<XT>(value);
           }
-          const float t = expf(-fabsf(gate));
-          const float sig = gate < 0.f ? t / (1.0f + t) : 1.0f / (1.0f + t);
-          float value = __fmul_rn(__fmul_rn(gate, sig), up);
-          if (residual) value += to_f32<XT>(residual[(size_t)b * half_n + col]);
-          out[(size_t)b * half_n + col] = from_f32<XT>(value);
         }
       }
       return;
@@ -508,6 +513,11 @@ int32_t pick_rows(krm_ctx* ctx, krm_buf x, krm_buf w, krm_buf scales, krm_buf bi
   // Rows per wave: two rows share one fetch of the activations; one row per wave keeps more
   // waves in flight when N is small.  The choice never changes a row's reduction order.
   const uint64_t cus = (uint64_t)ctx->num_cus;
+  // f32 activations of one row in few steps: four rows a wave halve the workgroups that each
+  // stage the row once more, as long as every CU still gets a few.
+  if constexpr (MB == 1 && sizeof(XT) == 4 && VEC == 4)
+    if (k <= 4096 && (uint64_t)n >= cus * 4 * 4 * 2)
+      return pick_steps<XT, ST, MB, 4, VEC>(ctx, x, w, scales, bias, out, m, n, k, group_shift, fuse);
   if (fuse.pair_silu || (uint64_t)n >= cus * 4 * 2)
     return pick_steps<XT, ST, MB, 2, VEC>(ctx, x, w, scales, bias, out, m, n, k, group_shift, fuse);
   return pick_steps<XT, ST, MB, 1, VEC>(ctx, x, w, scales, bias, out, m, n, k, group_shift, fuse);
