@@ -246,7 +246,8 @@ def main() -> int:
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-graph", action="store_true",
                     help="issue plain launches instead of replaying recorded graphs")
-    ap.add_argument("--only", default="", help="gemv | model: run only that part besides the headline GEMV")
+    ap.add_argument("--only", default="", help="gemv | gemm | attention | model | traffic: run only that part besides the "
+                         "headline GEMV")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build measures one GPU only (--gpus 1); no multi-GPU figure is "
@@ -296,19 +297,21 @@ def main() -> int:
         for _ in range(8):
             ctx.copy(dst, src, 8 << 20)
         ctx.sync()
+    steps2 = max(50, args.steps // 4)
     if args.only == "":
-        steps2 = max(50, args.steps // 4)
         log("[bench] GEMV M=16 (config 3)")
         ms16, _res16, algo16 = bench_gemv(ctx, ka, rng, steps2, max(10, args.warmup // 4), 16, n,
                                           k, g, copies)
         result["gemv_m16_gbs"] = round(algo16 / (ms16 / steps2 * 1e-3) / 1e9, 1)
         result["gemv_m16_us"] = round(ms16 / steps2 * 1e3, 3)
+    if args.only in ("", "attention"):
         log("[bench] decode attention (config 2)")
         ms_att, algo_att = bench_attention(ctx, ka, rng, steps2, max(10, args.warmup // 4), 20)
         att_gbs = algo_att / (ms_att / steps2 * 1e-3) / 1e9
         result["attention_decode_gbs"] = round(att_gbs, 1)
         result["attention_decode_us"] = round(ms_att / steps2 * 1e3, 3)
         result["attention_decode_pct_of_hbm_peak"] = round(100 * att_gbs / HBM_PEAK_GBS, 2)
+    if args.only in ("", "gemm"):
         for name, (gn, gk) in {"up": (11008, 4096), "down": (4096, 11008)}.items():
             log(f"[bench] prefill GEMM M=512 K={gk} N={gn} (config 1, {name}-projection)")
             ms_g, flops = bench_gemm(ctx, ka, rng, 40, 8, 512, gn, gk, g)

@@ -10,14 +10,15 @@
 // v_mfma_f32_32x32x16_f16.  The caller opts in with KRM_COMPUTE_F16.
 //
 // Workgroup tile BM x BN (waves in a WM x WN grid, 64 x 64 outputs per wave = 2 x 2 MFMA
-// tiles); K is walked 64 codes at a time through two LDS buffers:
-//   A tile  x[BM rows][64]  fp16, each group of 8 stored as (x0,x4,x1,x5,x2,x6,x3,x7)
-//   B tile  w[BN rows][64]  fp16 dequantised, the same order within each group of 8 — the
+// tiles); K is walked KC (64 or 128) codes at a time through one LDS copy of the chunk:
+//   A tile  x[BM rows][KC]  fp16, each group of 8 stored as (x0,x4,x1,x5,x2,x6,x3,x7)
+//   B tile  w[BN rows][KC]  fp16 dequantised, the same order within each group of 8 — the
 //           order the nibble trick produces (code i pairs with code i+4), so no shuffle is
 //           spent on the weights; the k index inside an MFMA is a free permutation as long as
 //           both operands use the same one.
 // Rows are padded by 16 bytes so the 16-byte fragment reads of 32 consecutive rows spread over
-// all LDS banks.  The next chunk's global loads are issued before the current chunk's MFMAs.
+// all LDS banks.  The next chunk's global loads are issued before the current chunk's MFMAs
+// and wait in registers; several workgroups share a CU to cover each other's barriers.
 #include "krm_internal.h"
 
 using namespace krm;
@@ -28,8 +29,12 @@ typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
 typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
 typedef float float16_t __attribute__((ext_vector_type(16)));
 
-constexpr int kChunk = 64;             // codes of K per LDS stage
-constexpr int kRowBytes = kChunk * 2 + 16;  // padded fp16 row
+// A K chunk of KC codes is staged per pass; rows are padded by 16 bytes so the 16-byte
+// fragment reads of 32 consecutive rows spread over all LDS banks.
+template <int KC>
+struct ChunkGeometry {
+  static constexpr int kRowBytes = KC * 2 + 16;
+};
 
 template <typename ST>
 __device__ inline _Float16 scale_as_half(const ST* s, size_t i);
@@ -42,6 +47,13 @@ __device__ inline _Float16 scale_as_half<float>(const float* s, size_t i) {
   return (_Float16)s[i];
 }
 
+// (a & mask) | bits in one VALU op (the compiler emits two when both constants are literals).
+__device__ inline uint32_t and_or(uint32_t a, uint32_t mask, uint32_t bits) {
+  uint32_t d;
+  asm("v_and_or_b32 %0, %1, %2, %3" : "=v"(d) : "v"(a), "s"(mask), "v"(bits));
+  return d;
+}
+
 // 8 codes of a word -> 8 fp16 values (u - 8) * scale, order (c0,c4,c1,c5,c2,c6,c3,c7).
 __device__ inline uint4 dequant_word(uint32_t word, _Float16 scale) {
   const uint32_t magic = 0x64006400u;  // (1024, 1024)
@@ -50,40 +62,55 @@ __device__ inline uint4 dequant_word(uint32_t word, _Float16 scale) {
   const half2_t off_hi = {(_Float16)-72.0f, (_Float16)-72.0f};
   const half2_t s2 = {scale, scale};
   const uint32_t upper = word >> 8;
-  const half2_t q0 = (__builtin_bit_cast(half2_t, (word & 0x000F000Fu) | magic) - off_lo) * s2;
-  const half2_t q1 =
-      (__builtin_elementwise_fma(__builtin_bit_cast(half2_t, (word & 0x00F000F0u) | magic), sixteenth, off_hi)) * s2;
-  const half2_t q2 = (__builtin_bit_cast(half2_t, (upper & 0x000F000Fu) | magic) - off_lo) * s2;
-  const half2_t q3 =
-      (__builtin_elementwise_fma(__builtin_bit_cast(half2_t, (upper & 0x00F000F0u) | magic), sixteenth, off_hi)) * s2;
+  const half2_t q0 = (__builtin_bit_cast(half2_t, and_or(word, 0x000F000Fu, magic)) - off_lo) * s2;
+  const half2_t q1 = (__builtin_elementwise_fma(
+                         __builtin_bit_cast(half2_t, and_or(word, 0x00F000F0u, magic)), sixteenth,
+                         off_hi)) * s2;
+  const half2_t q2 = (__builtin_bit_cast(half2_t, and_or(upper, 0x000F000Fu, magic)) - off_lo) * s2;
+  const half2_t q3 = (__builtin_elementwise_fma(
+                         __builtin_bit_cast(half2_t, and_or(upper, 0x00F000F0u, magic)), sixteenth,
+                         off_hi)) * s2;
   return make_uint4(__builtin_bit_cast(uint32_t, q0), __builtin_bit_cast(uint32_t, q1),
                     __builtin_bit_cast(uint32_t, q2), __builtin_bit_cast(uint32_t, q3));
 }
 
-// 8 consecutive activations -> fp16 in the order (x0,x4,x1,x5,x2,x6,x3,x7)
+// 8 consecutive activations as they arrive from memory; converted to fp16 in the order
+// (x0,x4,x1,x5,x2,x6,x3,x7) only when they are parked in LDS, so the loads stay in flight.
 template <typename XT>
-__device__ inline uint4 load_acts8(const XT* p, bool valid);
+struct Acts8;
 template <>
-__device__ inline uint4 load_acts8<__half>(const __half* p, bool valid) {
-  uint4 raw = *reinterpret_cast<const uint4*>(p);
-  const uint32_t keep = valid ? 0xFFFFFFFFu : 0u;
-  raw.x &= keep; raw.y &= keep; raw.z &= keep; raw.w &= keep;
-  return make_uint4(__builtin_amdgcn_perm(raw.z, raw.x, 0x05040100u),
-                    __builtin_amdgcn_perm(raw.z, raw.x, 0x07060302u),
-                    __builtin_amdgcn_perm(raw.w, raw.y, 0x05040100u),
-                    __builtin_amdgcn_perm(raw.w, raw.y, 0x07060302u));
-}
+struct Acts8<__half> {
+  uint4 raw;
+  __device__ inline void load(const __half* p) { raw = *reinterpret_cast<const uint4*>(p); }
+  __device__ inline void keep(uint32_t bits) {
+    raw.x &= bits; raw.y &= bits; raw.z &= bits; raw.w &= bits;
+  }
+  __device__ inline uint4 paired() const {
+    return make_uint4(__builtin_amdgcn_perm(raw.z, raw.x, 0x05040100u),
+                      __builtin_amdgcn_perm(raw.z, raw.x, 0x07060302u),
+                      __builtin_amdgcn_perm(raw.w, raw.y, 0x05040100u),
+                      __builtin_amdgcn_perm(raw.w, raw.y, 0x07060302u));
+  }
+};
 template <>
-__device__ inline uint4 load_acts8<float>(const float* p, bool valid) {
-  const float4 a = reinterpret_cast<const float4*>(p)[0];
-  const float4 b = reinterpret_cast<const float4*>(p)[1];
-  const float z = valid ? 1.0f : 0.0f;
-  auto pack = [&](float lo, float hi) {
-    const half2_t h = {(_Float16)(lo * z), (_Float16)(hi * z)};  // round to nearest even
-    return __builtin_bit_cast(uint32_t, h);
-  };
-  return make_uint4(pack(a.x, b.x), pack(a.y, b.y), pack(a.z, b.z), pack(a.w, b.w));
-}
+struct Acts8<float> {
+  uint4 a, b;  // raw bits of x0..x3, x4..x7
+  __device__ inline void load(const float* p) {
+    a = reinterpret_cast<const uint4*>(p)[0];
+    b = reinterpret_cast<const uint4*>(p)[1];
+  }
+  __device__ inline void keep(uint32_t bits) {
+    a.x &= bits; a.y &= bits; a.z &= bits; a.w &= bits;
+    b.x &= bits; b.y &= bits; b.z &= bits; b.w &= bits;
+  }
+  __device__ inline uint4 paired() const {
+    auto pack = [](uint32_t lo, uint32_t hi) {
+      const half2_t h = {(_Float16)__uint_as_float(lo), (_Float16)__uint_as_float(hi)};  // RNE
+      return __builtin_bit_cast(uint32_t, h);
+    };
+    return make_uint4(pack(a.x, b.x), pack(a.y, b.y), pack(a.z, b.z), pack(a.w, b.w));
+  }
+};
 
 template <typename T>
 __device__ inline float bias_f32(const T* p, size_t i);
@@ -100,24 +127,39 @@ __device__ inline void store_out<__half>(__half* p, size_t i, float v) {
   p[i] = __float2half_rn(v);
 }
 
-template <typename XT, typename ST, int WM, int WN>
-__global__ __launch_bounds__(WM * WN * 64) __attribute__((amdgpu_waves_per_eu(1, 2)))
+template <typename XT, typename ST, int WM, int WN, int KC, int KS, int DEPTH>
+__global__ __launch_bounds__(WM * WN * KS * 64) __attribute__((amdgpu_waves_per_eu(2, 2)))
 void gemm_i4_f16_kernel(const XT* __restrict__ x, const uint32_t* __restrict__ w,
                         const ST* __restrict__ scales, const XT* __restrict__ bias,
                         XT* __restrict__ out, uint32_t m, uint32_t n, uint32_t k,
                         uint32_t group_shift, uint32_t m_blocks, uint32_t n_blocks,
                         uint32_t wide_rows) {
-  constexpr int kThreads = WM * WN * 64;
+  // KS wave groups share the tile and split every chunk's K between them (their sums are
+  // added once at the end): more waves per output, so more work in flight per CU.
+  constexpr int kThreads = WM * WN * KS * 64;
   constexpr int BM = WM * 64, BN = WN * 64;
-  constexpr int kAPieces = BM * (kChunk / 8);        // 16-byte pieces of the A tile
+  constexpr int kRowBytes = ChunkGeometry<KC>::kRowBytes;
+  constexpr int kStepsPerGroup = KC / 16 / KS;
+  static_assert(KC % (16 * KS) == 0, "the K split divides the chunk");
+  constexpr int kRowPieces = KC / 8;                 // 16-byte pieces (or weight words) a row
+  constexpr int kAPieces = BM * kRowPieces;          // 16-byte pieces of the A tile
   constexpr int kAPer = kAPieces / kThreads;         // per thread
-  constexpr int kBPieces = BN * (kChunk / 8);        // words of the B tile
+  constexpr int kBPieces = BN * kRowPieces;          // words of the B tile
   constexpr int kBPer = kBPieces / kThreads;         // words per thread (consecutive in a row)
   static_assert(kAPieces % kThreads == 0 && kBPieces % kThreads == 0, "tile / thread mismatch");
-  static_assert(kBPer == 1 || kBPer == 2 || kBPer == 4 || kBPer == 8, "B words per thread");
+  static_assert(kBPer == 1 || kBPer == 2 || kBPer == 4 || kBPer == 8 || kBPer == 16,
+                "B words per thread");
+  static_assert(kRowPieces % kBPer == 0, "a thread's weight words stay inside one row");
 
-  __shared__ __attribute__((aligned(16))) unsigned char lds_a[2][BM * kRowBytes];
-  __shared__ __attribute__((aligned(16))) unsigned char lds_b[2][BN * kRowBytes];
+  // One LDS copy of the chunk; the NEXT chunk waits in registers (its loads are issued right
+  // after this chunk is parked), and several workgroups share a CU, so a workgroup that sits
+  // at a barrier or waits for memory leaves the matrix cores to the others.
+  constexpr int kTileBytes = (BM + BN) * kRowBytes;
+  constexpr int kReduceBytes = KS > 1 ? WM * WN * (KS - 1) * 64 * 64 * 4 : 0;
+  __shared__ __attribute__((aligned(16)))
+  unsigned char lds[kTileBytes > kReduceBytes ? kTileBytes : kReduceBytes];
+  unsigned char* lds_a = lds;
+  unsigned char* lds_b = lds + BM * kRowBytes;
 
   // Workgroups that share an x panel are placed on one XCD (ids are dealt round-robin over 8
   // XCDs), so that panel stays in that XCD's L2 while the weights stream through.
@@ -137,67 +179,89 @@ void gemm_i4_f16_kernel(const XT* __restrict__ x, const uint32_t* __restrict__ w
   const uint32_t m0 = mb * BM, n0 = nb * BN;
   const int tid = threadIdx.x;
   const int lane = tid & 63, wave = tid >> 6;
-  const int wm = wave % WM, wn = wave / WM;
+  const int wm = wave % WM, wn = (wave / WM) % WN, kg = wave / (WM * WN);
 
   const uint32_t words_per_row = k >> 3;
   const uint32_t groups_per_row = k >> group_shift;
-  const uint32_t chunks = (k + kChunk - 1) / kChunk;
+  const uint32_t chunks = (k + KC - 1) / KC;
 
-  // staging assignment
-  uint32_t a_row[kAPer], a_pc[kAPer];
+  // staging assignment: element offsets of the thread's pieces at chunk 0 (rows past M or N
+  // re-read the last row; their products are never stored)
+  uint32_t a_off[kAPer], a_lds[kAPer], a_k[kAPer];
 #pragma unroll
   for (int i = 0; i < kAPer; ++i) {
     const int p = tid + i * kThreads;
-    a_row[i] = p / (kChunk / 8);
-    a_pc[i] = p % (kChunk / 8);
+    const uint32_t row = p / kRowPieces, pc = p % kRowPieces;
+    a_off[i] = min(row, m - 1 - m0) * k + pc * 8;  // relative to the tile's first row
+    a_k[i] = pc * 8;
+    a_lds[i] = row * kRowBytes + pc * 16;
   }
-  const uint32_t b_row = (tid * kBPer) / (kChunk / 8);
-  const uint32_t b_w0 = (tid * kBPer) % (kChunk / 8);
-  const uint32_t b_grow = min(n0 + b_row, n - 1);  // rows past N re-read the last row, unused
+  const uint32_t b_row = (tid * kBPer) / kRowPieces;
+  const uint32_t b_w0 = (tid * kBPer) % kRowPieces;
+  const uint32_t b_grow = min(n0 + b_row, n - 1);
+  const uint32_t* b_src = w + (size_t)b_grow * words_per_row + b_w0;
+  const size_t b_scale_row = (size_t)b_grow * groups_per_row;
 
-  uint4 a_regs[kAPer];
-  uint32_t b_regs[kBPer];
-  _Float16 b_scale[kBPer];
+  const XT* x_tile = x + (size_t)m0 * k;
+  // A chunk's operands as they arrive from memory.  DEPTH of them are in flight: chunk c + DEPTH
+  // is requested as soon as chunk c has been parked in LDS.
+  struct Slot {
+    Acts8<XT> a[kAPer];
+    uint32_t b[kBPer];
+    _Float16 scale[kBPer];
+  };
+  // a thread's words are consecutive and aligned to their count, so they share one scale
+  // whenever a group covers them all
+  const bool one_scale = ((uint32_t)(kBPer * 8 - 1) >> group_shift) == 0;
 
-  auto fetch = [&](uint32_t chunk) {
-    const uint32_t k0 = chunk * kChunk;
+  auto fetch = [&](uint32_t chunk, Slot& slot) {
+    const uint32_t k0 = chunk * KC;
+    if (k0 + KC <= k) {  // uniform: the whole chunk lies inside K
 #pragma unroll
-    for (int i = 0; i < kAPer; ++i) {
-      const uint32_t row = m0 + a_row[i], kk = k0 + a_pc[i] * 8;
-      const bool valid = row < m && kk < k;
-      const uint32_t rr = valid ? row : 0u, kc = valid ? kk : 0u;
-      a_regs[i] = load_acts8<XT>(x + (size_t)rr * k + kc, valid);
-    }
-    // 16-byte weight loads when the rows are 16-byte aligned and the chunk lies inside K
-    // (both conditions are uniform over the workgroup).
-    const bool vec = kBPer >= 4 && wide_rows && k0 + kChunk <= k;
-    if (vec) {
+      for (int i = 0; i < kAPer; ++i) slot.a[i].load(x_tile + a_off[i] + k0);
+      if (kBPer >= 4 && wide_rows) {
 #pragma unroll
-      for (int j = 0; j < kBPer; j += 4) {
-        const uint4 v = *reinterpret_cast<const uint4*>(
-            w + (size_t)b_grow * words_per_row + (k0 >> 3) + b_w0 + j);
-        b_regs[j] = v.x;
-        if (j + 1 < kBPer) b_regs[j + 1] = v.y;
-        if (j + 2 < kBPer) b_regs[j + 2] = v.z;
-        if (j + 3 < kBPer) b_regs[j + 3] = v.w;
+        for (int j = 0; j + 3 < kBPer; j += 4) {
+          const uint4 v = *reinterpret_cast<const uint4*>(b_src + (k0 >> 3) + j);
+          slot.b[j] = v.x; slot.b[j + 1] = v.y; slot.b[j + 2] = v.z; slot.b[j + 3] = v.w;
+        }
+      } else {
+#pragma unroll
+        for (int j = 0; j < kBPer; ++j) slot.b[j] = b_src[(k0 >> 3) + j];
+      }
+      if (one_scale) {  // only scale[0] is loaded (no copies: a copy would wait for the load)
+        slot.scale[0] = scale_as_half<ST>(scales, b_scale_row + ((k0 + b_w0 * 8) >> group_shift));
+      } else {
+#pragma unroll
+        for (int j = 0; j < kBPer; ++j)
+          slot.scale[j] =
+              scale_as_half<ST>(scales, b_scale_row + ((k0 + (b_w0 + j) * 8) >> group_shift));
+      }
+    } else {  // last chunk of a K that is not a multiple of KC: zero activations past K
+#pragma unroll
+      for (int i = 0; i < kAPer; ++i) {
+        const bool inside = k0 + a_k[i] < k;
+        slot.a[i].load(x_tile + a_off[i] + (inside ? k0 : 0u));
+        slot.a[i].keep(inside ? 0xFFFFFFFFu : 0u);
+      }
+#pragma unroll
+      for (int j = 0; j < kBPer; ++j) {
+        const uint32_t kk = k0 + (b_w0 + j) * 8;
+        const uint32_t kc = kk < k ? kk : 0u;  // x is zero there; any finite weight will do
+        slot.b[j] = w[(size_t)b_grow * words_per_row + (kc >> 3)];
+        slot.scale[j] = scale_as_half<ST>(scales, b_scale_row + (kc >> group_shift));
       }
     }
-#pragma unroll
-    for (int j = 0; j < kBPer; ++j) {
-      const uint32_t kk = k0 + (b_w0 + j) * 8;
-      const uint32_t kc = kk < k ? kk : 0u;  // past the end of K: x is zero there, w is unused
-      if (!vec) b_regs[j] = w[(size_t)b_grow * words_per_row + (kc >> 3)];
-      b_scale[j] = scale_as_half<ST>(scales, (size_t)b_grow * groups_per_row + (kc >> group_shift));
-    }
   };
-  auto stage = [&](int buf) {
+  // `ragged`: the chunk reaches past K and carries one scale per word
+  auto stage = [&](const Slot& slot, bool ragged) {
 #pragma unroll
     for (int i = 0; i < kAPer; ++i)
-      *reinterpret_cast<uint4*>(&lds_a[buf][a_row[i] * kRowBytes + a_pc[i] * 16]) = a_regs[i];
+      *reinterpret_cast<uint4*>(&lds_a[a_lds[i]]) = slot.a[i].paired();
 #pragma unroll
     for (int j = 0; j < kBPer; ++j)
-      *reinterpret_cast<uint4*>(&lds_b[buf][b_row * kRowBytes + (b_w0 + j) * 16]) =
-          dequant_word(b_regs[j], b_scale[j]);
+      *reinterpret_cast<uint4*>(&lds_b[b_row * kRowBytes + (b_w0 + j) * 16]) =
+          dequant_word(slot.b[j], slot.scale[(one_scale && !ragged) ? 0 : j]);
   };
 
   float16_t acc[2][2];
@@ -208,37 +272,68 @@ void gemm_i4_f16_kernel(const XT* __restrict__ x, const uint32_t* __restrict__ w
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
-  fetch(0);
-  stage(0);
-  __syncthreads();
-
   const int frag_row = lane & 31, frag_g = lane >> 5;
-  for (uint32_t chunk = 0; chunk < chunks; ++chunk) {
-    const int buf = chunk & 1;
-    if (chunk + 1 < chunks) fetch(chunk + 1);
+  const unsigned char* a_frag =
+      lds_a + (wm * 64 + frag_row) * kRowBytes + frag_g * 16 + kg * kStepsPerGroup * 32;
+  const unsigned char* b_frag =
+      lds_b + (wn * 64 + frag_row) * kRowBytes + frag_g * 16 + kg * kStepsPerGroup * 32;
+
+  Slot slots[DEPTH];
 #pragma unroll
-    for (int ks = 0; ks < kChunk / 16; ++ks) {
-      half8_t af[2], bf[2];
+  for (int d = 0; d < DEPTH; ++d)
+    if ((uint32_t)d < chunks) fetch(d, slots[d]);
+  for (uint32_t base = 0; base < chunks; base += DEPTH) {
 #pragma unroll
-      for (int i = 0; i < 2; ++i) {
-        const int row = wm * 64 + i * 32 + frag_row;
-        af[i] = *reinterpret_cast<const half8_t*>(
-            &lds_a[buf][row * kRowBytes + (ks * 2 + frag_g) * 16]);
+    for (int d = 0; d < DEPTH; ++d) {  // unrolled: every slot has fixed registers
+      const uint32_t chunk = base + d;
+      if (chunk >= chunks) break;
+      stage(slots[d], chunk * KC + KC > k);
+      __syncthreads();
+      if (chunk + DEPTH < chunks) fetch(chunk + DEPTH, slots[d]);
+#pragma unroll
+      for (int ks = 0; ks < kStepsPerGroup; ++ks) {
+        half8_t af[2], bf[2];
+#pragma unroll
+        for (int i = 0; i < 2; ++i)
+          af[i] = *reinterpret_cast<const half8_t*>(a_frag + i * 32 * kRowBytes + ks * 32);
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+          bf[j] = *reinterpret_cast<const half8_t*>(b_frag + j * 32 * kRowBytes + ks * 32);
+#pragma unroll
+        for (int i = 0; i < 2; ++i)
+#pragma unroll
+          for (int j = 0; j < 2; ++j)
+            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[i], bf[j], acc[i][j], 0, 0, 0);
       }
-#pragma unroll
-      for (int j = 0; j < 2; ++j) {
-        const int row = wn * 64 + j * 32 + frag_row;
-        bf[j] = *reinterpret_cast<const half8_t*>(
-            &lds_b[buf][row * kRowBytes + (ks * 2 + frag_g) * 16]);
-      }
+      __syncthreads();  // every wave is done with this chunk before the next one is parked
+    }
+  }
+
+  if constexpr (KS > 1) {
+    // Sum of the K groups, group 0 + 1 + ... in that order; the tile's LDS is free again (the
+    // loop ended on a barrier).  Word (r, lane) of a wave's 64 x 64 block: conflict-free.
+    float* red = reinterpret_cast<float*>(lds);
+    if (kg > 0) {
+      float* dst = red + (size_t)(((kg - 1) * WN + wn) * WM + wm) * 64 * 64;
 #pragma unroll
       for (int i = 0; i < 2; ++i)
 #pragma unroll
         for (int j = 0; j < 2; ++j)
-          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[i], bf[j], acc[i][j], 0, 0, 0);
+#pragma unroll
+          for (int r = 0; r < 16; ++r) dst[((i * 2 + j) * 16 + r) * 64 + lane] = acc[i][j][r];
     }
-    if (chunk + 1 < chunks) stage(buf ^ 1);
     __syncthreads();
+    if (kg > 0) return;
+#pragma unroll
+    for (int g = 1; g < KS; ++g) {
+      const float* src = red + (size_t)(((g - 1) * WN + wn) * WM + wm) * 64 * 64;
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) acc[i][j][r] += src[((i * 2 + j) * 16 + r) * 64 + lane];
+    }
   }
 
   // epilogue: lane holds column (lane % 32); register r holds row 8*(r/4) + 4*(lane/32) + r%4
@@ -258,7 +353,7 @@ void gemm_i4_f16_kernel(const XT* __restrict__ x, const uint32_t* __restrict__ w
   }
 }
 
-template <typename XT, typename ST, int WM, int WN>
+template <typename XT, typename ST, int WM, int WN, int KC, int KS, int DEPTH>
 int32_t launch(krm_ctx* ctx, krm_buf x, krm_buf w, krm_buf scales, krm_buf bias, krm_buf out,
                uint32_t m, uint32_t n, uint32_t k, uint32_t group_shift) {
   constexpr int BM = WM * 64, BN = WN * 64;
@@ -271,7 +366,7 @@ int32_t launch(krm_ctx* ctx, krm_buf x, krm_buf w, krm_buf scales, krm_buf bias,
     total = (uint64_t)m_blocks * n_blocks;
   }
   if (total > 0x7fffffffull) return fail(ctx, KRM_ERR_VALIDATION, "linear: grid too large");
-  gemm_i4_f16_kernel<XT, ST, WM, WN><<<dim3((unsigned)total), dim3(WM * WN * 64), 0, ctx->stream>>>(
+  gemm_i4_f16_kernel<XT, ST, WM, WN, KC, KS, DEPTH><<<dim3((unsigned)total), dim3(WM * WN * KS * 64), 0, ctx->stream>>>(
       ptr<const XT>(x), ptr<const uint32_t>(w), ptr<const ST>(scales), ptr<const XT>(bias),
       ptr<XT>(out), m, n, k, group_shift, m_blocks, n_blocks,
       (k % 32 == 0 && aligned(w, 16)) ? 1u : 0u);
@@ -283,15 +378,16 @@ int32_t pick_tile(krm_ctx* ctx, krm_buf x, krm_buf w, krm_buf scales, krm_buf bi
                   uint32_t m, uint32_t n, uint32_t k, uint32_t group) {
   uint32_t group_shift = 0;
   while ((1u << group_shift) < group) ++group_shift;
-  // 128 x 128 tiles unless that leaves compute units idle; then 128 x 64 or 64 x 64.
+  // 128 x 64 tiles (two waves, chunks of 64 codes, two chunks in flight) when they fill the
+  // chip at least twice over.  Otherwise four wave groups split every 128-code chunk of K
+  // between them on a 64 x 64 tile: four times the waves for the same outputs.
   const uint64_t cus = (uint64_t)ctx->num_cus;
-  const uint64_t big = (uint64_t)((m + 127) / 128) * ((n + 127) / 128);
-  const uint64_t mid = (uint64_t)((m + 127) / 128) * ((n + 63) / 64);
-  if (m > 64 && big >= 2 * cus)
-    return launch<XT, ST, 2, 2>(ctx, x, w, scales, bias, out, m, n, k, group_shift);
-  if (m > 64 && mid >= cus)
-    return launch<XT, ST, 2, 1>(ctx, x, w, scales, bias, out, m, n, k, group_shift);
-  return launch<XT, ST, 1, 1>(ctx, x, w, scales, bias, out, m, n, k, group_shift);
+  const uint64_t wide = (uint64_t)((m + 127) / 128) * ((n + 63) / 64);
+  if (m > 64 && wide >= 2 * cus)
+    return launch<XT, ST, 2, 1, 64, 1, 2>(ctx, x, w, scales, bias, out, m, n, k, group_shift);
+  if (k >= 512)
+    return launch<XT, ST, 1, 1, 128, 4, 1>(ctx, x, w, scales, bias, out, m, n, k, group_shift);
+  return launch<XT, ST, 1, 1, 64, 1, 1>(ctx, x, w, scales, bias, out, m, n, k, group_shift);
 }
 
 }  // namespace
