@@ -10,15 +10,18 @@
 // v_mfma_f32_32x32x16_f16.  The caller opts in with KRM_COMPUTE_F16.
 //
 // Workgroup tile BM x BN (waves in a WM x WN grid, 64 x 64 outputs per wave = 2 x 2 MFMA
-// tiles); K is walked KC (64 or 128) codes at a time through one LDS copy of the chunk:
+// tiles, optionally KS wave groups that split each chunk's K and add their sums at the end);
+// K is walked KC (64 or 128) codes at a time through LDS:
 //   A tile  x[BM rows][KC]  fp16, each group of 8 stored as (x0,x4,x1,x5,x2,x6,x3,x7)
 //   B tile  w[BN rows][KC]  fp16 dequantised, the same order within each group of 8 — the
 //           order the nibble trick produces (code i pairs with code i+4), so no shuffle is
 //           spent on the weights; the k index inside an MFMA is a free permutation as long as
 //           both operands use the same one.
 // Rows are padded by 16 bytes so the 16-byte fragment reads of 32 consecutive rows spread over
-// all LDS banks.  The next chunk's global loads are issued before the current chunk's MFMAs
-// and wait in registers; several workgroups share a CU to cover each other's barriers.
+// all LDS banks.  Chunks travel memory -> registers (several in flight, no use of a loaded
+// value before it is parked, so the waits are counted) -> LDS -> fragments.  Pipelined form:
+// two LDS copies (distinct objects, so fragment reads may pass the parking writes), the
+// dequantisation of chunk c + 1 interleaved with the MFMAs of chunk c, one barrier a chunk.
 #include "krm_internal.h"
 
 using namespace krm;
@@ -36,15 +39,27 @@ struct ChunkGeometry {
   static constexpr int kRowBytes = KC * 2 + 16;
 };
 
+// A scale as it arrives from memory, kept in a whole 32-bit register until the chunk is parked
+// (narrowing it on arrival would be an ALU op that has to wait for the load).
 template <typename ST>
-__device__ inline _Float16 scale_as_half(const ST* s, size_t i);
+__device__ inline uint32_t scale_bits(const ST* s, size_t i);
 template <>
-__device__ inline _Float16 scale_as_half<__half>(const __half* s, size_t i) {
-  return __builtin_bit_cast(_Float16, s[i]);
+__device__ inline uint32_t scale_bits<__half>(const __half* s, size_t i) {
+  return reinterpret_cast<const uint16_t*>(s)[i];
 }
 template <>
-__device__ inline _Float16 scale_as_half<float>(const float* s, size_t i) {
-  return (_Float16)s[i];
+__device__ inline uint32_t scale_bits<float>(const float* s, size_t i) {
+  return reinterpret_cast<const uint32_t*>(s)[i];
+}
+template <typename ST>
+__device__ inline _Float16 scale_from_bits(uint32_t bits);
+template <>
+__device__ inline _Float16 scale_from_bits<__half>(uint32_t bits) {
+  return __builtin_bit_cast(_Float16, (uint16_t)bits);
+}
+template <>
+__device__ inline _Float16 scale_from_bits<float>(uint32_t bits) {
+  return (_Float16)__uint_as_float(bits);
 }
 
 // (a & mask) | bits in one VALU op (the compiler emits two when both constants are literals).
@@ -127,7 +142,7 @@ __device__ inline void store_out<__half>(__half* p, size_t i, float v) {
   p[i] = __float2half_rn(v);
 }
 
-template <typename XT, typename ST, int WM, int WN, int KC, int KS, int DEPTH>
+template <typename XT, typename ST, int WM, int WN, int KC, int KS, int DEPTH, bool PIPE, bool FAST>
 __global__ __launch_bounds__(WM * WN * KS * 64) __attribute__((amdgpu_waves_per_eu(2, 2)))
 void gemm_i4_f16_kernel(const XT* __restrict__ x, const uint32_t* __restrict__ w,
                         const ST* __restrict__ scales, const XT* __restrict__ bias,
@@ -154,12 +169,18 @@ void gemm_i4_f16_kernel(const XT* __restrict__ x, const uint32_t* __restrict__ w
   // One LDS copy of the chunk; the NEXT chunk waits in registers (its loads are issued right
   // after this chunk is parked), and several workgroups share a CU, so a workgroup that sits
   // at a barrier or waits for memory leaves the matrix cores to the others.
-  constexpr int kTileBytes = (BM + BN) * kRowBytes;
+  // PIPE: two LDS copies; while the matrix cores work on chunk c out of one copy, the same
+  // wave parks chunk c + 1 in the other (the two instruction streams interleave), one barrier
+  // per chunk.
+  constexpr int kStageBytes = (BM + BN) * kRowBytes;
+  constexpr int kStageValuPerMfma = (kAPer * 4 + kBPer * 13 + kStepsPerGroup * 4 - 1) / (kStepsPerGroup * 4);
   constexpr int kReduceBytes = KS > 1 ? WM * WN * (KS - 1) * 64 * 64 * 4 : 0;
+  // two separate objects, so the compiler knows that parking into one copy cannot touch the
+  // other and may move the fragment reads past those writes
   __shared__ __attribute__((aligned(16)))
-  unsigned char lds[kTileBytes > kReduceBytes ? kTileBytes : kReduceBytes];
-  unsigned char* lds_a = lds;
-  unsigned char* lds_b = lds + BM * kRowBytes;
+  unsigned char lds[kStageBytes > kReduceBytes ? kStageBytes : kReduceBytes];
+  __shared__ __attribute__((aligned(16))) unsigned char lds_other[PIPE ? kStageBytes : 16];
+  constexpr int kOffB = BM * kRowBytes;
 
   // Workgroups that share an x panel are placed on one XCD (ids are dealt round-robin over 8
   // XCDs), so that panel stays in that XCD's L2 while the weights stream through.
@@ -208,15 +229,27 @@ void gemm_i4_f16_kernel(const XT* __restrict__ x, const uint32_t* __restrict__ w
   struct Slot {
     Acts8<XT> a[kAPer];
     uint32_t b[kBPer];
-    _Float16 scale[kBPer];
+    uint32_t scale[kBPer];  // raw bits, see scale_bits
   };
   // a thread's words are consecutive and aligned to their count, so they share one scale
   // whenever a group covers them all
   const bool one_scale = ((uint32_t)(kBPer * 8 - 1) >> group_shift) == 0;
 
+  // FAST (16-byte aligned rows, one scale per thread, K a multiple of KC): a fetch is the same
+  // straight run of loads for every chunk, so waits on an older chunk can be counted and the
+  // younger requests stay in flight.  Any branch here would cost that.
   auto fetch = [&](uint32_t chunk, Slot& slot) {
     const uint32_t k0 = chunk * KC;
-    if (k0 + KC <= k) {  // uniform: the whole chunk lies inside K
+    if constexpr (FAST) {
+#pragma unroll
+      for (int i = 0; i < kAPer; ++i) slot.a[i].load(x_tile + a_off[i] + k0);
+#pragma unroll
+      for (int j = 0; j + 3 < kBPer; j += 4) {
+        const uint4 v = *reinterpret_cast<const uint4*>(b_src + (k0 >> 3) + j);
+        slot.b[j] = v.x; slot.b[j + 1] = v.y; slot.b[j + 2] = v.z; slot.b[j + 3] = v.w;
+      }
+      slot.scale[0] = scale_bits<ST>(scales, b_scale_row + ((k0 + b_w0 * 8) >> group_shift));
+    } else if (k0 + KC <= k) {  // uniform: the whole chunk lies inside K
 #pragma unroll
       for (int i = 0; i < kAPer; ++i) slot.a[i].load(x_tile + a_off[i] + k0);
       if (kBPer >= 4 && wide_rows) {
@@ -230,12 +263,12 @@ void gemm_i4_f16_kernel(const XT* __restrict__ x, const uint32_t* __restrict__ w
         for (int j = 0; j < kBPer; ++j) slot.b[j] = b_src[(k0 >> 3) + j];
       }
       if (one_scale) {  // only scale[0] is loaded (no copies: a copy would wait for the load)
-        slot.scale[0] = scale_as_half<ST>(scales, b_scale_row + ((k0 + b_w0 * 8) >> group_shift));
+        slot.scale[0] = scale_bits<ST>(scales, b_scale_row + ((k0 + b_w0 * 8) >> group_shift));
       } else {
 #pragma unroll
         for (int j = 0; j < kBPer; ++j)
           slot.scale[j] =
-              scale_as_half<ST>(scales, b_scale_row + ((k0 + (b_w0 + j) * 8) >> group_shift));
+              scale_bits<ST>(scales, b_scale_row + ((k0 + (b_w0 + j) * 8) >> group_shift));
       }
     } else {  // last chunk of a K that is not a multiple of KC: zero activations past K
 #pragma unroll
@@ -249,21 +282,10 @@ void gemm_i4_f16_kernel(const XT* __restrict__ x, const uint32_t* __restrict__ w
         const uint32_t kk = k0 + (b_w0 + j) * 8;
         const uint32_t kc = kk < k ? kk : 0u;  // x is zero there; any finite weight will do
         slot.b[j] = w[(size_t)b_grow * words_per_row + (kc >> 3)];
-        slot.scale[j] = scale_as_half<ST>(scales, b_scale_row + (kc >> group_shift));
+        slot.scale[j] = scale_bits<ST>(scales, b_scale_row + (kc >> group_shift));
       }
     }
   };
-  // `ragged`: the chunk reaches past K and carries one scale per word
-  auto stage = [&](const Slot& slot, bool ragged) {
-#pragma unroll
-    for (int i = 0; i < kAPer; ++i)
-      *reinterpret_cast<uint4*>(&lds_a[a_lds[i]]) = slot.a[i].paired();
-#pragma unroll
-    for (int j = 0; j < kBPer; ++j)
-      *reinterpret_cast<uint4*>(&lds_b[b_row * kRowBytes + (b_w0 + j) * 16]) =
-          dequant_word(slot.b[j], slot.scale[(one_scale && !ragged) ? 0 : j]);
-  };
-
   float16_t acc[2][2];
 #pragma unroll
   for (int i = 0; i < 2; ++i)
@@ -273,39 +295,129 @@ void gemm_i4_f16_kernel(const XT* __restrict__ x, const uint32_t* __restrict__ w
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
   const int frag_row = lane & 31, frag_g = lane >> 5;
-  const unsigned char* a_frag =
-      lds_a + (wm * 64 + frag_row) * kRowBytes + frag_g * 16 + kg * kStepsPerGroup * 32;
-  const unsigned char* b_frag =
-      lds_b + (wn * 64 + frag_row) * kRowBytes + frag_g * 16 + kg * kStepsPerGroup * 32;
+  const int a_frag = (wm * 64 + frag_row) * kRowBytes + frag_g * 16 + kg * kStepsPerGroup * 32;
+  const int b_frag =
+      kOffB + (wn * 64 + frag_row) * kRowBytes + frag_g * 16 + kg * kStepsPerGroup * 32;
 
-  Slot slots[DEPTH];
+  // `ragged`: the chunk reaches past K and carries one scale per word
+  auto stage = [&](const Slot& slot, bool ragged, int buf) {
 #pragma unroll
-  for (int d = 0; d < DEPTH; ++d)
-    if ((uint32_t)d < chunks) fetch(d, slots[d]);
-  for (uint32_t base = 0; base < chunks; base += DEPTH) {
+    for (int i = 0; i < kAPer; ++i)
+      *reinterpret_cast<uint4*>(&(buf ? lds_other : lds)[a_lds[i]]) = slot.a[i].paired();
 #pragma unroll
-    for (int d = 0; d < DEPTH; ++d) {  // unrolled: every slot has fixed registers
-      const uint32_t chunk = base + d;
-      if (chunk >= chunks) break;
-      stage(slots[d], chunk * KC + KC > k);
-      __syncthreads();
-      if (chunk + DEPTH < chunks) fetch(chunk + DEPTH, slots[d]);
+    for (int j = 0; j < kBPer; ++j)
+      *reinterpret_cast<uint4*>(&(buf ? lds_other : lds)[kOffB + b_row * kRowBytes + (b_w0 + j) * 16]) =
+          dequant_word(slot.b[j], scale_from_bits<ST>(
+                                      slot.scale[(FAST || (one_scale && !ragged)) ? 0 : j]));
+  };
+  // All fragments of the chunk are requested before the first matrix instruction, so only the
+  // first one waits for LDS.
+  auto compute = [&](int buf) {
+    half8_t af[kStepsPerGroup][2], bf[kStepsPerGroup][2];
 #pragma unroll
-      for (int ks = 0; ks < kStepsPerGroup; ++ks) {
-        half8_t af[2], bf[2];
+    for (int ks = 0; ks < kStepsPerGroup; ++ks) {
 #pragma unroll
-        for (int i = 0; i < 2; ++i)
-          af[i] = *reinterpret_cast<const half8_t*>(a_frag + i * 32 * kRowBytes + ks * 32);
+      for (int i = 0; i < 2; ++i)
+        af[ks][i] = *reinterpret_cast<const half8_t*>(
+            &(buf ? lds_other : lds)[a_frag + i * 32 * kRowBytes + ks * 32]);
+#pragma unroll
+      for (int j = 0; j < 2; ++j)
+        bf[ks][j] = *reinterpret_cast<const half8_t*>(
+            &(buf ? lds_other : lds)[b_frag + j * 32 * kRowBytes + ks * 32]);
+    }
+#pragma unroll
+    for (int ks = 0; ks < kStepsPerGroup; ++ks)
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
 #pragma unroll
         for (int j = 0; j < 2; ++j)
-          bf[j] = *reinterpret_cast<const half8_t*>(b_frag + j * 32 * kRowBytes + ks * 32);
+          acc[i][j] =
+              __builtin_amdgcn_mfma_f32_32x32x16_f16(af[ks][i], bf[ks][j], acc[i][j], 0, 0, 0);
+  };
+  if constexpr (PIPE) {
+    // chunk c travels slot[c % DEPTH] -> LDS copy c % 2 (DEPTH is even); DEPTH - 1 chunks are
+    // in flight behind the one being parked
+    static_assert(DEPTH % 2 == 0, "the LDS copy of a slot is fixed");
+    Slot slots[DEPTH];
 #pragma unroll
-        for (int i = 0; i < 2; ++i)
-#pragma unroll
-          for (int j = 0; j < 2; ++j)
-            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[i], bf[j], acc[i][j], 0, 0, 0);
+    for (int d = 0; d < DEPTH; ++d) {
+      if constexpr (FAST) {
+        fetch(min((uint32_t)d, chunks - 1), slots[d]);
+      } else {
+        if ((uint32_t)d < chunks) fetch(d, slots[d]);
       }
-      __syncthreads();  // every wave is done with this chunk before the next one is parked
+    }
+    stage(slots[0], KC > k, 0);
+    if constexpr (FAST) {
+      fetch(min((uint32_t)DEPTH, chunks - 1), slots[0]);
+    } else {
+      if ((uint32_t)DEPTH < chunks) fetch(DEPTH, slots[0]);
+    }
+    __syncthreads();
+    // steady state: every body parks its successor; straight-line code so the staging and the
+    // matrix instructions can be interleaved
+    auto body = [&](uint32_t chunk, int d) {
+      const int nd = (d + 1) % DEPTH;
+      stage(slots[nd], (chunk + 1) * KC + KC > k, nd % 2);
+      compute(d % 2);
+      // one matrix instruction, then a share of the staging work, in turn
+      constexpr int kMfmas = kStepsPerGroup * 4;
+      constexpr int kLead = kMfmas >= 8 ? 8 : kMfmas;  // fragment reads ahead of the first MFMA
+      __builtin_amdgcn_sched_group_barrier(0x100, kLead, 0);
+#pragma unroll
+      for (int i = 0; i < kMfmas; ++i) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x002, kStageValuPerMfma, 0);
+        if (i < kMfmas - kLead) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+        if (i % 2) __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);
+      }
+      if constexpr (FAST) {
+        fetch(min(chunk + 1 + DEPTH, chunks - 1), slots[nd]);  // past the end: a harmless re-read
+      } else {
+        if (chunk + 1 + DEPTH < chunks) fetch(chunk + 1 + DEPTH, slots[nd]);
+      }
+      __syncthreads();
+    };
+    uint32_t chunk = 0;
+    for (; chunk + DEPTH < chunks; chunk += DEPTH) {
+#pragma unroll
+      for (int d = 0; d < DEPTH; ++d) body(chunk + d, d);
+    }
+    // the last 1..DEPTH chunks: the final one has no successor to park
+#pragma unroll
+    for (int d = 0; d < DEPTH; ++d) {
+      if (chunk + d + 1 < chunks) {
+        body(chunk + d, d);
+      } else if (chunk + d < chunks) {
+        compute(d % 2);
+      }
+    }
+    __syncthreads();
+  } else {
+    Slot slots[DEPTH];
+#pragma unroll
+    for (int d = 0; d < DEPTH; ++d) {
+      if constexpr (FAST) {
+        fetch(min((uint32_t)d, chunks - 1), slots[d]);
+      } else {
+        if ((uint32_t)d < chunks) fetch(d, slots[d]);
+      }
+    }
+    for (uint32_t base = 0; base < chunks; base += DEPTH) {
+#pragma unroll
+      for (int d = 0; d < DEPTH; ++d) {  // unrolled: every slot has fixed registers
+        const uint32_t chunk = base + d;
+        if (chunk >= chunks) break;
+        stage(slots[d], chunk * KC + KC > k, 0);
+        __syncthreads();
+        if constexpr (FAST) {
+          fetch(min(chunk + DEPTH, chunks - 1), slots[d]);  // past the end: a harmless re-read
+        } else {
+          if (chunk + DEPTH < chunks) fetch(chunk + DEPTH, slots[d]);
+        }
+        compute(0);
+        __syncthreads();  // every wave is done with this chunk before the next one is parked
+      }
     }
   }
 
@@ -353,7 +465,7 @@ void gemm_i4_f16_kernel(const XT* __restrict__ x, const uint32_t* __restrict__ w
   }
 }
 
-template <typename XT, typename ST, int WM, int WN, int KC, int KS, int DEPTH>
+template <typename XT, typename ST, int WM, int WN, int KC, int KS, int DEPTH, bool PIPE = false>
 int32_t launch(krm_ctx* ctx, krm_buf x, krm_buf w, krm_buf scales, krm_buf bias, krm_buf out,
                uint32_t m, uint32_t n, uint32_t k, uint32_t group_shift) {
   constexpr int BM = WM * 64, BN = WN * 64;
@@ -366,10 +478,20 @@ int32_t launch(krm_ctx* ctx, krm_buf x, krm_buf w, krm_buf scales, krm_buf bias,
     total = (uint64_t)m_blocks * n_blocks;
   }
   if (total > 0x7fffffffull) return fail(ctx, KRM_ERR_VALIDATION, "linear: grid too large");
-  gemm_i4_f16_kernel<XT, ST, WM, WN, KC, KS, DEPTH><<<dim3((unsigned)total), dim3(WM * WN * KS * 64), 0, ctx->stream>>>(
-      ptr<const XT>(x), ptr<const uint32_t>(w), ptr<const ST>(scales), ptr<const XT>(bias),
-      ptr<XT>(out), m, n, k, group_shift, m_blocks, n_blocks,
-      (k % 32 == 0 && aligned(w, 16)) ? 1u : 0u);
+  constexpr int kWordsPerThread = BN * (KC / 8) / (WM * WN * KS * 64);
+  const uint32_t wide = (k % 32 == 0 && aligned(w, 16)) ? 1u : 0u;
+  const bool fast = wide && kWordsPerThread >= 4 && k % KC == 0 &&
+                    (((uint32_t)(kWordsPerThread * 8 - 1) >> group_shift) == 0);
+  if (fast)
+    gemm_i4_f16_kernel<XT, ST, WM, WN, KC, KS, DEPTH, PIPE, true>
+        <<<dim3((unsigned)total), dim3(WM * WN * KS * 64), 0, ctx->stream>>>(
+            ptr<const XT>(x), ptr<const uint32_t>(w), ptr<const ST>(scales), ptr<const XT>(bias),
+            ptr<XT>(out), m, n, k, group_shift, m_blocks, n_blocks, wide);
+  else
+    gemm_i4_f16_kernel<XT, ST, WM, WN, KC, KS, DEPTH, PIPE, false>
+        <<<dim3((unsigned)total), dim3(WM * WN * KS * 64), 0, ctx->stream>>>(
+            ptr<const XT>(x), ptr<const uint32_t>(w), ptr<const ST>(scales), ptr<const XT>(bias),
+            ptr<XT>(out), m, n, k, group_shift, m_blocks, n_blocks, wide);
   return launched(ctx, "gemm_i4_f16_kernel");
 }
 
@@ -381,10 +503,15 @@ int32_t pick_tile(krm_ctx* ctx, krm_buf x, krm_buf w, krm_buf scales, krm_buf bi
   // 128 x 64 tiles (two waves, chunks of 64 codes, two chunks in flight) when they fill the
   // chip at least twice over.  Otherwise four wave groups split every 128-code chunk of K
   // between them on a 64 x 64 tile: four times the waves for the same outputs.
+  // Enough 128 x 128 tiles for every CU: four waves a tile, chunks of 64 codes, pipelined with
+  // four chunks in flight.  Fewer (a narrow output with a long K, or few rows): 128 x 64 tiles
+  // whose two wave groups split every 128-code chunk of K, or 64 x 64 tiles with four groups.
   const uint64_t cus = (uint64_t)ctx->num_cus;
-  const uint64_t wide = (uint64_t)((m + 127) / 128) * ((n + 63) / 64);
-  if (m > 64 && wide >= 2 * cus)
-    return launch<XT, ST, 2, 1, 64, 1, 2>(ctx, x, w, scales, bias, out, m, n, k, group_shift);
+  const uint64_t tiles = (uint64_t)((m + 127) / 128) * ((n + 127) / 128);
+  if (m > 64 && tiles >= cus)
+    return launch<XT, ST, 2, 2, 64, 1, 4, true>(ctx, x, w, scales, bias, out, m, n, k, group_shift);
+  if (m > 64 && k >= 256)
+    return launch<XT, ST, 2, 1, 128, 2, 2, true>(ctx, x, w, scales, bias, out, m, n, k, group_shift);
   if (k >= 512)
     return launch<XT, ST, 1, 1, 128, 4, 1>(ctx, x, w, scales, bias, out, m, n, k, group_shift);
   return launch<XT, ST, 1, 1, 64, 1, 1>(ctx, x, w, scales, bias, out, m, n, k, group_shift);
