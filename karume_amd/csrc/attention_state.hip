@@ -176,6 +176,28 @@ __global__ __launch_bounds__(kThreads) void attention_generic_kernel(
 
 // ------------------------------------------------------------------------------ decode
 
+typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
+typedef float float4_t __attribute__((ext_vector_type(4)));
+
+// Value of lane `src` (0..15) of the caller's 16-lane row, in every lane of that row.
+template <int SRC>
+__device__ inline float row_broadcast_from(float v) {
+  return __builtin_bit_cast(
+      float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x150 + SRC, 0xf, 0xf, true));
+}
+__device__ inline float row_broadcast(float v, int src) {  // `src` is a constant after unrolling
+  switch (src) {
+    case 0: return row_broadcast_from<0>(v);
+    case 1: return row_broadcast_from<1>(v);
+    case 2: return row_broadcast_from<2>(v);
+    case 3: return row_broadcast_from<3>(v);
+    case 4: return row_broadcast_from<4>(v);
+    case 5: return row_broadcast_from<5>(v);
+    case 6: return row_broadcast_from<6>(v);
+    default: return row_broadcast_from<7>(v);
+  }
+}
+
 // Sum over the LPR consecutive lanes that share one K/V row; all of them get the total.
 template <int LPR>
 __device__ inline float group_sum(float v) {
@@ -290,6 +312,8 @@ void attention_decode_kernel(
   constexpr int D = LPR * E;
   constexpr int G = kThreads / LPR;
   constexpr int kChunkCols = kDecodeIter * G;
+  // fp16 queries and fp16 rows of 128 dims: the scores run on the matrix cores
+  constexpr bool kMfma = sizeof(XT) == 2 && sizeof(ST) == 2 && LPR == 16 && kDecodeIter == 8;
   constexpr int kOuts = (R * D + kThreads - 1) / kThreads;
   __shared__ float s_m[G][R];
   __shared__ float s_l[G][R];
@@ -360,6 +384,21 @@ void attention_decode_kernel(
       qf[h][e] = ((ld_f32<XT>(q, q_base + e) * a.scale) * a.scale) * kLog2e;
   }
 
+  // B operand of the score MFMAs: lane (n = lane % 16, g = lane / 16) holds head n's query at
+  // dims 32t + 8g.. as raw fp16 (exact products; the scale is applied to the f32 score)
+  half8_t qb[kMfma ? 4 : 1];
+  if constexpr (kMfma) {
+    const int n = tid & 15, g = (tid & 63) >> 4;
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+      const size_t at = ((size_t)seq * a.heads + head0 + (n < R ? n : 0)) * D + 32 * t + 8 * g;
+      uint4 raw = *reinterpret_cast<const uint4*>(reinterpret_cast<const __half*>(q) + at);
+      const uint32_t keep_bits = n < R ? 0xFFFFFFFFu : 0u;
+      raw.x &= keep_bits; raw.y &= keep_bits; raw.z &= keep_bits; raw.w &= keep_bits;
+      qb[t] = __builtin_bit_cast(half8_t, raw);
+    }
+  }
+
   float run_m[R], run_l[R], acc[R][E];
 #pragma unroll
   for (int h = 0; h < R; ++h) {
@@ -369,47 +408,102 @@ void attention_decode_kernel(
     for (int e = 0; e < E; ++e) acc[h][e] = 0.f;
   }
 
-  for (uint32_t chunk = 0; chunk < my_chunks; ++chunk) {
-    const uint64_t c_begin = c_first + (uint64_t)chunk * kChunkCols;
-    const uint64_t c_end = (c_begin + kChunkCols < past) ? c_begin + kChunkCols : past;
-    // requests first: every K row, then every V row of the chunk
-    uint4 kraw[kDecodeIter], vraw[kDecodeIter];
+  // The rows of a chunk as they arrive: K pieces (row-owner layout, or the MFMA A-operand
+  // layout: piece tile*4 + t) and V pieces (row-owner layout).
+  struct ChunkRows {
+    uint4 k[kDecodeIter];
+    uint4 v[kDecodeIter];
+  };
+  const int wave = tid >> 6, lane = tid & 63;
+  const int frag_row = lane & 15, frag_g = lane >> 4;
+  auto chunk_begin = [&](uint32_t chunk) { return c_first + (uint64_t)chunk * kChunkCols; };
+  auto chunk_end = [&](uint64_t c_begin) {
+    return (c_begin + kChunkCols < past) ? c_begin + kChunkCols : past;
+  };
+  // column that (lane group, iteration) owns inside a chunk
+  auto column_of = [&](uint64_t c_begin, int it) {
+    if constexpr (kMfma)
+      return c_begin + (uint64_t)((wave * 2 + it / 4) * 16 + 4 * frag_g + (it & 3));
+    else
+      return c_begin + (uint64_t)it * G + group;
+  };
+  // Requests only: every K row, then every V row of the chunk; unconditional (a column past
+  // the end re-reads the chunk's first column and is masked when it is used).
+  auto load_chunk = [&](uint32_t chunk, ChunkRows& rows) {
+    const uint64_t c_begin = chunk_begin(chunk), c_end = chunk_end(c_begin);
+    auto slot_row = [&](uint64_t col) {
+      const uint64_t c = col < c_end ? col : c_begin;
+      return row_base + (a.window ? c % a.window : c);
+    };
+    if constexpr (kMfma) {
+      // lane (r = lane % 16, g = lane / 16) takes 16 bytes of K row r of each 16-row tile at
+      // dims 32t + 8g..: the A-operand layout of v_mfma_f32_16x16x32_f16
+#pragma unroll
+      for (int tile = 0; tile < 2; ++tile) {
+        const uint64_t prow = slot_row(c_begin + (uint64_t)((wave * 2 + tile) * 16 + frag_row));
+#pragma unroll
+        for (int t = 0; t < 4; ++t)
+          rows.k[tile * 4 + t] =
+              *reinterpret_cast<const uint4*>(kslot + prow * D + 32 * t + 8 * frag_g);
+      }
+    } else {
+#pragma unroll
+      for (int it = 0; it < kDecodeIter; ++it)
+        rows.k[it] = *reinterpret_cast<const uint4*>(
+            kslot + slot_row(column_of(c_begin, it)) * D + sub * E);
+    }
+#pragma unroll
+    for (int it = 0; it < kDecodeIter; ++it)
+      rows.v[it] = *reinterpret_cast<const uint4*>(
+          vslot + slot_row(column_of(c_begin, it)) * D + sub * E);
+  };
+  auto consume_chunk = [&](uint32_t chunk, ChunkRows& rows) {
+    const uint64_t c_begin = chunk_begin(chunk), c_end = chunk_end(c_begin);
     bool valid[kDecodeIter];
 #pragma unroll
-    for (int it = 0; it < kDecodeIter; ++it) {
-      const uint64_t col = c_begin + (uint64_t)it * G + group;
-      valid[it] = col < c_end;
-      kraw[it] = make_uint4(0, 0, 0, 0);
-      if (valid[it]) {
-        const uint64_t prow = row_base + (a.window ? col % a.window : col);
-        kraw[it] = *reinterpret_cast<const uint4*>(kslot + prow * D + sub * E);
-      }
-    }
-#pragma unroll
-    for (int it = 0; it < kDecodeIter; ++it) {
-      const uint64_t col = c_begin + (uint64_t)it * G + group;
-      vraw[it] = make_uint4(0, 0, 0, 0);
-      if (valid[it]) {
-        const uint64_t prow = row_base + (a.window ? col % a.window : col);
-        vraw[it] = *reinterpret_cast<const uint4*>(vslot + prow * D + sub * E);
-      }
-    }
+    for (int it = 0; it < kDecodeIter; ++it) valid[it] = column_of(c_begin, it) < c_end;
     float sc[kDecodeIter][R];
     float cm[R];
 #pragma unroll
     for (int h = 0; h < R; ++h) cm[h] = -INFINITY;
+    if constexpr (kMfma) {
+      // Scores on the matrix cores: the query heads are the B operand (one column per head);
+      // lane (h, g) receives the scores of columns 4g..4g+3 of a tile for head h, and lane
+      // group g owns exactly those columns for P*V, so a score reaches its group with one
+      // broadcast inside the 16-lane row.
+      float4_t scores[2];
 #pragma unroll
-    for (int it = 0; it < kDecodeIter; ++it) {
-      float kf[E];
-      RowChunk<ST>::unpack(kraw[it], kf);
+      for (int tile = 0; tile < 2; ++tile) {
+        scores[tile] = float4_t{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-      for (int h = 0; h < R; ++h) {
-        float part = 0.f;
+        for (int t = 0; t < 4; ++t)
+          scores[tile] = __builtin_amdgcn_mfma_f32_16x16x32_f16(
+              __builtin_bit_cast(half8_t, rows.k[tile * 4 + t]), qb[t], scores[tile], 0, 0, 0);
+      }
+      const float qscale = (a.scale * a.scale) * kLog2e;
 #pragma unroll
-        for (int e = 0; e < E; ++e) part = fmaf(qf[h][e], kf[e], part);
-        part = group_sum<LPR>(part);
-        sc[it][h] = valid[it] ? part : -INFINITY;
-        cm[h] = fmaxf(cm[h], sc[it][h]);
+      for (int it = 0; it < kDecodeIter; ++it) {
+        const float mine = scores[it / 4][it & 3] * qscale;  // (column of `it`, head lane % 16)
+#pragma unroll
+        for (int h = 0; h < R; ++h) {
+          sc[it][h] = valid[it] ? row_broadcast(mine, h) : -INFINITY;
+          cm[h] = fmaxf(cm[h], sc[it][h]);
+        }
+      }
+    } else {
+#pragma unroll
+      for (int it = 0; it < kDecodeIter; ++it) {
+        float kf[E];
+        RowChunk<ST>::unpack(rows.k[it], kf);
+#pragma unroll
+        for (int h = 0; h < R; ++h) {
+          float part = 0.f;
+#pragma unroll
+          for (int e = 0; e < E; ++e) part = fmaf(qf[h][e], kf[e], part);
+          part = group_sum<LPR>(part);
+          sc[it][h] = valid[it] ? part : -INFINITY;
+          cm[h] = fmaxf(cm[h], sc[it][h]);
+        }
       }
     }
     float keep[R], ref[R];
@@ -425,8 +519,11 @@ void attention_decode_kernel(
     }
 #pragma unroll
     for (int it = 0; it < kDecodeIter; ++it) {
+      uint4 raw = rows.v[it];
+      const uint32_t keep_bits = valid[it] ? 0xFFFFFFFFu : 0u;  // a masked column: no Inf * 0
+      raw.x &= keep_bits; raw.y &= keep_bits; raw.z &= keep_bits; raw.w &= keep_bits;
       float vf[E];
-      RowChunk<ST>::unpack(vraw[it], vf);
+      RowChunk<ST>::unpack(raw, vf);
 #pragma unroll
       for (int h = 0; h < R; ++h) {
         const float p = __builtin_amdgcn_exp2f(sc[it][h] - ref[h]);  // 0 outside the chunk
@@ -435,6 +532,14 @@ void attention_decode_kernel(
         for (int e = 0; e < E; ++e) acc[h][e] = fmaf(p, vf[e], acc[h][e]);
       }
     }
+  };
+  // (Requesting chunk c + 1 before chunk c is used was tried for short pasts walked by one
+  // split: the second set of row registers halves the workgroups a CU holds, which costs the
+  // long pasts more than it gives the short ones.)
+  for (uint32_t chunk = 0; chunk < my_chunks; ++chunk) {
+    ChunkRows rows;
+    load_chunk(chunk, rows);
+    consume_chunk(chunk, rows);
   }
   // this step's own column: one more row for group 0 of the last split
 #pragma unroll
@@ -648,6 +753,7 @@ int32_t decode_dispatch(krm_ctx* ctx, DecodeLaunch& L, uint32_t repeat, uint32_t
     per_block >>= 1;
     blocks <<= 1;
   }
+
   L.args.repeat = repeat;
   L.args.head_groups = repeat / per_block;
   if ((uint64_t)L.args.kv_heads * L.args.head_groups > 65535 ||
@@ -763,7 +869,7 @@ static int32_t attention_state_impl(krm_ctx* ctx, krm_buf q, krm_buf ins_k, krm_
   const uint32_t repeat = heads / kv_heads;
   const uint32_t lpr = decode_lanes_per_row(depth, kv_dtype);
   const bool fast = (dyn || query == 1) && chunk_rows == 1 && lpr && decode_repeat_ok(repeat) &&
-                    aligned(slot_k, 16) && aligned(slot_v, 16) && batch <= 65535 &&
+                    aligned(slot_k, 16) && aligned(slot_v, 16) && aligned(q, 16) && batch <= 65535 &&
                     heads <= 65535 && (uint64_t)batch * heads <= kTicketSlots;
   if (fast) {
     const uint64_t low = window_low(window, past);
@@ -872,8 +978,9 @@ int32_t krm_attention_varlen(krm_ctx* ctx, krm_buf q, krm_buf ins_k, krm_buf ins
               depth, repeat);
   KRM_REQUIRE(ctx, q && ins_k && ins_v && slot_k && slot_v && out && workspace,
               "krm_attention_varlen: NULL buffer");
-  KRM_REQUIRE(ctx, aligned(slot_k, 16) && aligned(slot_v, 16) && aligned(workspace, 16),
-              "krm_attention_varlen: slots and workspace must be 16-byte aligned");
+  KRM_REQUIRE(ctx, aligned(slot_k, 16) && aligned(slot_v, 16) && aligned(workspace, 16) &&
+                       aligned(q, 16),
+              "krm_attention_varlen: q, slots and workspace must be 16-byte aligned");
   KRM_REQUIRE(ctx, cu_seqlens[0] >= 0, "krm_attention_varlen: cu_seqlens[0] is negative");
 
   // Host-side tables: slot row offsets and the first global split of each sequence.
