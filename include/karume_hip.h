@@ -275,6 +275,23 @@ int32_t krm_decode_rope_append(krm_ctx* ctx, krm_buf qkv, krm_buf positions_i32,
                                uint32_t depth, uint32_t table_rows, uint32_t capacity,
                                uint32_t window, uint32_t past, krm_buf lengths, int32_t io_dtype,
                                int32_t kv_dtype);
+/* A whole decode row's attention inputs in one launch: (optional rms_norm) -> the fused
+ * [q; k; v] projection (n = (H + 2*Hkv) * D rows, M = 1) -> half-split RoPE of q and k ->
+ * state_append of the roped k row and of the v row.  `out` receives [q_rot; k_rot; v] as
+ * [H + 2*Hkv, D].  The weight (and bias) rows of the q and k sections must be interleaved per
+ * head as (0, D/2, 1, D/2 + 1, ...), so that one lane finishes both halves of a rotation pair;
+ * the v section keeps its natural order.  Roundings are those of the separate ops
+ * (krm_linear_i4_fused, krm_rope_half, krm_state_append); `lengths` / `past` as in
+ * krm_decode_rope_append, and like it this may precede the step's attention.
+ * Fuses packages/runtime/src/kernels/linear.ts:34-64, packages/runtime/src/kernels/rope.ts:5-20,
+ * 52-80 and packages/runtime/src/kernels/state-append.ts:47-96. */
+int32_t krm_decode_qkv(krm_ctx* ctx, krm_buf x, krm_buf norm_weight_f32, float norm_eps,
+                       krm_buf w, krm_buf scales, krm_buf bias, krm_buf positions_i32,
+                       krm_buf cos_table_f32, krm_buf sin_table_f32, krm_buf out, krm_buf slot_k,
+                       krm_buf slot_v, uint32_t heads, uint32_t kv_heads, uint32_t depth,
+                       uint32_t k, uint32_t group, uint32_t table_rows, uint32_t capacity,
+                       uint32_t window, uint32_t past, krm_buf lengths, int32_t io_dtype,
+                       int32_t scale_dtype, int32_t kv_dtype);
 /* [a, b, d] -> [b, a, d] (the reshape + permute between linears and attention). */
 int32_t krm_transpose_01(krm_ctx* ctx, krm_buf x, krm_buf out, uint32_t a, uint32_t b, uint32_t d,
                          int32_t io_dtype);

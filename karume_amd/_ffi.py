@@ -69,6 +69,9 @@ PROTOTYPES = {
                             i32]),
     "krm_decode_rope_append": (i32, [c_ctx, c_buf, c_buf, c_buf, c_buf, c_buf, c_buf, c_buf, u32,
                                      u32, u32, u32, u32, u32, u32, c_buf, i32, i32]),
+    "krm_decode_qkv": (i32, [c_ctx, c_buf, c_buf, C.c_float, c_buf, c_buf, c_buf, c_buf, c_buf,
+                             c_buf, c_buf, c_buf, c_buf, u32, u32, u32, u32, u32, u32, u32, u32,
+                             u32, c_buf, i32, i32, i32]),
     "krm_transpose_01": (i32, [c_ctx, c_buf, c_buf, u32, u32, u32, i32]),
     "krm_silu_mul": (i32, [c_ctx, c_buf, c_buf, c_buf, u64, i32]),
     "krm_add": (i32, [c_ctx, c_buf, c_buf, c_buf, u64, i32]),

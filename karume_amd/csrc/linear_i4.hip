@@ -241,7 +241,27 @@ struct GemvFusion {
   float norm_eps;
   const void* residual;      // [M, N_out] added to the result (same element type as out)
   uint32_t pair_silu;        // rows (2i, 2i+1) = (gate_i, up_i): out[., i] = silu(gate) * up
+  // Decode row of a fused [q; k; v] projection (positions != null; M = 1).  Rows (2i, 2i+1) of
+  // the q and k sections hold dims (j, j + D/2) of one head, so the lane that finishes a pair
+  // rotates it (half-split RoPE, two rounded products then the add, as rope_kernel does) and
+  // writes it to its natural place in `out` ([H + 2*Hkv, D]); k pairs and the v rows (natural
+  // order) are also appended to the state slots (same rule as state_append_kernel).
+  const int32_t* positions;
+  const float* cos_table;
+  const float* sin_table;
+  void* slot_k;
+  void* slot_v;
+  uint32_t* lengths;         // device {past, query, fault, ...} or null: `past` below
+  uint32_t heads, kv_heads, depth, table_rows, capacity, window, past;
+  int32_t slot_f16;          // slot element type: 1 = fp16, 0 = f32
 };
+
+__device__ inline void slot_store(void* slot, int32_t is_f16, size_t i, float v) {
+  if (is_f16)
+    static_cast<__half*>(slot)[i] = __float2half_rn(v);
+  else
+    static_cast<float*>(slot)[i] = v;
+}
 
 // One wave = ROWS consecutive output rows over the whole K; a step covers 64 lanes x VEC
 // words (VEC*8 codes per lane, all inside one scale group).
@@ -456,6 +476,65 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 4))) voi
       }
       return;
     }
+    if (fuse.positions) {
+      const uint32_t half = fuse.depth >> 1;
+      const uint32_t rope_pairs = (fuse.heads + fuse.kv_heads) * half;
+      uint32_t past = fuse.past;
+      bool append = true;
+      if (fuse.lengths) {  // run-time lengths read on the device; same checks as the scalar form
+        past = fuse.lengths[0];
+        append = fuse.lengths[1] == 1u && (uint64_t)past + 1 <= 0xffffffffull &&
+                 (fuse.window != 0 || (uint64_t)past + 1 <= fuse.capacity);
+        if (!append && row0 == 0 && lane == 0) fuse.lengths[2] = 1u;
+      }
+      const uint64_t prow = fuse.window ? (uint64_t)past % fuse.window : (uint64_t)past;
+      const int32_t pos = fuse.positions[0];
+      const bool in_table = pos >= 0 && (uint32_t)pos < fuse.table_rows;
+#pragma unroll
+      for (int p = 0; p < ROWS / 2; ++p) {
+        const uint32_t row = row0 + 2 * p, pair = row >> 1;
+        float x0 = wave_sum(acc[2 * p][0]) * inv[0];
+        float x1 = wave_sum(acc[2 * p + 1][0]) * inv[0];
+        if (lane != p % kWave || row + 1 >= n) continue;
+        if (bias) {
+          x0 += to_f32<XT>(bias[row]);
+          x1 += to_f32<XT>(bias[row + 1]);
+        }
+        // what a separate linear would have stored (rounded to the activation type)
+        x0 = to_f32<XT>(from_f32<XT>(x0));
+        x1 = to_f32<XT>(from_f32<XT>(x1));
+        if (pair < rope_pairs) {
+          const uint32_t head = pair / half, j = pair - head * half;
+          float o0 = NAN, o1 = NAN;  // a position outside the table is never a valid rotation
+          if (in_table) {
+            const size_t t = (size_t)pos * fuse.depth + j;
+            o0 = __fadd_rn(__fmul_rn(x0, fuse.cos_table[t]), __fmul_rn(-x1, fuse.sin_table[t]));
+            o1 = __fadd_rn(__fmul_rn(x1, fuse.cos_table[t + half]),
+                           __fmul_rn(x0, fuse.sin_table[t + half]));
+          }
+          const size_t at = (size_t)head * fuse.depth + j;
+          out[at] = from_f32<XT>(o0);
+          out[at + half] = from_f32<XT>(o1);
+          if (head >= fuse.heads && append) {
+            const size_t dst = ((size_t)(head - fuse.heads) * fuse.capacity + prow) * fuse.depth + j;
+            slot_store(fuse.slot_k, fuse.slot_f16, dst, to_f32<XT>(from_f32<XT>(o0)));
+            slot_store(fuse.slot_k, fuse.slot_f16, dst + half, to_f32<XT>(from_f32<XT>(o1)));
+          }
+        } else {
+          const uint32_t e = (pair - rope_pairs) * 2;  // element of the v section, natural order
+          const size_t at = (size_t)(fuse.heads + fuse.kv_heads) * fuse.depth + e;
+          out[at] = from_f32<XT>(x0);
+          out[at + 1] = from_f32<XT>(x1);
+          if (append) {
+            const uint32_t plane = e / fuse.depth, d = e - plane * fuse.depth;
+            const size_t dst = ((size_t)plane * fuse.capacity + prow) * fuse.depth + d;
+            slot_store(fuse.slot_v, fuse.slot_f16, dst, x0);
+            slot_store(fuse.slot_v, fuse.slot_f16, dst + 1, x1);
+          }
+        }
+      }
+      return;
+    }
   }
 #pragma unroll
   for (int r = 0; r < ROWS; ++r) {
@@ -518,7 +597,7 @@ int32_t pick_rows(krm_ctx* ctx, krm_buf x, krm_buf w, krm_buf scales, krm_buf bi
   if constexpr (MB == 1 && sizeof(XT) == 4 && VEC == 4)
     if (k <= 4096 && (uint64_t)n >= cus * 4 * 4 * 2)
       return pick_steps<XT, ST, MB, 4, VEC>(ctx, x, w, scales, bias, out, m, n, k, group_shift, fuse);
-  if (fuse.pair_silu || (uint64_t)n >= cus * 4 * 2)
+  if (fuse.pair_silu || fuse.positions || (uint64_t)n >= cus * 4 * 2)
     return pick_steps<XT, ST, MB, 2, VEC>(ctx, x, w, scales, bias, out, m, n, k, group_shift, fuse);
   return pick_steps<XT, ST, MB, 1, VEC>(ctx, x, w, scales, bias, out, m, n, k, group_shift, fuse);
 }
@@ -645,6 +724,63 @@ int32_t krm_linear_i4_fused(krm_ctx* ctx, krm_buf x, krm_buf norm_weight_f32, fl
   fuse.residual = ptr<const void>(residual);
   fuse.pair_silu = epilogue == KRM_EPILOGUE_SILU_PAIRS ? 1u : 0u;
   return gemv_dispatch(ctx, x, w, scales, bias, out, m, n, k, group, io_dtype, scale_dtype, fuse);
+}
+
+int32_t krm_decode_qkv(krm_ctx* ctx, krm_buf x, krm_buf norm_weight_f32, float norm_eps,
+                       krm_buf w, krm_buf scales, krm_buf bias, krm_buf positions_i32,
+                       krm_buf cos_table_f32, krm_buf sin_table_f32, krm_buf out, krm_buf slot_k,
+                       krm_buf slot_v, uint32_t heads, uint32_t kv_heads, uint32_t depth,
+                       uint32_t k, uint32_t group, uint32_t table_rows, uint32_t capacity,
+                       uint32_t window, uint32_t past, krm_buf lengths, int32_t io_dtype,
+                       int32_t scale_dtype, int32_t kv_dtype) {
+  KRM_TRY(enter(ctx));
+  KRM_REQUIRE(ctx, valid_dtype(io_dtype) && valid_dtype(scale_dtype) && valid_dtype(kv_dtype),
+              "krm_decode_qkv: io_dtype %d / scale_dtype %d / kv_dtype %d", io_dtype, scale_dtype,
+              kv_dtype);
+  KRM_REQUIRE(ctx, is_pow2(group) && group >= 16 && k >= 1 && k % group == 0,
+              "krm_decode_qkv: group_size %u must be a power of two >= 16 dividing k = %u", group,
+              k);
+  KRM_REQUIRE(ctx, heads >= 1 && kv_heads >= 1 && depth >= 2 && depth % 2 == 0 && capacity >= 1 &&
+                       table_rows >= 1,
+              "krm_decode_qkv: H / Hkv / D / C / table rows (%u / %u / %u / %u / %u)", heads,
+              kv_heads, depth, capacity, table_rows);
+  KRM_REQUIRE(ctx, ((uint64_t)heads + 2ull * kv_heads) * depth <= 0x7fffffffull,
+              "krm_decode_qkv: the row is too long");
+  KRM_REQUIRE(ctx, window <= capacity, "krm_decode_qkv: window %u exceeds capacity %u", window,
+              capacity);
+  KRM_REQUIRE(ctx, !norm_weight_f32 || std::isfinite(norm_eps), "krm_decode_qkv: eps");
+  if (!lengths && window == 0 && (uint64_t)past + 1 > capacity)
+    return fail(ctx, KRM_ERR_EXECUTION,
+                "krm_decode_qkv: pastLength %u + queryLength 1 exceeds capacity %u", past, capacity);
+  KRM_REQUIRE(ctx, x && w && scales && positions_i32 && cos_table_f32 && sin_table_f32 && out &&
+                       slot_k && slot_v,
+              "krm_decode_qkv: NULL buffer");
+  KRM_REQUIRE(ctx, aligned(x, 16) && aligned(norm_weight_f32, 16) && aligned(w, 4) &&
+                       aligned(out, dtype_bytes(io_dtype)) && aligned(bias, dtype_bytes(io_dtype)) &&
+                       aligned(scales, dtype_bytes(scale_dtype)) && aligned(positions_i32, 4) &&
+                       aligned(cos_table_f32, 4) && aligned(sin_table_f32, 4) &&
+                       aligned(slot_k, dtype_bytes(kv_dtype)) &&
+                       aligned(slot_v, dtype_bytes(kv_dtype)) && aligned(lengths, 4),
+              "krm_decode_qkv: misaligned buffer");
+  GemvFusion fuse{};
+  fuse.norm_weight = ptr<const float>(norm_weight_f32);
+  fuse.norm_eps = norm_eps;
+  fuse.positions = ptr<const int32_t>(positions_i32);
+  fuse.cos_table = ptr<const float>(cos_table_f32);
+  fuse.sin_table = ptr<const float>(sin_table_f32);
+  fuse.slot_k = ptr<void>(slot_k);
+  fuse.slot_v = ptr<void>(slot_v);
+  fuse.lengths = ptr<uint32_t>(lengths);
+  fuse.heads = heads;
+  fuse.kv_heads = kv_heads;
+  fuse.depth = depth;
+  fuse.table_rows = table_rows;
+  fuse.capacity = capacity;
+  fuse.window = window;
+  fuse.past = past;
+  fuse.slot_f16 = kv_dtype == KRM_F16 ? 1 : 0;
+  const uint32_t n = (heads + 2 * kv_heads) * depth;
+  return gemv_dispatch(ctx, x, w, scales, bias, out, 1, n, k, group, io_dtype, scale_dtype, fuse);
 }
 
 int32_t krm_dequant_i4(krm_ctx* ctx, krm_buf w, krm_buf scales, krm_buf out_f32, uint64_t rows,

@@ -125,6 +125,17 @@ def _interleave_rows(a: Int4Linear, b: Int4Linear) -> Int4Linear:
     return Int4Linear(a.n * 2, a.k, packed, scales)
 
 
+def _rope_pair_rows(lin: Int4Linear, head_dim: int) -> Int4Linear:
+    """Rows of every head reordered to (0, D/2, 1, D/2 + 1, ...): the two halves of a rotation
+    pair become neighbours, which is what the fused qkv launch expects for q and k."""
+    half = head_dim // 2
+    heads = lin.n // head_dim
+    order = (np.arange(heads)[:, None, None] * head_dim
+             + np.arange(half)[None, :, None] + np.array([0, half])[None, None, :]).reshape(-1)
+    return Int4Linear(lin.n, lin.k, np.ascontiguousarray(lin.packed[order]),
+                      np.ascontiguousarray(lin.scales[order]))
+
+
 class LlamaDecoderSession:
     """Weights resident on the device + scratch activations for chunks of up to chunk_length
     rows.  io dtype selects f32 (the reference's semantic dtype) or fp16 activations; kv dtype
@@ -153,7 +164,9 @@ class LlamaDecoderSession:
                    for name in ("q", "k", "v", "o", "gate", "up", "down")},
             }
             if fuse_decode:
-                entry["qkv"] = _DeviceLinear(gpu, _stack_rows(lw["q"], lw["k"], lw["v"]))
+                entry["qkv"] = _DeviceLinear(gpu, _stack_rows(
+                    _rope_pair_rows(lw["q"], c.head_dim), _rope_pair_rows(lw["k"], c.head_dim),
+                    lw["v"]))
                 entry["gate_up"] = _DeviceLinear(gpu, _interleave_rows(lw["gate"], lw["up"]))
             self.layers.append(entry)
         self.final_norm = gpu.upload(weights.final_norm)
@@ -296,25 +309,26 @@ class LlamaDecoderSession:
 
     def _forward_fused_row(self, context: GenerationContext, past: int,
                            lengths: Optional[DeviceBuffer]) -> None:
-        """One decode row (M = Q = 1), 6 launches per layer instead of 16."""
+        """One decode row (M = Q = 1), 5 launches per layer instead of 16."""
         from .runtime import EPILOGUE_SILU_PAIRS
         g, c, b, io, eb = self.gpu, self.config, self.buf, self.io_dtype, self.eb
         hd, kvd = c.heads * c.head_dim, c.kv_heads * c.head_dim
-        q_r, k_r = b["qkr"], b["qkr"].offset(hd * eb)
+        # the qkv launch leaves [q_rot; k_rot; v] in one buffer
+        q_r, k_r = b["qkv"], b["qkv"].offset(hd * eb)
         v_row = b["qkv"].offset((hd + kvd) * eb)
         spec = dict(chunk_rows=1, depth=c.head_dim, capacity=context.capacity,
                     window=context.window)
         for li, lw in enumerate(self.layers):
-            self._fused(b["h"], lw["qkv"], b["qkv"], norm_weight=lw["attn_norm"],
-                        norm_eps=c.rms_eps)
-            # rope of the q and k heads and both appends in one launch; a one-row step's
-            # attention never reads the slot row this writes, so it may go first
-            g.decode_rope_append(b["qkv"], b["pos"], self.rope_cos, self.rope_sin, b["qkr"],
-                                 context.slots_k[li], context.slots_v[li], heads=c.heads,
-                                 kv_heads=c.kv_heads, depth=c.head_dim,
-                                 table_rows=c.max_position, capacity=context.capacity,
-                                 window=context.window, past=past, lengths=lengths, io_dtype=io,
-                                 kv_dtype=self.kv_dtype)
+            # rms_norm + [q; k; v] + rope of q and k + both appends in one launch; a one-row
+            # step's attention never reads the slot row this writes, so it may go first
+            lin = lw["qkv"]
+            g.decode_qkv(b["h"], lin.w, lin.s, b["pos"], self.rope_cos, self.rope_sin, b["qkv"],
+                         context.slots_k[li], context.slots_v[li], heads=c.heads,
+                         kv_heads=c.kv_heads, depth=c.head_dim, k=lin.k, group=c.group_size,
+                         table_rows=c.max_position, capacity=context.capacity,
+                         window=context.window, past=past, lengths=lengths,
+                         norm_weight=lw["attn_norm"], norm_eps=c.rms_eps, io_dtype=io,
+                         scale_dtype=F16, kv_dtype=self.kv_dtype)
             if lengths is None:
                 g.attention_state(q_r, k_r, v_row, context.slots_k[li], context.slots_v[li],
                                   b["att"], batch=1, heads=c.heads, kv_heads=c.kv_heads,

@@ -381,6 +381,23 @@ class GpuContext:
             capacity, window, past, _addr(lengths) if lengths is not None else 0, io_dtype,
             kv_dtype))
 
+    def decode_qkv(self, x: BufferLike, w: BufferLike, scales: BufferLike, positions: BufferLike,
+                   cos_table: BufferLike, sin_table: BufferLike, out: BufferLike,
+                   slot_k: BufferLike, slot_v: BufferLike, *, heads: int, kv_heads: int,
+                   depth: int, k: int, group: int, table_rows: int, capacity: int,
+                   window: int = 0, past: int = 0, lengths: Optional[BufferLike] = None,
+                   norm_weight: Optional[BufferLike] = None, norm_eps: float = 0.0,
+                   bias: Optional[BufferLike] = None, io_dtype: int = F32,
+                   scale_dtype: int = F32, kv_dtype: int = F32) -> None:
+        """(rms_norm ->) fused [q; k; v] projection of one decode row -> RoPE of q and k ->
+        state_append of k and v; q/k weight rows interleaved per head as (j, j + D/2)."""
+        self._check(self._lib.krm_decode_qkv(
+            self._handle, _addr(x), _addr(norm_weight) if norm_weight is not None else 0,
+            float(norm_eps), _addr(w), _addr(scales), _addr(bias) if bias is not None else 0,
+            _addr(positions), _addr(cos_table), _addr(sin_table), _addr(out), _addr(slot_k),
+            _addr(slot_v), heads, kv_heads, depth, k, group, table_rows, capacity, window, past,
+            _addr(lengths) if lengths is not None else 0, io_dtype, scale_dtype, kv_dtype))
+
     def transpose_01(self, x: BufferLike, out: BufferLike, a: int, b: int, d: int,
                      io_dtype: int = F32) -> None:
         self._check(self._lib.krm_transpose_01(self._handle, _addr(x), _addr(out), a, b, d,

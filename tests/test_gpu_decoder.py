@@ -147,6 +147,83 @@ def test_decode_rope_append_equals_rope_then_appends(gpu_ctx, io, kv, window, pa
         assert clean_v.download(kv_np, slot0_v.shape).tobytes() == slot0_v.tobytes()
 
 
+@pytest.mark.parametrize("io,kv", [(ka.F32, ka.F32), (ka.F32, ka.F16), (ka.F16, ka.F16)])
+@pytest.mark.parametrize("window,past,k", [(0, 5, 256), (4, 9, 2048), (0, 0, 4096)])
+def test_decode_qkv_equals_linear_rope_appends(gpu_ctx, io, kv, window, past, k):
+    """krm_decode_qkv (rms_norm + [q;k;v] + rope + appends, pair-interleaved q/k rows) writes
+    the same bits as krm_linear_i4_fused + krm_rope_half + two krm_state_append."""
+    from karume_amd.decoder import Int4Linear, _rope_pair_rows, _stack_rows
+    rng = np.random.default_rng(11 + past)
+    heads, kv_heads, d, table, cap, group = 4, 2, 32, 16, 12, 128
+    io_np = np.float32 if io == ka.F32 else np.float16
+    kv_np = np.float32 if kv == ka.F32 else np.float16
+    n = (heads + 2 * kv_heads) * d
+    packed, _codes, scales = helpers.synthetic_int4(rng, n, k, group)
+    packed = packed.reshape(n, k // 2)
+    x = rng.normal(size=(1, k)).astype(io_np)
+    norm_w = rng.normal(1.0, 0.1, size=k).astype(np.float32)
+    ang = rng.normal(size=(table, d))
+    cos, sin = np.cos(ang).astype(np.float32), np.sin(ang).astype(np.float32)
+    slot0_k = rng.normal(size=(kv_heads, cap, d)).astype(kv_np)
+    slot0_v = rng.normal(size=(kv_heads, cap, d)).astype(kv_np)
+    dx, dn, dc, ds = map(gpu_ctx.upload, (x, norm_w, cos, sin))
+    dp = gpu_ctx.upload(np.array([past], dtype=np.int32))
+    eb = x.itemsize
+    hq, hk = heads * d, kv_heads * d
+
+    # separate launches on the natural row order
+    dw, dsc = gpu_ctx.upload(packed), gpu_ctx.upload(scales)
+    qkv = gpu_ctx.alloc(n * eb)
+    gpu_ctx.linear_i4_fused(dx, dw, dsc, qkv, 1, n, k, group, io_dtype=io, scale_dtype=ka.F16,
+                            norm_weight=dn, norm_eps=1e-5)
+    want = gpu_ctx.alloc(n * eb)
+    gpu_ctx.rope_half(qkv, dp, dc, ds, want, 1, heads + kv_heads, d, table, True, io)
+    gpu_ctx.copy(want.offset((hq + hk) * eb), qkv.offset((hq + hk) * eb), hk * eb)
+    ref_k, ref_v = gpu_ctx.upload(slot0_k), gpu_ctx.upload(slot0_v)
+    spec = dict(kv_planes=kv_heads, chunk_rows=1, depth=d, capacity=cap, window=window,
+                x_dtype=io, slot_dtype=kv)
+    gpu_ctx.state_append(want.offset(hq * eb), ref_k, past=past, query=1, **spec)
+    gpu_ctx.state_append(want.offset((hq + hk) * eb), ref_v, past=past, query=1, **spec)
+    want_row = want.download(io_np, (n,))
+    want_k, want_v = ref_k.download(kv_np, slot0_k.shape), ref_v.download(kv_np, slot0_v.shape)
+
+    # one launch on the pair-interleaved rows
+    def part(lo, hi):
+        return Int4Linear(hi - lo, k, packed[lo:hi], scales[lo:hi])
+    fused = _stack_rows(_rope_pair_rows(part(0, hq), d), _rope_pair_rows(part(hq, hq + hk), d),
+                        part(hq + hk, n))
+    fw, fs = gpu_ctx.upload(fused.packed), gpu_ctx.upload(fused.scales)
+    lengths = gpu_ctx.zeros(16)
+    for dyn in (False, True):
+        got = gpu_ctx.zeros(n * eb)
+        got_k, got_v = gpu_ctx.upload(slot0_k), gpu_ctx.upload(slot0_v)
+        if dyn:
+            gpu_ctx.lengths_set(lengths, past, 1)
+        gpu_ctx.decode_qkv(dx, fw, fs, dp, dc, ds, got, got_k, got_v, heads=heads,
+                           kv_heads=kv_heads, depth=d, k=k, group=group, table_rows=table,
+                           capacity=cap, window=window, past=0 if dyn else past,
+                           lengths=lengths if dyn else None, norm_weight=dn, norm_eps=1e-5,
+                           io_dtype=io, scale_dtype=ka.F16, kv_dtype=kv)
+        assert got.download(io_np, (n,)).tobytes() == want_row.tobytes()
+        assert got_k.download(kv_np, want_k.shape).tobytes() == want_k.tobytes()
+        assert got_v.download(kv_np, want_v.shape).tobytes() == want_v.tobytes()
+    assert lengths.download(np.uint32, (4,))[2] == 0
+    if window == 0:
+        with pytest.raises(ka.ExecutionError):
+            gpu_ctx.decode_qkv(dx, fw, fs, dp, dc, ds, got, got_k, got_v, heads=heads,
+                               kv_heads=kv_heads, depth=d, k=k, group=group, table_rows=table,
+                               capacity=cap, past=cap, io_dtype=io, scale_dtype=ka.F16,
+                               kv_dtype=kv)
+        clean_k = gpu_ctx.upload(slot0_k)
+        gpu_ctx.lengths_set(lengths, cap, 1)
+        gpu_ctx.decode_qkv(dx, fw, fs, dp, dc, ds, got, clean_k, got_v, heads=heads,
+                           kv_heads=kv_heads, depth=d, k=k, group=group, table_rows=table,
+                           capacity=cap, lengths=lengths, io_dtype=io, scale_dtype=ka.F16,
+                           kv_dtype=kv)
+        assert lengths.download(np.uint32, (4,))[2] == 1
+        assert clean_k.download(kv_np, slot0_k.shape).tobytes() == slot0_k.tobytes()
+
+
 def test_transpose(gpu_ctx):
     x = np.arange(3 * 5 * 4, dtype=np.float32).reshape(3, 5, 4)
     dx = gpu_ctx.upload(x)
@@ -250,7 +327,7 @@ def test_greedy_loop_and_replayed_decode_agree(gpu_ctx):
 
 
 def test_fused_and_separate_decode_launches_agree(gpu_ctx):
-    """The fused one-row step (8 launches per layer) and the op-by-op step (16 launches) give
+    """The fused one-row step (5 launches per layer) and the op-by-op step (16 launches) give
     logits within 1e-4 of each other and the same tokens on a teacher-forced sequence."""
     weights = random_weights(SMALL, seed=7)
     ids = np.random.default_rng(2).integers(0, SMALL.vocab, size=14).astype(np.int32)
