@@ -328,8 +328,11 @@ void attention_decode_kernel(
   const uint32_t hk = blockIdx.y / a.head_groups;
   const uint32_t head0 = hk * a.repeat + (blockIdx.y - hk * a.head_groups) * R;  // first head
 
+  // Columns and slot rows are 32-bit (pastLength is a u32, a ragged batch holds < 2^31 rows);
+  // only the final byte address is 64-bit: 64-bit index math per load costs more than the
+  // attention arithmetic of a short past.
   uint32_t seq, split, nsplit, first_split;
-  uint64_t past, row_base;
+  uint32_t past, row_base;
   if constexpr (RAGGED) {
     // binary search: last sequence whose first split is <= blockIdx.x
     uint32_t lo_i = 0, hi_i = a.nseq;
@@ -341,8 +344,8 @@ void attention_decode_kernel(
     first_split = (uint32_t)a.split_prefix[seq];
     nsplit = (uint32_t)a.split_prefix[seq + 1] - first_split;
     split = blockIdx.x - first_split;
-    row_base = (uint64_t)a.cu_rows[seq];
-    past = (uint64_t)a.cu_rows[seq + 1] - row_base;
+    row_base = (uint32_t)a.cu_rows[seq];
+    past = (uint32_t)a.cu_rows[seq + 1] - row_base;
   } else {
     seq = blockIdx.z;
     uint32_t p32 = a.past, q32 = 1;
@@ -354,10 +357,10 @@ void attention_decode_kernel(
     if (split >= nsplit) return;  // the grid is sized for the longest past it may see
     first_split = seq * nsplit;
   }
-  const uint64_t low = window_low(a.window, past);  // limit of row 0 is `past`
+  const uint32_t low = (uint32_t)window_low(a.window, past);  // limit of row 0 is `past`
   const uint32_t total_chunks = decode_chunks(past - low, kChunkCols);
   const uint32_t my_chunks = nsplit == 1 ? total_chunks : 1u;
-  const uint64_t c_first = low + (uint64_t)split * kChunkCols;
+  const uint32_t c_first = low + split * kChunkCols;  // < past
   const bool last = split + 1 == nsplit;
 
   const size_t slot_base = (size_t)seq * a.slot_batch_stride + (size_t)hk * a.slot_plane_stride;
@@ -416,52 +419,50 @@ void attention_decode_kernel(
   };
   const int wave = tid >> 6, lane = tid & 63;
   const int frag_row = lane & 15, frag_g = lane >> 4;
-  auto chunk_begin = [&](uint32_t chunk) { return c_first + (uint64_t)chunk * kChunkCols; };
-  auto chunk_end = [&](uint64_t c_begin) {
-    return (c_begin + kChunkCols < past) ? c_begin + kChunkCols : past;
+  auto chunk_begin = [&](uint32_t chunk) { return c_first + chunk * kChunkCols; };
+  auto chunk_end = [&](uint32_t c_begin) {  // c_begin < past: no overflow
+    return past - c_begin > (uint32_t)kChunkCols ? c_begin + kChunkCols : past;
   };
-  // column that (lane group, iteration) owns inside a chunk
-  auto column_of = [&](uint64_t c_begin, int it) {
+  // offset inside a chunk of the column that (lane group, iteration) owns
+  auto column_of = [&](int it) -> uint32_t {
     if constexpr (kMfma)
-      return c_begin + (uint64_t)((wave * 2 + it / 4) * 16 + 4 * frag_g + (it & 3));
+      return (uint32_t)((wave * 2 + it / 4) * 16 + 4 * frag_g + (it & 3));
     else
-      return c_begin + (uint64_t)it * G + group;
+      return (uint32_t)(it * G + group);
   };
   // Requests only: every K row, then every V row of the chunk; unconditional (a column past
   // the end re-reads the chunk's first column and is masked when it is used).
   auto load_chunk = [&](uint32_t chunk, ChunkRows& rows) {
-    const uint64_t c_begin = chunk_begin(chunk), c_end = chunk_end(c_begin);
-    auto slot_row = [&](uint64_t col) {
-      const uint64_t c = col < c_end ? col : c_begin;
-      return row_base + (a.window ? c % a.window : c);
+    const uint32_t c_begin = chunk_begin(chunk), width = chunk_end(c_begin) - c_begin;
+    auto slot_row = [&](uint32_t offset) {  // element offset of the row's first dim
+      const uint32_t c = c_begin + (offset < width ? offset : 0u);
+      return (size_t)(row_base + (a.window ? c % a.window : c)) * D;
     };
     if constexpr (kMfma) {
       // lane (r = lane % 16, g = lane / 16) takes 16 bytes of K row r of each 16-row tile at
       // dims 32t + 8g..: the A-operand layout of v_mfma_f32_16x16x32_f16
 #pragma unroll
       for (int tile = 0; tile < 2; ++tile) {
-        const uint64_t prow = slot_row(c_begin + (uint64_t)((wave * 2 + tile) * 16 + frag_row));
+        const size_t at = slot_row((uint32_t)((wave * 2 + tile) * 16 + frag_row));
 #pragma unroll
         for (int t = 0; t < 4; ++t)
           rows.k[tile * 4 + t] =
-              *reinterpret_cast<const uint4*>(kslot + prow * D + 32 * t + 8 * frag_g);
+              *reinterpret_cast<const uint4*>(kslot + at + 32 * t + 8 * frag_g);
       }
     } else {
 #pragma unroll
       for (int it = 0; it < kDecodeIter; ++it)
-        rows.k[it] = *reinterpret_cast<const uint4*>(
-            kslot + slot_row(column_of(c_begin, it)) * D + sub * E);
+        rows.k[it] = *reinterpret_cast<const uint4*>(kslot + slot_row(column_of(it)) + sub * E);
     }
 #pragma unroll
     for (int it = 0; it < kDecodeIter; ++it)
-      rows.v[it] = *reinterpret_cast<const uint4*>(
-          vslot + slot_row(column_of(c_begin, it)) * D + sub * E);
+      rows.v[it] = *reinterpret_cast<const uint4*>(vslot + slot_row(column_of(it)) + sub * E);
   };
   auto consume_chunk = [&](uint32_t chunk, ChunkRows& rows) {
-    const uint64_t c_begin = chunk_begin(chunk), c_end = chunk_end(c_begin);
+    const uint32_t c_begin = chunk_begin(chunk), width = chunk_end(c_begin) - c_begin;
     bool valid[kDecodeIter];
 #pragma unroll
-    for (int it = 0; it < kDecodeIter; ++it) valid[it] = column_of(c_begin, it) < c_end;
+    for (int it = 0; it < kDecodeIter; ++it) valid[it] = column_of(it) < width;
     float sc[kDecodeIter][R];
     float cm[R];
 #pragma unroll
@@ -533,9 +534,8 @@ void attention_decode_kernel(
       }
     }
   };
-  // (Requesting chunk c + 1 before chunk c is used was tried for short pasts walked by one
-  // split: the second set of row registers halves the workgroups a CU holds, which costs the
-  // long pasts more than it gives the short ones.)
+  // (Requesting chunk c + 1 before chunk c is used, for short pasts walked by one split, was
+  // measured slower: 0.35 us more per launch at 1-4 chunks.)
   for (uint32_t chunk = 0; chunk < my_chunks; ++chunk) {
     ChunkRows rows;
     load_chunk(chunk, rows);

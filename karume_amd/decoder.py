@@ -303,6 +303,12 @@ class LlamaDecoderSession:
         self._linear(b["xn"], self.lm_head, b["logits"], 1)
         g.argmax(b["logits"], b["token"], 1, c.vocab, io)
 
+    def _replay_max_past(self, context: GenerationContext) -> int:
+        """Largest pastLength the recorded step will be replayed with: sizes the attention
+        launch (a short replay needs one split and takes the prefetching form)."""
+        hint = getattr(self, "_replay_last_past", None)
+        return context.capacity - 1 if hint is None else min(context.capacity - 1, hint)
+
     def _fused(self, x, lin: _DeviceLinear, out, **kw) -> None:
         self.gpu.linear_i4_fused(x, lin.w, lin.s, out, 1, lin.n, lin.k, self.config.group_size,
                                  io_dtype=self.io_dtype, scale_dtype=F16, **kw)
@@ -338,7 +344,7 @@ class LlamaDecoderSession:
                 g.attention_state_lengths(q_r, k_r, v_row, context.slots_k[li],
                                           context.slots_v[li], b["att"], batch=1, heads=c.heads,
                                           kv_heads=c.kv_heads, half_scale=c.half_scale,
-                                          lengths=lengths, max_past=context.capacity - 1,
+                                          lengths=lengths, max_past=self._replay_max_past(context),
                                           io_dtype=io, kv_dtype=self.kv_dtype,
                                           workspace=self.workspace, **spec)
             self._fused(b["att"], lw["o"], b["h"], residual=b["h"])
@@ -371,6 +377,7 @@ class LlamaDecoderSession:
             # embedding reads it
             b["token"].upload(np.array([first_token, 0, 0, 0], dtype=np.int32))
             g.lengths_set(context.lengths, context.past, 1)
+            self._replay_last_past = context.past + count - 1
             with g.record() as rec:
                 g.lengths_positions(context.lengths, b["pos"], 1)
                 self._forward(context, 1, 0, 1, 0, lengths=context.lengths, ids=b["token"])
@@ -385,6 +392,7 @@ class LlamaDecoderSession:
             context.poison()
             raise
         finally:
+            self._replay_last_past = None
             if graph is not None:
                 graph.destroy()
             history.free()
