@@ -246,7 +246,7 @@ def main() -> int:
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-graph", action="store_true",
                     help="issue plain launches instead of replaying recorded graphs")
-    ap.add_argument("--only", default="", help="gemv | gemm | attention | model | traffic: run only that part besides the "
+    ap.add_argument("--only", default="", help="gemv | gemv16 | gemm | attention | model | traffic: run only that part besides the "
                          "headline GEMV")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -302,7 +302,7 @@ def main() -> int:
         bench_gemm(ctx, ka, rng, 4, 2, 512, 11008, 4096, g)
         bench_gemm(ctx, ka, rng, 4, 2, 512, 4096, 11008, g)
     steps2 = max(50, args.steps // 4)
-    if args.only == "":
+    if args.only in ("", "gemv16"):
         log("[bench] GEMV M=16 (config 3)")
         ms16, _res16, algo16 = bench_gemv(ctx, ka, rng, steps2, max(10, args.warmup // 4), 16, n,
                                           k, g, copies)

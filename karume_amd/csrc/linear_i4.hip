@@ -222,6 +222,152 @@ struct Acts<float> {
   }
 };
 
+// ------------------------------------------------------------------ batched rows on MFMA
+//
+// 2 <= M <= 16 rows of fp16 activations: sixteen dot products per weight word on the VALU make
+// the kernel above compute-bound (about 400 GB/s at M = 16).  Here the products run on
+// v_mfma_f32_16x16x32_f16 and the VALU only dequantises: A = x (16 rows, rows past M repeat
+// the last one and are dropped), B = W^T, where lane (n = lane % 16, g = lane / 16) holds eight
+// codes of weight row n — one 32-bit word — as exact fp16 integers (u - 8), straight from the
+// load, no LDS.  A workgroup owns 16 weight rows; its four waves split K in quarters and walk
+// them in chunks of 256 codes.  Per chunk a lane loads the 16-byte pieces g and 4 + g of its
+// row, so that the four lane groups of MFMA step s < 4 (word 4g + s) cover codes 0..127 of the
+// chunk and steps 4..7 cover codes 128..255: each half lies inside one scale group (group >=
+// 128), is accumulated on its own and multiplied by the f32 scale of the lane's row afterwards
+// (the C layout keeps weight row n in lane % 16).  Products are exact, sums and scaling are
+// f32: the same arithmetic class as the kernel above, in a different order.
+typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
+typedef float float4_t __attribute__((ext_vector_type(4)));
+
+template <typename ST, int CHUNKS>
+__global__ __launch_bounds__(256) void gemv_i4_mfma_kernel(
+    const __half* __restrict__ x, const uint32_t* __restrict__ w, const ST* __restrict__ scales,
+    const __half* __restrict__ bias, __half* __restrict__ out, uint32_t m, uint32_t n, uint32_t k,
+    uint32_t group_shift) {
+  constexpr int kChunk = 256;
+  __shared__ float s_part[4][4][kWave];  // [wave][register][lane]
+  const int lane = threadIdx.x & (kWave - 1);
+  const int wave = threadIdx.x >> 6;
+  const int r16 = lane & 15, g = lane >> 4;
+  const uint32_t n0 = blockIdx.x * 16;
+  const uint32_t wrow = min(n0 + r16, n - 1);  // rows past N re-read the last row, unused
+  const uint32_t k_quarter = k >> 2;
+  const uint32_t k_first = wave * k_quarter;
+  const uint32_t chunks = k_quarter / kChunk;
+  const uint32_t* wptr = w + (size_t)wrow * (k >> 3) + (k_first >> 3) + 4 * g;
+  const ST* sptr = scales + (size_t)wrow * (k >> group_shift);
+
+  struct Weights {
+    uint4 words[2];   // pieces g and 4 + g of the row's 32 words
+    float scale[2];   // scale of each half of the chunk for this lane's row
+  };
+  // Activations: lane (row r, group g) needs x[r][16-byte piece 4g + s] at step s — a gather
+  // over 16 rows that the vector cache serves one row at a time.  So a wave first loads its
+  // chunk of x coalesced (32 lanes x 16 bytes = one row's 512 bytes), pairs the values for
+  // the nibble order and parks them in its own LDS strip, rows padded by 16 bytes so that
+  // the gather is conflict-free there.  Only this wave touches the strip: no barrier.
+  constexpr int kRowBytes = kChunk * 2 + 16;
+  constexpr int kStripBytes = 16 * kRowBytes;
+  __shared__ __attribute__((aligned(16))) unsigned char s_x[4][2][kStripBytes];
+  struct Acts {
+    uint4 piece[8];   // x pieces as loaded: rows 2j + lane / 32, piece lane % 32
+  };
+  auto fetch_w = [&](uint32_t chunk, Weights& c) {
+    const uint32_t kc = chunk * kChunk;
+    c.words[0] = *reinterpret_cast<const uint4*>(wptr + (kc >> 3));
+    c.words[1] = *reinterpret_cast<const uint4*>(wptr + (kc >> 3) + 16);
+    c.scale[0] = load_scale<ST>(sptr, (k_first + kc) >> group_shift);
+    c.scale[1] = load_scale<ST>(sptr, (k_first + kc + 128) >> group_shift);
+  };
+  const int load_row = lane >> 5, load_piece = lane & 31;
+  auto fetch_x = [&](uint32_t chunk, Acts& c) {
+    const uint32_t kc = chunk * kChunk;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const uint32_t row = min((uint32_t)(2 * j + load_row), m - 1);
+      c.piece[j] =
+          *reinterpret_cast<const uint4*>(x + (size_t)row * k + k_first + kc + 8 * load_piece);
+    }
+  };
+  auto park_x = [&](const Acts& c, int strip) {
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      half2_t p[4];
+      pair_activations(c.piece[j], p);
+      const uint4 v = make_uint4(__builtin_bit_cast(uint32_t, p[0]), __builtin_bit_cast(uint32_t, p[1]),
+                                 __builtin_bit_cast(uint32_t, p[2]), __builtin_bit_cast(uint32_t, p[3]));
+      *reinterpret_cast<uint4*>(&s_x[wave][strip][(2 * j + load_row) * kRowBytes + 16 * load_piece]) = v;
+    }
+  };
+  float4_t total = {0.f, 0.f, 0.f, 0.f};  // out[m = 4g + i][n = lane % 16] over this K quarter
+  auto consume = [&](const Weights& c, int strip) {
+    float4_t half_sum[2] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}};
+    half8_t a[8];
+#pragma unroll
+    for (int s = 0; s < 8; ++s)  // step s: word 4g + s (s < 4) or 16 + 4g + (s - 4)
+      a[s] = *reinterpret_cast<const half8_t*>(
+          &s_x[wave][strip][r16 * kRowBytes + 16 * ((s < 4 ? 4 * g + s : 16 + 4 * g + (s - 4)))]);
+#pragma unroll
+    for (int s = 0; s < 8; ++s) {
+      const uint32_t word = s < 4 ? (&c.words[0].x)[s] : (&c.words[1].x)[s - 4];
+      half2_t q[4];
+      codes_to_half2(word, q);
+      const half8_t b = {q[0].x, q[0].y, q[1].x, q[1].y, q[2].x, q[2].y, q[3].x, q[3].y};
+      half_sum[s >> 2] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[s], b, half_sum[s >> 2], 0, 0, 0);
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      total[i] = fmaf(half_sum[0][i], c.scale[0], total[i]);
+      total[i] = fmaf(half_sum[1][i], c.scale[1], total[i]);
+    }
+  };
+  if constexpr (CHUNKS > 0) {
+    // the wave's whole share of the weights is requested first (the long trip); activations
+    // run two chunks ahead in registers and one ahead in LDS; fixed registers, no branches
+    Weights wq[CHUNKS];
+#pragma unroll
+    for (int c = 0; c < CHUNKS; ++c) fetch_w(c, wq[c]);
+    Acts xa[2];
+    fetch_x(0, xa[0]);
+    if (CHUNKS > 1) fetch_x(1, xa[1]);
+    park_x(xa[0], 0);
+#pragma unroll
+    for (int c = 0; c < CHUNKS; ++c) {
+      if (c + 2 < CHUNKS) fetch_x(c + 2, xa[c & 1]);       // slot of the chunk parked last pass
+      if (c + 1 < CHUNKS) park_x(xa[(c + 1) & 1], (c + 1) & 1);
+      consume(wq[c], c & 1);
+    }
+  } else {
+    for (uint32_t chunk = 0; chunk < chunks; ++chunk) {
+      Weights wq;
+      Acts xa;
+      fetch_w(chunk, wq);
+      fetch_x(chunk, xa);
+      park_x(xa, 0);
+      consume(wq, 0);
+    }
+  }
+  // the four K quarters, added in wave order
+#pragma unroll
+  for (int i = 0; i < 4; ++i) s_part[wave][i][lane] = total[i];
+  __syncthreads();
+  if (wave == 0) {
+    const uint32_t col = n0 + r16;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      float v = s_part[0][i][lane];
+#pragma unroll
+      for (int q = 1; q < 4; ++q) v += s_part[q][i][lane];
+      const uint32_t row = 4 * g + i;
+      if (row < m && col < n) {
+        if (bias) v += __half2float(bias[col]);
+        out[(size_t)row * n + col] = __float2half_rn(v);
+      }
+    }
+  }
+}
+
+
 template <typename T>
 __device__ inline float to_f32(T v);
 template <>
@@ -633,6 +779,34 @@ static int32_t gemv_dispatch(krm_ctx* ctx, krm_buf x, krm_buf w, krm_buf scales,
                              krm_buf out, uint32_t m, uint32_t n, uint32_t k, uint32_t group,
                              int32_t io_dtype, int32_t scale_dtype, const GemvFusion& fuse) {
   if (io_dtype == KRM_F16) {
+    // batched fp16 rows on the matrix cores (plain op only)
+    const bool plain = !fuse.norm_weight && !fuse.residual && !fuse.pair_silu && !fuse.positions;
+    if (plain && m >= 2 && k % 1024 == 0 && group >= 128 && aligned(w, 16) && aligned(x, 16) &&
+        aligned(scales, 4)) {
+      uint32_t group_shift = 0;
+      while ((1u << group_shift) < group) ++group_shift;
+      const uint32_t blocks = (n + 15) / 16;
+#define KRM_MFMA_GEMV(ST, CH)                                                                  \
+  gemv_i4_mfma_kernel<ST, CH><<<dim3(blocks), dim3(256), 0, ctx->stream>>>(                    \
+      ptr<const __half>(x), ptr<const uint32_t>(w), ptr<const ST>(scales),                     \
+      ptr<const __half>(bias), ptr<__half>(out), m, n, k, group_shift)
+#define KRM_MFMA_GEMV_BY_K(ST)                      \
+  switch (k / 1024) {                               \
+    case 1: KRM_MFMA_GEMV(ST, 1); break;            \
+    case 2: KRM_MFMA_GEMV(ST, 2); break;            \
+    case 4: KRM_MFMA_GEMV(ST, 4); break;            \
+    case 8: KRM_MFMA_GEMV(ST, 8); break;            \
+    default: KRM_MFMA_GEMV(ST, 0); break;           \
+  }
+      if (scale_dtype == KRM_F16) {
+        KRM_MFMA_GEMV_BY_K(__half)
+      } else {
+        KRM_MFMA_GEMV_BY_K(float)
+      }
+#undef KRM_MFMA_GEMV_BY_K
+#undef KRM_MFMA_GEMV
+      return launched(ctx, "gemv_i4_mfma_kernel");
+    }
     if (scale_dtype == KRM_F16)
       return pick_vec<__half, __half>(ctx, x, w, scales, bias, out, m, n, k, group, fuse);
     return pick_vec<__half, float>(ctx, x, w, scales, bias, out, m, n, k, group, fuse);
