@@ -239,19 +239,19 @@ struct Acts<float> {
 typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
 typedef float float4_t __attribute__((ext_vector_type(4)));
 
-template <typename ST, int CHUNKS>
-__global__ __launch_bounds__(256) void gemv_i4_mfma_kernel(
+template <typename ST, int CHUNKS, int KW>
+__global__ __launch_bounds__(KW * 64) void gemv_i4_mfma_kernel(
     const __half* __restrict__ x, const uint32_t* __restrict__ w, const ST* __restrict__ scales,
     const __half* __restrict__ bias, __half* __restrict__ out, uint32_t m, uint32_t n, uint32_t k,
     uint32_t group_shift) {
   constexpr int kChunk = 256;
-  __shared__ float s_part[4][4][kWave];  // [wave][register][lane]
+  __shared__ float s_part[KW][4][kWave];  // [wave][register][lane]
   const int lane = threadIdx.x & (kWave - 1);
   const int wave = threadIdx.x >> 6;
   const int r16 = lane & 15, g = lane >> 4;
   const uint32_t n0 = blockIdx.x * 16;
   const uint32_t wrow = min(n0 + r16, n - 1);  // rows past N re-read the last row, unused
-  const uint32_t k_quarter = k >> 2;
+  const uint32_t k_quarter = k / KW;  // this wave's share of K
   const uint32_t k_first = wave * k_quarter;
   const uint32_t chunks = k_quarter / kChunk;
   const uint32_t* wptr = w + (size_t)wrow * (k >> 3) + (k_first >> 3) + 4 * g;
@@ -268,7 +268,7 @@ __global__ __launch_bounds__(256) void gemv_i4_mfma_kernel(
   // the gather is conflict-free there.  Only this wave touches the strip: no barrier.
   constexpr int kRowBytes = kChunk * 2 + 16;
   constexpr int kStripBytes = 16 * kRowBytes;
-  __shared__ __attribute__((aligned(16))) unsigned char s_x[4][2][kStripBytes];
+  __shared__ __attribute__((aligned(16))) unsigned char s_x[KW][CHUNKS == 1 ? 1 : 2][kStripBytes];
   struct Acts {
     uint4 piece[8];   // x pieces as loaded: rows 2j + lane / 32, piece lane % 32
   };
@@ -347,7 +347,7 @@ __global__ __launch_bounds__(256) void gemv_i4_mfma_kernel(
       consume(wq, 0);
     }
   }
-  // the four K quarters, added in wave order
+  // the waves' shares of K, added in wave order
 #pragma unroll
   for (int i = 0; i < 4; ++i) s_part[wave][i][lane] = total[i];
   __syncthreads();
@@ -357,7 +357,7 @@ __global__ __launch_bounds__(256) void gemv_i4_mfma_kernel(
     for (int i = 0; i < 4; ++i) {
       float v = s_part[0][i][lane];
 #pragma unroll
-      for (int q = 1; q < 4; ++q) v += s_part[q][i][lane];
+      for (int q = 1; q < KW; ++q) v += s_part[q][i][lane];
       const uint32_t row = 4 * g + i;
       if (row < m && col < n) {
         if (bias) v += __half2float(bias[col]);
@@ -786,17 +786,18 @@ static int32_t gemv_dispatch(krm_ctx* ctx, krm_buf x, krm_buf w, krm_buf scales,
       uint32_t group_shift = 0;
       while ((1u << group_shift) < group) ++group_shift;
       const uint32_t blocks = (n + 15) / 16;
-#define KRM_MFMA_GEMV(ST, CH)                                                                  \
-  gemv_i4_mfma_kernel<ST, CH><<<dim3(blocks), dim3(256), 0, ctx->stream>>>(                    \
+#define KRM_MFMA_GEMV(ST, CH, KW)                                                              \
+  gemv_i4_mfma_kernel<ST, CH, KW><<<dim3(blocks), dim3(KW * 64), 0, ctx->stream>>>(            \
       ptr<const __half>(x), ptr<const uint32_t>(w), ptr<const ST>(scales),                     \
       ptr<const __half>(bias), ptr<__half>(out), m, n, k, group_shift)
-#define KRM_MFMA_GEMV_BY_K(ST)                      \
-  switch (k / 1024) {                               \
-    case 1: KRM_MFMA_GEMV(ST, 1); break;            \
-    case 2: KRM_MFMA_GEMV(ST, 2); break;            \
-    case 4: KRM_MFMA_GEMV(ST, 4); break;            \
-    case 8: KRM_MFMA_GEMV(ST, 8); break;            \
-    default: KRM_MFMA_GEMV(ST, 0); break;           \
+  // eight waves a workgroup (two per SIMD) when K gives each at least one chunk
+#define KRM_MFMA_GEMV_BY_K(ST)                         \
+  switch (k / 1024) {                                  \
+    case 1: KRM_MFMA_GEMV(ST, 1, 4); break;            \
+    case 2: KRM_MFMA_GEMV(ST, 1, 8); break;            \
+    case 4: KRM_MFMA_GEMV(ST, 2, 8); break;            \
+    case 8: KRM_MFMA_GEMV(ST, 4, 8); break;            \
+    default: KRM_MFMA_GEMV(ST, 0, 4); break;           \
   }
       if (scale_dtype == KRM_F16) {
         KRM_MFMA_GEMV_BY_K(__half)
