@@ -154,6 +154,25 @@ def test_linear_batched_rows_equal_single_rows_bitwise(gpu_ctx, io):
     assert np.max(np.abs(batched.astype(np.float32) - want)) <= tol
 
 
+@pytest.mark.parametrize("m,n,k,g,scale_f16,with_bias", [
+    (2, 16, 1024, 128, True, False), (16, 4096, 4096, 128, True, True),
+    (7, 100, 2048, 128, False, True), (16, 33, 8192, 256, True, False),
+    (3, 250, 3072, 128, True, True), (16, 64, 5120, 1024, False, False)])
+def test_batched_fp16_rows_on_matrix_cores_match_oracle(gpu_ctx, m, n, k, g, scale_f16, with_bias):
+    """2..16 fp16 rows take the MFMA kernel (K a multiple of 1024, group >= 128): ragged N,
+    every compile-time chunk count and the loop form (K = 3072, 5120), group sizes up to
+    1024, f32 and fp16 scales, bias.  Gate: the oracle's f32 result rounded to fp16, one ulp."""
+    rng = np.random.default_rng(m * 1000 + n)
+    packed, _q, scale = helpers.synthetic_int4(rng, n, k, g, scale_f16=scale_f16)
+    x = rng.normal(size=(m, k)).astype(np.float16)
+    bias = rng.normal(size=n).astype(np.float16) if with_bias else None
+    got = run_linear(gpu_ctx, x, packed, scale, bias, n, k, g)
+    want = oracle.linear_i4(x.astype(np.float32), packed, scale.astype(np.float32),
+                            (bias if with_bias else np.zeros(n)).astype(np.float32), n, k, g)
+    err = np.abs(got.astype(np.float32) - want)
+    assert np.all(err <= 2.0 ** -10 * np.abs(want) + 4e-5), float(err.max())
+
+
 @pytest.mark.parametrize("shape", [(1, 256, 2048, 128), (3, 2048, 5632, 128), (1, 100, 11008, 128),
                                    (7, 33, 96, 32), (2, 5, 64, 16), (16, 32000, 2048, 128)])
 def test_linear_shapes_of_the_decoder(gpu_ctx, shape):
