@@ -28,7 +28,7 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
 # HBM bytes per config-0 GEMV launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled
 # by an 8 MiB copy kernel's readings (profiles/gemv_i4_config0_pmc_traffic.txt).
-GEMV_PMC_TRAFFIC_BYTES = 8_797_800
+GEMV_PMC_TRAFFIC_BYTES = 8_816_800
 USE_GRAPHS = True       # --no-graph: plain launches (rocprofv3's kernel trace crashes on graph launches)
 
 
