@@ -182,15 +182,16 @@ void gemm_i4_f16_kernel(const XT* __restrict__ x, const uint32_t* __restrict__ w
   __shared__ __attribute__((aligned(16))) unsigned char lds_other[PIPE ? kStageBytes : 16];
   constexpr int kOffB = BM * kRowBytes;
 
-  // Workgroups that share an x panel are placed on one XCD (ids are dealt round-robin over 8
-  // XCDs), so that panel stays in that XCD's L2 while the weights stream through.
+  // Workgroup ids are dealt round-robin over the 8 XCDs, each with its own L2.  The row panels
+  // of one column block get consecutive slots of ONE XCD, so its weights cross the fabric once
+  // and the other panels find them in that L2 (x, the smaller operand, is re-read instead).
   uint32_t mb, nb;
   {
     const uint32_t id = blockIdx.x;
     if (8 % m_blocks == 0) {
-      const uint32_t xcd = id & 7, slot = id >> 3, per = 8 / m_blocks;
-      mb = xcd % m_blocks;
-      nb = slot * per + xcd / m_blocks;
+      const uint32_t xcd = id & 7, slot = id >> 3;
+      mb = slot % m_blocks;
+      nb = (slot / m_blocks) * 8 + xcd;
     } else {
       mb = id % m_blocks;
       nb = id / m_blocks;
@@ -472,8 +473,7 @@ int32_t launch(krm_ctx* ctx, krm_buf x, krm_buf w, krm_buf scales, krm_buf bias,
   const uint32_t m_blocks = (m + BM - 1) / BM, n_blocks = (n + BN - 1) / BN;
   uint64_t total;
   if (8 % m_blocks == 0) {
-    const uint32_t per = 8 / m_blocks;
-    total = (uint64_t)((n_blocks + per - 1) / per) * 8;
+    total = (uint64_t)((n_blocks + 7) / 8) * 8 * m_blocks;
   } else {
     total = (uint64_t)m_blocks * n_blocks;
   }
