@@ -234,8 +234,42 @@ def cpu_baseline(n: int, k: int, g: int, budget_s: float = 12.0):
     dt = time.perf_counter() - t0
     algo = n * k // 2 + n * (k // g) * 2 + k * 2 + n * 2
     cores = int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1))
-    return {"value": algo * reps / dt / 1e9, "unit": "GB/s", "cores": cores, "kind": "port",
-            "sample": f"{reps} repetitions of the config-0 GEMV (M=1,K=N=4096) in {dt:.1f} s"}
+    result = {"value": algo * reps / dt / 1e9, "unit": "GB/s", "cores": cores, "kind": "port",
+              "sample": f"{reps} repetitions of the config-0 GEMV (M=1,K=N=4096) in {dt:.1f} s"}
+    result.update(cpu_decode_baseline(g))
+    return result
+
+
+def cpu_decode_baseline(g: int, tokens: int = 3):
+    """Decode tokens/s of the 1.1B-shape model (config 4) on the host cores, from the oracle's
+    linear over the eight weight shapes of one decode step (the linears are all but a few
+    thousandths of a step's arithmetic): one layer's seven projections x 22 layers + lm_head."""
+    from oracle import oracle
+    from karume_amd.decoder import LlamaConfig
+
+    c = LlamaConfig()
+    d, hd, kvd = c.d_model, c.heads * c.head_dim, c.kv_heads * c.head_dim
+    shapes = [(hd, d), (kvd, d), (kvd, d), (d, hd), (c.ffn, d), (c.ffn, d), (d, c.ffn)]
+    rng = np.random.default_rng(2)
+    ops = {}
+    for n, k in set(shapes + [(c.vocab, d)]):
+        ops[(n, k)] = (rng.integers(0, 256, size=n * k // 2, dtype=np.uint8),
+                       np.abs(rng.normal(0, 0.02, size=(n, k // g))).astype(np.float32),
+                       rng.normal(size=(1, k)).astype(np.float32), np.zeros(n, dtype=np.float32))
+
+    def step():
+        for n, k in shapes * c.layers + [(c.vocab, d)]:
+            packed, scale, x, bias = ops[(n, k)]
+            oracle.linear_i4(x, packed, scale, bias, n, k, g)
+
+    step()  # warm
+    t0 = time.perf_counter()
+    for _ in range(tokens):
+        step()
+    dt = (time.perf_counter() - t0) / tokens
+    return {"decode_tokens_per_s": round(1.0 / dt, 2),
+            "decode_sample": f"{tokens} decode steps' linears (config 4: 22 layers x 7 projections "
+                             f"+ lm_head, int4 g{g}) through the oracle, {dt * 1e3:.0f} ms each"}
 
 
 def main() -> int:
