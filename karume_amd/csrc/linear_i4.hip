@@ -426,7 +426,9 @@ constexpr bool share_x_in_lds() {
   return sizeof(XT) == 4 && MB == 1 && NSTEP > 0 && NSTEP <= 4;
 }
 
-template <typename XT, typename ST, int MB, int ROWS, int VEC, int NSTEP, bool NORM>
+// NORM and DECODE_ROW are compile-time so that the plain kernel carries neither their branches
+// nor their registers (a run-time test at the top of the kernel cost the plain GEMV 8 %).
+template <typename XT, typename ST, int MB, int ROWS, int VEC, int NSTEP, bool NORM, bool DECODE_ROW>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 4))) void gemv_i4_kernel(
     const XT* __restrict__ x, const uint32_t* __restrict__ w, const ST* __restrict__ scales,
     const XT* __restrict__ bias, XT* __restrict__ out, uint32_t m, uint32_t n, uint32_t k,
@@ -460,6 +462,29 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 4))) voi
     squares[b] = 0.f;
 #pragma unroll
     for (int r = 0; r < ROWS; ++r) acc[r][b] = 0.f;
+  }
+
+  // Decode-row epilogue: the rotation's table entries are requested now, so that they arrive
+  // with the weights instead of after the reductions.
+  float rope_cos[ROWS / 2 > 0 ? ROWS / 2 : 1][2], rope_sin[ROWS / 2 > 0 ? ROWS / 2 : 1][2];
+  bool rope_in_table = false;
+  if constexpr (DECODE_ROW) {
+    {
+      const uint32_t half = fuse.depth >> 1;
+      const uint32_t rope_pairs = (fuse.heads + fuse.kv_heads) * half;
+      const int32_t pos = fuse.positions[0];
+      rope_in_table = pos >= 0 && (uint32_t)pos < fuse.table_rows;
+#pragma unroll
+      for (int p = 0; p < ROWS / 2; ++p) {
+        const uint32_t pair = (row0 >> 1) + p;
+        const bool rotates = rope_in_table && pair < rope_pairs;
+        const size_t t = rotates ? (size_t)pos * fuse.depth + pair % half : 0;
+        rope_cos[p][0] = fuse.cos_table[t];
+        rope_sin[p][0] = fuse.sin_table[t];
+        rope_cos[p][1] = fuse.cos_table[rotates ? t + half : 0];
+        rope_sin[p][1] = fuse.sin_table[rotates ? t + half : 0];
+      }
+    }
   }
 
   // Lanes past the end of K (last step of a K that is not a multiple of the step) read the
@@ -622,7 +647,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 4))) voi
       }
       return;
     }
-    if (fuse.positions) {
+    if constexpr (DECODE_ROW) {
       const uint32_t half = fuse.depth >> 1;
       const uint32_t rope_pairs = (fuse.heads + fuse.kv_heads) * half;
       uint32_t past = fuse.past;
@@ -634,8 +659,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 4))) voi
         if (!append && row0 == 0 && lane == 0) fuse.lengths[2] = 1u;
       }
       const uint64_t prow = fuse.window ? (uint64_t)past % fuse.window : (uint64_t)past;
-      const int32_t pos = fuse.positions[0];
-      const bool in_table = pos >= 0 && (uint32_t)pos < fuse.table_rows;
+      const bool in_table = rope_in_table;
 #pragma unroll
       for (int p = 0; p < ROWS / 2; ++p) {
         const uint32_t row = row0 + 2 * p, pair = row >> 1;
@@ -653,10 +677,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 4))) voi
           const uint32_t head = pair / half, j = pair - head * half;
           float o0 = NAN, o1 = NAN;  // a position outside the table is never a valid rotation
           if (in_table) {
-            const size_t t = (size_t)pos * fuse.depth + j;
-            o0 = __fadd_rn(__fmul_rn(x0, fuse.cos_table[t]), __fmul_rn(-x1, fuse.sin_table[t]));
-            o1 = __fadd_rn(__fmul_rn(x1, fuse.cos_table[t + half]),
-                           __fmul_rn(x0, fuse.sin_table[t + half]));
+            o0 = __fadd_rn(__fmul_rn(x0, rope_cos[p][0]), __fmul_rn(-x1, rope_sin[p][0]));
+            o1 = __fadd_rn(__fmul_rn(x1, rope_cos[p][1]), __fmul_rn(x0, rope_sin[p][1]));
           }
           const size_t at = (size_t)head * fuse.depth + j;
           out[at] = from_f32<XT>(o0);
@@ -703,14 +725,20 @@ int32_t launch_gemv(krm_ctx* ctx, krm_buf x, krm_buf w, krm_buf scales, krm_buf 
                     const GemvFusion& fuse = GemvFusion{}) {
   const uint32_t rows_per_block = 4 * ROWS;
   const uint32_t blocks = (n + rows_per_block - 1) / rows_per_block;
-  if (fuse.norm_weight)
-    gemv_i4_kernel<XT, ST, MB, ROWS, VEC, NSTEP, true><<<dim3(blocks), dim3(256), 0, ctx->stream>>>(
-        ptr<const XT>(x), ptr<const uint32_t>(w), ptr<const ST>(scales), ptr<const XT>(bias),
-        ptr<XT>(out), m, n, k, group_shift, fuse);
-  else
-    gemv_i4_kernel<XT, ST, MB, ROWS, VEC, NSTEP, false><<<dim3(blocks), dim3(256), 0, ctx->stream>>>(
-        ptr<const XT>(x), ptr<const uint32_t>(w), ptr<const ST>(scales), ptr<const XT>(bias),
-        ptr<XT>(out), m, n, k, group_shift, fuse);
+#define KRM_GEMV_LAUNCH(NORM, ROW)                                                              \
+  gemv_i4_kernel<XT, ST, MB, ROWS, VEC, NSTEP, NORM, ROW>                                       \
+      <<<dim3(blocks), dim3(256), 0, ctx->stream>>>(ptr<const XT>(x), ptr<const uint32_t>(w),  \
+                                                    ptr<const ST>(scales), ptr<const XT>(bias), \
+                                                    ptr<XT>(out), m, n, k, group_shift, fuse)
+  if constexpr (MB == 1 && ROWS % 2 == 0) {
+    if (fuse.positions) {
+      if (fuse.norm_weight) KRM_GEMV_LAUNCH(true, true); else KRM_GEMV_LAUNCH(false, true);
+      return launched(ctx, "gemv_i4_kernel");
+    }
+  }
+  if (fuse.positions) return fail(ctx, KRM_ERR_VALIDATION, "decode row: one row, even row count");
+  if (fuse.norm_weight) KRM_GEMV_LAUNCH(true, false); else KRM_GEMV_LAUNCH(false, false);
+#undef KRM_GEMV_LAUNCH
   return launched(ctx, "gemv_i4_kernel");
 }
 
