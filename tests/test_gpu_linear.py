@@ -251,3 +251,40 @@ def test_linear_fused_decode_forms(gpu_ctx):
         gpu_ctx.linear_i4_fused(buf, buf, buf, buf, 1, 63, 128, 128,
                                 epilogue=ka.EPILOGUE_SILU_PAIRS)
     buf.free()
+
+
+def test_linear_from_a_model_file(gpu_ctx):
+    """File -> reader -> device: an int4 `linear` weight written as an I4 tensor with its F32
+    group scale is handed to the kernel as the reader's views of the file (no re-packing) and
+    must match the oracle run on the same bytes.  Gate as in the reference cases above."""
+    import json
+    from karume_amd.format_model import (build_safetensors, i4_resident_initializers, open_model,
+                                         packed_int4)
+    rng = np.random.default_rng(11)
+    n, k, g, m = 96, 512, 64, 3
+    q = rng.integers(-8, 8, size=(n, k), dtype=np.int8)
+    scale = rng.uniform(0.005, 0.05, size=(n, k // g)).astype(np.float32)
+    bias = rng.normal(size=n).astype(np.float32)
+    graph = {
+        "format": "karume-ir", "version": 1, "requires": {"ops": ["linear"]}, "symbols": [],
+        "inputs": [{"name": "x", "dtype": "f32", "shape": [m, k]}], "outputs": ["y"],
+        "initializers": {
+            "w": {"tensor": "proj.weight",
+                  "storage": {"dtype": "i4", "scale": "karume.scale.proj.weight", "group_size": g}},
+            "b": {"tensor": "proj.bias", "storage": {"dtype": "f32"}}},
+        "values": {"w": {"dtype": "f32", "shape": [n, k]}, "b": {"dtype": "f32", "shape": [n]},
+                   "y": {"dtype": "f32", "shape": [m, n]}},
+        "nodes": [{"op": "linear", "ins": ["x", "w", "b"], "outs": ["y"], "attrs": {}}]}
+    blob = build_safetensors(
+        [("karume.scale.proj.weight", "F32", [n, k // g], scale.tobytes()),
+         ("proj.bias", "F32", [n], bias.tobytes()),
+         ("proj.weight", "I4", [n, k], oracle.pack_i4(q).tobytes())],
+        {"karume_ir": json.dumps(graph)})
+    model = open_model(blob)
+    assert i4_resident_initializers(model) == {"w"}
+    weight = packed_int4(model, "w")
+    x = rng.normal(size=(m, k)).astype(np.float32)
+    want = oracle.linear_i4(x, weight.packed, weight.scales, bias, n, k, g)
+    got = run_linear(gpu_ctx, x, weight.packed, weight.scales, bias, n, k, g)
+    ok, fails, max_abs, worst = oracle.allclose(got, want, atol=1e-5, rtol=1e-3)
+    assert ok, (fails, max_abs, worst)
