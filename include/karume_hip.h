@@ -292,6 +292,33 @@ int32_t krm_decode_qkv(krm_ctx* ctx, krm_buf x, krm_buf norm_weight_f32, float n
                        uint32_t k, uint32_t group, uint32_t table_rows, uint32_t capacity,
                        uint32_t window, uint32_t past, krm_buf lengths, int32_t io_dtype,
                        int32_t scale_dtype, int32_t kv_dtype);
+/* ---- w4a8: `linear` with int4 weights on integer dot products (the reference's opt-in
+ *      SessionOptions.linearCompute "i8a8" with int4-resident weights,
+ *      packages/runtime/src/runtime/recipe-builder.ts:1320-1341,1407-1488;
+ *      contract docs/decisions/0076-w4a8-linear-execution.md:40-60) --------------------------
+ * Step 1, the activation quantiser (params {rows, dim} + bindings x, xq, xs:
+ * packages/runtime/src/kernels/quantize-rows.ts:89-146):
+ *   xs[row] = max(f32(max|x[row, :]| * f32(1/127)), f32 tiny); a NaN in the row makes it NaN
+ *   xq[row, i] = clamp(round-half-even(x[row, i] / xs[row]), -127, 127), int8, row-major
+ * x / xs is the correctly rounded division (the reference's WGSL division is not, and its
+ * codes may differ by one next to a tie; these never do).  A NaN quotient stores 0.
+ * Requires dim >= 1 and dim % 4 == 0 (quantize-rows.ts:160-173), x 16-byte aligned. */
+int32_t krm_quantize_rows(krm_ctx* ctx, krm_buf x_f32, krm_buf xq_i8, krm_buf xs_f32,
+                          uint32_t rows, uint32_t dim);
+/* Step 2, the product (params {m, n, k} + bindings xq, w, bias, out, scales, xs:
+ * packages/runtime/src/kernels/linear-i8a8.ts:47-72,376-510,589-625):
+ *   accf = 0; for each group gi ascending: accf = fma(f32(sum_group xq * wq), scales[col, gi], accf)
+ *   out[row, col] = fma(accf, xs[row], bias[col])
+ * the group sums are exact int32, every fma is fused and correctly rounded, so the result is
+ * bit-identical to packages/runtime/src/reference/i8a8.ts:209-231 evaluated with a fused
+ * multiply-add, for every tiling.
+ *   xq [m, k] int8, xs [m] f32 (from krm_quantize_rows), w [n, k] packed int4,
+ *   scales [n, k/group] scale_dtype, bias [n] f32 or 0 (= zeros), out [m, n] f32.
+ * Requires k > 0, k % 4 == 0 (recipe-builder.ts:1336-1338), group a power of two >= 16
+ * dividing k, group <= 2113664 (the int32 gate LINEAR_W4A8_MAX_GROUP, linear-i8a8.ts:124-132). */
+int32_t krm_linear_w4a8(krm_ctx* ctx, krm_buf xq_i8, krm_buf xs_f32, krm_buf w, krm_buf scales,
+                        krm_buf bias_f32, krm_buf out_f32, uint32_t m, uint32_t n, uint32_t k,
+                        uint32_t group, int32_t scale_dtype);
 /* [a, b, d] -> [b, a, d] (the reshape + permute between linears and attention). */
 int32_t krm_transpose_01(krm_ctx* ctx, krm_buf x, krm_buf out, uint32_t a, uint32_t b, uint32_t d,
                          int32_t io_dtype);

@@ -1,0 +1,352 @@
+// w4a8 `linear` for gfx950: per-token int8 activations x int4 group-quantised weights with
+// integer dot products.
+//
+// Semantics follow the reference's opt-in integer-dot path for int4-resident weights
+// (packages/runtime/src/kernels/quantize-rows.ts:89-146 for the activation quantiser,
+// packages/runtime/src/kernels/linear-i8a8.ts:47-72,376-510 for the product, contract
+// docs/decisions/0076-w4a8-linear-execution.md:40-60, CPU reference
+// packages/runtime/src/reference/i8a8.ts:92-118,209-231):
+//
+//   xs[row]  = max(f32(amax(|x[row]|) * f32(1/127)), f32 tiny)      NaN in the row -> NaN
+//   xq       = clamp(round-half-even(x / xs[row]), -127, +127)
+//   accf     = 0;  for each group gi of the row, ascending:
+//                acci = sum over the group of xq * wq               exact, int32
+//                accf = fma(f32(acci), wscale[col, gi], accf)       one rounding per group
+//   out      = fma(accf, xs[row], bias[col])
+//
+// Every floating-point operation is a correctly rounded IEEE operation in a fixed order, and
+// everything inside a group is exact integer arithmetic, so the result does not depend on how
+// a kernel tiles the problem: the kernels here differ in speed only and agree bit for bit with
+// each other and with the CPU statement of the formula.
+//
+// The weight nibbles are stored u = q + 8.  u ^ 8 is q's 4-bit two's complement, and a
+// two's-complement nibble in the upper half of a byte reads as the signed byte 16 * q; the
+// integer dot products therefore run on bytes 16 * q (two ops per four codes, no sign
+// extension) and the exact factor 16 is shifted out of the group sum before it is converted.
+#include "krm_internal.h"
+
+namespace {
+
+using namespace krm;
+
+typedef int v4i_t __attribute__((ext_vector_type(4)));
+typedef int v16i_t __attribute__((ext_vector_type(16)));
+
+constexpr float kF32Tiny = 1.1754943508222875e-38f;
+constexpr uint32_t kMaxGroup = 2113664;      // int32 holds g * 127 * 8 (linear-i8a8.ts:124-132)
+constexpr uint32_t kMaxGroupTimes16 = 131072;  // int32 holds g * 127 * 8 * 16
+
+template <typename ST>
+__device__ inline float scale_f32(const ST* s, size_t i);
+template <>
+__device__ inline float scale_f32<float>(const float* s, size_t i) { return s[i]; }
+template <>
+__device__ inline float scale_f32<__half>(const __half* s, size_t i) { return __half2float(s[i]); }
+
+__device__ inline bool is_nan_bits(float v) {
+  return (__float_as_uint(v) & 0x7fffffffu) > 0x7f800000u;
+}
+
+// ------------------------------------------------------------------------- quantize_rows
+//
+// One workgroup per row (grid-stride over rows), two passes over the row: |x| maximum with NaN
+// propagation, then the quotients.  x / s is the correctly rounded f32 division, so the codes
+// equal the CPU formula's for every input, also next to a rounding tie.
+__global__ __launch_bounds__(256) void quantize_rows_kernel(const float* __restrict__ x,
+                                                            uint32_t* __restrict__ xq,
+                                                            float* __restrict__ xs,
+                                                            uint32_t rows, uint32_t dim) {
+  __shared__ float s_max[4];
+  __shared__ uint32_t s_nan[4];
+  const uint32_t quads = dim >> 2;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  for (uint32_t row = blockIdx.x; row < rows; row += gridDim.x) {
+    const float4* xr = reinterpret_cast<const float4*>(x + (size_t)row * dim);
+    float amax = 0.f;
+    bool nan = false;
+    for (uint32_t i = threadIdx.x; i < quads; i += 256) {
+      const float4 v = xr[i];
+      const float a[4] = {fabsf(v.x), fabsf(v.y), fabsf(v.z), fabsf(v.w)};
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        nan = nan || is_nan_bits(a[e]);
+        amax = fmaxf(amax, a[e]);  // ignores a NaN operand; the flag carries it
+      }
+    }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) amax = fmaxf(amax, __shfl_xor(amax, off));
+    const bool wave_nan = __any(nan);
+    if (lane == 0) {
+      s_max[wave] = amax;
+      s_nan[wave] = wave_nan ? 1u : 0u;
+    }
+    __syncthreads();
+    amax = fmaxf(fmaxf(s_max[0], s_max[1]), fmaxf(s_max[2], s_max[3]));
+    const bool row_nan = (s_nan[0] | s_nan[1] | s_nan[2] | s_nan[3]) != 0u;
+    float s = fmaxf(amax * (float)(1.0 / 127.0), kF32Tiny);
+    if (row_nan) s = __uint_as_float(0x7fc00000u);
+    if (threadIdx.x == 0) xs[row] = s;
+    uint32_t* qr = xq + (size_t)row * quads;
+    for (uint32_t i = threadIdx.x; i < quads; i += 256) {
+      const float4 v = xr[i];
+      const float f[4] = {v.x, v.y, v.z, v.w};
+      uint32_t packed = 0;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        float r = rintf(f[e] / s);
+        r = is_nan_bits(r) ? 0.f : fminf(fmaxf(r, -127.f), 127.f);
+        packed |= ((uint32_t)(int32_t)r & 0xffu) << (8 * e);
+      }
+      qr[i] = packed;
+    }
+    __syncthreads();  // s_max / s_nan are rewritten by the next row
+  }
+}
+
+// ------------------------------------------------------------------- any shape (fallback)
+//
+// One wave per output column, one x row at a time; the lanes share the words of a group and
+// add their exact partial sums.  Covers every group size the format allows; the kernels below
+// take the shapes that matter for speed.
+template <typename ST>
+__global__ __launch_bounds__(256) void linear_w4a8_generic_kernel(
+    const uint32_t* __restrict__ xq, const float* __restrict__ xs, const uint32_t* __restrict__ w,
+    const ST* __restrict__ scales, const float* __restrict__ bias, float* __restrict__ out,
+    uint32_t m, uint32_t n, uint32_t k, uint32_t group) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const uint32_t col = blockIdx.x * 4 + wave;
+  if (col >= n) return;
+  const uint32_t words_per_group = group >> 3, groups = k / group;
+  const uint32_t* wrow = w + (size_t)col * (k >> 3);
+  for (uint32_t row = blockIdx.y; row < m; row += gridDim.y) {
+    const uint32_t* xrow = xq + (size_t)row * (k >> 2);
+    float accf = 0.f;
+    for (uint32_t gi = 0; gi < groups; ++gi) {
+      int32_t acci = 0;
+      for (uint32_t j = lane; j < words_per_group; j += 64) {
+        const uint32_t word = wrow[(size_t)gi * words_per_group + j];
+        const uint32_t x0 = xrow[((size_t)gi * group >> 2) + 2 * j];
+        const uint32_t x1 = xrow[((size_t)gi * group >> 2) + 2 * j + 1];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          const int32_t q = (int32_t)((word >> (4 * e)) & 15u) - 8;
+          const int32_t xv = (int32_t)(int8_t)(((e < 4 ? x0 : x1) >> (8 * (e & 3))) & 0xffu);
+          acci += q * xv;
+        }
+      }
+#pragma unroll
+      for (int off = 32; off > 0; off >>= 1) acci += __shfl_xor(acci, off);
+      accf = fmaf((float)acci, scale_f32<ST>(scales, (size_t)col * groups + gi), accf);
+    }
+    if (lane == 0) out[(size_t)row * n + col] = fmaf(accf, xs[row], bias ? bias[col] : 0.f);
+  }
+}
+
+// --------------------------------------------------------------- few rows of x (decode)
+//
+// Weight-streaming form for M <= 8 and 32 <= group <= 2048.  A wave owns two weight rows over
+// the whole K and MB rows of x; a step is 64 lanes x 16 bytes = 2048 codes per weight row, a
+// lane's 32 codes lie inside one group.  Per word: u ^ 8 once, the odd codes are the upper
+// nibbles in place, the even codes one shift away; x's bytes are regrouped (even, odd) to
+// match and two v_dot4_i32_i8 add eight products.  The lanes of a group add their sums
+// (exact), the group totals and scales go through LDS to one lane per output, which runs the
+// ascending fma chain.
+template <typename ST, int MB>
+__global__ __launch_bounds__(256) void linear_w4a8_rows_kernel(
+    const uint32_t* __restrict__ xq, const float* __restrict__ xs, const uint32_t* __restrict__ w,
+    const ST* __restrict__ scales, const float* __restrict__ bias, float* __restrict__ out,
+    uint32_t m, uint32_t n, uint32_t k, uint32_t group_shift) {
+  constexpr int ROWS = 2;
+  constexpr int kStep = 64 * 32;
+  __shared__ int32_t s_sum[4][ROWS * MB][64];
+  __shared__ float s_ws[4][ROWS][64];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const uint32_t row0 = (blockIdx.x * 4 + wave) * ROWS;
+  const uint32_t b0 = blockIdx.y * MB;
+  const uint32_t span = 1u << (group_shift - 5);  // lanes per group
+  const uint32_t per_step = 64u / span;           // groups per step
+  const uint32_t groups = k >> group_shift;
+  const uint32_t steps = (k + kStep - 1) / kStep;
+
+  const uint32_t* wrow[ROWS];
+  const ST* srow[ROWS];
+#pragma unroll
+  for (int r = 0; r < ROWS; ++r) {
+    const uint32_t row = min(row0 + r, n - 1);  // rows past N re-read the last row, unused
+    wrow[r] = w + (size_t)row * (k >> 3);
+    srow[r] = scales + (size_t)row * groups;
+  }
+  const uint32_t* xrow[MB];
+#pragma unroll
+  for (int b = 0; b < MB; ++b) xrow[b] = xq + (size_t)min(b0 + b, m - 1) * (k >> 2);
+
+  struct Step {
+    uint4 w[ROWS];
+    float s[ROWS];
+    uint4 x[MB][2];
+  };
+  // requests only; lanes past the end of K re-read the row's start and are masked later
+  auto fetch = [&](uint32_t step, Step& d) {
+    const uint32_t k0 = step * kStep + lane * 32;
+    const uint32_t kc = k0 < k ? k0 : 0u;
+#pragma unroll
+    for (int r = 0; r < ROWS; ++r) {
+      d.w[r] = *reinterpret_cast<const uint4*>(wrow[r] + (kc >> 3));
+      d.s[r] = scale_f32<ST>(srow[r], kc >> group_shift);
+    }
+#pragma unroll
+    for (int b = 0; b < MB; ++b) {
+      d.x[b][0] = *reinterpret_cast<const uint4*>(xrow[b] + (kc >> 2));
+      d.x[b][1] = *reinterpret_cast<const uint4*>(xrow[b] + (kc >> 2) + 4);
+    }
+  };
+
+  const int chain_r = lane / MB, chain_b = lane % MB;  // the output a chain lane owns
+  const bool chain = lane < ROWS * MB;
+  float accf = 0.f;
+
+  Step cur, nxt;
+  fetch(0, cur);
+  for (uint32_t step = 0; step < steps; ++step) {
+    if (step + 1 < steps) fetch(step + 1, nxt);
+    const bool active = step * kStep + lane * 32 < k;
+    int32_t acc[ROWS][MB];
+#pragma unroll
+    for (int r = 0; r < ROWS; ++r)
+#pragma unroll
+      for (int b = 0; b < MB; ++b) acc[r][b] = 0;
+    uint32_t hi[ROWS][4], lo[ROWS][4];
+#pragma unroll
+    for (int r = 0; r < ROWS; ++r) {
+      const uint32_t words[4] = {cur.w[r].x, cur.w[r].y, cur.w[r].z, cur.w[r].w};
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const uint32_t t = words[j] ^ 0x88888888u;
+        hi[r][j] = t & 0xF0F0F0F0u;          // bytes 16 * q of codes 1, 3, 5, 7
+        lo[r][j] = (t << 4) & 0xF0F0F0F0u;   // bytes 16 * q of codes 0, 2, 4, 6
+      }
+    }
+#pragma unroll
+    for (int b = 0; b < MB; ++b) {
+      const uint32_t xw[8] = {cur.x[b][0].x, cur.x[b][0].y, cur.x[b][0].z, cur.x[b][0].w,
+                              cur.x[b][1].x, cur.x[b][1].y, cur.x[b][1].z, cur.x[b][1].w};
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const uint32_t even = __builtin_amdgcn_perm(xw[2 * j + 1], xw[2 * j], 0x06040200u);
+        const uint32_t odd = __builtin_amdgcn_perm(xw[2 * j + 1], xw[2 * j], 0x07050301u);
+#pragma unroll
+        for (int r = 0; r < ROWS; ++r) {
+          acc[r][b] = __builtin_amdgcn_sdot4((int)lo[r][j], (int)even, acc[r][b], false);
+          acc[r][b] = __builtin_amdgcn_sdot4((int)hi[r][j], (int)odd, acc[r][b], false);
+        }
+      }
+    }
+#pragma unroll
+    for (int r = 0; r < ROWS; ++r)
+#pragma unroll
+      for (int b = 0; b < MB; ++b) {
+        int32_t v = active ? acc[r][b] : 0;
+        for (uint32_t off = 1; off < span; off <<= 1) v += __shfl_xor(v, (int)off);
+        acc[r][b] = v;
+      }
+    if ((lane & (span - 1)) == 0) {
+      const uint32_t slot = lane >> (group_shift - 5);
+#pragma unroll
+      for (int r = 0; r < ROWS; ++r) {
+        s_ws[wave][r][slot] = cur.s[r];
+#pragma unroll
+        for (int b = 0; b < MB; ++b) s_sum[wave][r * MB + b][slot] = acc[r][b];
+      }
+    }
+    __syncthreads();
+    if (chain) {
+      const uint32_t first = step * per_step;
+      const uint32_t count = groups - first < per_step ? groups - first : per_step;
+      for (uint32_t j = 0; j < count; ++j)
+        accf = fmaf((float)(s_sum[wave][lane][j] >> 4), s_ws[wave][chain_r][j], accf);
+    }
+    __syncthreads();
+    cur = nxt;
+  }
+  if (chain) {
+    const uint32_t row = row0 + chain_r, xb = b0 + chain_b;
+    if (row < n && xb < m)
+      out[(size_t)xb * n + row] = fmaf(accf, xs[xb], bias ? bias[row] : 0.f);
+  }
+}
+
+template <typename ST>
+int32_t launch_w4a8(krm_ctx* ctx, krm_buf xq, krm_buf xs, krm_buf w, krm_buf scales,
+                    krm_buf bias, krm_buf out, uint32_t m, uint32_t n, uint32_t k,
+                    uint32_t group) {
+  const uint32_t* pxq = ptr<const uint32_t>(xq);
+  const float* pxs = ptr<const float>(xs);
+  const uint32_t* pw = ptr<const uint32_t>(w);
+  const ST* ps = ptr<const ST>(scales);
+  const float* pb = ptr<const float>(bias);
+  float* po = ptr<float>(out);
+  uint32_t shift = 0;
+  while ((1u << shift) < group) ++shift;
+  const bool rows_form = group >= 32 && group <= 2048 && m <= 8 && aligned(xq, 16) &&
+                         aligned(w, 16);
+  if (rows_form) {
+    const dim3 grid((n + 7) / 8, m <= 1 ? 1 : m <= 2 ? 1 : (m + 3) / 4);
+    if (m <= 1)
+      hipLaunchKernelGGL((linear_w4a8_rows_kernel<ST, 1>), grid, dim3(256), 0, ctx->stream, pxq,
+                         pxs, pw, ps, pb, po, m, n, k, shift);
+    else if (m <= 2)
+      hipLaunchKernelGGL((linear_w4a8_rows_kernel<ST, 2>), grid, dim3(256), 0, ctx->stream, pxq,
+                         pxs, pw, ps, pb, po, m, n, k, shift);
+    else
+      hipLaunchKernelGGL((linear_w4a8_rows_kernel<ST, 4>), grid, dim3(256), 0, ctx->stream, pxq,
+                         pxs, pw, ps, pb, po, m, n, k, shift);
+    return launched(ctx, "linear_w4a8_rows_kernel");
+  }
+  const dim3 grid((n + 3) / 4, m < 65535u ? m : 65535u);
+  hipLaunchKernelGGL((linear_w4a8_generic_kernel<ST>), grid, dim3(256), 0, ctx->stream, pxq, pxs,
+                     pw, ps, pb, po, m, n, k, group);
+  return launched(ctx, "linear_w4a8_generic_kernel");
+}
+
+}  // namespace
+
+extern "C" int32_t krm_quantize_rows(krm_ctx* ctx, krm_buf x, krm_buf xq, krm_buf xs,
+                                     uint32_t rows, uint32_t dim) {
+  KRM_TRY(enter(ctx));
+  KRM_REQUIRE(ctx, dim >= 1, "quantize_rows: dim must be positive (%u)", dim);
+  KRM_REQUIRE(ctx, dim % 4 == 0, "quantize_rows: dim must be a multiple of 4 (%u)", dim);
+  if (rows == 0) return KRM_OK;
+  KRM_REQUIRE(ctx, x && xq && xs, "quantize_rows: null buffer");
+  KRM_REQUIRE(ctx, aligned(x, 16) && aligned(xq, 4) && aligned(xs, 4),
+              "quantize_rows: x needs 16-byte, xq and xs 4-byte alignment");
+  const uint32_t blocks = rows < (1u << 16) ? rows : (1u << 16);
+  hipLaunchKernelGGL(quantize_rows_kernel, dim3(blocks), dim3(256), 0, ctx->stream,
+                     krm::ptr<const float>(x), krm::ptr<uint32_t>(xq), krm::ptr<float>(xs), rows,
+                     dim);
+  return krm::launched(ctx, "quantize_rows_kernel");
+}
+
+extern "C" int32_t krm_linear_w4a8(krm_ctx* ctx, krm_buf xq, krm_buf xs, krm_buf w,
+                                   krm_buf scales, krm_buf bias, krm_buf out, uint32_t m,
+                                   uint32_t n, uint32_t k, uint32_t group, int32_t scale_dtype) {
+  KRM_TRY(enter(ctx));
+  KRM_REQUIRE(ctx, krm::valid_dtype(scale_dtype), "linear w4a8: unknown scale dtype %d",
+              scale_dtype);
+  KRM_REQUIRE(ctx, k > 0 && k % 4 == 0, "linear w4a8: k must be a positive multiple of 4 (%u)", k);
+  KRM_REQUIRE(ctx, krm::is_pow2(group) && group >= 16,
+              "linear w4a8: group_size %u is not a power of two >= 16", group);
+  KRM_REQUIRE(ctx, k % group == 0, "linear w4a8: k=%u is not a multiple of group_size %u", k,
+              group);
+  KRM_REQUIRE(ctx, group <= kMaxGroup,
+              "linear w4a8: group_size %u exceeds the int32 reduction limit %u", group, kMaxGroup);
+  if (m == 0 || n == 0) return KRM_OK;
+  KRM_REQUIRE(ctx, xq && xs && w && scales && out, "linear w4a8: null buffer");
+  KRM_REQUIRE(ctx, krm::aligned(xq, 4) && krm::aligned(xs, 4) && krm::aligned(w, 4) &&
+                       krm::aligned(out, 4) && krm::aligned(bias, 4) &&
+                       krm::aligned(scales, krm::dtype_bytes(scale_dtype)),
+              "linear w4a8: misaligned buffer");
+  (void)kMaxGroupTimes16;
+  if (scale_dtype == KRM_F16)
+    return launch_w4a8<__half>(ctx, xq, xs, w, scales, bias, out, m, n, k, group);
+  return launch_w4a8<float>(ctx, xq, xs, w, scales, bias, out, m, n, k, group);
+}

@@ -263,6 +263,18 @@ class GpuContext:
             _addr(bias), _addr(residual), _addr(out), m, n, k, group, io_dtype, scale_dtype,
             epilogue))
 
+    def quantize_rows(self, x_f32: BufferLike, xq_i8: BufferLike, xs_f32: BufferLike, rows: int,
+                      dim: int) -> None:
+        self._check(self._lib.krm_quantize_rows(self._handle, _addr(x_f32), _addr(xq_i8),
+                                                _addr(xs_f32), rows, dim))
+
+    def linear_w4a8(self, xq_i8: BufferLike, xs_f32: BufferLike, w: BufferLike,
+                    scales: BufferLike, bias_f32: BufferLike, out_f32: BufferLike, m: int, n: int,
+                    k: int, group: int, scale_dtype: int = F32) -> None:
+        self._check(self._lib.krm_linear_w4a8(self._handle, _addr(xq_i8), _addr(xs_f32), _addr(w),
+                                              _addr(scales), _addr(bias_f32), _addr(out_f32), m, n,
+                                              k, group, scale_dtype))
+
     def attention_state_workspace(self, batch: int, heads: int, kv_heads: int, chunk_rows: int,
                                   depth: int, window: int, max_past: int, max_query: int = 1
                                   ) -> int:

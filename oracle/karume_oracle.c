@@ -186,6 +186,114 @@ int krmo_linear_i4_mt(const float* x, const uint8_t* bytes, const float* scale,
 }
 
 /* ---------------------------------------------------------------------------------------
+ * w4a8: per-token int8 activations x int4 group-quantised weights, integer dot products.
+ * ------------------------------------------------------------------------------------- */
+
+/* Per-row (= per-token) symmetric int8 quantisation.
+ * packages/runtime/src/reference/i8a8.ts:92-118 (kernel: src/kernels/quantize-rows.ts:89-146):
+ *   amax = max |x| over the row, NaN propagates to the row's scale;
+ *   s    = max(f32(amax * f32(1/127)), f32 tiny)   -- a multiplication, never amax / 127;
+ *   q    = clamp(round-half-to-even(f32(x / s)), -127, +127).
+ * The JavaScript computes amax * (1/127) and x / s in double and rounds once to f32; both
+ * equal the IEEE f32 operation (the product of two f32 is exact in double, and a double
+ * quotient rounded to f32 is the correctly rounded f32 quotient), so plain float arithmetic
+ * is used here.  A NaN quotient (NaN or Inf scale) stores 0, like an Int8Array store. */
+void krmo_quantize_rows(const float* x, size_t rows, size_t dim, int8_t* q, float* scale) {
+  const float inv_abs_max = (float)(1.0 / 127.0);
+  const float tiny = 1.1754943508222875e-38f;
+  for (size_t row = 0; row < rows; ++row) {
+    const float* xr = x + row * dim;
+    float amax = 0.0f;
+    int saw_nan = 0;
+    for (size_t i = 0; i < dim; ++i) {
+      const float value = fabsf(xr[i]);
+      if (isnan(value)) saw_nan = 1;
+      else if (value > amax) amax = value;
+    }
+    float s = amax * inv_abs_max;
+    if (!(s > tiny)) s = tiny;  /* Math.max(s, tiny); s is never NaN here */
+    if (saw_nan) s = NAN;
+    scale[row] = s;
+    for (size_t i = 0; i < dim; ++i) {
+      float r = rintf(xr[i] / s);  /* default rounding mode: ties to even */
+      if (isnan(r)) r = 0.0f;
+      if (r > 127.0f) r = 127.0f;
+      if (r < -127.0f) r = -127.0f;
+      q[row * dim + i] = (int8_t)r;
+    }
+  }
+}
+
+/* Smallest distance of x / s from a half-integer over all finite quotients
+ * (packages/runtime/src/reference/i8a8.ts:129-146): data with a large margin quantises the
+ * same way under a division that is a few ulp off. */
+double krmo_quantize_rows_tie_margin(const float* x, size_t rows, size_t dim) {
+  double margin = INFINITY;
+  int8_t* q = (int8_t*)malloc((rows * dim) ? rows * dim : 1);
+  float* s = (float*)malloc(sizeof(float) * (rows ? rows : 1));
+  if (!q || !s) { free(q); free(s); return -1.0; }
+  krmo_quantize_rows(x, rows, dim, q, s);
+  for (size_t row = 0; row < rows; ++row)
+    for (size_t i = 0; i < dim; ++i) {
+      const float ratio = x[row * dim + i] / s[row];
+      if (!isfinite(ratio)) continue;
+      const double fraction = (double)ratio - floor((double)ratio);
+      const double d = fabs(fraction - 0.5);
+      if (d < margin) margin = d;
+    }
+  free(q);
+  free(s);
+  return margin;
+}
+
+/* w4a8 linear.  packages/runtime/src/reference/i8a8.ts:209-231 (contract:
+ * docs/decisions/0076-w4a8-linear-execution.md:40-60):
+ *   accf = 0;  for each group gi, ascending:
+ *       acci = sum over the group of xq[row, i] * wq[col, i]           exact integer
+ *       accf = fma(f32(acci), wscale[col, gi], accf)                   one rounding per group
+ *   out = fma(accf, xs[row], bias[col])
+ * The activation scale is applied once, last; groups are never merged into one integer sum.
+ * fused != 0: each fma is a true fused multiply-add (what the reference's GPU kernel
+ * executes).  fused == 0: the JavaScript reference's stand-in, (double)a * b + c rounded to
+ * f32 -- the product is exact in double; the sum is rounded twice, which can differ from the
+ * fused result only when the exact sum needs more than 53 bits.
+ * Weights are the packed int4 bytes (flat element i in byte i / 2, low nibble first, stored
+ * u = q + 8); `group` may be any divisor of k (the reference's known-answer cases use 2). */
+int krmo_linear_w4a8(const float* x, const uint8_t* bytes, const float* wscale,
+                     const float* bias, size_t m, size_t n, size_t k, size_t group, int fused,
+                     float* out) {
+  if (group < 1 || k % group != 0 || (n * k) % 2 != 0) return KRMO_ERR_SHAPE;
+  const size_t groups = k / group;
+  int8_t* q = (int8_t*)malloc((m * k) ? m * k : 1);
+  float* xs = (float*)malloc(sizeof(float) * (m ? m : 1));
+  if (!q || !xs) { free(q); free(xs); return KRMO_ERR_SHAPE; }
+  krmo_quantize_rows(x, m, k, q, xs);
+#pragma omp parallel for schedule(static)
+  for (long long col = 0; col < (long long)n; ++col) {
+    for (size_t row = 0; row < m; ++row) {
+      float accf = 0.0f;
+      for (size_t gi = 0; gi < groups; ++gi) {
+        int64_t acci = 0;
+        for (size_t i = gi * group; i < (gi + 1) * group; ++i) {
+          const size_t flat = (size_t)col * k + i;
+          const uint8_t byte = bytes[flat >> 1];
+          const int u = (flat & 1) ? (byte >> 4) : (byte & 0x0f);
+          acci += (int64_t)q[row * k + i] * (int64_t)(u - 8);
+        }
+        const float a = (float)acci, w = wscale[(size_t)col * groups + gi];
+        accf = fused ? fmaf(a, w, accf) : (float)((double)a * (double)w + (double)accf);
+      }
+      out[row * n + (size_t)col] =
+          fused ? fmaf(accf, xs[row], bias[col])
+                : (float)((double)accf * (double)xs[row] + (double)bias[col]);
+    }
+  }
+  free(q);
+  free(xs);
+  return KRMO_OK;
+}
+
+/* ---------------------------------------------------------------------------------------
  * states-form attention geometry.  packages/runtime/src/kernels/state-attention.ts:714-733
  * ------------------------------------------------------------------------------------- */
 static int sliding(uint64_t window) { return window > 0; } /* state-attention.ts:148 */

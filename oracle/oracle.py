@@ -72,6 +72,12 @@ def _declare(L: C.CDLL) -> None:
         f.argtypes = [p, p, p, z, z, z, p]
     L.krmo_linear_i4_mt.restype = C.c_int
     L.krmo_linear_i4_mt.argtypes = [p, p, p, p, z, z, z, z, p]
+    L.krmo_quantize_rows.restype = None
+    L.krmo_quantize_rows.argtypes = [p, z, z, p, p]
+    L.krmo_quantize_rows_tie_margin.restype = C.c_double
+    L.krmo_quantize_rows_tie_margin.argtypes = [p, z, z]
+    L.krmo_linear_w4a8.restype = C.c_int
+    L.krmo_linear_w4a8.argtypes = [p, p, p, p, z, z, z, z, C.c_int, p]
     L.krmo_state_column_base.restype = u64
     L.krmo_state_column_base.argtypes = [u64, u64]
     L.krmo_state_live_columns.restype = u64
@@ -188,6 +194,38 @@ def linear_i4(x, packed, scale, bias, n: int, k: int, group: int) -> np.ndarray:
                                  _ptr(out))
     if rc != 0:
         raise OracleError("linear_i4 rejected the shapes")
+    return out.reshape(x.shape[:-1] + (n,))
+
+
+def quantize_rows(x, dim: int):
+    """Per-row symmetric int8 quantisation -> (q int8 [rows, dim], scale f32 [rows])."""
+    x = _f32(x).reshape(-1, dim) if dim else _f32(x).reshape(0, 0)
+    rows = x.shape[0]
+    q = np.empty((rows, dim), dtype=np.int8)
+    scale = np.empty(rows, dtype=np.float32)
+    lib().krmo_quantize_rows(_ptr(x), rows, dim, _ptr(q), _ptr(scale))
+    return q, scale
+
+
+def quantize_rows_tie_margin(x, dim: int) -> float:
+    x = _f32(x).reshape(-1, dim)
+    return float(lib().krmo_quantize_rows_tie_margin(_ptr(x), x.shape[0], dim))
+
+
+def linear_w4a8(x, packed, scale, bias, n: int, k: int, group: int, fused: bool = True):
+    """w4a8 linear: int8 rows of x against packed int4 weights, one f32 flush per group."""
+    x = _f32(x)
+    packed = np.ascontiguousarray(packed, dtype=np.uint8).reshape(-1)
+    scale = _f32(scale).reshape(-1)
+    bias = _f32(bias) if bias is not None else np.zeros(n, dtype=np.float32)
+    if packed.size * 2 != n * k or scale.size * group != n * k or x.shape[-1] != k:
+        raise OracleError("linear_w4a8 shapes")
+    m = x.size // k
+    out = np.empty((m, n), dtype=np.float32)
+    rc = lib().krmo_linear_w4a8(_ptr(x), _ptr(packed), _ptr(scale), _ptr(bias), m, n, k, group,
+                                1 if fused else 0, _ptr(out))
+    if rc != 0:
+        raise OracleError("linear_w4a8 rejected the shapes")
     return out.reshape(x.shape[:-1] + (n,))
 
 

@@ -251,3 +251,43 @@ def oracle_decoder_logits(weights, ids) -> np.ndarray:
         h = (h + lin(act, lw["down"])).astype(np.float32)
     xn = oracle.rms_norm(h, weights.final_norm, c.rms_eps)
     return lin(xn, weights.lm_head)
+
+
+# ---------------------------------------------------------------------------- w4a8
+
+def SIGNED_A8(i: int) -> float:
+    """x / bias generator of the integer-dot tests (packages/runtime/tests/gpu_i8a8_test.ts:82)."""
+    return ((i % 29) - 14) * 0.3717 + 0.0131
+
+
+TIE_MARGIN = 1e-3  # gpu_i8a8_test.ts:86
+
+
+@dataclass(frozen=True)
+class W4a8Case:
+    name: str
+    m: int
+    n: int
+    k: int
+    group: int
+
+
+# packages/runtime/tests/gpu_i8a8_test.ts:758-769
+W4A8_CASES = [
+    W4a8Case("v4 [130,96] x W[68,96] g32", 130, 68, 96, 32),
+    W4a8Case("scalar [129,48] x W[67,48] g16", 129, 67, 48, 16),
+    W4a8Case("v4 small [3,32] x W[8,32] g32", 3, 8, 32, 32),
+    W4a8Case("scalar small [17,96] x W[19,96] g32", 17, 19, 96, 32),
+]
+
+
+def make_w4a8(case: W4a8Case, x_value=None):
+    """Inputs of one case as the reference prepares them (gpu_i8a8_test.ts:777-821): weights
+    from group_varying through the test-side quantiser, bias and x from SIGNED_A8.
+    x_value(index, m, k) replaces single elements of x."""
+    w = seeded(case.n * case.k, group_varying(case.k, case.group)).reshape(case.n, case.k)
+    packed, q, scale = quantize_i4(w, (case.n, case.k), case.group)
+    bias = seeded(case.n, SIGNED_A8)
+    fn = (lambda i: x_value(i, case.m, case.k)) if x_value else SIGNED_A8
+    x = seeded(case.m * case.k, fn).reshape(case.m, case.k)
+    return x, packed, q, scale, bias

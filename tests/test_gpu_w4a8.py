@@ -1,0 +1,201 @@
+"""GPU parity of the w4a8 path (activation quantiser + integer-dot `linear`, through the C ABI)
+against the CPU oracle.  The contract is atol = 0: group sums are exact integers and every
+floating-point step is one correctly rounded operation in a fixed order
+(docs/decisions/0076-w4a8-linear-execution.md:40-60), so every comparison here is bitwise
+(NaN where the oracle has NaN)."""
+import numpy as np
+import pytest
+
+import helpers
+import karume_amd as ka
+from helpers import oracle
+
+pytestmark = pytest.mark.gpu
+
+
+def assert_exact(got, want, what):
+    got, want = np.asarray(got), np.asarray(want)
+    assert got.shape == want.shape, what
+    nan = np.isnan(want) if want.dtype.kind == "f" else np.zeros(want.shape, bool)
+    assert np.array_equal(np.isnan(got) if got.dtype.kind == "f" else nan, nan), what
+    assert np.array_equal(got[~nan], want[~nan]), (what, np.argwhere(got != want)[:5])
+
+
+def run_quantize(ctx, x):
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    rows, dim = x.shape
+    dx = ctx.upload(x)
+    dq, ds = ctx.alloc(max(rows * dim, 16)), ctx.alloc(max(rows * 4, 16))
+    ctx.quantize_rows(dx, dq, ds, rows, dim)
+    q = dq.download(np.int8, (rows, dim))
+    s = ds.download(np.float32, (rows,))
+    for b in (dx, dq, ds):
+        b.free()
+    return q, s
+
+
+def run_w4a8(ctx, x, packed, scale, bias, n, k, group):
+    """quantize_rows + linear_w4a8 with node-local temporaries, as the reference's builder
+    issues them (packages/runtime/src/runtime/recipe-builder.ts:1428-1488)."""
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    scale = np.ascontiguousarray(scale)
+    m = x.shape[0]
+    dx, dw, dsc = ctx.upload(x), ctx.upload(packed), ctx.upload(scale)
+    db = ctx.upload(np.ascontiguousarray(bias, dtype=np.float32)) if bias is not None else None
+    dq, dxs = ctx.alloc(max(m * k, 16)), ctx.alloc(max(m * 4, 16))
+    out = ctx.alloc(max(m * n * 4, 16))
+    ctx.quantize_rows(dx, dq, dxs, m, k)
+    ctx.linear_w4a8(dq, dxs, dw, dsc, db, out, m, n, k, group, ka.dtype_code(scale.dtype))
+    got = out.download(np.float32, (m, n))
+    for b in (dx, dw, dsc, dq, dxs, out) + ((db,) if db is not None else ()):
+        b.free()
+    return got
+
+
+# ---- quantize_rows: packages/runtime/tests/gpu_i8a8_test.ts:216-330 ---------------------------
+
+def test_quantize_ties_round_to_even(gpu_ctx):
+    values = np.array([[127, 0.5, 1.5, -0.5, -1.5, 2.5, 3.5, -3.5]], dtype=np.float32)
+    q, s = run_quantize(gpu_ctx, values)
+    assert float(s[0]) == 1.0
+    assert q.tolist() == [[127, 0, 2, 0, -2, 2, 4, -4]]
+
+
+def test_quantize_matches_oracle_rows_of_different_size(gpu_ctx):
+    rows, dim = 7, 20  # a multiple of 4 that is no multiple of 16
+    x = np.array([[0 if r == 3 else helpers.SIGNED_A8(r * dim + i) * (1 + r * 3)
+                   for i in range(dim)] for r in range(rows)], dtype=np.float32)
+    q, s = run_quantize(gpu_ctx, x)
+    want_q, want_s = oracle.quantize_rows(x, dim)
+    assert_exact(s, want_s, "scale")
+    assert_exact(q, want_q, "codes")
+    assert float(s[3]) == 1.1754943508222875e-38 and not q[3].any()
+
+
+def test_quantize_propagates_nan_and_inf_to_the_row_scale(gpu_ctx):
+    rows, dim = 4, 8
+    x = helpers.seeded(rows * dim, helpers.SIGNED_A8).reshape(rows, dim)
+    x[1, dim - 1] = np.nan
+    x[2, 3] = np.inf
+    x[3, 3] = -np.inf
+    q, s = run_quantize(gpu_ctx, x)
+    want_q, want_s = oracle.quantize_rows(x, dim)
+    assert_exact(s, want_s, "scale")
+    assert np.isfinite(s[0]) and np.isnan(s[1]) and s[2] == np.inf and s[3] == np.inf
+    assert_exact(q, want_q, "codes")  # also the non-finite rows: a NaN quotient stores 0
+
+
+@pytest.mark.parametrize("rows, dim", [(1, 4096), (3, 11008), (300, 260), (2, 4)])
+def test_quantize_random_rows_bit_exact_without_a_tie_margin(gpu_ctx, rows, dim):
+    """Random data, no margin gate: the device division is correctly rounded, so the codes
+    equal the oracle's even where x / s sits next to a half-integer."""
+    rng = np.random.default_rng(rows * 131 + dim)
+    x = (rng.normal(size=(rows, dim)) * rng.uniform(0.01, 30, size=(rows, 1))).astype(np.float32)
+    x[0, : min(dim, 8)] = [0.5, 1.5, 2.5, -0.5, 127, -127, 63.5, 0][: min(dim, 8)]
+    q, s = run_quantize(gpu_ctx, x)
+    want_q, want_s = oracle.quantize_rows(x, dim)
+    assert_exact(s, want_s, "scale")
+    assert_exact(q, want_q, "codes")
+
+
+def test_quantize_rejections(gpu_ctx):
+    buf = gpu_ctx.alloc(256)
+    with pytest.raises(ka.GpuValidationError, match="multiple of 4"):
+        gpu_ctx.quantize_rows(buf, buf, buf, 1, 6)
+    with pytest.raises(ka.GpuValidationError, match="positive"):
+        gpu_ctx.quantize_rows(buf, buf, buf, 1, 0)
+    gpu_ctx.quantize_rows(buf, buf, buf, 0, 8)  # no rows: nothing to do
+    buf.free()
+
+
+# ---- linear: packages/runtime/tests/gpu_i8a8_test.ts:758-912 ----------------------------------
+
+@pytest.mark.parametrize("case", helpers.W4A8_CASES, ids=lambda c: c.name)
+def test_w4a8_reference_cases_bit_exact(gpu_ctx, case):
+    x, packed, q, scale, bias = helpers.make_w4a8(case)
+    want = oracle.linear_w4a8(x, packed, scale, bias, case.n, case.k, case.group)
+    got = run_w4a8(gpu_ctx, x, packed, scale, bias, case.n, case.k, case.group)
+    assert_exact(got, want, case.name)
+    assert len(set(got.reshape(-1).tolist())) > 1
+
+
+def test_w4a8_nan_row_zero_row(gpu_ctx):
+    case = helpers.W4A8_CASES[0]
+    nan_row, zero_row = 2, 5
+
+    def x_value(i, m, k):
+        row = i // k
+        if row == zero_row:
+            return 0.0
+        if row == nan_row and i % k == k - 3:
+            return float("nan")
+        return helpers.SIGNED_A8(i)
+
+    x, packed, q, scale, bias = helpers.make_w4a8(case, x_value)
+    want = oracle.linear_w4a8(x, packed, scale, bias, case.n, case.k, case.group)
+    got = run_w4a8(gpu_ctx, x, packed, scale, bias, case.n, case.k, case.group)
+    assert_exact(got, want, "nan / zero rows")
+    assert np.isnan(got[nan_row]).all() and np.isfinite(got[nan_row + 1]).all()
+    assert np.array_equal(got[zero_row], bias)
+
+
+def test_w4a8_differs_from_the_f32_activation_path(gpu_ctx):
+    case = helpers.W4A8_CASES[3]
+    x, packed, q, scale, bias = helpers.make_w4a8(case)
+    got = run_w4a8(gpu_ctx, x, packed, scale, bias, case.n, case.k, case.group)
+    f32_path = oracle.linear_i4(x, packed, scale, bias, case.n, case.k, case.group)
+    assert not np.array_equal(got, f32_path)
+    assert np.allclose(got, f32_path, rtol=0.05, atol=0.5)  # same op, coarser activations
+
+
+SHAPES = [  # (m, n, k, group, fp16 scales, bias)
+    (1, 4096, 4096, 128, True, False),    # the decode GEMV shape
+    (1, 130, 2048, 32, False, True),      # one group per lane
+    (1, 64, 6144, 2048, True, True),      # one group per step
+    (2, 70, 4096, 64, True, True),
+    (4, 100, 1024, 128, False, True),     # K shorter than a step
+    (7, 33, 5632, 128, True, True),       # K with a partial last step
+    (8, 16, 11008, 64, True, False),
+    (1, 9, 8192, 4096, True, True),       # a group longer than a step (fallback form)
+    (3, 21, 64, 16, False, True),         # two groups per lane (fallback form)
+    (16, 4096, 4096, 128, True, True),    # the ragged batch's GEMV shape
+    (40, 300, 1024, 128, True, True),
+]
+
+
+@pytest.mark.parametrize("m, n, k, group, scale_f16, with_bias", SHAPES)
+def test_w4a8_random_shapes_bit_exact(gpu_ctx, m, n, k, group, scale_f16, with_bias):
+    rng = np.random.default_rng(m * 7919 + n * 31 + k + group)
+    packed, q, scale = helpers.synthetic_int4(rng, n, k, group, scale_f16)
+    x = rng.normal(size=(m, k)).astype(np.float32)
+    bias = rng.normal(size=n).astype(np.float32) if with_bias else None
+    want = oracle.linear_w4a8(x, packed, np.asarray(scale, dtype=np.float32), bias, n, k, group)
+    got = run_w4a8(gpu_ctx, x, packed, scale, bias, n, k, group)
+    assert_exact(got, want, (m, n, k, group))
+
+
+def test_w4a8_rows_do_not_depend_on_the_batch(gpu_ctx):
+    rng = np.random.default_rng(3)
+    n, k, group = 512, 4096, 128
+    packed, q, scale = helpers.synthetic_int4(rng, n, k, group)
+    x = rng.normal(size=(16, k)).astype(np.float32)
+    whole = run_w4a8(gpu_ctx, x, packed, scale, None, n, k, group)
+    for rows in (1, 3, 8):
+        part = run_w4a8(gpu_ctx, x[:rows], packed, scale, None, n, k, group)
+        assert np.array_equal(part, whole[:rows])
+
+
+def test_w4a8_rejections(gpu_ctx):
+    buf = gpu_ctx.alloc(4096)
+    args = (buf, buf, buf, buf, None, buf)
+    with pytest.raises(ka.GpuValidationError, match="multiple of 4"):
+        gpu_ctx.linear_w4a8(*args, 1, 4, 0, 16)
+    with pytest.raises(ka.GpuValidationError, match="power of two"):
+        gpu_ctx.linear_w4a8(*args, 1, 4, 48, 24)
+    with pytest.raises(ka.GpuValidationError, match="power of two"):
+        gpu_ctx.linear_w4a8(*args, 1, 4, 32, 8)
+    with pytest.raises(ka.GpuValidationError, match="not a multiple of group_size"):
+        gpu_ctx.linear_w4a8(*args, 1, 4, 48, 32)
+    with pytest.raises(ka.GpuValidationError, match="int32 reduction limit"):
+        gpu_ctx.linear_w4a8(*args, 1, 1, 1 << 22, 1 << 22)
+    buf.free()
