@@ -275,6 +275,185 @@ __global__ __launch_bounds__(256) void linear_w4a8_rows_kernel(
   }
 }
 
+// ------------------------------------------------------------------ many rows (prefill)
+//
+// Matrix-core form for M > 8 and 64 <= group <= 131072: v_mfma_i32_32x32x32_i8 with A = xq
+// (rows of the tile), B = the weight bytes 16 * q (columns), int32 accumulators.  A workgroup
+// owns 64 rows of x and 256 weight rows; each of its four waves owns 64 of those weight rows
+// (two column tiles) against both row tiles.
+//  * B never touches LDS: lane (n = lane % 32, h = lane / 32) loads 16 bytes = codes
+//    64c + 32h .. + 31 of weight row n per 64-code chunk and expands words 2s, 2s + 1 into the
+//    operand of the chunk's MFMA step s: (even codes of word 2s, odd codes of word 2s,
+//    even codes of word 2s + 1, odd codes of word 2s + 1).
+//  * A goes through LDS in stages of 256 codes, its bytes regrouped (even, odd) per 8 codes on
+//    the way in, so that lane (m, h) reads its 16 operand bytes at 64c + 32h + 16s in one piece
+//    and byte j of A meets byte j of B.  Rows are padded by 16 bytes.
+//  * After the last chunk of a group the 64 int32 sums of a wave are shifted (the exact factor
+//    16), converted and fused into the f32 accumulators with the lane's column scale; the
+//    activation scale and the bias follow once, at the store.
+// Workgroup ids are dealt so that the row blocks of a column block run on one XCD.
+template <typename ST>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1)))
+void linear_w4a8_mfma_kernel(
+    const uint8_t* __restrict__ xq, const float* __restrict__ xs, const uint8_t* __restrict__ w,
+    const ST* __restrict__ scales, const float* __restrict__ bias, float* __restrict__ out,
+    uint32_t m, uint32_t n, uint32_t k, uint32_t group_shift, uint32_t m_blocks,
+    uint32_t n_blocks) {
+  constexpr int BM = 64, WN = 2, MT = BM / 32;
+  constexpr int kStage = 256;            // codes of x per LDS stage
+  constexpr int kRow = kStage + 16;      // bytes per LDS row
+  __shared__ __align__(16) uint8_t s_x[2][BM * kRow];
+
+  const uint32_t xcd = blockIdx.x & 7u, slot = blockIdx.x >> 3;
+  const uint32_t mb = slot % m_blocks, nb = (slot / m_blocks) * 8u + xcd;
+  if (nb >= n_blocks) return;  // the whole workgroup leaves before any barrier
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int frag_row = lane & 31, frag_h = lane >> 5;
+  const uint32_t m0 = mb * BM, n0 = nb * (4 * WN * 32) + wave * (WN * 32);
+  const uint32_t groups = k >> group_shift;
+  const uint32_t chunks_total = k >> 6;
+  const uint32_t chunks_per_group = 1u << (group_shift - 6);
+  const uint32_t stages = (k + kStage - 1) / kStage;
+
+  const uint8_t* wrow[WN];
+  const ST* srow[WN];
+#pragma unroll
+  for (int nt = 0; nt < WN; ++nt) {
+    const uint32_t row = min(n0 + nt * 32 + frag_row, n - 1);  // past N: last row, unused
+    wrow[nt] = w + (size_t)row * (k >> 1) + frag_h * 16;
+    srow[nt] = scales + (size_t)row * groups;
+  }
+  // staging: 64 rows x 16 units of 16 bytes, four units per thread
+  const uint8_t* xsrc[4];
+  uint32_t xunit[4], xdst[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const uint32_t u = tid + 256 * i, row = u >> 4;
+    xunit[i] = (u & 15u) * 16u;
+    xsrc[i] = xq + (size_t)min(m0 + row, m - 1) * k;
+    xdst[i] = row * kRow + xunit[i];
+  }
+  auto load_x = [&](uint32_t stage, uint4 (&r)[4]) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const uint32_t at = stage * kStage + xunit[i];
+      r[i] = *reinterpret_cast<const uint4*>(xsrc[i] + (at < k ? at : 0u));
+    }
+  };
+  auto park_x = [&](int buf, const uint4 (&r)[4]) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      uint4 v;
+      v.x = __builtin_amdgcn_perm(r[i].y, r[i].x, 0x06040200u);
+      v.y = __builtin_amdgcn_perm(r[i].y, r[i].x, 0x07050301u);
+      v.z = __builtin_amdgcn_perm(r[i].w, r[i].z, 0x06040200u);
+      v.w = __builtin_amdgcn_perm(r[i].w, r[i].z, 0x07050301u);
+      *reinterpret_cast<uint4*>(&s_x[buf][xdst[i]]) = v;
+    }
+  };
+  struct Weights {
+    uint4 w[WN][4];
+    float s[WN][4];
+  };
+  auto load_w = [&](uint32_t stage, Weights& d) {
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+      const uint32_t code = stage * kStage + 64u * c;
+      const uint32_t kc = code < k ? code : 0u;
+#pragma unroll
+      for (int nt = 0; nt < WN; ++nt) {
+        d.w[nt][c] = *reinterpret_cast<const uint4*>(wrow[nt] + (kc >> 1));
+        d.s[nt][c] = scale_f32<ST>(srow[nt], kc >> group_shift);
+      }
+    }
+  };
+
+  v16i_t acc[MT][WN];
+  float accf[MT][WN][16];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+    for (int nt = 0; nt < WN; ++nt)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        acc[mt][nt][r] = 0;
+        accf[mt][nt][r] = 0.f;
+      }
+
+  uint4 xr[4];
+  Weights cur, nxt;
+  load_x(0, xr);
+  load_w(0, cur);
+  park_x(0, xr);
+  __syncthreads();
+  int buf = 0;
+  for (uint32_t stage = 0; stage < stages; ++stage) {
+    const bool more = stage + 1 < stages;
+    if (more) {
+      load_x(stage + 1, xr);
+      load_w(stage + 1, nxt);
+    }
+    const uint32_t first_chunk = stage * 4u;
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+      if (first_chunk + c >= chunks_total) break;
+#pragma unroll
+      for (int s = 0; s < 2; ++s) {
+        v4i_t a[MT];
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt)
+          a[mt] = *reinterpret_cast<const v4i_t*>(
+              &s_x[buf][(mt * 32 + frag_row) * kRow + 64 * c + 32 * frag_h + 16 * s]);
+#pragma unroll
+        for (int nt = 0; nt < WN; ++nt) {
+          const uint32_t w0 = (s == 0 ? cur.w[nt][c].x : cur.w[nt][c].z) ^ 0x88888888u;
+          const uint32_t w1 = (s == 0 ? cur.w[nt][c].y : cur.w[nt][c].w) ^ 0x88888888u;
+          v4i_t b;
+          b[0] = (int)((w0 << 4) & 0xF0F0F0F0u);
+          b[1] = (int)(w0 & 0xF0F0F0F0u);
+          b[2] = (int)((w1 << 4) & 0xF0F0F0F0u);
+          b[3] = (int)(w1 & 0xF0F0F0F0u);
+#pragma unroll
+          for (int mt = 0; mt < MT; ++mt)
+            acc[mt][nt] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[mt], b, acc[mt][nt], 0, 0, 0);
+        }
+      }
+      if (((first_chunk + c + 1) & (chunks_per_group - 1)) == 0) {  // the group ends here
+#pragma unroll
+        for (int nt = 0; nt < WN; ++nt) {
+          const float ws = cur.s[nt][c];
+#pragma unroll
+          for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+              accf[mt][nt][r] = fmaf((float)(acc[mt][nt][r] >> 4), ws, accf[mt][nt][r]);
+              acc[mt][nt][r] = 0;
+            }
+        }
+      }
+    }
+    if (more) {
+      park_x(buf ^ 1, xr);
+      cur = nxt;
+    }
+    __syncthreads();
+    buf ^= 1;
+  }
+
+#pragma unroll
+  for (int nt = 0; nt < WN; ++nt) {
+    const uint32_t col = n0 + nt * 32 + frag_row;
+    const float b = (bias && col < n) ? bias[col] : 0.f;
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const uint32_t row = m0 + mt * 32 + 8 * (r / 4) + 4 * frag_h + (r % 4);
+        if (row < m && col < n) out[(size_t)row * n + col] = fmaf(accf[mt][nt][r], xs[row], b);
+      }
+  }
+}
+
 template <typename ST>
 int32_t launch_w4a8(krm_ctx* ctx, krm_buf xq, krm_buf xs, krm_buf w, krm_buf scales,
                     krm_buf bias, krm_buf out, uint32_t m, uint32_t n, uint32_t k,
@@ -301,6 +480,16 @@ int32_t launch_w4a8(krm_ctx* ctx, krm_buf xq, krm_buf xs, krm_buf w, krm_buf sca
       hipLaunchKernelGGL((linear_w4a8_rows_kernel<ST, 4>), grid, dim3(256), 0, ctx->stream, pxq,
                          pxs, pw, ps, pb, po, m, n, k, shift);
     return launched(ctx, "linear_w4a8_rows_kernel");
+  }
+  if (m > 8 && group >= 64 && group <= kMaxGroupTimes16 && aligned(xq, 16) && aligned(w, 16)) {
+    const uint32_t m_blocks = (m + 63) / 64, n_blocks = (n + 255) / 256;
+    const uint64_t blocks = (uint64_t)((n_blocks + 7) / 8) * 8u * m_blocks;
+    if (blocks <= 0x7fffffffull) {
+      hipLaunchKernelGGL((linear_w4a8_mfma_kernel<ST>), dim3((uint32_t)blocks), dim3(256), 0,
+                         ctx->stream, ptr<const uint8_t>(xq), pxs, ptr<const uint8_t>(w), ps, pb,
+                         po, m, n, k, shift, m_blocks, n_blocks);
+      return launched(ctx, "linear_w4a8_mfma_kernel");
+    }
   }
   const dim3 grid((n + 3) / 4, m < 65535u ? m : 65535u);
   hipLaunchKernelGGL((linear_w4a8_generic_kernel<ST>), grid, dim3(256), 0, ctx->stream, pxq, pxs,
@@ -345,7 +534,6 @@ extern "C" int32_t krm_linear_w4a8(krm_ctx* ctx, krm_buf xq, krm_buf xs, krm_buf
                        krm::aligned(out, 4) && krm::aligned(bias, 4) &&
                        krm::aligned(scales, krm::dtype_bytes(scale_dtype)),
               "linear w4a8: misaligned buffer");
-  (void)kMaxGroupTimes16;
   if (scale_dtype == KRM_F16)
     return launch_w4a8<__half>(ctx, xq, xs, w, scales, bias, out, m, n, k, group);
   return launch_w4a8<float>(ctx, xq, xs, w, scales, bias, out, m, n, k, group);

@@ -160,6 +160,13 @@ SHAPES = [  # (m, n, k, group, fp16 scales, bias)
     (3, 21, 64, 16, False, True),         # two groups per lane (fallback form)
     (16, 4096, 4096, 128, True, True),    # the ragged batch's GEMV shape
     (40, 300, 1024, 128, True, True),
+    # the matrix-core form (M > 8, group >= 64)
+    (70, 260, 5696, 64, True, True),      # K ends inside an LDS stage; N one past a block
+    (9, 31, 512, 512, False, True),       # a group over two stages
+    (33, 64, 4096, 2048, True, False),
+    (100, 257, 1024, 256, False, True),
+    (512, 1000, 4096, 128, True, True),   # the prefill row count
+    (130, 96, 11008, 128, True, True),    # the down-projection's K
 ]
 
 
