@@ -161,6 +161,37 @@ def bench_gemm(ctx, ka, rng, steps: int, warmup: int, m: int, n: int, k: int, g:
     return ms / steps, 2.0 * m * n * k
 
 
+def bench_w4a8(ctx, ka, rng, steps: int, warmup: int, m: int, n: int, k: int, g: int,
+               copies: int):
+    """w4a8 `linear` (int8 activations x int4 weights, integer dot products): one step = the
+    activation quantiser + the product, f32 x in, f32 out, fp16 group scales.
+    Returns (ms per step, ms per step of the product alone)."""
+    weights, scales = [], []
+    for _ in range(copies):
+        weights.append(ctx.upload(rng.integers(0, 256, size=n * k // 2, dtype=np.uint8)))
+        scales.append(ctx.upload(np.maximum(
+            np.abs(rng.normal(0, 0.02, size=(n, k // g))).astype(np.float16),
+            np.float16(6.104e-05))))
+    x = ctx.upload(rng.normal(size=(m, k)).astype(np.float32))
+    xq, xs = ctx.alloc(max(16, m * k)), ctx.alloc(max(16, m * 4))
+    out = ctx.alloc(m * n * 4)
+
+    def step(i: int) -> None:
+        j = i % copies
+        ctx.quantize_rows(x, xq, xs, m, k)
+        ctx.linear_w4a8(xq, xs, weights[j], scales[j], None, out, m, n, k, g, ka.F16)
+
+    def product(i: int) -> None:
+        j = i % copies
+        ctx.linear_w4a8(xq, xs, weights[j], scales[j], None, out, m, n, k, g, ka.F16)
+
+    ms = timed(ctx, step, steps, warmup, copies)
+    ms_product = timed(ctx, product, steps, warmup, copies)
+    for b in weights + scales + [x, xq, xs, out]:
+        b.free()
+    return ms / steps, ms_product / steps
+
+
 def bench_model(ctx, ka, io_dtype, kv_dtype, prompt_len: int = 128, new_tokens: int = 256):
     """BASELINE config 4: random-init 1.1B-shape int4 decoder, 128-token random prompt, 256
     greedy decode steps, batch 1.  The decode steps replay one recorded step (lengths and the
@@ -280,7 +311,7 @@ def main() -> int:
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-graph", action="store_true",
                     help="issue plain launches instead of replaying recorded graphs")
-    ap.add_argument("--only", default="", help="gemv | gemv16 | gemm | attention | model | traffic: run only that part besides the "
+    ap.add_argument("--only", default="", help="gemv | gemv16 | gemm | attention | w4a8 | model | traffic: run only that part besides the "
                          "headline GEMV")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -357,6 +388,21 @@ def main() -> int:
             result[f"gemm_{name}_us"] = round(ms_g * 1e3, 2)
             result[f"gemm_{name}_pct_of_f16_mfma_peak"] = round(
                 100 * flops / (ms_g * 1e-3) / 2.5e15, 2)
+    if args.only in ("", "w4a8"):
+        log("[bench] w4a8 linear: M=1 GEMV and M=512 up/down-projections")
+        ms_q, ms_p = bench_w4a8(ctx, ka, rng, steps2, max(10, args.warmup // 4), 1, n, k, g, copies)
+        w4_bytes = n * k // 2 + n * (k // g) * 2 + k + 4 + n * 4
+        result["w4a8_gemv_us"] = round(ms_q * 1e3, 3)
+        result["w4a8_gemv_product_us"] = round(ms_p * 1e3, 3)
+        result["w4a8_gemv_product_gbs"] = round(w4_bytes / (ms_p * 1e-3) / 1e9, 1)
+        for name, (gn, gk) in {"up": (11008, 4096), "down": (4096, 11008)}.items():
+            ms_q, ms_p = bench_w4a8(ctx, ka, rng, 40, 8, 512, gn, gk, g, 4)
+            ops = 2.0 * 512 * gn * gk
+            result[f"w4a8_gemm_{name}_us"] = round(ms_q * 1e3, 2)
+            result[f"w4a8_gemm_{name}_product_us"] = round(ms_p * 1e3, 2)
+            result[f"w4a8_gemm_{name}_product_tops"] = round(ops / (ms_p * 1e-3) / 1e12, 1)
+            result[f"w4a8_gemm_{name}_pct_of_i8_mfma_peak"] = round(
+                100 * ops / (ms_p * 1e-3) / 5.0e15, 2)
     if args.only in ("", "model"):
         # f32 activations: with this random init (|N(0,0.02)| scales on uniform codes) the
         # residual stream passes 65504 after a few layers, so fp16 activations are not usable
