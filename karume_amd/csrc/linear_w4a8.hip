@@ -25,6 +25,8 @@
 // extension) and the exact factor 16 is shifted out of the group sum before it is converted.
 #include "krm_internal.h"
 
+#include <cstdlib>
+
 namespace {
 
 using namespace krm;
@@ -495,6 +497,197 @@ void linear_w4a8_mfma_kernel(
   }
 }
 
+// Matrix-core form with both operands through LDS: eight waves, workgroup tile
+// (64 * MT) x 256, wave (wm, wn) = (32 * MT) ... rows wm and 64 columns wn.  The packed weight
+// bytes are staged as they are (coalesced 16-byte loads, 128 bytes of a row per stage) and
+// expanded to the bytes 16 * q in registers after the LDS read, so LDS holds a quarter of what
+// dequantised bytes would take; xq is staged with its bytes regrouped (even, odd) as above.
+// The stage's group scales are staged too, already converted.  Two waves share a SIMD: one
+// wave's group flush (VALU) runs under the other's MFMAs.
+template <typename ST, int GSH, int MT>
+__global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2)))
+void linear_w4a8_tile_kernel(
+    const uint8_t* __restrict__ xq, const float* __restrict__ xs, const uint8_t* __restrict__ w,
+    const ST* __restrict__ scales, const float* __restrict__ bias, float* __restrict__ out,
+    uint32_t m, uint32_t n, uint32_t k, uint32_t group_shift, uint32_t m_blocks,
+    uint32_t n_blocks) {
+  constexpr int WN = 2;                       // 32-column tiles per wave
+  constexpr int BM = 2 * 32 * MT, BN = 256;   // two wave rows, four wave columns
+  constexpr int kStage = 256;                 // codes per LDS stage
+  constexpr int kRowA = kStage + 16;          // bytes per LDS row of xq
+  constexpr int kRowB = kStage / 2 + 16;      // bytes per LDS row of packed weights
+  constexpr int kChunksPerGroup = GSH ? (1 << (GSH - 6)) : 4;  // inside a stage
+  constexpr int kScalesPerStage = GSH ? (kStage >> GSH) : 1;
+  constexpr int kAUnits = BM * 16 / 512;      // 16-byte units of xq per thread and stage
+  __shared__ __align__(16) uint8_t s_a[2][BM * kRowA];
+  __shared__ __align__(16) uint8_t s_b[2][BN * kRowB];
+  __shared__ __align__(16) float s_s[2][BN][4];
+
+  const uint32_t xcd = blockIdx.x & 7u, slot = blockIdx.x >> 3;
+  const uint32_t mb = slot % m_blocks, nb = (slot / m_blocks) * 8u + xcd;
+  if (nb >= n_blocks) return;  // the whole workgroup leaves before any barrier
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = wave >> 2, wn = wave & 3;
+  const int frag_row = lane & 31, frag_h = lane >> 5;
+  const uint32_t m0 = mb * BM, n0 = nb * BN;
+  const uint32_t shift = GSH ? (uint32_t)GSH : group_shift;
+  const uint32_t groups = k >> shift;
+  const uint32_t chunks_total = k >> 6;
+  const uint32_t stages = (k + kStage - 1) / kStage;
+  const uint32_t stages_per_group = GSH ? 1u : 1u << (shift - 8);
+
+  // staging roles: xq rows in 16 units of 16 bytes (rows tid / 16 + 32 i), weight rows in 8
+  // (rows tid / 8 + 64 i), one scale row per thread; 32-bit offsets from the three bases
+  const uint32_t arow0 = tid >> 4, aunit = (tid & 15u) * 16u;
+  const uint32_t brow0 = tid >> 3, bunit = (tid & 7u) * 16u;
+  const ST* ssrc = scales + (size_t)min(n0 + (uint32_t)(tid & 255), n - 1) * groups;
+  struct Staged {
+    uint4 a[kAUnits];
+    uint4 b[4];
+    ST s[kScalesPerStage];
+  };
+  // Requests only, clamped addresses: every stage issues the same loads in the same order.
+  auto load_stage = [&](uint32_t stage, Staged& d) {
+    const uint32_t a_at = stage * kStage + aunit, b_at = stage * (kStage / 2) + bunit;
+    const uint32_t a_off = a_at < k ? a_at : 0u, b_off = b_at < (k >> 1) ? b_at : 0u;
+#pragma unroll
+    for (int i = 0; i < kAUnits; ++i)
+      d.a[i] = *reinterpret_cast<const uint4*>(
+          xq + (size_t)min(m0 + arow0 + 32u * i, m - 1) * k + a_off);
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      d.b[i] = *reinterpret_cast<const uint4*>(
+          w + (size_t)min(n0 + brow0 + 64u * i, n - 1) * (k >> 1) + b_off);
+#pragma unroll
+    for (int j = 0; j < kScalesPerStage; ++j) {
+      const uint32_t code = stage * kStage + (j << (GSH ? GSH : 8));
+      d.s[j] = ssrc[(code < k ? code : 0u) >> shift];
+    }
+  };
+  // codes past the end of K are parked as zeros in xq: their products vanish whatever B holds
+  auto park_stage = [&](uint32_t stage, int buf, const Staged& d) {
+    const uint32_t keep = stage * kStage + aunit < k ? 0xFFFFFFFFu : 0u;
+#pragma unroll
+    for (int i = 0; i < kAUnits; ++i) {
+      uint4 v;
+      v.x = __builtin_amdgcn_perm(d.a[i].y, d.a[i].x, 0x06040200u) & keep;
+      v.y = __builtin_amdgcn_perm(d.a[i].y, d.a[i].x, 0x07050301u) & keep;
+      v.z = __builtin_amdgcn_perm(d.a[i].w, d.a[i].z, 0x06040200u) & keep;
+      v.w = __builtin_amdgcn_perm(d.a[i].w, d.a[i].z, 0x07050301u) & keep;
+      *reinterpret_cast<uint4*>(&s_a[buf][(arow0 + 32u * i) * kRowA + aunit]) = v;
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      *reinterpret_cast<uint4*>(&s_b[buf][(brow0 + 64u * i) * kRowB + bunit]) = d.b[i];
+    if (tid < 256) {
+#pragma unroll
+      for (int j = 0; j < kScalesPerStage; ++j) s_s[buf][tid][j] = scale_f32<ST>(&d.s[j], 0);
+    }
+  };
+
+  v16i_t acc[MT][WN];
+  float accf[MT][WN][16];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+    for (int nt = 0; nt < WN; ++nt)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        acc[mt][nt][r] = 0;
+        accf[mt][nt][r] = 0.f;
+      }
+  const v16i_t zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+
+  Staged staged;
+  load_stage(0, staged);
+  park_stage(0, 0, staged);
+  __syncthreads();
+
+  const uint32_t a_base = (uint32_t)((wm * 32 * MT + frag_row) * kRowA + 32 * frag_h);
+  const uint32_t b_base = (uint32_t)((wn * 64 + frag_row) * kRowB + 16 * frag_h);
+  auto run_stage = [&](uint32_t stage, int buf) {
+    load_stage(stage + 1, staged);
+    const uint32_t first_chunk = stage * 4u;
+    const bool stage_opens = GSH ? true : (stage & (stages_per_group - 1)) == 0;
+    const bool stage_closes = GSH ? true : ((stage + 1) & (stages_per_group - 1)) == 0;
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+      const bool valid = first_chunk + c < chunks_total;
+      const bool opens_static = GSH != 0 && (c % kChunksPerGroup) == 0;
+      const bool closes = GSH ? ((c + 1) % kChunksPerGroup) == 0 : (stage_closes && c == 3);
+      if (GSH == 0 && stage_opens && c == 0) {
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+          for (int nt = 0; nt < WN; ++nt) acc[mt][nt] = zero;
+      }
+      uint4 braw[WN];
+#pragma unroll
+      for (int nt = 0; nt < WN; ++nt)
+        braw[nt] = *reinterpret_cast<const uint4*>(&s_b[buf][b_base + nt * 32 * kRowB + 32 * c]);
+#pragma unroll
+      for (int s = 0; s < 2; ++s) {
+        v4i_t a[MT];
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt)
+          a[mt] = *reinterpret_cast<const v4i_t*>(
+              &s_a[buf][a_base + mt * 32 * kRowA + 64 * c + 16 * s]);
+#pragma unroll
+        for (int nt = 0; nt < WN; ++nt) {
+          const uint32_t w0 = (s == 0 ? braw[nt].x : braw[nt].z) ^ 0x88888888u;
+          const uint32_t w1 = (s == 0 ? braw[nt].y : braw[nt].w) ^ 0x88888888u;
+          v4i_t b;
+          b[0] = (int)((w0 << 4) & 0xF0F0F0F0u);
+          b[1] = (int)(w0 & 0xF0F0F0F0u);
+          b[2] = (int)((w1 << 4) & 0xF0F0F0F0u);
+          b[3] = (int)(w1 & 0xF0F0F0F0u);
+#pragma unroll
+          for (int mt = 0; mt < MT; ++mt)
+            acc[mt][nt] = __builtin_amdgcn_mfma_i32_32x32x32_i8(
+                a[mt], b, (opens_static && s == 0) ? zero : acc[mt][nt], 0, 0, 0);
+        }
+      }
+      if (closes) {
+#pragma unroll
+        for (int nt = 0; nt < WN; ++nt) {
+          const float ws = s_s[buf][wn * 64 + nt * 32 + frag_row][GSH ? c / kChunksPerGroup : 0];
+          // an fp16 scale / 16 is always exact in f32; an f32 scale below 2^-122 may not be
+          const float ws16 = ws * 0.0625f;
+          const bool exact = sizeof(ST) == 2 || __all(ws16 * 16.0f == ws);
+          const float mult = valid ? (exact ? ws16 : ws) : 0.f;  // past K: accf + 0 * 0
+          const int down = exact ? 0 : 4;
+#pragma unroll
+          for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+              const int32_t sum = sizeof(ST) == 2 ? acc[mt][nt][r] : acc[mt][nt][r] >> down;
+              accf[mt][nt][r] = fmaf((float)sum, mult, accf[mt][nt][r]);
+            }
+        }
+      }
+    }
+    park_stage(stage + 1, buf ^ 1, staged);
+    __syncthreads();
+  };
+  for (uint32_t stage = 0; stage < stages; stage += 2) {
+    run_stage(stage, 0);
+    run_stage(stage + 1, 1);  // past the last stage: zeros, fused with a zero scale
+  }
+
+#pragma unroll
+  for (int nt = 0; nt < WN; ++nt) {
+    const uint32_t col = n0 + wn * 64 + nt * 32 + frag_row;
+    const float b = (bias && col < n) ? bias[col] : 0.f;
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const uint32_t row = m0 + wm * 32 * MT + mt * 32 + 8 * (r / 4) + 4 * frag_h + (r % 4);
+        if (row < m && col < n) out[(size_t)row * n + col] = fmaf(accf[mt][nt][r], xs[row], b);
+      }
+  }
+}
+
 template <typename ST>
 int32_t launch_w4a8(krm_ctx* ctx, krm_buf xq, krm_buf xs, krm_buf w, krm_buf scales,
                     krm_buf bias, krm_buf out, uint32_t m, uint32_t n, uint32_t k,
@@ -523,7 +716,30 @@ int32_t launch_w4a8(krm_ctx* ctx, krm_buf xq, krm_buf xs, krm_buf w, krm_buf sca
     return launched(ctx, "linear_w4a8_rows_kernel");
   }
   if (m > 8 && group >= 64 && group <= kMaxGroupTimes16 && aligned(xq, 16) && aligned(w, 16)) {
-    const uint32_t m_blocks = (m + 63) / 64, n_blocks = (n + 255) / 256;
+    const uint32_t n_blocks = (n + 255) / 256;
+    const char* form = getenv("KRM_W4A8_FORM");
+    if (!form || strcmp(form, "direct") != 0) {
+      // rows of 128 per workgroup when that still covers most of the chip, else 64
+      const bool tall = getenv("KRM_W4A8_TALL") != nullptr;
+      const uint32_t m_blocks = tall ? (m + 127) / 128 : (m + 63) / 64;
+      const uint64_t blocks = (uint64_t)((n_blocks + 7) / 8) * 8u * m_blocks;
+      if (blocks <= 0x7fffffffull) {
+#define KRM_W4A8_TILE(GSH, MT)                                                                  \
+  hipLaunchKernelGGL((linear_w4a8_tile_kernel<ST, GSH, MT>), dim3((uint32_t)blocks), dim3(512), \
+                     0, ctx->stream, ptr<const uint8_t>(xq), pxs, ptr<const uint8_t>(w), ps,   \
+                     pb, po, m, n, k, shift, m_blocks, n_blocks)
+#define KRM_W4A8_TILE_G(GSH) \
+  do { if (tall) KRM_W4A8_TILE(GSH, 2); else KRM_W4A8_TILE(GSH, 1); } while (0)
+        if (shift == 6) KRM_W4A8_TILE_G(6);
+        else if (shift == 7) KRM_W4A8_TILE_G(7);
+        else if (shift == 8) KRM_W4A8_TILE_G(8);
+        else KRM_W4A8_TILE_G(0);
+#undef KRM_W4A8_TILE_G
+#undef KRM_W4A8_TILE
+        return launched(ctx, "linear_w4a8_tile_kernel");
+      }
+    }
+    const uint32_t m_blocks = (m + 63) / 64;
     const uint64_t blocks = (uint64_t)((n_blocks + 7) / 8) * 8u * m_blocks;
     if (blocks <= 0x7fffffffull) {
 #define KRM_W4A8_MFMA(GSH)                                                                    \
