@@ -25,8 +25,6 @@
 // extension) and the exact factor 16 is shifted out of the group sum before it is converted.
 #include "krm_internal.h"
 
-#include <cstdlib>
-
 namespace {
 
 using namespace krm;
@@ -280,224 +278,30 @@ __global__ __launch_bounds__(256) void linear_w4a8_rows_kernel(
 // ------------------------------------------------------------------ many rows (prefill)
 //
 // Matrix-core form for M > 8 and 64 <= group <= 131072: v_mfma_i32_32x32x32_i8 with A = xq
-// (rows of the tile), B = the weight bytes 16 * q (columns), int32 accumulators.  A workgroup
-// owns 64 rows of x and 256 weight rows; each of its four waves owns 64 of those weight rows
-// (two column tiles) against both row tiles.
-//  * B never touches LDS: lane (n = lane % 32, h = lane / 32) loads 16 bytes = codes
+// (rows of the tile), B = the weight bytes 16 * q (columns), int32 accumulators.
+//  * Lane (n = lane % 32, h = lane / 32) of a column tile holds 16 bytes = codes
 //    64c + 32h .. + 31 of weight row n per 64-code chunk and expands words 2s, 2s + 1 into the
 //    operand of the chunk's MFMA step s: (even codes of word 2s, odd codes of word 2s,
-//    even codes of word 2s + 1, odd codes of word 2s + 1).  Two stages of four chunks are in
-//    flight; a stage's registers are requested again, for two stages ahead, when its last
-//    chunk is consumed.
-//  * A goes through LDS in stages of 256 codes, its bytes regrouped (even, odd) per 8 codes on
-//    the way in, so that lane (m, h) reads its 16 operand bytes at 64c + 32h + 16s in one piece
-//    and byte j of A meets byte j of B.  Rows are padded by 16 bytes.
+//    even codes of word 2s + 1, odd codes of word 2s + 1).
+//  * xq's bytes are regrouped (even, odd) per 8 codes on the way into LDS, so that lane (m, h)
+//    reads its 16 operand bytes at 64c + 32h + 16s in one piece and byte j of A meets byte j
+//    of B.  LDS rows are padded by 16 bytes.
 //  * The first MFMA of a group starts from a zero accumulator; after the group's last chunk
-//    the 64 int32 sums of a wave (16 x the group sums) are converted and fused into the f32
-//    accumulators with the lane's column scale / 16 — the same real product, hence the same
-//    rounded result; where an f32 scale / 16 is not exact (a subnormal quotient) the sums are
-//    shifted instead.  The activation scale and the bias follow once, at the store.
+//    the int32 sums (16 x the group sums) are converted and fused into the f32 accumulators
+//    with the lane's column scale / 16 — the same real product, hence the same rounded result;
+//    where an f32 scale / 16 is not exact (a subnormal quotient) the sums are shifted instead.
+//    The activation scale and the bias follow once, at the store.
+//  * Every stage issues the same loads in the same order whatever K is (addresses past K are
+//    clamped, chunks past K multiply zeros and are fused with a zero scale): a branch around a
+//    load would make the compiler's wait counts assume the worst path.
 // GSH = log2(group) for groups of 64, 128, 256 (group boundaries known at compile time);
 // GSH = 0: any larger group (a whole number of stages).
 // Workgroup ids are dealt so that the row blocks of a column block run on one XCD.
-template <typename ST, int GSH>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1)))
-void linear_w4a8_mfma_kernel(
-    const uint8_t* __restrict__ xq, const float* __restrict__ xs, const uint8_t* __restrict__ w,
-    const ST* __restrict__ scales, const float* __restrict__ bias, float* __restrict__ out,
-    uint32_t m, uint32_t n, uint32_t k, uint32_t group_shift, uint32_t m_blocks,
-    uint32_t n_blocks) {
-  constexpr int BM = 64, WN = 2, MT = BM / 32;
-  constexpr int kStage = 256;            // codes of x per LDS stage
-  constexpr int kRow = kStage + 16;      // bytes per LDS row
-  constexpr int kChunksPerGroup = GSH ? (1 << (GSH - 6)) : 4;  // inside a stage
-  __shared__ __align__(16) uint8_t s_x[2][BM * kRow];
-
-  const uint32_t xcd = blockIdx.x & 7u, slot = blockIdx.x >> 3;
-  const uint32_t mb = slot % m_blocks, nb = (slot / m_blocks) * 8u + xcd;
-  if (nb >= n_blocks) return;  // the whole workgroup leaves before any barrier
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int frag_row = lane & 31, frag_h = lane >> 5;
-  const uint32_t m0 = mb * BM, n0 = nb * (4 * WN * 32) + wave * (WN * 32);
-  const uint32_t shift = GSH ? (uint32_t)GSH : group_shift;
-  const uint32_t groups = k >> shift;
-  const uint32_t chunks_total = k >> 6;
-  const uint32_t stages = (k + kStage - 1) / kStage;
-  const uint32_t stages_per_group = GSH ? 1u : 1u << (shift - 8);
-
-  const uint8_t* wrow[WN];
-  const ST* srow[WN];
-#pragma unroll
-  for (int nt = 0; nt < WN; ++nt) {
-    const uint32_t row = min(n0 + nt * 32 + frag_row, n - 1);  // past N: last row, unused
-    wrow[nt] = w + (size_t)row * (k >> 1) + frag_h * 16;
-    srow[nt] = scales + (size_t)row * groups;
-  }
-  // staging: 64 rows x 16 units of 16 bytes, four units per thread
-  const uint8_t* xsrc[4];
-  uint32_t xunit[4], xdst[4];
-#pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    const uint32_t u = tid + 256 * i, row = u >> 4;
-    xunit[i] = (u & 15u) * 16u;
-    xsrc[i] = xq + (size_t)min(m0 + row, m - 1) * k;
-    xdst[i] = row * kRow + xunit[i];
-  }
-  auto load_x = [&](uint32_t stage, uint4 (&r)[4]) {
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const uint32_t at = stage * kStage + xunit[i];
-      r[i] = *reinterpret_cast<const uint4*>(xsrc[i] + (at < k ? at : 0u));
-    }
-  };
-  // codes past the end of K are parked as zeros: their products vanish whatever B holds
-  auto park_x = [&](uint32_t stage, int buf, const uint4 (&r)[4]) {
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const uint32_t keep = stage * kStage + xunit[i] < k ? 0xFFFFFFFFu : 0u;
-      uint4 v;
-      v.x = __builtin_amdgcn_perm(r[i].y, r[i].x, 0x06040200u) & keep;
-      v.y = __builtin_amdgcn_perm(r[i].y, r[i].x, 0x07050301u) & keep;
-      v.z = __builtin_amdgcn_perm(r[i].w, r[i].z, 0x06040200u) & keep;
-      v.w = __builtin_amdgcn_perm(r[i].w, r[i].z, 0x07050301u) & keep;
-      *reinterpret_cast<uint4*>(&s_x[buf][xdst[i]]) = v;
-    }
-  };
-  struct StageWeights {
-    uint4 w[4][WN];  // the weight bytes of a stage's four chunks
-    ST s[4][WN];     // and the scale of the group each of them lies in, as stored: a
-                     // conversion here would make the wave wait for the load it just issued
-  };
-  // A stage's chunks are requested together (a lane's four 16-byte pieces share one 128-byte
-  // line of its weight row), two stages before they are used.
-  auto load_stage = [&](uint32_t stage, StageWeights& d) {
-#pragma unroll
-    for (int c = 0; c < 4; ++c) {
-      const uint32_t code = stage * kStage + 64u * c;
-      const uint32_t kc = code < k ? code : 0u;  // past K: the row's start again, never used
-#pragma unroll
-      for (int nt = 0; nt < WN; ++nt) {
-        d.w[c][nt] = *reinterpret_cast<const uint4*>(wrow[nt] + (kc >> 1));
-        d.s[c][nt] = srow[nt][kc >> shift];
-      }
-    }
-  };
-
-  v16i_t acc[MT][WN];
-  float accf[MT][WN][16];
-#pragma unroll
-  for (int mt = 0; mt < MT; ++mt)
-#pragma unroll
-    for (int nt = 0; nt < WN; ++nt)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        acc[mt][nt][r] = 0;
-        accf[mt][nt][r] = 0.f;
-      }
-  const v16i_t zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
-
-  uint4 xr[4];
-  StageWeights ring[2];
-  load_x(0, xr);
-  load_stage(0, ring[0]);
-  load_stage(1, ring[1]);
-  park_x(0, 0, xr);
-  __syncthreads();
-
-  // One stage: x from LDS buffer `buf`, weights from `sw`, which is requested again for two
-  // stages ahead once its last chunk is consumed.  Every stage issues the same loads in the
-  // same order whatever K is (addresses past K are clamped, chunks past K multiply zeros and
-  // are fused with a zero scale), so the waits the compiler places count exactly the loads
-  // that are younger than the one needed — a branch around a load would make it wait for all.
-  auto run_stage = [&](uint32_t stage, int buf, StageWeights& sw) {
-    load_x(stage + 1, xr);
-    const uint32_t first_chunk = stage * 4u;
-    // larger groups: boundaries fall on stages
-    const bool stage_opens = GSH ? true : (stage & (stages_per_group - 1)) == 0;
-    const bool stage_closes = GSH ? true : ((stage + 1) & (stages_per_group - 1)) == 0;
-    float ws[4][WN];
-#pragma unroll
-    for (int c = 0; c < 4; ++c)
-#pragma unroll
-      for (int nt = 0; nt < WN; ++nt) ws[c][nt] = scale_f32<ST>(&sw.s[c][nt], 0);
-#pragma unroll
-    for (int c = 0; c < 4; ++c) {
-      const bool valid = first_chunk + c < chunks_total;
-      const bool opens_static = GSH != 0 && (c % kChunksPerGroup) == 0;
-      const bool closes = GSH ? ((c + 1) % kChunksPerGroup) == 0 : (stage_closes && c == 3);
-      if (GSH == 0 && stage_opens && c == 0) {
-#pragma unroll
-        for (int mt = 0; mt < MT; ++mt)
-#pragma unroll
-          for (int nt = 0; nt < WN; ++nt) acc[mt][nt] = zero;
-      }
-#pragma unroll
-      for (int s = 0; s < 2; ++s) {
-        v4i_t a[MT];
-#pragma unroll
-        for (int mt = 0; mt < MT; ++mt)
-          a[mt] = *reinterpret_cast<const v4i_t*>(
-              &s_x[buf][(mt * 32 + frag_row) * kRow + 64 * c + 32 * frag_h + 16 * s]);
-#pragma unroll
-        for (int nt = 0; nt < WN; ++nt) {
-          const uint32_t w0 = (s == 0 ? sw.w[c][nt].x : sw.w[c][nt].z) ^ 0x88888888u;
-          const uint32_t w1 = (s == 0 ? sw.w[c][nt].y : sw.w[c][nt].w) ^ 0x88888888u;
-          v4i_t b;
-          b[0] = (int)((w0 << 4) & 0xF0F0F0F0u);
-          b[1] = (int)(w0 & 0xF0F0F0F0u);
-          b[2] = (int)((w1 << 4) & 0xF0F0F0F0u);
-          b[3] = (int)(w1 & 0xF0F0F0F0u);
-#pragma unroll
-          for (int mt = 0; mt < MT; ++mt)
-            acc[mt][nt] = __builtin_amdgcn_mfma_i32_32x32x32_i8(
-                a[mt], b, (opens_static && s == 0) ? zero : acc[mt][nt], 0, 0, 0);
-        }
-      }
-      if (c == 3) load_stage(stage + 2, sw);
-      if (closes) {
-#pragma unroll
-        for (int nt = 0; nt < WN; ++nt) {
-          // an fp16 scale / 16 is always exact in f32; an f32 scale below 2^-122 may not be
-          const float ws16 = ws[c][nt] * 0.0625f;
-          const bool exact = sizeof(ST) == 2 || __all(ws16 * 16.0f == ws[c][nt]);
-          const float mult = valid ? (exact ? ws16 : ws[c][nt]) : 0.f;  // past K: accf + 0 * 0
-          const int down = exact ? 0 : 4;
-#pragma unroll
-          for (int mt = 0; mt < MT; ++mt)
-#pragma unroll
-            for (int r = 0; r < 16; ++r) {
-              const int32_t sum = sizeof(ST) == 2 ? acc[mt][nt][r] : acc[mt][nt][r] >> down;
-              accf[mt][nt][r] = fmaf((float)sum, mult, accf[mt][nt][r]);
-            }
-        }
-      }
-    }
-    park_x(stage + 1, buf ^ 1, xr);
-    __syncthreads();
-    // nothing of the next stage moves up here: its weights were requested one stage later
-    // and expanding them early would wait for those requests
-    __builtin_amdgcn_sched_barrier(0);
-  };
-  for (uint32_t stage = 0; stage < stages; stage += 2) {
-    run_stage(stage, 0, ring[0]);
-    run_stage(stage + 1, 1, ring[1]);  // past the last stage: zeros, fused with a zero scale
-  }
-
-#pragma unroll
-  for (int nt = 0; nt < WN; ++nt) {
-    const uint32_t col = n0 + nt * 32 + frag_row;
-    const float b = (bias && col < n) ? bias[col] : 0.f;
-#pragma unroll
-    for (int mt = 0; mt < MT; ++mt)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const uint32_t row = m0 + mt * 32 + 8 * (r / 4) + 4 * frag_h + (r % 4);
-        if (row < m && col < n) out[(size_t)row * n + col] = fmaf(accf[mt][nt][r], xs[row], b);
-      }
-  }
-}
-
-// Matrix-core form with both operands through LDS: eight waves, workgroup tile
+// (Weights loaded straight from global memory into the operand registers, without LDS, were
+// measured 1.5 x slower: a lane's own 16 bytes of its own row make every quad of lanes touch
+// four cache lines, and the vector cache's tag lookups become the bound.)
+//
+// Both operands go through LDS: eight waves, workgroup tile
 // (64 * MT) x 256, wave (wm, wn) = (32 * MT) ... rows wm and 64 columns wn.  The packed weight
 // bytes are staged as they are (coalesced 16-byte loads, 128 bytes of a row per stage) and
 // expanded to the bytes 16 * q in registers after the LDS read, so LDS holds a quarter of what
@@ -716,42 +520,19 @@ int32_t launch_w4a8(krm_ctx* ctx, krm_buf xq, krm_buf xs, krm_buf w, krm_buf sca
     return launched(ctx, "linear_w4a8_rows_kernel");
   }
   if (m > 8 && group >= 64 && group <= kMaxGroupTimes16 && aligned(xq, 16) && aligned(w, 16)) {
-    const uint32_t n_blocks = (n + 255) / 256;
-    const char* form = getenv("KRM_W4A8_FORM");
-    if (!form || strcmp(form, "direct") != 0) {
-      // rows of 128 per workgroup when that still covers most of the chip, else 64
-      const bool tall = getenv("KRM_W4A8_TALL") != nullptr;
-      const uint32_t m_blocks = tall ? (m + 127) / 128 : (m + 63) / 64;
-      const uint64_t blocks = (uint64_t)((n_blocks + 7) / 8) * 8u * m_blocks;
-      if (blocks <= 0x7fffffffull) {
-#define KRM_W4A8_TILE(GSH, MT)                                                                  \
-  hipLaunchKernelGGL((linear_w4a8_tile_kernel<ST, GSH, MT>), dim3((uint32_t)blocks), dim3(512), \
-                     0, ctx->stream, ptr<const uint8_t>(xq), pxs, ptr<const uint8_t>(w), ps,   \
-                     pb, po, m, n, k, shift, m_blocks, n_blocks)
-#define KRM_W4A8_TILE_G(GSH) \
-  do { if (tall) KRM_W4A8_TILE(GSH, 2); else KRM_W4A8_TILE(GSH, 1); } while (0)
-        if (shift == 6) KRM_W4A8_TILE_G(6);
-        else if (shift == 7) KRM_W4A8_TILE_G(7);
-        else if (shift == 8) KRM_W4A8_TILE_G(8);
-        else KRM_W4A8_TILE_G(0);
-#undef KRM_W4A8_TILE_G
-#undef KRM_W4A8_TILE
-        return launched(ctx, "linear_w4a8_tile_kernel");
-      }
-    }
-    const uint32_t m_blocks = (m + 63) / 64;
+    const uint32_t m_blocks = (m + 63) / 64, n_blocks = (n + 255) / 256;
     const uint64_t blocks = (uint64_t)((n_blocks + 7) / 8) * 8u * m_blocks;
     if (blocks <= 0x7fffffffull) {
-#define KRM_W4A8_MFMA(GSH)                                                                    \
-  hipLaunchKernelGGL((linear_w4a8_mfma_kernel<ST, GSH>), dim3((uint32_t)blocks), dim3(256), 0,  \
-                     ctx->stream, ptr<const uint8_t>(xq), pxs, ptr<const uint8_t>(w), ps, pb,  \
-                     po, m, n, k, shift, m_blocks, n_blocks)
-      if (shift == 6) KRM_W4A8_MFMA(6);
-      else if (shift == 7) KRM_W4A8_MFMA(7);
-      else if (shift == 8) KRM_W4A8_MFMA(8);
-      else KRM_W4A8_MFMA(0);
-#undef KRM_W4A8_MFMA
-      return launched(ctx, "linear_w4a8_mfma_kernel");
+#define KRM_W4A8_TILE(GSH)                                                                     \
+  hipLaunchKernelGGL((linear_w4a8_tile_kernel<ST, GSH, 1>), dim3((uint32_t)blocks), dim3(512), \
+                     0, ctx->stream, ptr<const uint8_t>(xq), pxs, ptr<const uint8_t>(w), ps,  \
+                     pb, po, m, n, k, shift, m_blocks, n_blocks)
+      if (shift == 6) KRM_W4A8_TILE(6);
+      else if (shift == 7) KRM_W4A8_TILE(7);
+      else if (shift == 8) KRM_W4A8_TILE(8);
+      else KRM_W4A8_TILE(0);
+#undef KRM_W4A8_TILE
+      return launched(ctx, "linear_w4a8_tile_kernel");
     }
   }
   const dim3 grid((n + 3) / 4, m < 65535u ? m : 65535u);
