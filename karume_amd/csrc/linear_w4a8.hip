@@ -438,13 +438,15 @@ void linear_w4a8_tile_kernel(
               &s_a[buf][a_base + mt * 32 * kRowA + 64 * c + 16 * s]);
 #pragma unroll
         for (int nt = 0; nt < WN; ++nt) {
-          const uint32_t w0 = (s == 0 ? braw[nt].x : braw[nt].z) ^ 0x88888888u;
-          const uint32_t w1 = (s == 0 ? braw[nt].y : braw[nt].w) ^ 0x88888888u;
+          // (w ^ c) & m is one three-input bit operation; the shifted form folds the shift of
+          // the constant: ((w ^ 0x88888888) << 4) & m == ((w << 4) ^ 0x80808080) & m
+          const uint32_t w0 = s == 0 ? braw[nt].x : braw[nt].z;
+          const uint32_t w1 = s == 0 ? braw[nt].y : braw[nt].w;
           v4i_t b;
-          b[0] = (int)((w0 << 4) & 0xF0F0F0F0u);
-          b[1] = (int)(w0 & 0xF0F0F0F0u);
-          b[2] = (int)((w1 << 4) & 0xF0F0F0F0u);
-          b[3] = (int)(w1 & 0xF0F0F0F0u);
+          b[0] = (int)(((w0 << 4) ^ 0x80808080u) & 0xF0F0F0F0u);
+          b[1] = (int)((w0 ^ 0x88888888u) & 0xF0F0F0F0u);
+          b[2] = (int)(((w1 << 4) ^ 0x80808080u) & 0xF0F0F0F0u);
+          b[3] = (int)((w1 ^ 0x88888888u) & 0xF0F0F0F0u);
 #pragma unroll
           for (int mt = 0; mt < MT; ++mt)
             acc[mt][nt] = __builtin_amdgcn_mfma_i32_32x32x32_i8(
