@@ -466,6 +466,168 @@ void gemm_i4_f16_kernel(const XT* __restrict__ x, const uint32_t* __restrict__ w
   }
 }
 
+// ---------------------------------------------------------------- packed weights in LDS
+//
+// Eight waves, workgroup tile (64 * MT) x 256, wave (wm, wn) = 32 * MT rows x 64 columns, K in
+// stages of 128 codes.  The weight bytes are staged as they are — coalesced 16-byte loads, a
+// quarter of the LDS bytes the dequantised fp16 tile takes — and every wave dequantises the
+// words of its own 64 columns after reading them back: lane (n = lane % 32, h = lane / 32)
+// reads 16 bytes = codes 64c + 32h .. + 31 of column n per 64-code chunk, word j of which is
+// the B operand of the chunk's MFMA step j (fp16(u - 8) * fp16(scale), order
+// c0,c4,c1,c5,c2,c6,c3,c7); the A operand of that step is x[m][64c + 32h + 8j ..] in the
+// same order, 16 bytes of the staged x row.  The same arithmetic as the kernel above, so the
+// two agree up to the order of the f32 additions.  Two waves share a SIMD: one wave's
+// dequantisation runs under the other's MFMAs.  Every stage issues the same loads whatever K
+// is (clamped addresses; x past K is parked as zeros).
+template <typename XT, typename ST, int MT>
+__global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2)))
+void gemm_i4_f16_packed_kernel(const XT* __restrict__ x, const uint8_t* __restrict__ w,
+                               const ST* __restrict__ scales, const XT* __restrict__ bias,
+                               XT* __restrict__ out, uint32_t m, uint32_t n, uint32_t k,
+                               uint32_t group_shift, uint32_t m_blocks, uint32_t n_blocks) {
+  constexpr int WN = 2;
+  constexpr int BM = 2 * 32 * MT, BN = 256;
+  constexpr int kStage = 128;                 // codes per LDS stage
+  constexpr int kRowA = kStage * 2 + 16;      // bytes per LDS row of fp16 x
+  constexpr int kRowB = kStage / 2 + 16;      // bytes per LDS row of packed weights
+  constexpr int kAUnits = BM * (kStage / 8) / 512;  // 8-element units of x per thread and stage
+  __shared__ __align__(16) uint8_t s_a[2][BM * kRowA];
+  __shared__ __align__(16) uint8_t s_b[2][BN * kRowB];
+  __shared__ _Float16 s_s[2][BN][2];
+
+  const uint32_t xcd = blockIdx.x & 7u, slot = blockIdx.x >> 3;
+  const uint32_t mb = slot % m_blocks, nb = (slot / m_blocks) * 8u + xcd;
+  if (nb >= n_blocks) return;  // the whole workgroup leaves before any barrier
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = wave >> 2, wn = wave & 3;
+  const int frag_row = lane & 31, frag_h = lane >> 5;
+  const uint32_t m0 = mb * BM, n0 = nb * BN;
+  const uint32_t groups = k >> group_shift;
+  const uint32_t stages = (k + kStage - 1) / kStage;
+
+  // staging roles: x rows in 16 units of 8 elements (rows tid / 16 + 32 i), weight rows in 4
+  // units of 16 bytes (rows tid / 4 + 128 i), one scale row per thread of the first four waves
+  const uint32_t arow0 = tid >> 4, aunit = (tid & 15u) * 8u;      // element offset in the stage
+  const uint32_t brow0 = tid >> 2, bunit = (tid & 3u) * 16u;      // byte offset in the stage
+  const ST* ssrc = scales + (size_t)min(n0 + (uint32_t)(tid & 255), n - 1) * groups;
+
+  struct Staged {
+    Acts8<XT> a[kAUnits];
+    uint4 b[2];
+  };
+  auto load_stage = [&](uint32_t stage, Staged& d) {
+    const uint32_t a_at = stage * kStage + aunit, b_at = stage * (kStage / 2) + bunit;
+    const uint32_t a_off = a_at < k ? a_at : 0u, b_off = b_at < (k >> 1) ? b_at : 0u;
+#pragma unroll
+    for (int i = 0; i < kAUnits; ++i)
+      d.a[i].load(x + (size_t)min(m0 + arow0 + 32u * i, m - 1) * k + a_off);
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+      d.b[i] = *reinterpret_cast<const uint4*>(
+          w + (size_t)min(n0 + brow0 + 128u * i, n - 1) * (k >> 1) + b_off);
+  };
+  auto park_stage = [&](uint32_t stage, int buf, Staged& d) {
+    const uint32_t keep = stage * kStage + aunit < k ? 0xFFFFFFFFu : 0u;
+#pragma unroll
+    for (int i = 0; i < kAUnits; ++i) {
+      uint4 v = d.a[i].paired();
+      v.x &= keep; v.y &= keep; v.z &= keep; v.w &= keep;  // past K: zeros, whatever B holds
+      *reinterpret_cast<uint4*>(&s_a[buf][(arow0 + 32u * i) * kRowA + aunit * 2u]) = v;
+    }
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+      *reinterpret_cast<uint4*>(&s_b[buf][(brow0 + 128u * i) * kRowB + bunit]) = d.b[i];
+    // The stage's (at most two) group scales of this thread's column, fetched here by the first
+    // four waves.  (Requested a stage ahead like the tiles, or all at once into an LDS table,
+    // measured 5-8 % slower: every lane's scale sits in another cache line.)
+    if (tid < 256) {
+      const uint32_t c0 = stage * kStage, c1 = stage * kStage + 64u;
+      s_s[buf][tid][0] = scale_from_bits<ST>(scale_bits<ST>(ssrc, (c0 < k ? c0 : 0u) >> group_shift));
+      s_s[buf][tid][1] = scale_from_bits<ST>(scale_bits<ST>(ssrc, (c1 < k ? c1 : 0u) >> group_shift));
+    }
+  };
+
+  float16_t acc[MT][WN];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+    for (int nt = 0; nt < WN; ++nt)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[mt][nt][r] = 0.f;
+
+  Staged staged;
+  load_stage(0, staged);
+  park_stage(0, 0, staged);
+  __syncthreads();
+
+  const uint32_t a_base = (uint32_t)((wm * 32 * MT + frag_row) * kRowA + 64 * frag_h);
+  const uint32_t b_base = (uint32_t)((wn * 64 + frag_row) * kRowB + 16 * frag_h);
+  auto run_stage = [&](uint32_t stage, int buf) {
+    load_stage(stage + 1, staged);
+    // the requests stay here, a whole stage ahead of their use (left alone, the scheduler
+    // moves them down to the parking code, where their latency is in the open)
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int c = 0; c < 2; ++c) {
+      uint4 braw[WN];
+      _Float16 ws[WN];
+#pragma unroll
+      for (int nt = 0; nt < WN; ++nt) {
+        braw[nt] = *reinterpret_cast<const uint4*>(&s_b[buf][b_base + nt * 32 * kRowB + 32 * c]);
+        ws[nt] = s_s[buf][wn * 64 + nt * 32 + frag_row][c];
+      }
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        half8_t a[MT];
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt)
+          a[mt] = *reinterpret_cast<const half8_t*>(
+              &s_a[buf][a_base + mt * 32 * kRowA + 128 * c + 16 * j]);
+#pragma unroll
+        for (int nt = 0; nt < WN; ++nt) {
+          const uint32_t word = j == 0 ? braw[nt].x : j == 1 ? braw[nt].y : j == 2 ? braw[nt].z
+                                                                                  : braw[nt].w;
+          const half8_t b = __builtin_bit_cast(half8_t, dequant_word(word, ws[nt]));
+#pragma unroll
+          for (int mt = 0; mt < MT; ++mt)
+            acc[mt][nt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[mt], b, acc[mt][nt], 0, 0, 0);
+        }
+      }
+    }
+    park_stage(stage + 1, buf ^ 1, staged);
+    __syncthreads();
+  };
+  for (uint32_t stage = 0; stage < stages; stage += 2) {
+    run_stage(stage, 0);
+    run_stage(stage + 1, 1);  // past the last stage: x is zeros
+  }
+
+#pragma unroll
+  for (int nt = 0; nt < WN; ++nt) {
+    const uint32_t col = n0 + wn * 64 + nt * 32 + frag_row;
+    const float b = (bias && col < n) ? bias_f32<XT>(bias, col) : 0.f;
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const uint32_t row = m0 + wm * 32 * MT + mt * 32 + 8 * (r / 4) + 4 * frag_h + (r % 4);
+        if (row < m && col < n) store_out<XT>(out, (size_t)row * n + col, acc[mt][nt][r] + b);
+      }
+  }
+}
+
+template <typename XT, typename ST, int MT>
+int32_t launch_packed(krm_ctx* ctx, krm_buf x, krm_buf w, krm_buf scales, krm_buf bias,
+                      krm_buf out, uint32_t m, uint32_t n, uint32_t k, uint32_t group_shift) {
+  const uint32_t m_blocks = (m + 64 * MT - 1) / (64 * MT), n_blocks = (n + 255) / 256;
+  const uint64_t total = (uint64_t)((n_blocks + 7) / 8) * 8 * m_blocks;
+  if (total > 0x7fffffffull) return fail(ctx, KRM_ERR_VALIDATION, "linear: grid too large");
+  gemm_i4_f16_packed_kernel<XT, ST, MT><<<dim3((unsigned)total), dim3(512), 0, ctx->stream>>>(
+      ptr<const XT>(x), ptr<const uint8_t>(w), ptr<const ST>(scales), ptr<const XT>(bias),
+      ptr<XT>(out), m, n, k, group_shift, m_blocks, n_blocks);
+  return launched(ctx, "gemm_i4_f16_packed_kernel");
+}
+
 template <typename XT, typename ST, int WM, int WN, int KC, int KS, int DEPTH, bool PIPE = false>
 int32_t launch(krm_ctx* ctx, krm_buf x, krm_buf w, krm_buf scales, krm_buf bias, krm_buf out,
                uint32_t m, uint32_t n, uint32_t k, uint32_t group_shift) {
@@ -507,6 +669,13 @@ int32_t pick_tile(krm_ctx* ctx, krm_buf x, krm_buf w, krm_buf scales, krm_buf bi
   // four chunks in flight.  Fewer (a narrow output with a long K, or few rows): 128 x 64 tiles
   // whose two wave groups split every 128-code chunk of K, or 64 x 64 tiles with four groups.
   const uint64_t cus = (uint64_t)ctx->num_cus;
+  // 128 x 256 tiles with the packed weights in LDS when they cover most of the chip (measured
+  // 77 us against 85 us on the 512 x 11008 x 4096 up-projection; with fewer tiles than that the
+  // forms below, which split K inside a workgroup, are faster).
+  const uint64_t packed_tiles = (uint64_t)((m + 127) / 128) * ((n + 255) / 256);
+  if (m > 64 && group >= 64 && k % 8 == 0 && aligned(w, 16) && aligned(x, 16) &&
+      packed_tiles * 5 >= cus * 3)
+    return launch_packed<XT, ST, 2>(ctx, x, w, scales, bias, out, m, n, k, group_shift);
   const uint64_t tiles = (uint64_t)((m + 127) / 128) * ((n + 127) / 128);
   if (m > 64 && tiles >= cus)
     return launch<XT, ST, 2, 2, 64, 1, 4, true>(ctx, x, w, scales, bias, out, m, n, k, group_shift);

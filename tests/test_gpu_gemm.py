@@ -66,7 +66,10 @@ def test_config1_prefill_gemm(gpu_ctx, m, n, k, g, io):
 
 @pytest.mark.parametrize("shape", [(17, 64, 64, 16), (65, 68, 48, 16), (130, 200, 96, 32),
                                    (100, 129, 320, 64), (300, 1000, 2048, 128),
-                                   (64, 256, 512, 128), (33, 8, 128, 128)])
+                                   (64, 256, 512, 128), (33, 8, 128, 128),
+                                   # enough 128 x 256 tiles for the packed-weights form, with
+                                   # ragged edges in M, N and K (K ends inside a 128-code stage)
+                                   (300, 13349, 320, 64)])
 def test_gemm_edges_exact_weights(gpu_ctx, shape):
     """Tile edges in M, N and K (K not a multiple of the 64-code stage, N not a multiple of
     the tile) with power-of-two scales: dequantised weights are exact in fp16, x is fp16, so
