@@ -3,14 +3,14 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W]
 
-A step is one int4 g128 GEMV at M=1, K=N=4096 (BASELINE config 0: fp16 activations and
+A step is one int4 g128 GEMV at M=1, K=N=4096 (benchmark config 0: fp16 activations and
 scales, f32 accumulation, fp16 output) through the C ABI.  Steps rotate over enough distinct
 weight buffers (> 512 MiB) that no step finds its weights in the 256 MB Infinity Cache, so
 `value` is an HBM number; the cache-resident figure is reported beside it.  Inputs are
 resident in HBM before the timed region; timing uses HIP events recorded on the stream the
 kernels are launched on.
 
-Prints ONE JSON line.  Extra keys report the other BASELINE configs measured the same way.
+Prints ONE JSON line.  Extra keys report the other benchmark configs measured the same way.
 """
 from __future__ import annotations
 
@@ -108,7 +108,7 @@ def bench_gemv(ctx, ka, rng, steps: int, warmup: int, m: int, n: int, k: int, g:
 
 
 def bench_attention(ctx, ka, rng, steps: int, warmup: int, copies: int):
-    """BASELINE config 2: B=1, H=32, Hkv=8, D=128, 4095 cached rows + this step's row, fp16."""
+    """benchmark config 2: B=1, H=32, Hkv=8, D=128, 4095 cached rows + this step's row, fp16."""
     heads, kv_heads, depth, past, cap = 32, 8, 128, 4095, 4096
     slots = []
     for _ in range(copies):
@@ -139,7 +139,7 @@ def bench_attention(ctx, ka, rng, steps: int, warmup: int, copies: int):
 
 
 def bench_gemm(ctx, ka, rng, steps: int, warmup: int, m: int, n: int, k: int, g: int):
-    """BASELINE config 1: prefill GEMM on the matrix cores, fp16 activations and output."""
+    """benchmark config 1: prefill GEMM on the matrix cores, fp16 activations and output."""
     copies = 4
     weights, scales = [], []
     for _ in range(copies):
@@ -193,7 +193,7 @@ def bench_w4a8(ctx, ka, rng, steps: int, warmup: int, m: int, n: int, k: int, g:
 
 
 def bench_model(ctx, ka, io_dtype, kv_dtype, prompt_len: int = 128, new_tokens: int = 256):
-    """BASELINE config 4: random-init 1.1B-shape int4 decoder, 128-token random prompt, 256
+    """benchmark config 4: random-init 1.1B-shape int4 decoder, 128-token random prompt, 256
     greedy decode steps, batch 1.  The decode steps replay one recorded step (lengths and the
     fed-back token stay on the device); timing covers the replays only, then prefill + decode."""
     from karume_amd.decoder import LlamaConfig, LlamaDecoderSession, random_weights

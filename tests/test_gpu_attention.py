@@ -105,7 +105,7 @@ def test_decode_split_k(gpu_ctx, case, io, kv):
 
 
 def test_config2_decode_attention(gpu_ctx):
-    """BASELINE config 2: B=1, H=32, Hkv=8, D=128, 4095 slot rows + this step's row, fp16."""
+    """benchmark config 2: B=1, H=32, Hkv=8, D=128, 4095 slot rows + this step's row, fp16."""
     case = StateCase("config 2", 1, 32, 8, 1, 128, 4096, 0, 4095, 1)
     x = random_state_inputs(case, seed=2, f16_values=True)
     want = oracle_state_attention(case, x)
@@ -284,7 +284,7 @@ def test_chain_prefill_then_decode_on_device(gpu_ctx):
 # ---------------------------------------------------------------------------- ragged batch
 
 def test_config3_ragged_batch_equals_one_at_a_time(gpu_ctx):
-    """BASELINE config 3: 16 sequences, KV lengths ~ U{128..4096} (seeded), packed with
+    """benchmark config 3: 16 sequences, KV lengths ~ U{128..4096} (seeded), packed with
     prefix-sum offsets, H=32, Hkv=8, D=128, fp16 KV.  One launch; every sequence is then run
     alone through krm_attention_state and the bits must agree; a few are checked against the
     oracle (atol 5e-6 on f32 output)."""

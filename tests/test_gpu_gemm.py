@@ -41,7 +41,7 @@ def check(got, want, exact_weights=False):
 @pytest.mark.parametrize("m,n,k,g", [(512, 11008, 4096, 128), (512, 4096, 11008, 128)])
 @pytest.mark.parametrize("io", [np.float16, np.float32])
 def test_config1_prefill_gemm(gpu_ctx, m, n, k, g, io):
-    """BASELINE config 1 at full size (up- and down-projection); 192 sampled output columns
+    """benchmark config 1 at full size (up- and down-projection); 192 sampled output columns
     are checked against the f64 oracle, all rows."""
     rng = np.random.default_rng(n + k)
     packed, _q, scale = helpers.synthetic_int4(rng, n, k, g)

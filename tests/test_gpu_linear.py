@@ -101,7 +101,7 @@ def test_linear_packed_equals_preexpanded_through_same_kernel(gpu_ctx):
 
 @pytest.mark.parametrize("io", [np.float16, np.float32])
 def test_linear_config0_gemv(gpu_ctx, io):
-    """BASELINE config 0: M=1, K=N=4096, int4 g128, fp16 scales |N(0,0.02)|, x ~ N(0,1) in fp16.
+    """benchmark config 0: M=1, K=N=4096, int4 g128, fp16 scales |N(0,0.02)|, x ~ N(0,1) in fp16.
     f32 output: atol 2e-5 (|out| ~ 5, f32 accumulation; measured worst 4e-6), rtol 0.
     fp16 output: the oracle's f32 result rounded to fp16, within 1 fp16 ulp."""
     rng = np.random.default_rng(40960)
@@ -124,7 +124,7 @@ def test_linear_config0_gemv(gpu_ctx, io):
 
 @pytest.mark.parametrize("io", [np.float16, np.float32])
 def test_linear_batched_rows_equal_single_rows_bitwise(gpu_ctx, io):
-    """BASELINE config 3 (GEMV part): M = 16 in one launch vs the rows in smaller launches.
+    """benchmark config 3 (GEMV part): M = 16 in one launch vs the rows in smaller launches.
     f32 activations: the per-row reduction order does not depend on M, so the bits agree with
     single-row launches.  fp16 activations: batches of 2..16 rows run on the matrix cores,
     where a row's bits do not depend on the batch it sits in; a single row takes the
