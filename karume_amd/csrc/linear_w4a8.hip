@@ -49,9 +49,25 @@ __device__ inline bool is_nan_bits(float v) {
 
 // ------------------------------------------------------------------------- quantize_rows
 //
-// One workgroup per row (grid-stride over rows), two passes over the row: |x| maximum with NaN
-// propagation, then the quotients.  x / s is the correctly rounded f32 division, so the codes
-// equal the CPU formula's for every input, also next to a rounding tie.
+// One workgroup per row (grid-stride over rows): |x| maximum with NaN propagation, then the
+// quotients.  Rows of up to 256 * 4 * kQuantCache elements stay in registers between the two
+// (one trip to memory, all loads in flight together); longer rows are read twice.  x / s is the
+// correctly rounded f32 division, so the codes equal the CPU formula's for every input, also
+// next to a rounding tie.
+constexpr int kQuantCache = 12;  // float4 per thread: rows of up to 12288 elements
+
+__device__ inline uint32_t quantize4(const float4& v, float s) {
+  const float f[4] = {v.x, v.y, v.z, v.w};
+  uint32_t packed = 0;
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    float r = rintf(f[e] / s);
+    r = is_nan_bits(r) ? 0.f : fminf(fmaxf(r, -127.f), 127.f);
+    packed |= ((uint32_t)(int32_t)r & 0xffu) << (8 * e);
+  }
+  return packed;
+}
+
 __global__ __launch_bounds__(256) void quantize_rows_kernel(const float* __restrict__ x,
                                                             uint32_t* __restrict__ xq,
                                                             float* __restrict__ xs,
@@ -59,19 +75,33 @@ __global__ __launch_bounds__(256) void quantize_rows_kernel(const float* __restr
   __shared__ float s_max[4];
   __shared__ uint32_t s_nan[4];
   const uint32_t quads = dim >> 2;
+  const bool cached = quads <= 256u * kQuantCache;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   for (uint32_t row = blockIdx.x; row < rows; row += gridDim.x) {
     const float4* xr = reinterpret_cast<const float4*>(x + (size_t)row * dim);
+    float4 cache[kQuantCache];
     float amax = 0.f;
     bool nan = false;
-    for (uint32_t i = threadIdx.x; i < quads; i += 256) {
-      const float4 v = xr[i];
+    auto fold = [&](const float4& v) {
       const float a[4] = {fabsf(v.x), fabsf(v.y), fabsf(v.z), fabsf(v.w)};
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
         nan = nan || is_nan_bits(a[e]);
         amax = fmaxf(amax, a[e]);  // ignores a NaN operand; the flag carries it
       }
+    };
+    if (cached) {
+#pragma unroll
+      for (int i = 0; i < kQuantCache; ++i) {
+        if (256u * i >= quads) break;  // uniform: the row ends before this stride
+        const uint32_t at = threadIdx.x + 256u * i;
+        cache[i] = xr[at < quads ? at : 0u];  // past the row: its first quad again, not folded
+      }
+#pragma unroll
+      for (int i = 0; i < kQuantCache; ++i)
+        if (threadIdx.x + 256u * i < quads) fold(cache[i]);
+    } else {
+      for (uint32_t i = threadIdx.x; i < quads; i += 256) fold(xr[i]);
     }
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) amax = fmaxf(amax, __shfl_xor(amax, off));
@@ -87,17 +117,14 @@ __global__ __launch_bounds__(256) void quantize_rows_kernel(const float* __restr
     if (row_nan) s = __uint_as_float(0x7fc00000u);
     if (threadIdx.x == 0) xs[row] = s;
     uint32_t* qr = xq + (size_t)row * quads;
-    for (uint32_t i = threadIdx.x; i < quads; i += 256) {
-      const float4 v = xr[i];
-      const float f[4] = {v.x, v.y, v.z, v.w};
-      uint32_t packed = 0;
+    if (cached) {
 #pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        float r = rintf(f[e] / s);
-        r = is_nan_bits(r) ? 0.f : fminf(fmaxf(r, -127.f), 127.f);
-        packed |= ((uint32_t)(int32_t)r & 0xffu) << (8 * e);
+      for (int i = 0; i < kQuantCache; ++i) {
+        const uint32_t at = threadIdx.x + 256u * i;
+        if (at < quads) qr[at] = quantize4(cache[i], s);
       }
-      qr[i] = packed;
+    } else {
+      for (uint32_t i = threadIdx.x; i < quads; i += 256) qr[i] = quantize4(xr[i], s);
     }
     __syncthreads();  // s_max / s_nan are rewritten by the next row
   }
