@@ -268,6 +268,13 @@ def cpu_baseline(n: int, k: int, g: int, budget_s: float = 12.0):
     result = {"value": algo * reps / dt / 1e9, "unit": "GB/s", "cores": cores, "kind": "port",
               "sample": f"{reps} repetitions of the config-0 GEMV (M=1,K=N=4096) in {dt:.1f} s"}
     result.update(cpu_decode_baseline(g))
+    # the integer-dot form of the same GEMV (quantiser + product) through the oracle, ~2 s
+    reps, t0 = 0, time.perf_counter()
+    while time.perf_counter() - t0 < 2.0 and reps < 2000:
+        oracle.linear_w4a8(x, packed, scale, bias, n, k, g)
+        reps += 1
+    dt = time.perf_counter() - t0
+    result["w4a8_gemv_us"] = round(dt / reps * 1e6, 1)
     return result
 
 
