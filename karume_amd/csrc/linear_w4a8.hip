@@ -521,6 +521,185 @@ void linear_w4a8_tile_kernel(
   }
 }
 
+// The same staging with a 128 x 256 workgroup tile, wave = 64 x 64, for groups of 64 or 128
+// codes.  Four 32 x 32 tiles per wave would need 64 int32 and 64 f32 accumulators at once, more
+// than two waves per SIMD leave room for, so the work is ordered by group: the group's weight
+// words are expanded once (both column tiles, all MFMA steps of the group), then each row tile
+// in turn runs its two MFMA chains over the group and is fused into its f32 accumulators — 32
+// int32 accumulators live at a time, and the expansion is shared by the two row tiles.
+template <typename ST, int GSH>
+__global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2)))
+void linear_w4a8_tall_kernel(
+    const uint8_t* __restrict__ xq, const float* __restrict__ xs, const uint8_t* __restrict__ w,
+    const ST* __restrict__ scales, const float* __restrict__ bias, float* __restrict__ out,
+    uint32_t m, uint32_t n, uint32_t k, uint32_t m_blocks, uint32_t n_blocks) {
+  static_assert(GSH == 6 || GSH == 7, "groups of 64 or 128 codes");
+  constexpr int MT = 2, WN = 2;
+  constexpr int BM = 128, BN = 256;
+  constexpr int kStage = 128;                          // codes per LDS stage
+  constexpr int kRowA = kStage + 16, kRowB = kStage / 2 + 16;
+  constexpr int kGroupsPerStage = kStage >> GSH;       // 2 or 1
+  constexpr int kStepsPerGroup = 1 << (GSH - 5);       // MFMA steps of 32 codes: 2 or 4
+  constexpr int kAUnits = BM * (kStage / 16) / 512;    // 16-byte units of xq per thread: 2
+  constexpr int kBUnits = BN * (kStage / 32) / 512;    // and of packed weights: 2
+  __shared__ __align__(16) uint8_t s_a[2][BM * kRowA];
+  __shared__ __align__(16) uint8_t s_b[2][BN * kRowB];
+  __shared__ __align__(16) float s_s[2][BN][2];
+
+  const uint32_t xcd = blockIdx.x & 7u, slot = blockIdx.x >> 3;
+  const uint32_t mb = slot % m_blocks, nb = (slot / m_blocks) * 8u + xcd;
+  if (nb >= n_blocks) return;  // the whole workgroup leaves before any barrier
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = wave >> 2, wn = wave & 3;
+  const int frag_row = lane & 31, frag_h = lane >> 5;
+  const uint32_t m0 = mb * BM, n0 = nb * BN;
+  const uint32_t groups = k >> GSH;
+  const uint32_t chunks_total = k >> 6;
+  const uint32_t stages = (k + kStage - 1) / kStage;
+
+  // staging roles: xq rows in 8 units of 16 bytes (rows tid / 8 + 64 i), weight rows in 4
+  // (rows tid / 4 + 128 i)
+  const uint32_t arow0 = tid >> 3, aunit = (tid & 7u) * 16u;
+  const uint32_t brow0 = tid >> 2, bunit = (tid & 3u) * 16u;
+  const ST* ssrc = scales + (size_t)min(n0 + (uint32_t)(tid & 255), n - 1) * groups;
+
+  struct Staged {
+    uint4 a[kAUnits];
+    uint4 b[kBUnits];
+    ST s[kGroupsPerStage];
+  };
+  auto load_stage = [&](uint32_t stage, Staged& d) {
+    const uint32_t a_at = stage * kStage + aunit, b_at = stage * (kStage / 2) + bunit;
+    const uint32_t a_off = a_at < k ? a_at : 0u, b_off = b_at < (k >> 1) ? b_at : 0u;
+#pragma unroll
+    for (int i = 0; i < kAUnits; ++i)
+      d.a[i] = *reinterpret_cast<const uint4*>(
+          xq + (size_t)min(m0 + arow0 + 64u * i, m - 1) * k + a_off);
+#pragma unroll
+    for (int i = 0; i < kBUnits; ++i)
+      d.b[i] = *reinterpret_cast<const uint4*>(
+          w + (size_t)min(n0 + brow0 + 128u * i, n - 1) * (k >> 1) + b_off);
+#pragma unroll
+    for (int j = 0; j < kGroupsPerStage; ++j) {
+      const uint32_t code = stage * kStage + (j << GSH);
+      d.s[j] = ssrc[(code < k ? code : 0u) >> GSH];
+    }
+  };
+  auto park_stage = [&](uint32_t stage, int buf, const Staged& d) {
+    const uint32_t keep = stage * kStage + aunit < k ? 0xFFFFFFFFu : 0u;
+#pragma unroll
+    for (int i = 0; i < kAUnits; ++i) {
+      uint4 v;
+      v.x = __builtin_amdgcn_perm(d.a[i].y, d.a[i].x, 0x06040200u) & keep;
+      v.y = __builtin_amdgcn_perm(d.a[i].y, d.a[i].x, 0x07050301u) & keep;
+      v.z = __builtin_amdgcn_perm(d.a[i].w, d.a[i].z, 0x06040200u) & keep;
+      v.w = __builtin_amdgcn_perm(d.a[i].w, d.a[i].z, 0x07050301u) & keep;
+      *reinterpret_cast<uint4*>(&s_a[buf][(arow0 + 64u * i) * kRowA + aunit]) = v;
+    }
+#pragma unroll
+    for (int i = 0; i < kBUnits; ++i)
+      *reinterpret_cast<uint4*>(&s_b[buf][(brow0 + 128u * i) * kRowB + bunit]) = d.b[i];
+    if (tid < 256) {
+#pragma unroll
+      for (int j = 0; j < kGroupsPerStage; ++j) s_s[buf][tid][j] = scale_f32<ST>(&d.s[j], 0);
+    }
+  };
+
+  float accf[MT][WN][16];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+    for (int nt = 0; nt < WN; ++nt)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) accf[mt][nt][r] = 0.f;
+  const v16i_t zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+
+  Staged staged;
+  load_stage(0, staged);
+  park_stage(0, 0, staged);
+  __syncthreads();
+
+  const uint32_t a_base = (uint32_t)((wm * 64 + frag_row) * kRowA + 32 * frag_h);
+  const uint32_t b_base = (uint32_t)((wn * 64 + frag_row) * kRowB + 16 * frag_h);
+  auto run_stage = [&](uint32_t stage, int buf) {
+    load_stage(stage + 1, staged);
+    __builtin_amdgcn_sched_barrier(0);  // the requests stay a stage ahead of their use
+#pragma unroll
+    for (int gi = 0; gi < kGroupsPerStage; ++gi) {
+      // codes 0 .. (1 << GSH) - 1 of the group = MFMA steps 0 .. kStepsPerGroup - 1;
+      // step st lies in chunk (gi << GSH) / 64 + st / 2, half st % 2
+      const int first_chunk_in_stage = (gi << GSH) >> 6;
+      const bool valid = stage * 2u + first_chunk_in_stage < chunks_total;
+      v4i_t bexp[WN][kStepsPerGroup];
+      float mult[WN];
+#pragma unroll
+      for (int nt = 0; nt < WN; ++nt) {
+#pragma unroll
+        for (int cc = 0; cc < kStepsPerGroup / 2; ++cc) {
+          const uint4 braw = *reinterpret_cast<const uint4*>(
+              &s_b[buf][b_base + nt * 32 * kRowB + 32 * (first_chunk_in_stage + cc)]);
+          const uint32_t words[4] = {braw.x, braw.y, braw.z, braw.w};
+#pragma unroll
+          for (int s = 0; s < 2; ++s) {
+            v4i_t b;
+            b[0] = (int)(((words[2 * s] << 4) ^ 0x80808080u) & 0xF0F0F0F0u);
+            b[1] = (int)((words[2 * s] ^ 0x88888888u) & 0xF0F0F0F0u);
+            b[2] = (int)(((words[2 * s + 1] << 4) ^ 0x80808080u) & 0xF0F0F0F0u);
+            b[3] = (int)((words[2 * s + 1] ^ 0x88888888u) & 0xF0F0F0F0u);
+            bexp[nt][2 * cc + s] = b;
+          }
+        }
+        const float ws = s_s[buf][wn * 64 + nt * 32 + frag_row][gi];
+        // an fp16 scale / 16 is exact in f32; an f32 scale may not be (subnormal quotient):
+        // then the sums are shifted instead (below)
+        mult[nt] = valid ? ws : 0.f;  // past K: accf + 0 * 0
+      }
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) {
+        v16i_t acc[WN];
+#pragma unroll
+        for (int st = 0; st < kStepsPerGroup; ++st) {
+          const v4i_t a = *reinterpret_cast<const v4i_t*>(
+              &s_a[buf][a_base + mt * 32 * kRowA + 64 * (first_chunk_in_stage + st / 2) +
+                        16 * (st & 1)]);
+#pragma unroll
+          for (int nt = 0; nt < WN; ++nt)
+            acc[nt] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, bexp[nt][st],
+                                                            st == 0 ? zero : acc[nt], 0, 0, 0);
+        }
+#pragma unroll
+        for (int nt = 0; nt < WN; ++nt) {
+          const float ws16 = mult[nt] * 0.0625f;
+          const bool exact = sizeof(ST) == 2 || __all(ws16 * 16.0f == mult[nt]);
+          const float factor = exact ? ws16 : mult[nt];
+          const int down = exact ? 0 : 4;
+#pragma unroll
+          for (int r = 0; r < 16; ++r) {
+            const int32_t sum = sizeof(ST) == 2 ? acc[nt][r] : acc[nt][r] >> down;
+            accf[mt][nt][r] = fmaf((float)sum, factor, accf[mt][nt][r]);
+          }
+        }
+      }
+    }
+    park_stage(stage + 1, buf ^ 1, staged);
+    __syncthreads();
+  };
+  for (uint32_t stage = 0; stage < stages; ++stage) run_stage(stage, (int)(stage & 1u));
+
+#pragma unroll
+  for (int nt = 0; nt < WN; ++nt) {
+    const uint32_t col = n0 + wn * 64 + nt * 32 + frag_row;
+    const float b = (bias && col < n) ? bias[col] : 0.f;
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const uint32_t row = m0 + wm * 64 + mt * 32 + 8 * (r / 4) + 4 * frag_h + (r % 4);
+        if (row < m && col < n) out[(size_t)row * n + col] = fmaf(accf[mt][nt][r], xs[row], b);
+      }
+  }
+}
+
 template <typename ST>
 int32_t launch_w4a8(krm_ctx* ctx, krm_buf xq, krm_buf xs, krm_buf w, krm_buf scales,
                     krm_buf bias, krm_buf out, uint32_t m, uint32_t n, uint32_t k,
@@ -549,7 +728,25 @@ int32_t launch_w4a8(krm_ctx* ctx, krm_buf xq, krm_buf xs, krm_buf w, krm_buf sca
     return launched(ctx, "linear_w4a8_rows_kernel");
   }
   if (m > 8 && group >= 64 && group <= kMaxGroupTimes16 && aligned(xq, 16) && aligned(w, 16)) {
-    const uint32_t m_blocks = (m + 63) / 64, n_blocks = (n + 255) / 256;
+    const uint32_t n_blocks = (n + 255) / 256;
+    // 128-row tiles for groups of 64 / 128 when they still cover most of the chip
+    const uint32_t tall_blocks = (m + 127) / 128;
+    if ((shift == 6 || shift == 7) &&
+        (uint64_t)tall_blocks * n_blocks * 5 >= (uint64_t)ctx->num_cus * 3) {
+      const uint64_t blocks = (uint64_t)((n_blocks + 7) / 8) * 8u * tall_blocks;
+      if (blocks <= 0x7fffffffull) {
+        if (shift == 6)
+          hipLaunchKernelGGL((linear_w4a8_tall_kernel<ST, 6>), dim3((uint32_t)blocks), dim3(512),
+                             0, ctx->stream, ptr<const uint8_t>(xq), pxs, ptr<const uint8_t>(w),
+                             ps, pb, po, m, n, k, tall_blocks, n_blocks);
+        else
+          hipLaunchKernelGGL((linear_w4a8_tall_kernel<ST, 7>), dim3((uint32_t)blocks), dim3(512),
+                             0, ctx->stream, ptr<const uint8_t>(xq), pxs, ptr<const uint8_t>(w),
+                             ps, pb, po, m, n, k, tall_blocks, n_blocks);
+        return launched(ctx, "linear_w4a8_tall_kernel");
+      }
+    }
+    const uint32_t m_blocks = (m + 63) / 64;
     const uint64_t blocks = (uint64_t)((n_blocks + 7) / 8) * 8u * m_blocks;
     if (blocks <= 0x7fffffffull) {
 #define KRM_W4A8_TILE(GSH)                                                                     \
