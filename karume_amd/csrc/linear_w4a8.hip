@@ -328,28 +328,29 @@ __global__ __launch_bounds__(256) void linear_w4a8_rows_kernel(
 // measured 1.5 x slower: a lane's own 16 bytes of its own row make every quad of lanes touch
 // four cache lines, and the vector cache's tag lookups become the bound.)
 //
-// Both operands go through LDS: eight waves, workgroup tile
-// (64 * MT) x 256, wave (wm, wn) = (32 * MT) ... rows wm and 64 columns wn.  The packed weight
+// Both operands go through LDS: eight waves, workgroup tile (64 * MT) x (128 * WN), wave
+// (wm, wn) = 32 * MT rows x 32 * WN columns (WN = 1 when 256-column tiles would leave a
+// quarter of the chip without work).  The packed weight
 // bytes are staged as they are (coalesced 16-byte loads, 128 bytes of a row per stage) and
 // expanded to the bytes 16 * q in registers after the LDS read, so LDS holds a quarter of what
 // dequantised bytes would take; xq is staged with its bytes regrouped (even, odd) as above.
 // The stage's group scales are staged too, already converted.  Two waves share a SIMD: one
 // wave's group flush (VALU) runs under the other's MFMAs.
-template <typename ST, int GSH, int MT>
+template <typename ST, int GSH, int MT, int WN>
 __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2)))
 void linear_w4a8_tile_kernel(
     const uint8_t* __restrict__ xq, const float* __restrict__ xs, const uint8_t* __restrict__ w,
     const ST* __restrict__ scales, const float* __restrict__ bias, float* __restrict__ out,
     uint32_t m, uint32_t n, uint32_t k, uint32_t group_shift, uint32_t m_blocks,
     uint32_t n_blocks) {
-  constexpr int WN = 2;                       // 32-column tiles per wave
-  constexpr int BM = 2 * 32 * MT, BN = 256;   // two wave rows, four wave columns
+  constexpr int BM = 2 * 32 * MT, BN = 4 * 32 * WN;  // two wave rows, four wave columns
   constexpr int kStage = 256;                 // codes per LDS stage
   constexpr int kRowA = kStage + 16;          // bytes per LDS row of xq
   constexpr int kRowB = kStage / 2 + 16;      // bytes per LDS row of packed weights
   constexpr int kChunksPerGroup = GSH ? (1 << (GSH - 6)) : 4;  // inside a stage
   constexpr int kScalesPerStage = GSH ? (kStage >> GSH) : 1;
   constexpr int kAUnits = BM * 16 / 512;      // 16-byte units of xq per thread and stage
+  constexpr int kBUnits = BN * 8 / 512;       // and of packed weights
   __shared__ __align__(16) uint8_t s_a[2][BM * kRowA];
   __shared__ __align__(16) uint8_t s_b[2][BN * kRowB];
   __shared__ __align__(16) float s_s[2][BN][4];
@@ -371,10 +372,10 @@ void linear_w4a8_tile_kernel(
   // (rows tid / 8 + 64 i), one scale row per thread; 32-bit offsets from the three bases
   const uint32_t arow0 = tid >> 4, aunit = (tid & 15u) * 16u;
   const uint32_t brow0 = tid >> 3, bunit = (tid & 7u) * 16u;
-  const ST* ssrc = scales + (size_t)min(n0 + (uint32_t)(tid & 255), n - 1) * groups;
+  const ST* ssrc = scales + (size_t)min(n0 + (uint32_t)(tid % BN), n - 1) * groups;
   struct Staged {
     uint4 a[kAUnits];
-    uint4 b[4];
+    uint4 b[kBUnits];
     ST s[kScalesPerStage];
   };
   // Requests only, clamped addresses: every stage issues the same loads in the same order.
@@ -386,7 +387,7 @@ void linear_w4a8_tile_kernel(
       d.a[i] = *reinterpret_cast<const uint4*>(
           xq + (size_t)min(m0 + arow0 + 32u * i, m - 1) * k + a_off);
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
+    for (int i = 0; i < kBUnits; ++i)
       d.b[i] = *reinterpret_cast<const uint4*>(
           w + (size_t)min(n0 + brow0 + 64u * i, n - 1) * (k >> 1) + b_off);
 #pragma unroll
@@ -408,9 +409,9 @@ void linear_w4a8_tile_kernel(
       *reinterpret_cast<uint4*>(&s_a[buf][(arow0 + 32u * i) * kRowA + aunit]) = v;
     }
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
+    for (int i = 0; i < kBUnits; ++i)
       *reinterpret_cast<uint4*>(&s_b[buf][(brow0 + 64u * i) * kRowB + bunit]) = d.b[i];
-    if (tid < 256) {
+    if (tid < BN) {
 #pragma unroll
       for (int j = 0; j < kScalesPerStage; ++j) s_s[buf][tid][j] = scale_f32<ST>(&d.s[j], 0);
     }
@@ -435,7 +436,7 @@ void linear_w4a8_tile_kernel(
   __syncthreads();
 
   const uint32_t a_base = (uint32_t)((wm * 32 * MT + frag_row) * kRowA + 32 * frag_h);
-  const uint32_t b_base = (uint32_t)((wn * 64 + frag_row) * kRowB + 16 * frag_h);
+  const uint32_t b_base = (uint32_t)((wn * 32 * WN + frag_row) * kRowB + 16 * frag_h);
   auto run_stage = [&](uint32_t stage, int buf) {
     load_stage(stage + 1, staged);
     const uint32_t first_chunk = stage * 4u;
@@ -483,7 +484,8 @@ void linear_w4a8_tile_kernel(
       if (closes) {
 #pragma unroll
         for (int nt = 0; nt < WN; ++nt) {
-          const float ws = s_s[buf][wn * 64 + nt * 32 + frag_row][GSH ? c / kChunksPerGroup : 0];
+          const float ws =
+              s_s[buf][wn * 32 * WN + nt * 32 + frag_row][GSH ? c / kChunksPerGroup : 0];
           // an fp16 scale / 16 is always exact in f32; an f32 scale below 2^-122 may not be
           const float ws16 = ws * 0.0625f;
           const bool exact = sizeof(ST) == 2 || __all(ws16 * 16.0f == ws);
@@ -509,7 +511,7 @@ void linear_w4a8_tile_kernel(
 
 #pragma unroll
   for (int nt = 0; nt < WN; ++nt) {
-    const uint32_t col = n0 + wn * 64 + nt * 32 + frag_row;
+    const uint32_t col = n0 + wn * 32 * WN + nt * 32 + frag_row;
     const float b = (bias && col < n) ? bias[col] : 0.f;
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt)
@@ -747,16 +749,22 @@ int32_t launch_w4a8(krm_ctx* ctx, krm_buf xq, krm_buf xs, krm_buf w, krm_buf sca
       }
     }
     const uint32_t m_blocks = (m + 63) / 64;
-    const uint64_t blocks = (uint64_t)((n_blocks + 7) / 8) * 8u * m_blocks;
+    // 64 x 256 tiles, or 64 x 128 when those would leave a quarter of the chip without work
+    const bool narrow = (uint64_t)m_blocks * n_blocks * 4 < (uint64_t)ctx->num_cus * 3;
+    const uint32_t nb = narrow ? (n + 127) / 128 : n_blocks;
+    const uint64_t blocks = (uint64_t)((nb + 7) / 8) * 8u * m_blocks;
     if (blocks <= 0x7fffffffull) {
-#define KRM_W4A8_TILE(GSH)                                                                     \
-  hipLaunchKernelGGL((linear_w4a8_tile_kernel<ST, GSH, 1>), dim3((uint32_t)blocks), dim3(512), \
-                     0, ctx->stream, ptr<const uint8_t>(xq), pxs, ptr<const uint8_t>(w), ps,  \
-                     pb, po, m, n, k, shift, m_blocks, n_blocks)
-      if (shift == 6) KRM_W4A8_TILE(6);
-      else if (shift == 7) KRM_W4A8_TILE(7);
-      else if (shift == 8) KRM_W4A8_TILE(8);
-      else KRM_W4A8_TILE(0);
+#define KRM_W4A8_TILE(GSH, WN)                                                                 \
+  hipLaunchKernelGGL((linear_w4a8_tile_kernel<ST, GSH, 1, WN>), dim3((uint32_t)blocks),        \
+                     dim3(512), 0, ctx->stream, ptr<const uint8_t>(xq), pxs,                  \
+                     ptr<const uint8_t>(w), ps, pb, po, m, n, k, shift, m_blocks, nb)
+#define KRM_W4A8_TILE_G(GSH) \
+  do { if (narrow) KRM_W4A8_TILE(GSH, 1); else KRM_W4A8_TILE(GSH, 2); } while (0)
+      if (shift == 6) KRM_W4A8_TILE_G(6);
+      else if (shift == 7) KRM_W4A8_TILE_G(7);
+      else if (shift == 8) KRM_W4A8_TILE_G(8);
+      else KRM_W4A8_TILE_G(0);
+#undef KRM_W4A8_TILE_G
 #undef KRM_W4A8_TILE
       return launched(ctx, "linear_w4a8_tile_kernel");
     }
