@@ -169,7 +169,7 @@ __device__ inline bool beats(float va, uint32_t ia, float vb, uint32_t ib) {
   return ia < ib;
 }
 constexpr int kArgmaxThreads = 1024;
-constexpr int kArgmaxUnroll = 16;  // independent loads in flight per thread
+constexpr int kArgmaxUnroll = 32;  // independent loads in flight per thread (one pass up to 32768)
 template <typename XT>
 __global__ __launch_bounds__(kArgmaxThreads) void argmax_kernel(const XT* __restrict__ x,
                                                                int32_t* __restrict__ out,
