@@ -260,7 +260,7 @@ struct DecodeArgs {
   uint32_t nseq;             // ragged batch: sequences; single: batch
   const int32_t* cu_rows;    // ragged batch: [nseq+1] first slot row of each sequence
   const int32_t* split_prefix;  // ragged batch: [nseq+1] first global split of each sequence
-  uint32_t* tickets;         // [nseq * kv_heads] arrival counters, zero between launches
+  uint32_t* tickets;         // arrival counter (sequence, head unit) at index * kTicketStride, zero between launches
   uint32_t* lengths;         // single sequence: device {past, query, fault} or null
   uint32_t capacity;         // single sequence: slot rows (checked against device lengths)
 };
@@ -609,25 +609,27 @@ void attention_decode_kernel(
   // Arrival: the partial was written through to memory (device-scope stores); once every
   // thread's stores have completed, take a ticket.  The last arrival merges, reading the
   // partials with device-scope loads.  No cache-wide write-back or invalidate is involved.
-  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+  // The wait is spelled out: a workgroup-scope release fence does not wait for global stores
+  // on this target, and a device-scope one writes the whole L2 back.
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   __syncthreads();
+  uint32_t* ticket = &a.tickets[(size_t)(seq * gridDim.y + blockIdx.y) * kTicketStride];
   if (tid == 0)
-    s_ticket = __hip_atomic_fetch_add(&a.tickets[seq * gridDim.y + blockIdx.y], 1u,
-                                      __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    s_ticket = __hip_atomic_fetch_add(ticket, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   __syncthreads();
   if (s_ticket + 1 != nsplit) return;
 
   // Merge nsplit partials of each of the R heads, kMergeChunk at a time, ascending order; the
   // partial rows of a pass are all requested before any is used.
-  float tot_m[R], tot_l[R];
-  float tot_o[kOuts];
+  // Every output element tracks the running (max, sum) of its own head: the same numbers in
+  // all elements of a head, and one exponential per partial instead of one per use.
+  float tot_m[kOuts], tot_l[kOuts], tot_o[kOuts];
 #pragma unroll
-  for (int h = 0; h < R; ++h) {
-    tot_m[h] = -INFINITY;
-    tot_l[h] = 0.f;
+  for (int i = 0; i < kOuts; ++i) {
+    tot_m[i] = -INFINITY;
+    tot_l[i] = 0.f;
+    tot_o[i] = 0.f;
   }
-#pragma unroll
-  for (int i = 0; i < kOuts; ++i) tot_o[i] = 0.f;
   for (uint32_t s0 = 0; s0 < nsplit; s0 += kMergeChunk) {
     const uint32_t cnt = nsplit - s0 < (uint32_t)kMergeChunk ? nsplit - s0 : (uint32_t)kMergeChunk;
     // the weighted rows first (long latency), the small (max, sum) pairs next
@@ -651,35 +653,23 @@ void attention_decode_kernel(
       s_wl[h][s] = s < cnt ? observe(&ws_ml[slot_index * 2 + 1]) : 0.f;
     }
     __syncthreads();
-    float keep[R];
-#pragma unroll
-    for (int h = 0; h < R; ++h) {  // every thread tracks every head (uniform work)
-      float m = tot_m[h];
-#pragma unroll
-      for (int j = 0; j < kMergeChunk; ++j) m = fmaxf(m, s_w[h][j]);
-      keep[h] = __builtin_amdgcn_exp2f(tot_m[h] - m);  // 0 on the first pass
-      float l = tot_l[h] * keep[h];
-#pragma unroll
-      for (int j = 0; j < kMergeChunk; ++j)
-        l = fmaf(__builtin_amdgcn_exp2f(s_w[h][j] - m), s_wl[h][j], l);
-      tot_m[h] = m;
-      tot_l[h] = l;
-    }
 #pragma unroll
     for (int i = 0; i < kOuts; ++i) {
       const int o = tid + i * kThreads;
-      const int oo = o < R * D ? o : 0;
-      const int h = oo / D;
-      float k_h = keep[0], m_h = tot_m[0];
+      const int h = (o < R * D ? o : 0) / D;
+      float m = tot_m[i];
 #pragma unroll
-      for (int hh = 1; hh < R; ++hh) {
-        k_h = (h == hh) ? keep[hh] : k_h;
-        m_h = (h == hh) ? tot_m[hh] : m_h;
+      for (int j = 0; j < kMergeChunk; ++j) m = fmaxf(m, s_w[h][j]);
+      const float keep = __builtin_amdgcn_exp2f(tot_m[i] - m);  // 0 on the first pass
+      float l = tot_l[i] * keep, total = tot_o[i] * keep;
+#pragma unroll
+      for (int j = 0; j < kMergeChunk; ++j) {
+        const float wgt = __builtin_amdgcn_exp2f(s_w[h][j] - m);
+        l = fmaf(wgt, s_wl[h][j], l);
+        total = fmaf(wgt, rows[i][j], total);
       }
-      float total = tot_o[i] * k_h;
-#pragma unroll
-      for (int j = 0; j < kMergeChunk; ++j)
-        total = fmaf(__builtin_amdgcn_exp2f(s_w[h][j] - m_h), rows[i][j], total);
+      tot_m[i] = m;
+      tot_l[i] = l;
       tot_o[i] = total;
     }
   }
@@ -688,14 +678,10 @@ void attention_decode_kernel(
     const int o = tid + i * kThreads;
     if (o >= R * D) break;
     const int h = o / D, d = o - h * D;
-    float l_h = tot_l[0];
-#pragma unroll
-    for (int hh = 1; hh < R; ++hh) l_h = (h == hh) ? tot_l[hh] : l_h;
-    st_f32<XT>(out, ((size_t)seq * a.heads + head0 + h) * D + d, tot_o[i] / l_h);
+    st_f32<XT>(out, ((size_t)seq * a.heads + head0 + h) * D + d, tot_o[i] / tot_l[i]);
   }
   if (tid == 0)  // ready for the next launch
-    __hip_atomic_store(&a.tickets[seq * gridDim.y + blockIdx.y], 0u, __ATOMIC_RELAXED,
-                       __HIP_MEMORY_SCOPE_AGENT);
+    __hip_atomic_store(ticket, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
 struct DecodeLaunch {

@@ -39,6 +39,10 @@ namespace krm {
 
 constexpr int kWave = 64;
 constexpr uint32_t kTicketSlots = 1u << 16;
+// Words between two arrival counters: one counter per 128 bytes.  Atomics on one cache line
+// execute one after the other (11 ns each, measured); the 512 workgroups of a 4096-column
+// decode step, counting on 16 neighbouring words, spent 5.8 us queueing there.
+constexpr uint32_t kTicketStride = 32;
 
 // Records the message on the context (or on the context-less slot) and returns `code`.
 int32_t fail(krm_ctx* ctx, int32_t code, const char* fmt, ...);

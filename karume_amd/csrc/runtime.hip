@@ -83,8 +83,9 @@ int32_t krm_ctx_create_on_stream(int32_t device, void* hip_stream, krm_ctx** out
     delete ctx;
     return hip_status(nullptr, st, "hipHostMalloc");
   }
-  st = hipMalloc(reinterpret_cast<void**>(&ctx->tickets), kTicketSlots * sizeof(uint32_t));
-  if (st == hipSuccess) st = hipMemset(ctx->tickets, 0, kTicketSlots * sizeof(uint32_t));
+  const size_t ticket_bytes = (size_t)kTicketSlots * kTicketStride * sizeof(uint32_t);
+  st = hipMalloc(reinterpret_cast<void**>(&ctx->tickets), ticket_bytes);
+  if (st == hipSuccess) st = hipMemset(ctx->tickets, 0, ticket_bytes);
   if (st == hipSuccess) st = hipDeviceSynchronize();
   if (st != hipSuccess) {
     if (ctx->tickets) (void)hipFree(ctx->tickets);
