@@ -179,21 +179,46 @@ struct Acts<float> {
   struct Regs {
     float v[VEC][8];
   };
+  // The loads of `load` alone (activations, then norm weights), so that a caller can put other
+  // requests between them and their first use.
+  template <int VEC, bool NORM>
+  struct Raw {
+    uint4 x[VEC][2];
+    float4 g[NORM ? VEC : 1][2];
+  };
+  template <int VEC, bool NORM>
+  __device__ static inline void request(const float* x, const float* g, Raw<VEC, NORM>& raw) {
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) {
+      raw.x[j][0] = reinterpret_cast<const uint4*>(x)[2 * j];
+      raw.x[j][1] = reinterpret_cast<const uint4*>(x)[2 * j + 1];
+      if constexpr (NORM) {
+        raw.g[j][0] = reinterpret_cast<const float4*>(g)[2 * j];
+        raw.g[j][1] = reinterpret_cast<const float4*>(g)[2 * j + 1];
+      }
+    }
+  }
   template <int VEC, bool NORM>
   __device__ static inline void load(const float* x, const float* g, bool active, Regs<VEC>& r,
                                      float& squares) {
+    Raw<VEC, NORM> raw;
+    request<VEC, NORM>(x, g, raw);
+    finish<VEC, NORM>(raw, active, r, squares);
+  }
+  template <int VEC, bool NORM>
+  __device__ static inline void finish(const Raw<VEC, NORM>& raw, bool active, Regs<VEC>& r,
+                                       float& squares) {
 #pragma unroll
     for (int j = 0; j < VEC; ++j) {
-      uint4 ua = reinterpret_cast<const uint4*>(x)[2 * j];
-      uint4 ub = reinterpret_cast<const uint4*>(x)[2 * j + 1];
+      const uint4 ua = raw.x[j][0], ub = raw.x[j][1];
       const uint32_t keep = (!NORM || active) ? 0xFFFFFFFFu : 0u;  // x^2 past K must be 0
       float4 a = make_float4(__uint_as_float(ua.x & keep), __uint_as_float(ua.y & keep),
                              __uint_as_float(ua.z & keep), __uint_as_float(ua.w & keep));
       float4 b = make_float4(__uint_as_float(ub.x & keep), __uint_as_float(ub.y & keep),
                              __uint_as_float(ub.z & keep), __uint_as_float(ub.w & keep));
       if constexpr (NORM) {
-        const float4 ga = reinterpret_cast<const float4*>(g)[2 * j];
-        const float4 gb = reinterpret_cast<const float4*>(g)[2 * j + 1];
+        const float4 ga = raw.g[j][0];
+        const float4 gb = raw.g[j][1];
         squares = fmaf(a.x, a.x, squares); squares = fmaf(a.y, a.y, squares);
         squares = fmaf(a.z, a.z, squares); squares = fmaf(a.w, a.w, squares);
         squares = fmaf(b.x, b.x, squares); squares = fmaf(b.y, b.y, squares);
@@ -439,8 +464,10 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 4))) voi
   const int lane = threadIdx.x & (kWave - 1);
   const int wave = threadIdx.x >> 6;
   constexpr bool XLDS = share_x_in_lds<XT, MB, NSTEP>();
-  const uint32_t row0 = (blockIdx.x * (blockDim.x >> 6) + wave) * ROWS;
-  if (!XLDS && row0 >= n) return;  // whole wave leaves together (XLDS: it still stages x)
+  // Four waves a workgroup (the launch below).  A wave whose rows lie past N stays: it re-reads
+  // the last row and stores nothing, so no branch stands between the kernel's entry and its
+  // loads (an early exit made the pointer arguments wait for the row test).
+  const uint32_t row0 = (blockIdx.x * 4u + wave) * ROWS;
 
   const uint32_t words_per_row = k >> 3;
   const uint32_t groups_per_row = k >> group_shift;
@@ -527,17 +554,26 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 4))) voi
   if constexpr (NSTEP > 0) {
     uint32_t all_w[NSTEP][ROWS][VEC];
     float all_s[NSTEP][ROWS];
-#pragma unroll
-    for (int step = 0; step < NSTEP; ++step) fetch(step, all_w[step], all_s[step]);
     if constexpr (XLDS) {
       // 16-byte units, unit u of lane l at [(step * kUnits + u) * 64 + l]: conflict-free
       constexpr int kUnits = sizeof(Regs) / 16;
       static_assert(sizeof(Regs) % 16 == 0, "activation registers are whole 16-byte units");
       __shared__ uint4 s_x[NSTEP * kUnits * kWave];
       __shared__ float s_squares[NSTEP];
+      // The staging waves ask for the activations first: loads return in order, and x (in the
+      // cache) would otherwise arrive behind the weights (from memory) and hold the whole
+      // workgroup at the barrier until then; with x early, every wave starts on its rows as
+      // soon as its own weights are there.
+      typename Acts<XT>::template Raw<VEC, NORM> raw_x;
+      const uint32_t x_k0 = (uint32_t)wave * kStepElems + lane * kLaneElems;
+      const uint32_t x_kc = x_k0 < k ? x_k0 : 0u;
+      if (wave < NSTEP)
+        Acts<XT>::template request<VEC, NORM>(x + x_kc, fuse.norm_weight + x_kc, raw_x);
+#pragma unroll
+      for (int step = 0; step < NSTEP; ++step) fetch(step, all_w[step], all_s[step]);
       if (wave < NSTEP) {
         Regs regs;
-        fetch_x(wave, 0, regs);
+        Acts<XT>::template finish<VEC, NORM>(raw_x, x_k0 < k, regs, squares[0]);
         uint4 units[kUnits];
         __builtin_memcpy(units, &regs, sizeof(Regs));
 #pragma unroll
@@ -564,12 +600,16 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 4))) voi
         consume(step, all_w[step], all_s[step], 0, regs);
       }
     } else if constexpr (MB == 1) {
+#pragma unroll
+      for (int step = 0; step < NSTEP; ++step) fetch(step, all_w[step], all_s[step]);
       Regs regs[NSTEP];
 #pragma unroll
       for (int step = 0; step < NSTEP; ++step) fetch_x(step, 0, regs[step]);
 #pragma unroll
       for (int step = 0; step < NSTEP; ++step) consume(step, all_w[step], all_s[step], 0, regs[step]);
     } else {
+#pragma unroll
+      for (int step = 0; step < NSTEP; ++step) fetch(step, all_w[step], all_s[step]);
 #pragma unroll
       for (int step = 0; step < NSTEP; ++step) {
 #pragma unroll
