@@ -616,6 +616,312 @@ void gemm_i4_f16_packed_kernel(const XT* __restrict__ x, const uint8_t* __restri
   }
 }
 
+// ------------------------------------------------ packed weights in LDS, K dealt by units
+//
+// The same 128 x 256 tile and stage loop as above, for outputs whose tiles do not fill the
+// chip evenly (172 tiles on 256 CUs leave a third idle; 64 tiles three quarters).  The work is
+// the list of (tile, stage) units, tiles in column-block-major order; it is cut into one
+// contiguous range per workgroup (the grid is one workgroup per CU, ranges differ by at most
+// one unit), so a tile is computed by up to a few workgroups, each over a slice of K.  A
+// workgroup that computes a whole tile stores it.  Otherwise it writes its 128 x 256 f32
+// partial (device-scope stores, each thread its own registers, 16 bytes at a time), waits for
+// the stores, and takes a ticket on the tile's counter; the workgroup that arrives last adds
+// the partials in ascending K order — its own from registers — so the bits do not depend on
+// who arrives last.  No workgroup ever waits for another.
+struct UnitDeal {
+  uint32_t stages_per_tile;
+  uint32_t units_lo, extra;  // workgroup v owns units_lo + (v < extra) units from deal_begin(v)
+  float* partials;           // [2 * workgroups] slots of 128 x 256 floats
+  uint32_t* tickets;         // one counter per tile, kTicketStride words apart, zero at rest
+};
+__host__ __device__ inline uint32_t deal_begin(const UnitDeal& d, uint32_t v) {
+  return v * d.units_lo + (v < d.extra ? v : d.extra);
+}
+__device__ inline uint32_t deal_owner(const UnitDeal& d, uint32_t unit) {
+  const uint32_t big = d.extra * (d.units_lo + 1u);
+  return unit < big ? unit / (d.units_lo + 1u) : d.extra + (unit - big) / d.units_lo;
+}
+constexpr uint32_t kPartialFloats = 128u * 256u;
+
+typedef float float4_t __attribute__((ext_vector_type(4)));
+// 16 bytes written through to / read from memory that every XCD sees (device scope).
+__device__ inline void publish4(float4_t* p, float4_t v) {
+  asm volatile("global_store_dwordx4 %0, %1, off sc1" ::"v"(p), "v"(v) : "memory");
+}
+__device__ inline float4_t observe4(const float4_t* p) {
+  float4_t v;
+  asm volatile("global_load_dwordx4 %0, %1, off sc1" : "=v"(v) : "v"(p) : "memory");
+  return v;
+}
+// The eight requests above have landed; the values pass through so that no use moves ahead.
+__device__ inline void landed(float4_t (&p)[8]) {
+  asm volatile("s_waitcnt vmcnt(0)"
+               : "+v"(p[0]), "+v"(p[1]), "+v"(p[2]), "+v"(p[3]), "+v"(p[4]), "+v"(p[5]), "+v"(p[6]),
+                 "+v"(p[7])::"memory");
+}
+
+// WM = 2 (the one in use): eight waves, wave = 64 x 64, two waves a SIMD, as above.  WM = 1: four
+// waves, wave = 128 x 64, every weight word dequantised once for four MFMAs instead of twice for
+// two — measured 101 us against 78 us on the 512 x 11008 x 4096 product: the single wave of a
+// SIMD does not hide its own LDS reads and dequantisation under its MFMAs as compiled (and
+// spills 31 registers).
+template <typename XT, typename ST, int WM>
+__global__ __launch_bounds__(WM * 256) __attribute__((amdgpu_waves_per_eu(WM, WM)))
+void gemm_i4_f16_dealt_kernel(const XT* __restrict__ x, const uint8_t* __restrict__ w,
+                              const ST* __restrict__ scales, const XT* __restrict__ bias,
+                              XT* __restrict__ out, uint32_t m, uint32_t n, uint32_t k,
+                              uint32_t group_shift, uint32_t m_blocks, UnitDeal deal) {
+  constexpr int MT = 4 / WM, WN = 2;
+  constexpr int T = WM * 256;  // threads
+  constexpr int BM = WM * 32 * MT, BN = 256;
+  static_assert(BM == 128, "the partial layout and the deal assume 128 x 256 tiles");
+  constexpr int kStage = 128;
+  constexpr int kRowA = kStage * 2 + 16;
+  constexpr int kRowB = kStage / 2 + 16;
+  constexpr int kAUnits = BM * (kStage / 8) / T;
+  constexpr int kBUnits = BN * (kStage / 32) / T;
+  __shared__ __align__(16) uint8_t s_a[2][BM * kRowA];
+  __shared__ __align__(16) uint8_t s_b[2][BN * kRowB];
+  __shared__ _Float16 s_s[2][BN][2];
+  __shared__ uint32_t s_ticket;
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = wave >> 2, wn = wave & 3;
+  const int frag_row = lane & 31, frag_h = lane >> 5;
+  const uint32_t groups = k >> group_shift;
+  const uint32_t spt = deal.stages_per_tile;
+  const uint32_t arow0 = tid >> 4, aunit = (tid & 15u) * 8u;
+  const uint32_t brow0 = tid >> 2, bunit = (tid & 3u) * 16u;
+  const uint32_t a_base = (uint32_t)((wm * 32 * MT + frag_row) * kRowA + 64 * frag_h);
+  const uint32_t b_base = (uint32_t)((wn * 64 + frag_row) * kRowB + 16 * frag_h);
+
+  // the workgroups of one XCD (ids equal mod 8) take neighbouring ranges: the row panels of a
+  // column block then mostly share an L2
+  uint32_t v = blockIdx.x;
+  if ((gridDim.x & 7u) == 0) v = (blockIdx.x & 7u) * (gridDim.x >> 3) + (blockIdx.x >> 3);
+  const uint32_t my_begin = deal_begin(deal, v);
+  uint32_t unit = my_begin;
+  uint32_t left = deal.units_lo + (v < deal.extra ? 1u : 0u);
+  while (left > 0) {
+    const uint32_t tile = unit / spt, s0 = unit - tile * spt;
+    const uint32_t s1 = spt - s0 < left ? spt : s0 + left;
+    const uint32_t nb = tile / m_blocks, mb = tile - nb * m_blocks;
+    const uint32_t m0 = mb * BM, n0 = nb * BN;
+    const ST* ssrc = scales + (size_t)min(n0 + (uint32_t)(tid & 255), n - 1) * groups;
+
+    struct Staged {
+      Acts8<XT> a[kAUnits];
+      uint4 b[kBUnits];
+    };
+    auto load_stage = [&](uint32_t stage, Staged& d) {
+      const uint32_t a_at = stage * kStage + aunit, b_at = stage * (kStage / 2) + bunit;
+      const uint32_t a_off = a_at < k ? a_at : 0u, b_off = b_at < (k >> 1) ? b_at : 0u;
+#pragma unroll
+      for (int i = 0; i < kAUnits; ++i)
+        d.a[i].load(x + (size_t)min(m0 + arow0 + (uint32_t)(T / 16) * i, m - 1) * k + a_off);
+#pragma unroll
+      for (int i = 0; i < kBUnits; ++i)
+        d.b[i] = *reinterpret_cast<const uint4*>(
+            w + (size_t)min(n0 + brow0 + (uint32_t)(T / 4) * i, n - 1) * (k >> 1) + b_off);
+    };
+    auto park_stage = [&](uint32_t stage, int buf, Staged& d) {
+      const uint32_t keep = stage * kStage + aunit < k ? 0xFFFFFFFFu : 0u;
+#pragma unroll
+      for (int i = 0; i < kAUnits; ++i) {
+        uint4 pv = d.a[i].paired();
+        pv.x &= keep; pv.y &= keep; pv.z &= keep; pv.w &= keep;
+        *reinterpret_cast<uint4*>(&s_a[buf][(arow0 + (uint32_t)(T / 16) * i) * kRowA + aunit * 2u]) = pv;
+      }
+#pragma unroll
+      for (int i = 0; i < kBUnits; ++i)
+        *reinterpret_cast<uint4*>(&s_b[buf][(brow0 + (uint32_t)(T / 4) * i) * kRowB + bunit]) = d.b[i];
+      if (tid < 256) {
+        const uint32_t c0 = stage * kStage, c1 = stage * kStage + 64u;
+        s_s[buf][tid][0] = scale_from_bits<ST>(scale_bits<ST>(ssrc, (c0 < k ? c0 : 0u) >> group_shift));
+        s_s[buf][tid][1] = scale_from_bits<ST>(scale_bits<ST>(ssrc, (c1 < k ? c1 : 0u) >> group_shift));
+      }
+    };
+
+    float16_t acc[MT][WN];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+      for (int nt = 0; nt < WN; ++nt)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[mt][nt][r] = 0.f;
+
+    Staged staged;
+    load_stage(s0, staged);
+    park_stage(s0, 0, staged);
+    __syncthreads();
+
+    auto run_stage = [&](uint32_t stage, int buf) {
+      load_stage(stage + 1, staged);
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int c = 0; c < 2; ++c) {
+        uint4 braw[WN];
+        _Float16 ws[WN];
+#pragma unroll
+        for (int nt = 0; nt < WN; ++nt) {
+          braw[nt] = *reinterpret_cast<const uint4*>(&s_b[buf][b_base + nt * 32 * kRowB + 32 * c]);
+          ws[nt] = s_s[buf][wn * 64 + nt * 32 + frag_row][c];
+        }
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          half8_t a[MT];
+#pragma unroll
+          for (int mt = 0; mt < MT; ++mt)
+            a[mt] = *reinterpret_cast<const half8_t*>(
+                &s_a[buf][a_base + mt * 32 * kRowA + 128 * c + 16 * j]);
+#pragma unroll
+          for (int nt = 0; nt < WN; ++nt) {
+            const uint32_t word = j == 0 ? braw[nt].x : j == 1 ? braw[nt].y : j == 2 ? braw[nt].z
+                                                                                    : braw[nt].w;
+            const half8_t b = __builtin_bit_cast(half8_t, dequant_word(word, ws[nt]));
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt)
+              acc[mt][nt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[mt], b, acc[mt][nt], 0, 0, 0);
+          }
+        }
+      }
+      park_stage(stage + 1, buf ^ 1, staged);
+      __syncthreads();
+    };
+    for (uint32_t stage = s0; stage < s1; stage += 2) {
+      run_stage(stage, 0);
+      if (stage + 1 < s1) run_stage(stage + 1, 1);
+    }
+
+    auto store_block = [&](int mt, int nt, const float16_t& total) {
+      const uint32_t col = n0 + wn * 64 + nt * 32 + frag_row;
+      const float b = (bias && col < n) ? bias_f32<XT>(bias, col) : 0.f;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const uint32_t row = m0 + wm * 32 * MT + mt * 32 + 8 * (r / 4) + 4 * frag_h + (r % 4);
+        if (row < m && col < n) store_out<XT>(out, (size_t)row * n + col, total[r] + b);
+      }
+    };
+
+    if (s0 == 0 && s1 == spt) {
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+        for (int nt = 0; nt < WN; ++nt) store_block(mt, nt, acc[mt][nt]);
+    } else {
+      // Slot of workgroup u's partial of this tile: its second slot when its range began at or
+      // before the tile's first unit, its first slot otherwise (a range holds at most one
+      // partial of either kind).  16-byte piece c of thread t sits at [c * threads + t].
+      const uint32_t tile_begin = tile * spt;
+      auto slot_of = [&](uint32_t u) {
+        return 2u * u + (deal_begin(deal, u) <= tile_begin ? 1u : 0u);
+      };
+      uint32_t* ticket = deal.tickets + (size_t)tile * kTicketStride;
+      const uint32_t first = deal_owner(deal, tile_begin), last = deal_owner(deal, tile_begin + spt - 1u);
+      // Every other partial already there (the usual case for the slice computed last: slices
+      // that open a range finish early)?  Then this one need not be written at all.
+      if (tid == 0)
+        s_ticket = __hip_atomic_load(ticket, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      __syncthreads();
+      bool merge = s_ticket == last - first;
+      __syncthreads();  // s_ticket is written again below
+      if (!merge) {
+        float4_t* mine =
+            reinterpret_cast<float4_t*>(deal.partials + (size_t)slot_of(v) * kPartialFloats);
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+          for (int nt = 0; nt < WN; ++nt)
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+              const float4_t piece = {acc[mt][nt][4 * q], acc[mt][nt][4 * q + 1],
+                                      acc[mt][nt][4 * q + 2], acc[mt][nt][4 * q + 3]};
+              publish4(mine + (size_t)(((mt * WN + nt) * 4 + q) * T + tid), piece);
+            }
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this thread's partial is in memory
+        __syncthreads();
+        if (tid == 0)
+          s_ticket = __hip_atomic_fetch_add(ticket, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __syncthreads();
+        merge = s_ticket == last - first;  // arrived last after all
+      }
+      if (merge) {  // every other partial of the tile is complete
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+          float16_t total[WN];
+          for (uint32_t u = first; u <= last; ++u) {
+            float16_t part[WN];
+#pragma unroll
+            for (int nt = 0; nt < WN; ++nt) part[nt] = acc[mt][nt];
+            if (u != v) {
+              const float4_t* src =
+                  reinterpret_cast<const float4_t*>(deal.partials + (size_t)slot_of(u) * kPartialFloats) +
+                  (size_t)(mt * WN * 4 * T + tid);
+              float4_t p[8];
+#pragma unroll
+              for (int i = 0; i < 8; ++i) p[i] = observe4(src + (size_t)i * T);
+              landed(p);
+#pragma unroll
+              for (int nt = 0; nt < WN; ++nt)
+#pragma unroll
+                for (int q = 0; q < 4; ++q)
+#pragma unroll
+                  for (int i = 0; i < 4; ++i) part[nt][4 * q + i] = p[nt * 4 + q][i];
+            }
+#pragma unroll
+            for (int nt = 0; nt < WN; ++nt) {
+              if (u == first) {
+                total[nt] = part[nt];
+              } else {
+#pragma unroll
+                for (int r = 0; r < 16; ++r) total[nt][r] += part[nt][r];
+              }
+            }
+          }
+#pragma unroll
+          for (int nt = 0; nt < WN; ++nt) store_block(mt, nt, total[nt]);
+        }
+        if (tid == 0)
+          __hip_atomic_store(ticket, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      }
+    }
+    unit += s1 - s0;
+    left -= s1 - s0;
+  }
+}
+
+// Workgroups, units and scratch of a dealt launch; false when the shape is not worth it.
+bool plan_deal(krm_ctx* ctx, uint32_t m, uint32_t n, uint32_t k, uint32_t& grid, UnitDeal& deal) {
+  const uint64_t cus = (uint64_t)ctx->num_cus;
+  const uint64_t tiles = (uint64_t)((m + 127) / 128) * ((n + 255) / 256);
+  const uint32_t spt = (k + 127) / 128;
+  const uint64_t units = tiles * spt;
+  if (tiles > kTicketSlots || units > 0x7fffffffull || units < cus) return false;
+  // whole rounds of tiles already use the chip well
+  const uint64_t rounds = (tiles + cus - 1) / cus;
+  if (tiles * 10 >= rounds * cus * 9) return false;
+  // a tile shared by many workgroups costs more in partials than the idle CUs did
+  if (tiles * 6 < cus) return false;
+  if (!ctx->gemm_partials) return false;
+  grid = (uint32_t)cus;
+  deal.stages_per_tile = spt;
+  deal.units_lo = (uint32_t)(units / cus);
+  deal.extra = (uint32_t)(units % cus);
+  deal.partials = ctx->gemm_partials;
+  deal.tickets = ctx->tickets;
+  return true;
+}
+
+template <typename XT, typename ST, int WM>
+int32_t launch_dealt(krm_ctx* ctx, krm_buf x, krm_buf w, krm_buf scales, krm_buf bias, krm_buf out,
+                     uint32_t m, uint32_t n, uint32_t k, uint32_t group_shift, uint32_t grid,
+                     const UnitDeal& deal) {
+  gemm_i4_f16_dealt_kernel<XT, ST, WM><<<dim3(grid), dim3(WM * 256), 0, ctx->stream>>>(
+      ptr<const XT>(x), ptr<const uint8_t>(w), ptr<const ST>(scales), ptr<const XT>(bias),
+      ptr<XT>(out), m, n, k, group_shift, (m + 127) / 128, deal);
+  return launched(ctx, "gemm_i4_f16_dealt_kernel");
+}
+
 template <typename XT, typename ST, int MT>
 int32_t launch_packed(krm_ctx* ctx, krm_buf x, krm_buf w, krm_buf scales, krm_buf bias,
                       krm_buf out, uint32_t m, uint32_t n, uint32_t k, uint32_t group_shift) {
@@ -673,8 +979,14 @@ int32_t pick_tile(krm_ctx* ctx, krm_buf x, krm_buf w, krm_buf scales, krm_buf bi
   // 77 us against 85 us on the 512 x 11008 x 4096 up-projection; with fewer tiles than that the
   // forms below, which split K inside a workgroup, are faster).
   const uint64_t packed_tiles = (uint64_t)((m + 127) / 128) * ((n + 255) / 256);
-  if (m > 64 && group >= 64 && k % 8 == 0 && aligned(w, 16) && aligned(x, 16) &&
-      packed_tiles * 5 >= cus * 3)
+  const bool packed_ok = m > 64 && group >= 64 && k % 8 == 0 && aligned(w, 16) && aligned(x, 16);
+  if (packed_ok) {
+    uint32_t grid = 0;
+    UnitDeal deal{};
+    if (plan_deal(ctx, m, n, k, grid, deal))
+      return launch_dealt<XT, ST, 2>(ctx, x, w, scales, bias, out, m, n, k, group_shift, grid, deal);
+  }
+  if (packed_ok && packed_tiles * 5 >= cus * 3)
     return launch_packed<XT, ST, 2>(ctx, x, w, scales, bias, out, m, n, k, group_shift);
   const uint64_t tiles = (uint64_t)((m + 127) / 128) * ((n + 127) / 128);
   if (m > 64 && tiles >= cus)

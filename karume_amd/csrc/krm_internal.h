@@ -22,6 +22,9 @@ struct krm_ctx {
   // Arrival counters of the split-K attention (device memory, zeroed at creation; the last
   // workgroup of every (sequence, kv head) puts its counter back to zero).
   uint32_t* tickets = nullptr;
+  // Scratch of the unit-dealt GEMM: two 128 x 256 f32 partials per CU (64 MiB on 256 CUs),
+  // allocated with the context so that launches can be recorded into graphs.
+  float* gemm_partials = nullptr;
   bool recording = false;  // between krm_graph_begin and krm_graph_end
   char error[512] = {0};
 };
@@ -43,6 +46,7 @@ constexpr uint32_t kTicketSlots = 1u << 16;
 // execute one after the other (11 ns each, measured); the 512 workgroups of a 4096-column
 // decode step, counting on 16 neighbouring words, spent 5.8 us queueing there.
 constexpr uint32_t kTicketStride = 32;
+constexpr size_t kGemmPartialBytes = 128u * 256u * sizeof(float);
 
 // Records the message on the context (or on the context-less slot) and returns `code`.
 int32_t fail(krm_ctx* ctx, int32_t code, const char* fmt, ...);

@@ -86,8 +86,12 @@ int32_t krm_ctx_create_on_stream(int32_t device, void* hip_stream, krm_ctx** out
   const size_t ticket_bytes = (size_t)kTicketSlots * kTicketStride * sizeof(uint32_t);
   st = hipMalloc(reinterpret_cast<void**>(&ctx->tickets), ticket_bytes);
   if (st == hipSuccess) st = hipMemset(ctx->tickets, 0, ticket_bytes);
+  if (st == hipSuccess)
+    st = hipMalloc(reinterpret_cast<void**>(&ctx->gemm_partials),
+                   (size_t)2 * ctx->num_cus * kGemmPartialBytes);
   if (st == hipSuccess) st = hipDeviceSynchronize();
   if (st != hipSuccess) {
+    if (ctx->gemm_partials) (void)hipFree(ctx->gemm_partials);
     if (ctx->tickets) (void)hipFree(ctx->tickets);
     (void)hipHostFree(ctx->pinned);
     delete ctx;
@@ -103,6 +107,7 @@ int32_t krm_ctx_create(int32_t device, krm_ctx** out) {
   // Default priority on purpose: mixed stream priorities are not used anywhere.
   hipError_t st = hipStreamCreateWithFlags(&ctx->stream, hipStreamNonBlocking);
   if (st != hipSuccess) {
+    (void)hipFree(ctx->gemm_partials);
     (void)hipFree(ctx->tickets);
     (void)hipHostFree(ctx->pinned);
     delete ctx;
@@ -120,6 +125,7 @@ int32_t krm_ctx_destroy(krm_ctx* ctx) {
   if (ctx->owns_stream) (void)hipStreamDestroy(ctx->stream);
   if (ctx->pinned) (void)hipHostFree(ctx->pinned);
   if (ctx->tickets) (void)hipFree(ctx->tickets);
+  if (ctx->gemm_partials) (void)hipFree(ctx->gemm_partials);
   delete ctx;
   return KRM_OK;
 }

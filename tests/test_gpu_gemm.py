@@ -92,6 +92,25 @@ def test_gemm_edges_exact_weights(gpu_ctx, shape):
                   - 1e-3 * np.abs(want_h)) <= 2e-3  # fp16 output rounding
 
 
+def test_gemm_with_tiles_shared_between_workgroups_is_reproducible(gpu_ctx):
+    """43 tiles of 8 stages on 256 CUs: the (tile, stage) units are dealt one or two to a
+    workgroup, so every tile is the sum of 4-8 partials added by whichever workgroup arrives
+    last.  The sum is taken in K order whoever that is: repeated runs give the same bits, and
+    the result meets the exact-weights gate."""
+    m, n, k, g = 128, 11008, 1024, 128
+    rng = np.random.default_rng(77)
+    q = rng.integers(-8, 8, size=(n, k), dtype=np.int8)
+    scale = (2.0 ** rng.integers(-8, -3, size=(n, k // g))).astype(np.float32)
+    packed = oracle.pack_i4(q)
+    x = rng.normal(size=(m, k)).astype(np.float16).astype(np.float32)
+    bias = rng.normal(size=n).astype(np.float32)
+    first = run_linear(gpu_ctx, x, packed, scale, bias, n, k, g, compute=ka.COMPUTE_F16)
+    for _ in range(4):
+        again = run_linear(gpu_ctx, x, packed, scale, bias, n, k, g, compute=ka.COMPUTE_F16)
+        assert np.array_equal(first.view(np.uint32), again.view(np.uint32))
+    check(first, oracle.linear_i4(x, packed, scale, bias, n, k, g), exact_weights=True)
+
+
 def test_gemm_reference_cases(gpu_ctx):
     """The reference's tile-edge shapes with its own generators (M = 65 and 17 take the MFMA
     path with KRM_COMPUTE_F16); arbitrary f32 scales, f32 x that is not fp16-representable."""
