@@ -700,11 +700,18 @@ void gemm_i4_f16_dealt_kernel(const XT* __restrict__ x, const uint8_t* __restric
   uint32_t v = blockIdx.x;
   if ((gridDim.x & 7u) == 0) v = (blockIdx.x & 7u) * (gridDim.x >> 3) + (blockIdx.x >> 3);
   const uint32_t my_begin = deal_begin(deal, v);
-  uint32_t unit = my_begin;
   uint32_t left = deal.units_lo + (v < deal.extra ? 1u : 0u);
+
+  // The tiles of the range are taken last to first: a range usually ends with the first stages
+  // of a tile and begins with the last stages of the one before, so every workgroup then walks
+  // K upwards from (about) stage 0 and, at any moment, the chip reads few distinct K slices of
+  // x, which stay in the L2s.
   while (left > 0) {
-    const uint32_t tile = unit / spt, s0 = unit - tile * spt;
-    const uint32_t s1 = spt - s0 < left ? spt : s0 + left;
+    const uint32_t range_end = my_begin + left;
+    const uint32_t tile = (range_end - 1u) / spt;
+    const uint32_t tile_first = tile * spt;
+    const uint32_t s0 = my_begin > tile_first ? my_begin - tile_first : 0u;
+    const uint32_t s1 = range_end - tile_first;
     const uint32_t nb = tile / m_blocks, mb = tile - nb * m_blocks;
     const uint32_t m0 = mb * BM, n0 = nb * BN;
     const ST* ssrc = scales + (size_t)min(n0 + (uint32_t)(tid & 255), n - 1) * groups;
@@ -885,7 +892,6 @@ void gemm_i4_f16_dealt_kernel(const XT* __restrict__ x, const uint8_t* __restric
           __hip_atomic_store(ticket, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       }
     }
-    unit += s1 - s0;
     left -= s1 - s0;
   }
 }
