@@ -58,6 +58,10 @@ typedef struct krm_event krm_event;
 #define KRM_COMPUTE_F16 1
 
 /* ---- context (acquireGpu / GpuContext.destroy, packages/runtime/mod.ts:13-113) ---------- */
+/* A context owns, besides its stream, 1 MiB of pinned host staging and device scratch that its
+ * kernels share: 8 MiB of arrival counters (split attention, shared GEMM tiles) and two
+ * 128 x 256 f32 tile partials per CU (64 MiB on 256 CUs) for the prefill GEMM.  Calls on one
+ * context are ordered on its stream; two contexts never share scratch. */
 int32_t krm_ctx_create(int32_t device, krm_ctx** out);
 /* Same, but launches go to an existing hipStream_t (0 = the device's default stream); the
  * stream stays owned by the caller. */
