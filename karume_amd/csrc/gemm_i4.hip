@@ -981,9 +981,11 @@ int32_t pick_tile(krm_ctx* ctx, krm_buf x, krm_buf w, krm_buf scales, krm_buf bi
   // four chunks in flight.  Fewer (a narrow output with a long K, or few rows): 128 x 64 tiles
   // whose two wave groups split every 128-code chunk of K, or 64 x 64 tiles with four groups.
   const uint64_t cus = (uint64_t)ctx->num_cus;
-  // 128 x 256 tiles with the packed weights in LDS when they cover most of the chip (measured
-  // 77 us against 85 us on the 512 x 11008 x 4096 up-projection; with fewer tiles than that the
-  // forms below, which split K inside a workgroup, are faster).
+  // 128 x 256 tiles with the packed weights in LDS.  Dealt by (tile, stage) units over all CUs
+  // when whole rounds of tiles would leave part of the chip idle (512 x 11008 x 4096: 69 us
+  // against 77 us for one workgroup per tile; 512 x 4096 x 11008: 75 us against 93 us for the
+  // K-splitting form below); one workgroup per tile when the tiles cover most of the chip; with
+  // fewer tiles the forms below, which split K inside a workgroup.
   const uint64_t packed_tiles = (uint64_t)((m + 127) / 128) * ((n + 255) / 256);
   const bool packed_ok = m > 64 && group >= 64 && k % 8 == 0 && aligned(w, 16) && aligned(x, 16);
   if (packed_ok) {
