@@ -328,6 +328,69 @@ void attention_decode_kernel(
   const uint32_t hk = blockIdx.y / a.head_groups;
   const uint32_t head0 = hk * a.repeat + (blockIdx.y - hk * a.head_groups) * R;  // first head
 
+  // The rows of a chunk as they arrive: K pieces (row-owner layout, or the MFMA A-operand
+  // layout: piece tile*4 + t) and V pieces (row-owner layout).
+  struct ChunkRows {
+    uint4 k[kDecodeIter];
+    uint4 v[kDecodeIter];
+  };
+  const int wave = tid >> 6, lane = tid & 63;
+  const int frag_row = lane & 15, frag_g = lane >> 4;
+  // offset inside a chunk of the column that (lane group, iteration) owns
+  auto column_of = [&](int it) -> uint32_t {
+    if constexpr (kMfma)
+      return (uint32_t)((wave * 2 + it / 4) * 16 + 4 * frag_g + (it & 3));
+    else
+      return (uint32_t)(it * G + group);
+  };
+  // Requests only: every K row, then every V row of the `width` columns from c_begin of a slot;
+  // unconditional (a column past the end re-reads the first column and is masked when used).
+  auto request_rows = [&](const ST* kslot, const ST* vslot, uint32_t first_row, uint32_t c_begin,
+                          uint32_t width, ChunkRows& rows) {
+    auto slot_row = [&](uint32_t offset) {  // element offset of the row's first dim
+      const uint32_t c = c_begin + (offset < width ? offset : 0u);
+      return (size_t)(first_row + (a.window ? c % a.window : c)) * D;
+    };
+    if constexpr (kMfma) {
+      // lane (r = lane % 16, g = lane / 16) takes 16 bytes of K row r of each 16-row tile at
+      // dims 32t + 8g..: the A-operand layout of v_mfma_f32_16x16x32_f16
+#pragma unroll
+      for (int tile = 0; tile < 2; ++tile) {
+        const size_t at = slot_row((uint32_t)((wave * 2 + tile) * 16 + frag_row));
+#pragma unroll
+        for (int t = 0; t < 4; ++t)
+          rows.k[tile * 4 + t] =
+              *reinterpret_cast<const uint4*>(kslot + at + 32 * t + 8 * frag_g);
+      }
+    } else {
+#pragma unroll
+      for (int it = 0; it < kDecodeIter; ++it)
+        rows.k[it] = *reinterpret_cast<const uint4*>(kslot + slot_row(column_of(it)) + sub * E);
+    }
+#pragma unroll
+    for (int it = 0; it < kDecodeIter; ++it)
+      rows.v[it] = *reinterpret_cast<const uint4*>(vslot + slot_row(column_of(it)) + sub * E);
+  };
+
+  // Lengths that live on the device (a recorded decode step) cost a dependent round trip before
+  // the first address is known.  Without a window the first chunk of a split does not depend
+  // on them — only how many of its columns count does — so its rows are asked for right away,
+  // bounded by the slot's capacity instead of the past; columns that turn out to lie beyond
+  // the past are masked when the chunk is used, like any ragged end.
+  ChunkRows rows0;
+  bool early = false;
+  if constexpr (!RAGGED) {
+    early = a.lengths != nullptr && a.window == 0;
+    if (early) {
+      const size_t base = (size_t)blockIdx.z * a.slot_batch_stride + (size_t)hk * a.slot_plane_stride;
+      const uint32_t want = blockIdx.x * (uint32_t)kChunkCols;
+      const uint32_t c_begin = want < a.capacity ? want : a.capacity - 1u;
+      const uint32_t room = a.capacity - c_begin;
+      request_rows(slot_k + base, slot_v + base, 0u, c_begin,
+                   room < (uint32_t)kChunkCols ? room : (uint32_t)kChunkCols, rows0);
+    }
+  }
+
   // Columns and slot rows are 32-bit (pastLength is a u32, a ragged batch holds < 2^31 rows);
   // only the final byte address is 64-bit: 64-bit index math per load costs more than the
   // attention arithmetic of a short past.
@@ -411,52 +474,13 @@ void attention_decode_kernel(
     for (int e = 0; e < E; ++e) acc[h][e] = 0.f;
   }
 
-  // The rows of a chunk as they arrive: K pieces (row-owner layout, or the MFMA A-operand
-  // layout: piece tile*4 + t) and V pieces (row-owner layout).
-  struct ChunkRows {
-    uint4 k[kDecodeIter];
-    uint4 v[kDecodeIter];
-  };
-  const int wave = tid >> 6, lane = tid & 63;
-  const int frag_row = lane & 15, frag_g = lane >> 4;
   auto chunk_begin = [&](uint32_t chunk) { return c_first + chunk * kChunkCols; };
   auto chunk_end = [&](uint32_t c_begin) {  // c_begin < past: no overflow
     return past - c_begin > (uint32_t)kChunkCols ? c_begin + kChunkCols : past;
   };
-  // offset inside a chunk of the column that (lane group, iteration) owns
-  auto column_of = [&](int it) -> uint32_t {
-    if constexpr (kMfma)
-      return (uint32_t)((wave * 2 + it / 4) * 16 + 4 * frag_g + (it & 3));
-    else
-      return (uint32_t)(it * G + group);
-  };
-  // Requests only: every K row, then every V row of the chunk; unconditional (a column past
-  // the end re-reads the chunk's first column and is masked when it is used).
   auto load_chunk = [&](uint32_t chunk, ChunkRows& rows) {
-    const uint32_t c_begin = chunk_begin(chunk), width = chunk_end(c_begin) - c_begin;
-    auto slot_row = [&](uint32_t offset) {  // element offset of the row's first dim
-      const uint32_t c = c_begin + (offset < width ? offset : 0u);
-      return (size_t)(row_base + (a.window ? c % a.window : c)) * D;
-    };
-    if constexpr (kMfma) {
-      // lane (r = lane % 16, g = lane / 16) takes 16 bytes of K row r of each 16-row tile at
-      // dims 32t + 8g..: the A-operand layout of v_mfma_f32_16x16x32_f16
-#pragma unroll
-      for (int tile = 0; tile < 2; ++tile) {
-        const size_t at = slot_row((uint32_t)((wave * 2 + tile) * 16 + frag_row));
-#pragma unroll
-        for (int t = 0; t < 4; ++t)
-          rows.k[tile * 4 + t] =
-              *reinterpret_cast<const uint4*>(kslot + at + 32 * t + 8 * frag_g);
-      }
-    } else {
-#pragma unroll
-      for (int it = 0; it < kDecodeIter; ++it)
-        rows.k[it] = *reinterpret_cast<const uint4*>(kslot + slot_row(column_of(it)) + sub * E);
-    }
-#pragma unroll
-    for (int it = 0; it < kDecodeIter; ++it)
-      rows.v[it] = *reinterpret_cast<const uint4*>(vslot + slot_row(column_of(it)) + sub * E);
+    const uint32_t c_begin = chunk_begin(chunk);
+    request_rows(kslot, vslot, row_base, c_begin, chunk_end(c_begin) - c_begin, rows);
   };
   auto consume_chunk = [&](uint32_t chunk, ChunkRows& rows) {
     const uint32_t c_begin = chunk_begin(chunk), width = chunk_end(c_begin) - c_begin;
@@ -539,18 +563,17 @@ void attention_decode_kernel(
   // trip; 3 x 32 registers of rows fit beside one head's state).  Each case holds its loads and
   // their uses in one branch: a branch between a load and its use makes the compiler wait
   // inside it.
+  if (!early) load_chunk(0, rows0);  // harmless when the split has no column at all
   bool walked = false;
   if constexpr (R == 1) {
     if (nsplit == 1 && total_chunks == 2) {
-      ChunkRows rows0, rows1;
-      load_chunk(0, rows0);
+      ChunkRows rows1;
       load_chunk(1, rows1);
       consume_chunk(0, rows0);
       consume_chunk(1, rows1);
       walked = true;
     } else if (nsplit == 1 && total_chunks > 2) {
-      ChunkRows rows0, rows1, rows2;
-      load_chunk(0, rows0);
+      ChunkRows rows1, rows2;
       load_chunk(1, rows1);
       load_chunk(2, rows2);
       consume_chunk(0, rows0);
@@ -563,11 +586,11 @@ void attention_decode_kernel(
       walked = true;
     }
   }
-  if (!walked) {
-    for (uint32_t chunk = 0; chunk < my_chunks; ++chunk) {
-      ChunkRows rows;
-      load_chunk(chunk, rows);
-      consume_chunk(chunk, rows);
+  if (!walked && my_chunks > 0) {
+    consume_chunk(0, rows0);
+    for (uint32_t chunk = 1; chunk < my_chunks; ++chunk) {
+      load_chunk(chunk, rows0);
+      consume_chunk(chunk, rows0);
     }
   }
   // this step's own column: one more row for group 0 of the last split
