@@ -104,6 +104,40 @@ def test_decode_split_k(gpu_ctx, case, io, kv):
         assert np.all(err <= ulp), float(np.max(err))
 
 
+@pytest.mark.parametrize("case", DECODE_CASES, ids=lambda c: c.name)
+@pytest.mark.parametrize("io,kv", [(np.float32, np.float32), (np.float16, np.float16)])
+def test_decode_with_device_lengths_equals_scalar_form(gpu_ctx, case, io, kv):
+    """pastLength read on the device (a recorded decode step) gives the bits of the call that
+    carries it as an argument.  Without a window the device form asks for the first chunk's
+    rows before the lengths arrive, bounded by the capacity only: every slot row the step must
+    not see (columns >= pastLength) holds NaN here and must not reach the result."""
+    x = random_state_inputs(case, seed=case.past * 3 + case.depth, f16_values=True)
+    if case.window == 0:
+        x["slot_k"][:, :, case.past:] = np.nan
+        x["slot_v"][:, :, case.past:] = np.nan
+    want = run_attention(gpu_ctx, case, x, io=io, kv=kv)
+    assert np.all(np.isfinite(want.astype(np.float32)))
+    bufs = {k: gpu_ctx.upload(np.ascontiguousarray(
+        v, dtype=io if k in ("q", "ins_k", "ins_v") else kv)) for k, v in x.items()}
+    out = gpu_ctx.upload(np.full(want.size, 123.0, dtype=io))
+    max_past = case.past if case.window else case.capacity - 1
+    ws = gpu_ctx.alloc(max(16, gpu_ctx.attention_state_workspace(
+        case.batch, case.heads, case.kv_heads, 1, case.depth, case.window, max_past, 1)))
+    lengths = gpu_ctx.zeros(16)
+    gpu_ctx.lengths_set(lengths, case.past, 1)
+    gpu_ctx.attention_state_lengths(
+        bufs["q"], bufs["ins_k"], bufs["ins_v"], bufs["slot_k"], bufs["slot_v"], out,
+        batch=case.batch, heads=case.heads, kv_heads=case.kv_heads, chunk_rows=1,
+        depth=case.depth, capacity=case.capacity, window=case.window,
+        half_scale=oracle.half_scale(case.depth), lengths=lengths, max_past=max_past,
+        io_dtype=ka.dtype_code(io), kv_dtype=ka.dtype_code(kv), workspace=ws)
+    got = out.download(io, want.shape)
+    assert lengths.download(np.uint32, (4,))[2] == 0
+    assert got.tobytes() == want.tobytes()
+    for b in list(bufs.values()) + [out, ws, lengths]:
+        b.free()
+
+
 def test_config2_decode_attention(gpu_ctx):
     """benchmark config 2: B=1, H=32, Hkv=8, D=128, 4095 slot rows + this step's row, fp16."""
     case = StateCase("config 2", 1, 32, 8, 1, 128, 4096, 0, 4095, 1)
