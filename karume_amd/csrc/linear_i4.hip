@@ -347,14 +347,17 @@ __global__ __launch_bounds__(KW * 64) void gemv_i4_mfma_kernel(
     }
   };
   if constexpr (CHUNKS > 0) {
-    // the wave's whole share of the weights is requested first (the long trip); activations
-    // run two chunks ahead in registers and one ahead in LDS; fixed registers, no branches
-    Weights wq[CHUNKS];
-#pragma unroll
-    for (int c = 0; c < CHUNKS; ++c) fetch_w(c, wq[c]);
+    // The activations of the first two chunks are requested first: they come from the cache and
+    // loads return in order, so they are parked while the wave's whole share of the weights
+    // (requested next, the long trip) is still on its way.  Activations then run two chunks
+    // ahead in registers and one ahead in LDS; fixed registers, no branches.
     Acts xa[2];
     fetch_x(0, xa[0]);
     if (CHUNKS > 1) fetch_x(1, xa[1]);
+    Weights wq[CHUNKS];
+#pragma unroll
+    for (int c = 0; c < CHUNKS; ++c) fetch_w(c, wq[c]);
+    __builtin_amdgcn_sched_barrier(0);
     park_x(xa[0], 0);
 #pragma unroll
     for (int c = 0; c < CHUNKS; ++c) {
