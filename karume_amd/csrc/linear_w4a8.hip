@@ -216,15 +216,16 @@ __global__ __launch_bounds__(256) void linear_w4a8_rows_kernel(
   auto fetch = [&](uint32_t step, Step& d) {
     const uint32_t k0 = step * kStep + lane * 32;
     const uint32_t kc = k0 < k ? k0 : 0u;
-#pragma unroll
-    for (int r = 0; r < ROWS; ++r) {
-      d.w[r] = *reinterpret_cast<const uint4*>(wrow[r] + (kc >> 3));
-      d.s[r] = scale_f32<ST>(srow[r], kc >> group_shift);
-    }
+    // activations first: they come from the cache, and loads return in order
 #pragma unroll
     for (int b = 0; b < MB; ++b) {
       d.x[b][0] = *reinterpret_cast<const uint4*>(xrow[b] + (kc >> 2));
       d.x[b][1] = *reinterpret_cast<const uint4*>(xrow[b] + (kc >> 2) + 4);
+    }
+#pragma unroll
+    for (int r = 0; r < ROWS; ++r) {
+      d.w[r] = *reinterpret_cast<const uint4*>(wrow[r] + (kc >> 3));
+      d.s[r] = scale_f32<ST>(srow[r], kc >> group_shift);
     }
   };
 
@@ -235,7 +236,7 @@ __global__ __launch_bounds__(256) void linear_w4a8_rows_kernel(
   Step cur, nxt;
   fetch(0, cur);
   for (uint32_t step = 0; step < steps; ++step) {
-    if (step + 1 < steps) fetch(step + 1, nxt);
+    fetch(step + 1 < steps ? step + 1 : step, nxt);  // unconditional: no wait inside a branch
     const bool active = step * kStep + lane * 32 < k;
     int32_t acc[ROWS][MB];
 #pragma unroll
