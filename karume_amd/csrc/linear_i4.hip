@@ -536,12 +536,13 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 4))) voi
       dst_s[r] = load_scale<ST>(srow[r], kc >> group_shift);
     }
   };
-  auto fetch_x = [&](uint32_t step, int b, Regs& regs) {
+  // `counted` = false: a repeated request whose values are not used (its x^2 must not be added)
+  auto fetch_x = [&](uint32_t step, int b, Regs& regs, bool counted = true) {
     const uint32_t k0 = step * kStepElems + lane * kLaneElems;
     const uint32_t xrow = min((uint32_t)b, m - 1);  // rows past M re-read the last row, unused
     const uint32_t kc = k0 < k ? k0 : 0u;
-    Acts<XT>::template load<VEC, NORM>(x + (size_t)xrow * k + kc, fuse.norm_weight + kc, k0 < k,
-                                       regs, squares[b]);
+    Acts<XT>::template load<VEC, NORM>(x + (size_t)xrow * k + kc, fuse.norm_weight + kc,
+                                       k0 < k && counted, regs, squares[b]);
   };
   auto consume = [&](uint32_t step, const uint32_t (&cw)[ROWS][VEC], const float (&cs)[ROWS],
                      int b, const Regs& regs) {
@@ -628,13 +629,14 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 4))) voi
     uint32_t cur_w[ROWS][VEC], nxt_w[ROWS][VEC];
     float cur_s[ROWS], nxt_s[ROWS];
     Regs cur_x, nxt_x;  // MB == 1 only: activations travel with the weights
-    fetch(0, cur_w, cur_s);
     if constexpr (MB == 1) fetch_x(0, 0, cur_x);
+    fetch(0, cur_w, cur_s);
     for (uint32_t step = 0; step < steps; ++step) {
-      if (step + 1 < steps) {
-        fetch(step + 1, nxt_w, nxt_s);
-        if constexpr (MB == 1) fetch_x(step + 1, 0, nxt_x);
-      }
+      // unconditional (the last pass asks for its own step again, a cache hit that is not
+      // used): a branch around loads makes the compiler wait for everything inside it
+      const uint32_t ahead = step + 1 < steps ? step + 1 : step;
+      if constexpr (MB == 1) fetch_x(ahead, 0, nxt_x, step + 1 < steps);
+      fetch(ahead, nxt_w, nxt_s);
       if constexpr (MB == 1) {
         consume(step, cur_w, cur_s, 0, cur_x);
         cur_x = nxt_x;
