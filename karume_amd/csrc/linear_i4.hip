@@ -366,13 +366,20 @@ __global__ __launch_bounds__(KW * 64) void gemv_i4_mfma_kernel(
       consume(wq[c], c & 1);
     }
   } else {
+    // any chunk count: the next chunk's requests are out (unconditionally; the last pass asks
+    // for its own chunk again) before this chunk is used
+    Weights wq, wq_next;
+    Acts xa, xa_next;
+    fetch_x(0, xa);
+    fetch_w(0, wq);
     for (uint32_t chunk = 0; chunk < chunks; ++chunk) {
-      Weights wq;
-      Acts xa;
-      fetch_w(chunk, wq);
-      fetch_x(chunk, xa);
+      const uint32_t ahead = chunk + 1 < chunks ? chunk + 1 : chunk;
+      fetch_x(ahead, xa_next);
+      fetch_w(ahead, wq_next);
       park_x(xa, 0);
       consume(wq, 0);
+      wq = wq_next;
+      xa = xa_next;
     }
   }
   // the waves' shares of K, added in wave order
