@@ -276,9 +276,18 @@ __global__ __launch_bounds__(KW * 64) void gemv_i4_mfma_kernel(
   const int r16 = lane & 15, g = lane >> 4;
   const uint32_t n0 = blockIdx.x * 16;
   const uint32_t wrow = min(n0 + r16, n - 1);  // rows past N re-read the last row, unused
-  const uint32_t k_quarter = k / KW;  // this wave's share of K
-  const uint32_t k_first = wave * k_quarter;
-  const uint32_t chunks = k_quarter / kChunk;
+  // This wave's share of K: an equal part with a compile-time chunk count, or (loop form) the
+  // chunks of 256 codes dealt to the waves in order, the first k/256 % KW waves one more.
+  uint32_t k_first, chunks;
+  if constexpr (CHUNKS > 0) {
+    k_first = wave * (k / KW);
+    chunks = CHUNKS;
+  } else {
+    const uint32_t total = k / kChunk, base = total / KW, extra = total % KW;
+    chunks = base + ((uint32_t)wave < extra ? 1u : 0u);
+    k_first = (wave * base + ((uint32_t)wave < extra ? (uint32_t)wave : extra)) * kChunk;
+    if (chunks == 0) k_first = 0;  // nothing to do: its (unused) requests stay inside the row
+  }
   const uint32_t* wptr = w + (size_t)wrow * (k >> 3) + (k_first >> 3) + 4 * g;
   const ST* sptr = scales + (size_t)wrow * (k >> group_shift);
 
@@ -861,7 +870,7 @@ static int32_t gemv_dispatch(krm_ctx* ctx, krm_buf x, krm_buf w, krm_buf scales,
   if (io_dtype == KRM_F16) {
     // batched fp16 rows on the matrix cores (plain op only)
     const bool plain = !fuse.norm_weight && !fuse.residual && !fuse.pair_silu && !fuse.positions;
-    if (plain && m >= 2 && k % 1024 == 0 && group >= 128 && aligned(w, 16) && aligned(x, 16) &&
+    if (plain && m >= 2 && k % 256 == 0 && group >= 128 && aligned(w, 16) && aligned(x, 16) &&
         aligned(scales, 4)) {
       uint32_t group_shift = 0;
       while ((1u << group_shift) < group) ++group_shift;
@@ -872,12 +881,18 @@ static int32_t gemv_dispatch(krm_ctx* ctx, krm_buf x, krm_buf w, krm_buf scales,
       ptr<const __half>(bias), ptr<__half>(out), m, n, k, group_shift)
   // eight waves a workgroup (two per SIMD) when K gives each at least one chunk
 #define KRM_MFMA_GEMV_BY_K(ST)                         \
-  switch (k / 1024) {                                  \
+  switch (k % 1024 ? 0u : k / 1024) {                  \
     case 1: KRM_MFMA_GEMV(ST, 1, 4); break;            \
     case 2: KRM_MFMA_GEMV(ST, 1, 8); break;            \
     case 4: KRM_MFMA_GEMV(ST, 2, 8); break;            \
     case 8: KRM_MFMA_GEMV(ST, 4, 8); break;            \
-    default: KRM_MFMA_GEMV(ST, 0, 4); break;           \
+    default:                                           \
+      if (k >= 2048) {                                 \
+        KRM_MFMA_GEMV(ST, 0, 8);                       \
+      } else {                                         \
+        KRM_MFMA_GEMV(ST, 0, 4);                       \
+      }                                                \
+      break;                                           \
   }
       if (scale_dtype == KRM_F16) {
         KRM_MFMA_GEMV_BY_K(__half)

@@ -157,9 +157,12 @@ def test_linear_batched_rows_equal_single_rows_bitwise(gpu_ctx, io):
 @pytest.mark.parametrize("m,n,k,g,scale_f16,with_bias", [
     (2, 16, 1024, 128, True, False), (16, 4096, 4096, 128, True, True),
     (7, 100, 2048, 128, False, True), (16, 33, 8192, 256, True, False),
-    (3, 250, 3072, 128, True, True), (16, 64, 5120, 1024, False, False)])
+    (3, 250, 3072, 128, True, True), (16, 64, 5120, 1024, False, False),
+    # K a multiple of 256 only: the chunks are dealt unevenly to the waves (some get none)
+    (16, 2048, 5632, 128, True, True), (5, 100, 11008, 128, True, False),
+    (3, 40, 256, 128, False, True), (16, 64, 768, 256, True, False)])
 def test_batched_fp16_rows_on_matrix_cores_match_oracle(gpu_ctx, m, n, k, g, scale_f16, with_bias):
-    """2..16 fp16 rows take the MFMA kernel (K a multiple of 1024, group >= 128): ragged N,
+    """2..16 fp16 rows take the MFMA kernel (K a multiple of 256, group >= 128): ragged N,
     every compile-time chunk count and the loop form (K = 3072, 5120), group sizes up to
     1024, f32 and fp16 scales, bias.  Gate: the oracle's f32 result rounded to fp16, one ulp."""
     rng = np.random.default_rng(m * 1000 + n)
