@@ -786,9 +786,12 @@ void gemm_i4_f16_dealt_kernel(const XT* __restrict__ x, const uint8_t* __restric
             const uint32_t word = j == 0 ? braw[nt].x : j == 1 ? braw[nt].y : j == 2 ? braw[nt].z
                                                                                     : braw[nt].w;
             const half8_t b = __builtin_bit_cast(half8_t, dequant_word(word, ws[nt]));
+            // the wave that feeds the matrix pipe goes first; the other one dequantises meanwhile
+            __builtin_amdgcn_s_setprio(1);
 #pragma unroll
             for (int mt = 0; mt < MT; ++mt)
               acc[mt][nt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[mt], b, acc[mt][nt], 0, 0, 0);
+            __builtin_amdgcn_s_setprio(0);
           }
         }
       }
