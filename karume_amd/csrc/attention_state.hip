@@ -573,13 +573,21 @@ void attention_decode_kernel(
       consume_chunk(1, rows1);
       walked = true;
     } else if (nsplit == 1 && total_chunks > 2) {
-      ChunkRows rows1, rows2;
+      // (the variant that scores on the matrix cores holds more state: two chunks at once keep
+      // it within 256 registers, i.e. two workgroups a CU for its many-split launches)
+      ChunkRows rows1;
       load_chunk(1, rows1);
-      load_chunk(2, rows2);
-      consume_chunk(0, rows0);
-      consume_chunk(1, rows1);
-      consume_chunk(2, rows2);
-      for (uint32_t chunk = 3; chunk < total_chunks; ++chunk) {
+      if constexpr (!kMfma) {
+        ChunkRows rows2;
+        load_chunk(2, rows2);
+        consume_chunk(0, rows0);
+        consume_chunk(1, rows1);
+        consume_chunk(2, rows2);
+      } else {
+        consume_chunk(0, rows0);
+        consume_chunk(1, rows1);
+      }
+      for (uint32_t chunk = kMfma ? 2 : 3; chunk < total_chunks; ++chunk) {
         load_chunk(chunk, rows0);
         consume_chunk(chunk, rows0);
       }
