@@ -56,6 +56,8 @@ DECODE_CASES = [
     StateCase("decode r4 D128 P128 boundary", 1, 8, 2, 1, 128, 256, 0, 128, 1),
     StateCase("decode r8 D64 P383", 1, 32, 4, 1, 64, 512, 0, 383, 1),
     StateCase("decode r1 D64 P0", 1, 4, 4, 1, 64, 16, 0, 0, 1),
+    StateCase("decode r1 D128 P700 six splits", 1, 4, 4, 1, 128, 1024, 0, 700, 1),
+    StateCase("decode r1 D64 P300 chunks together", 1, 4, 4, 1, 64, 512, 0, 300, 1),
     StateCase("decode r2 D32 B3 P77", 3, 4, 2, 1, 32, 96, 0, 77, 1),
     StateCase("decode sliding W100 P1000 C128", 1, 8, 2, 1, 128, 128, 100, 1000, 1),
     StateCase("decode sliding W300 P299", 1, 8, 2, 1, 64, 300, 300, 299, 1),
