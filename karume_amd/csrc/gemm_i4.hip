@@ -905,7 +905,10 @@ bool plan_deal(krm_ctx* ctx, uint32_t m, uint32_t n, uint32_t k, uint32_t& grid,
   const uint64_t tiles = (uint64_t)((m + 127) / 128) * ((n + 255) / 256);
   const uint32_t spt = (k + 127) / 128;
   const uint64_t units = tiles * spt;
-  if (tiles > kTicketSlots || units > 0x7fffffffull || units < cus) return false;
+  // at least four stages to a workgroup: with less, a tile is the sum of so many short slices
+  // that writing and merging the partials costs more than the idle CUs did (128 x 11264 x 2048:
+  // 2.75 stages each, 36.8 us against 30.9 us for one workgroup per 128 x 64 tile)
+  if (tiles > kTicketSlots || units > 0x7fffffffull || units < 4 * cus) return false;
   // whole rounds of tiles already use the chip well
   const uint64_t rounds = (tiles + cus - 1) / cus;
   if (tiles * 10 >= rounds * cus * 9) return false;

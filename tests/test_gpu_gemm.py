@@ -69,7 +69,10 @@ def test_config1_prefill_gemm(gpu_ctx, m, n, k, g, io):
                                    (64, 256, 512, 128), (33, 8, 128, 128),
                                    # enough 128 x 256 tiles for the packed-weights form, with
                                    # ragged edges in M, N and K (K ends inside a 128-code stage)
-                                   (300, 13349, 320, 64)])
+                                   (300, 13349, 320, 64),
+                                   # the same with a K long enough for the (tile, stage) units to
+                                   # be dealt over the CUs: tiles shared by 2-3 workgroups
+                                   (300, 13349, 2624, 64)])
 def test_gemm_edges_exact_weights(gpu_ctx, shape):
     """Tile edges in M, N and K (K not a multiple of the 64-code stage, N not a multiple of
     the tile) with power-of-two scales: dequantised weights are exact in fp16, x is fp16, so
@@ -93,11 +96,11 @@ def test_gemm_edges_exact_weights(gpu_ctx, shape):
 
 
 def test_gemm_with_tiles_shared_between_workgroups_is_reproducible(gpu_ctx):
-    """43 tiles of 8 stages on 256 CUs: the (tile, stage) units are dealt one or two to a
-    workgroup, so every tile is the sum of 4-8 partials added by whichever workgroup arrives
+    """86 tiles of 32 stages on 256 CUs: the (tile, stage) units are dealt 10 or 11 to a
+    workgroup, so every tile is the sum of 3-4 partials added by whichever workgroup arrives
     last.  The sum is taken in K order whoever that is: repeated runs give the same bits, and
     the result meets the exact-weights gate."""
-    m, n, k, g = 128, 11008, 1024, 128
+    m, n, k, g = 256, 11008, 4096, 128
     rng = np.random.default_rng(77)
     q = rng.integers(-8, 8, size=(n, k), dtype=np.int8)
     scale = (2.0 ** rng.integers(-8, -3, size=(n, k // g))).astype(np.float32)
