@@ -601,23 +601,26 @@ void attention_decode_kernel(
       consume_chunk(chunk, rows0);
     }
   }
-  // this step's own column: one more row for group 0 of the last split
+  // this step's own column: one more row for group 0 of the last split (for every other lane
+  // the update below is the identity, so the other splits skip it)
+  if (last) {
 #pragma unroll
-  for (int h = 0; h < R; ++h) {
-    float part = 0.f;
+    for (int h = 0; h < R; ++h) {
+      float part = 0.f;
 #pragma unroll
-    for (int e = 0; e < E; ++e) part = fmaf(qf[h][e], kx[e], part);
-    part = group_sum<LPR>(part);
-    const float s_own = own ? part : -INFINITY;
-    const float m_new = fmaxf(run_m[h], s_own);
-    const float ref = m_new == -INFINITY ? 0.f : m_new;
-    const float keep = __builtin_amdgcn_exp2f(run_m[h] - ref);
-    const float p = __builtin_amdgcn_exp2f(s_own - ref);
-    run_m[h] = m_new;
-    run_l[h] = run_l[h] * keep + p;
+      for (int e = 0; e < E; ++e) part = fmaf(qf[h][e], kx[e], part);
+      part = group_sum<LPR>(part);
+      const float s_own = own ? part : -INFINITY;
+      const float m_new = fmaxf(run_m[h], s_own);
+      const float ref = m_new == -INFINITY ? 0.f : m_new;
+      const float keep = __builtin_amdgcn_exp2f(run_m[h] - ref);
+      const float p = __builtin_amdgcn_exp2f(s_own - ref);
+      run_m[h] = m_new;
+      run_l[h] = run_l[h] * keep + p;
 #pragma unroll
-    for (int e = 0; e < E; ++e)
-      acc[h][e] = fmaf(p, own ? vx[e] : 0.f, acc[h][e] * keep);  // 0 * NaN must not leak
+      for (int e = 0; e < E; ++e)
+        acc[h][e] = fmaf(p, own ? vx[e] : 0.f, acc[h][e] * keep);  // 0 * NaN must not leak
+    }
   }
 
   // merge of the G group states, ascending group order
