@@ -390,7 +390,9 @@ def main() -> int:
     if args.only in ("", "gemm"):
         for name, (gn, gk) in {"up": (11008, 4096), "down": (4096, 11008)}.items():
             log(f"[bench] prefill GEMM M=512 K={gk} N={gn} (config 1, {name}-projection)")
-            ms_g, flops = bench_gemm(ctx, ka, rng, 40, 8, 512, gn, gk, g)
+            # 400 warm-up launches (30 ms): a shorter run still sees the clocks ramping up from
+            # idle (100 launches from idle measure 81 us each, 2000 measure 68 us)
+            ms_g, flops = bench_gemm(ctx, ka, rng, 400, 400, 512, gn, gk, g)
             result[f"gemm_{name}_tflops"] = round(flops / (ms_g * 1e-3) / 1e12, 1)
             result[f"gemm_{name}_us"] = round(ms_g * 1e3, 2)
             result[f"gemm_{name}_pct_of_f16_mfma_peak"] = round(
@@ -403,7 +405,7 @@ def main() -> int:
         result["w4a8_gemv_product_us"] = round(ms_p * 1e3, 3)
         result["w4a8_gemv_product_gbs"] = round(w4_bytes / (ms_p * 1e-3) / 1e9, 1)
         for name, (gn, gk) in {"up": (11008, 4096), "down": (4096, 11008)}.items():
-            ms_q, ms_p = bench_w4a8(ctx, ka, rng, 40, 8, 512, gn, gk, g, 4)
+            ms_q, ms_p = bench_w4a8(ctx, ka, rng, 400, 400, 512, gn, gk, g, 4)
             ops = 2.0 * 512 * gn * gk
             result[f"w4a8_gemm_{name}_us"] = round(ms_q * 1e3, 2)
             result[f"w4a8_gemm_{name}_product_us"] = round(ms_p * 1e3, 2)
