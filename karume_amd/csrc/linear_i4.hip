@@ -579,36 +579,73 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 4))) voi
       constexpr int kUnits = sizeof(Regs) / 16;
       static_assert(sizeof(Regs) % 16 == 0, "activation registers are whole 16-byte units");
       __shared__ uint4 s_x[NSTEP * kUnits * kWave];
-      __shared__ float s_squares[NSTEP];
-      // The staging waves ask for the activations first: loads return in order, and x (in the
-      // cache) would otherwise arrive behind the weights (from memory) and hold the whole
-      // workgroup at the barrier until then; with x early, every wave starts on its rows as
-      // soon as its own weights are there.
-      typename Acts<XT>::template Raw<VEC, NORM> raw_x;
-      const uint32_t x_k0 = (uint32_t)wave * kStepElems + lane * kLaneElems;
-      const uint32_t x_kc = x_k0 < k ? x_k0 : 0u;
-      if (wave < NSTEP)
-        Acts<XT>::template request<VEC, NORM>(x + x_kc, fuse.norm_weight + x_kc, raw_x);
+      __shared__ float s_squares[VEC == 4 ? 4 : NSTEP];
+      if constexpr (VEC == 4) {
+        // Every wave stages a quarter of each step (8 elements a lane) and asks for it before
+        // its weights.  Loads return in order — also across the waves of a CU, whose requests
+        // share one queue in the vector cache — so x lines asked for after any weight line
+        // arrive behind it: with one staging wave the barrier below opened only when weights
+        // had come back from HBM (1.2-3.9 us after the launch), and all waves then ran their
+        // dot products at once.  With x first in every wave the barrier opens after a cache
+        // round trip and each wave starts on its rows as soon as its own weights are there.
+        using Quarter = typename Acts<XT>::template Raw<1, NORM>;
+        Quarter raw_q[NSTEP];
 #pragma unroll
-      for (int step = 0; step < NSTEP; ++step) fetch(step, all_w[step], all_s[step]);
-      if (wave < NSTEP) {
-        Regs regs;
-        Acts<XT>::template finish<VEC, NORM>(raw_x, x_k0 < k, regs, squares[0]);
-        uint4 units[kUnits];
-        __builtin_memcpy(units, &regs, sizeof(Regs));
+        for (int step = 0; step < NSTEP; ++step) {
+          const uint32_t q_k0 = (uint32_t)step * kStepElems + wave * 512 + lane * 8;
+          const uint32_t q_kc = q_k0 < k ? q_k0 : 0u;
+          Acts<XT>::template request<1, NORM>(x + q_kc, fuse.norm_weight + q_kc, raw_q[step]);
+        }
 #pragma unroll
-        for (int u = 0; u < kUnits; ++u) s_x[(wave * kUnits + u) * kWave + lane] = units[u];
+        for (int step = 0; step < NSTEP; ++step) fetch(step, all_w[step], all_s[step]);
+#pragma unroll
+        for (int step = 0; step < NSTEP; ++step) {
+          const uint32_t q_k0 = (uint32_t)step * kStepElems + wave * 512 + lane * 8;
+          typename Acts<XT>::template Regs<1> part;
+          Acts<XT>::template finish<1, NORM>(raw_q[step], q_k0 < k, part, squares[0]);
+          uint4 units[2];
+          __builtin_memcpy(units, &part, sizeof(part));
+          // elements wave * 512 + lane * 8 .. + 8 of the step are units 2 * (lane % 4) and
+          // the next one of the consuming lane wave * 16 + lane / 4
+#pragma unroll
+          for (int j = 0; j < 2; ++j)
+            s_x[(step * kUnits + (lane & 3) * 2 + j) * kWave + wave * 16 + (lane >> 2)] = units[j];
+        }
         if constexpr (NORM) {
           const float total = wave_sum(squares[0]);
           if (lane == 0) s_squares[wave] = total;
         }
-      }
-      __syncthreads();
-      if constexpr (NORM) {
-        float total = 0.f;
+        __syncthreads();
+        if constexpr (NORM)
+          shared_squares = ((s_squares[0] + s_squares[1]) + s_squares[2]) + s_squares[3];
+      } else {
+        // narrow steps (4-byte loads): wave s stages step s, its activations requested first
+        typename Acts<XT>::template Raw<VEC, NORM> raw_x;
+        const uint32_t x_k0 = (uint32_t)wave * kStepElems + lane * kLaneElems;
+        const uint32_t x_kc = x_k0 < k ? x_k0 : 0u;
+        if (wave < NSTEP)
+          Acts<XT>::template request<VEC, NORM>(x + x_kc, fuse.norm_weight + x_kc, raw_x);
 #pragma unroll
-        for (int step = 0; step < NSTEP; ++step) total += s_squares[step];
-        shared_squares = total;
+        for (int step = 0; step < NSTEP; ++step) fetch(step, all_w[step], all_s[step]);
+        if (wave < NSTEP) {
+          Regs regs;
+          Acts<XT>::template finish<VEC, NORM>(raw_x, x_k0 < k, regs, squares[0]);
+          uint4 units[kUnits];
+          __builtin_memcpy(units, &regs, sizeof(Regs));
+#pragma unroll
+          for (int u = 0; u < kUnits; ++u) s_x[(wave * kUnits + u) * kWave + lane] = units[u];
+          if constexpr (NORM) {
+            const float total = wave_sum(squares[0]);
+            if (lane == 0) s_squares[wave] = total;
+          }
+        }
+        __syncthreads();
+        if constexpr (NORM) {
+          float total = 0.f;
+#pragma unroll
+          for (int step = 0; step < NSTEP; ++step) total += s_squares[step];
+          shared_squares = total;
+        }
       }
 #pragma unroll
       for (int step = 0; step < NSTEP; ++step) {
