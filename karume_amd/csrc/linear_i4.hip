@@ -129,17 +129,41 @@ struct Acts<__half> {
   };
   // `g` (optional): rms_norm weights of the same 8*VEC positions; the lane then carries
   // fp16(x * g) and adds its x^2 to `squares`.
+  // The loads of `load` alone (see Acts<float>::Raw).
+  template <int VEC, bool NORM>
+  struct Raw {
+    uint4 x[VEC];
+    float4 g[NORM ? VEC : 1][2];
+  };
+  template <int VEC, bool NORM>
+  __device__ static inline void request(const __half* x, const float* g, Raw<VEC, NORM>& raw) {
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) {
+      raw.x[j] = reinterpret_cast<const uint4*>(x)[j];
+      if constexpr (NORM) {
+        raw.g[j][0] = reinterpret_cast<const float4*>(g)[2 * j];
+        raw.g[j][1] = reinterpret_cast<const float4*>(g)[2 * j + 1];
+      }
+    }
+  }
   template <int VEC, bool NORM>
   __device__ static inline void load(const __half* x, const float* g, bool active, Regs<VEC>& r,
                                      float& squares) {
+    Raw<VEC, NORM> raw;
+    request<VEC, NORM>(x, g, raw);
+    finish<VEC, NORM>(raw, active, r, squares);
+  }
+  template <int VEC, bool NORM>
+  __device__ static inline void finish(const Raw<VEC, NORM>& in, bool active, Regs<VEC>& r,
+                                       float& squares) {
 #pragma unroll
     for (int j = 0; j < VEC; ++j) {
-      uint4 raw = reinterpret_cast<const uint4*>(x)[j];
+      uint4 raw = in.x[j];
       if constexpr (NORM) {
         const uint32_t keep = active ? 0xFFFFFFFFu : 0u;  // x^2 of a lane past K must be 0
         raw.x &= keep; raw.y &= keep; raw.z &= keep; raw.w &= keep;
-        const float4 ga = reinterpret_cast<const float4*>(g)[2 * j];
-        const float4 gb = reinterpret_cast<const float4*>(g)[2 * j + 1];
+        const float4 ga = in.g[j][0];
+        const float4 gb = in.g[j][1];
         const float gw[8] = {ga.x, ga.y, ga.z, ga.w, gb.x, gb.y, gb.z, gb.w};
         uint32_t words[4] = {raw.x, raw.y, raw.z, raw.w};
 #pragma unroll
@@ -467,7 +491,7 @@ __device__ inline void slot_store(void* slot, int32_t is_f16, size_t i, float v)
 //  weight requests are out.
 template <typename XT, int MB, int NSTEP>
 constexpr bool share_x_in_lds() {
-  return sizeof(XT) == 4 && MB == 1 && NSTEP > 0 && NSTEP <= 4;
+  return MB == 1 && NSTEP > 0 && NSTEP <= 4;
 }
 
 // NORM and DECODE_ROW are compile-time so that the plain kernel carries neither their branches
@@ -603,13 +627,15 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 4))) voi
           const uint32_t q_k0 = (uint32_t)step * kStepElems + wave * 512 + lane * 8;
           typename Acts<XT>::template Regs<1> part;
           Acts<XT>::template finish<1, NORM>(raw_q[step], q_k0 < k, part, squares[0]);
-          uint4 units[2];
+          constexpr int kQuarterUnits = sizeof(part) / 16;  // 2 (f32) or 1 (fp16)
+          uint4 units[kQuarterUnits];
           __builtin_memcpy(units, &part, sizeof(part));
-          // elements wave * 512 + lane * 8 .. + 8 of the step are units 2 * (lane % 4) and
-          // the next one of the consuming lane wave * 16 + lane / 4
+          // elements wave * 512 + lane * 8 .. + 8 of the step are the units from
+          // kQuarterUnits * (lane % 4) on of the consuming lane wave * 16 + lane / 4
 #pragma unroll
-          for (int j = 0; j < 2; ++j)
-            s_x[(step * kUnits + (lane & 3) * 2 + j) * kWave + wave * 16 + (lane >> 2)] = units[j];
+          for (int j = 0; j < kQuarterUnits; ++j)
+            s_x[(step * kUnits + (lane & 3) * kQuarterUnits + j) * kWave + wave * 16 + (lane >> 2)] =
+                units[j];
         }
         if constexpr (NORM) {
           const float total = wave_sum(squares[0]);
