@@ -210,6 +210,10 @@ int32_t krm_lengths_positions(krm_ctx* ctx, krm_buf lengths, krm_buf positions_i
  * step (packages/models/src/generation/greedy.ts:245-252 reads back every step). */
 int32_t krm_lengths_log_token(krm_ctx* ctx, krm_buf lengths, krm_buf token_i32,
                               krm_buf history_i32, uint32_t history_len);
+/* krm_lengths_log_token, krm_lengths_advance and krm_lengths_positions (one row) in one launch:
+ * the end of a recorded one-row decode step, which leaves the next step's position behind. */
+int32_t krm_lengths_step_end(krm_ctx* ctx, krm_buf lengths, krm_buf token_i32,
+                             krm_buf history_i32, uint32_t history_len, krm_buf positions_i32);
 /* krm_attention_state with device lengths; `max_past` sizes the launch and the workspace. */
 int32_t krm_attention_state_lengths(krm_ctx* ctx, krm_buf q, krm_buf ins_k, krm_buf ins_v,
                                     krm_buf slot_k, krm_buf slot_v, krm_buf out, uint32_t batch,

@@ -62,6 +62,7 @@ PROTOTYPES = {
     "krm_lengths_advance": (i32, [c_ctx, c_buf]),
     "krm_lengths_positions": (i32, [c_ctx, c_buf, c_buf, u32]),
     "krm_lengths_log_token": (i32, [c_ctx, c_buf, c_buf, c_buf, u32]),
+    "krm_lengths_step_end": (i32, [c_ctx, c_buf, c_buf, c_buf, u32, c_buf]),
     "krm_attention_state_lengths": (i32, [c_ctx, c_buf, c_buf, c_buf, c_buf, c_buf, c_buf, u32,
                                           u32, u32, u32, u32, u32, u32, C.c_float, c_buf, u32,
                                           i32, i32, c_buf, size_t]),

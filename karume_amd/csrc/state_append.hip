@@ -255,7 +255,33 @@ __global__ void lengths_log_token_kernel(uint32_t* lengths, const int32_t* token
   lengths[3] = at + 1;
 }
 
+// End of a one-row decode step in one launch: the three kernels above in their order.
+__global__ void lengths_step_end_kernel(uint32_t* lengths, const int32_t* token, int32_t* history,
+                                        uint32_t history_len, int32_t* positions) {
+  const uint32_t at = lengths[3];
+  if (at < history_len) history[at] = token[0];
+  lengths[3] = at + 1;
+  uint32_t past = lengths[0];
+  if (lengths[2] == 0u) {
+    past += lengths[1];
+    lengths[0] = past;
+  }
+  positions[0] = (int32_t)past;
+}
+
 extern "C" {
+
+int32_t krm_lengths_step_end(krm_ctx* ctx, krm_buf lengths, krm_buf token_i32,
+                             krm_buf history_i32, uint32_t history_len, krm_buf positions_i32) {
+  KRM_TRY(enter(ctx));
+  KRM_REQUIRE(ctx, lengths && token_i32 && history_i32 && positions_i32 && lengths % 4 == 0 &&
+                       token_i32 % 4 == 0 && history_i32 % 4 == 0 && positions_i32 % 4 == 0,
+              "krm_lengths_step_end: bad buffer");
+  lengths_step_end_kernel<<<dim3(1), dim3(1), 0, ctx->stream>>>(
+      ptr<uint32_t>(lengths), ptr<const int32_t>(token_i32), ptr<int32_t>(history_i32),
+      history_len, ptr<int32_t>(positions_i32));
+  return launched(ctx, "lengths_step_end_kernel");
+}
 
 int32_t krm_lengths_log_token(krm_ctx* ctx, krm_buf lengths, krm_buf token_i32,
                               krm_buf history_i32, uint32_t history_len) {

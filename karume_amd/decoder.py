@@ -378,11 +378,11 @@ class LlamaDecoderSession:
             b["token"].upload(np.array([first_token, 0, 0, 0], dtype=np.int32))
             g.lengths_set(context.lengths, context.past, 1)
             self._replay_last_past = context.past + count - 1
+            g.lengths_positions(context.lengths, b["pos"], 1)
             with g.record() as rec:
-                g.lengths_positions(context.lengths, b["pos"], 1)
                 self._forward(context, 1, 0, 1, 0, lengths=context.lengths, ids=b["token"])
-                g.lengths_log_token(context.lengths, b["token"], history, count)
-                g.lengths_advance(context.lengths)
+                # token logged, lengths advanced, the next replay's position written: one launch
+                g.lengths_step_end(context.lengths, b["token"], history, count, b["pos"])
             graph = rec.graph
             for _ in range(count):
                 graph.launch()

@@ -344,6 +344,13 @@ class GpuContext:
         self._check(self._lib.krm_lengths_log_token(self._handle, _addr(lengths), _addr(token),
                                                     _addr(history), history_len))
 
+    def lengths_step_end(self, lengths: BufferLike, token: BufferLike, history: BufferLike,
+                         history_len: int, positions: BufferLike) -> None:
+        """log the token, advance the lengths, leave the next one-row step's position."""
+        self._check(self._lib.krm_lengths_step_end(self._handle, _addr(lengths), _addr(token),
+                                                   _addr(history), history_len,
+                                                   _addr(positions)))
+
     def attention_state_lengths(self, q: BufferLike, ins_k: BufferLike, ins_v: BufferLike,
                                 slot_k: BufferLike, slot_v: BufferLike, out: BufferLike, *,
                                 batch: int, heads: int, kv_heads: int, chunk_rows: int,

@@ -366,3 +366,26 @@ def test_context_capacity_and_poison(gpu_ctx):
     ctx.dispose()
     with pytest.raises(ka.KarumeError):
         session.run(ids[:, :1], ids[:, :1], 0, context=ctx, query_length=1)
+
+
+def test_lengths_step_end_equals_the_three_launches(gpu_ctx):
+    """krm_lengths_step_end = log_token + advance + positions (one row), clean and faulted."""
+    for fault in (0, 1):
+        state = np.array([41, 1, fault, 2], dtype=np.uint32)
+        token = gpu_ctx.upload(np.array([777, 0, 0, 0], dtype=np.int32))
+        outs = []
+        for fused in (False, True):
+            lengths = gpu_ctx.upload(state.copy())
+            history = gpu_ctx.upload(np.full(4, -1, dtype=np.int32))
+            pos = gpu_ctx.upload(np.full(4, -5, dtype=np.int32))
+            if fused:
+                gpu_ctx.lengths_step_end(lengths, token, history, 4, pos)
+            else:
+                gpu_ctx.lengths_log_token(lengths, token, history, 4)
+                gpu_ctx.lengths_advance(lengths)
+                gpu_ctx.lengths_positions(lengths, pos, 1)
+            outs.append((lengths.download(np.uint32, (4,)).tolist(),
+                         history.download(np.int32, (4,)).tolist(),
+                         pos.download(np.int32, (4,)).tolist()))
+        assert outs[0] == outs[1]
+        assert outs[1][0][0] == (41 if fault else 42) and outs[1][1][2] == 777
