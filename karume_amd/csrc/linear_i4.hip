@@ -741,8 +741,12 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 4))) voi
   float inv[MB];
 #pragma unroll
   for (int b = 0; b < MB; ++b)
-    inv[b] = NORM ? 1.0f / sqrtf((XLDS ? shared_squares : wave_sum(squares[b])) / (float)k +
-                                 fuse.norm_eps)
+    // v_rsq_f32 (1 ulp) here, v_exp_f32 and v_rcp_f32 in the silu below: the IEEE sequences of
+    // sqrt, division and expf were a third of this epilogue's instructions, issued by every wave
+    // of the CU at the same moment (gate/up launch: 1.4 us between the last dot product and the
+    // end); the stand-alone rms_norm and silu kernels keep the exact forms
+    inv[b] = NORM ? __builtin_amdgcn_rsqf((XLDS ? shared_squares : wave_sum(squares[b])) / (float)k +
+                                          fuse.norm_eps)
                   : 1.0f;
   const XT* residual = static_cast<const XT*>(fuse.residual);
   if constexpr (ROWS % 2 == 0) {
@@ -761,8 +765,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 4))) voi
               gate += to_f32<XT>(bias[row]);
               up += to_f32<XT>(bias[row + 1]);
             }
-            const float t = expf(-fabsf(gate));
-            const float sig = gate < 0.f ? t / (1.0f + t) : 1.0f / (1.0f + t);
+            const float t = __builtin_amdgcn_exp2f(-fabsf(gate) * 1.4426950408889634f);
+            const float r = __builtin_amdgcn_rcpf(1.0f + t);
+            const float sig = gate < 0.f ? t * r : r;
             float value = __fmul_rn(__fmul_rn(gate, sig), up);
             if (residual) value += to_f32<XT>(residual[(size_t)b * half_n + col]);
             out[(size_t)b * half_n + col] = from_f32<XT>(value);
