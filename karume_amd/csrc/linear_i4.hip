@@ -63,24 +63,49 @@ __global__ __launch_bounds__(256) void dequant_i4_kernel(const uint32_t* __restr
 
 // ------------------------------------------------------------------------------------ GEMV
 
-// Sum over the 64 lanes of a wave; every lane returns the total.  Fixed tree: quad swaps,
-// half-row mirror, row mirror (16-lane rows), then the four row sums in ascending order.
+// Sums over the 64 lanes of a wave.  One fixed order of additions for every form, so a row's
+// bits do not depend on how many rows its wave reduces: partner lane ^ 1, lane ^ 2 (quad
+// permutes), then the quads of a 16-lane row (rotate by 4, by 8), the rows 16 apart (swizzle) and
+// the halves 32 apart; the value of lane 0 (or of lane r for row r) is the result.
+template <int CTRL>
+__device__ inline float dpp_from(float v) {
+  return __builtin_bit_cast(
+      float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, true));
+}
+// levels 3..6: every lane adds lanes at the same position mod 4
+__device__ inline float wave_sum_tail(float v) {
+  v += dpp_from<0x124>(v);  // row_ror:4
+  v += dpp_from<0x128>(v);  // row_ror:8
+  v += __builtin_bit_cast(float, __builtin_amdgcn_ds_swizzle(__builtin_bit_cast(int, v), 0x401F));  // lane ^ 16
+  v += __shfl_xor(v, 32, kWave);
+  return v;
+}
+__device__ inline float lane_value(float v, int lane) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), lane));
+}
+// every lane returns the total
 __device__ inline float wave_sum(float v) {
-  int t;
-  t = __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0xB1, 0xf, 0xf, true);
-  v += __builtin_bit_cast(float, t);  // quad_perm [1,0,3,2]
-  t = __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x4E, 0xf, 0xf, true);
-  v += __builtin_bit_cast(float, t);  // quad_perm [2,3,0,1]
-  t = __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x141, 0xf, 0xf, true);
-  v += __builtin_bit_cast(float, t);  // row_half_mirror
-  t = __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x140, 0xf, 0xf, true);
-  v += __builtin_bit_cast(float, t);  // row_mirror
-  const int bits = __builtin_bit_cast(int, v);
-  const float r0 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(bits, 0));
-  const float r1 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(bits, 16));
-  const float r2 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(bits, 32));
-  const float r3 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(bits, 48));
-  return ((r0 + r1) + r2) + r3;
+  v += dpp_from<0xB1>(v);  // quad_perm [1,0,3,2]
+  v += dpp_from<0x4E>(v);  // quad_perm [2,3,0,1]
+  v += dpp_from<0x124>(v);
+  v += dpp_from<0x128>(v);
+  // the last two levels through scalar registers: the same pairs as wave_sum_tail
+  return (lane_value(v, 0) + lane_value(v, 16)) + (lane_value(v, 32) + lane_value(v, 48));
+}
+// Two and four sums at once: after the first level a lane keeps one of two values, after the
+// second one of four, so the later levels run once.  Lane r ends with the total of value r.
+__device__ inline float wave_sum2(float a, float b, int lane) {
+  const bool odd = lane & 1;
+  float p = (odd ? b : a) + dpp_from<0xB1>(odd ? a : b);
+  p += dpp_from<0x4E>(p);
+  return wave_sum_tail(p);
+}
+__device__ inline float wave_sum4(float a, float b, float c, float d, int lane) {
+  const bool odd = lane & 1, high = lane & 2;
+  const float p0 = (odd ? b : a) + dpp_from<0xB1>(odd ? a : b);  // even lanes: a, odd lanes: b
+  const float p1 = (odd ? d : c) + dpp_from<0xB1>(odd ? c : d);  // even lanes: c, odd lanes: d
+  const float q = (high ? p1 : p0) + dpp_from<0x4E>(high ? p0 : p1);
+  return wave_sum_tail(q);
 }
 
 // Eight codes of one u32 as four fp16 pairs holding the exact integers (u - 8):
@@ -749,6 +774,22 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 4))) voi
                                           fuse.norm_eps)
                   : 1.0f;
   const XT* residual = static_cast<const XT*>(fuse.residual);
+  // the rows' totals, uniform (one row of x: two or four rows are reduced together)
+  float total[ROWS][MB];
+  if constexpr (MB == 1 && ROWS == 4) {
+    const float t = wave_sum4(acc[0][0], acc[1][0], acc[2][0], acc[3][0], lane);
+#pragma unroll
+    for (int r = 0; r < ROWS; ++r) total[r][0] = lane_value(t, r);
+  } else if constexpr (MB == 1 && ROWS == 2) {
+    const float t = wave_sum2(acc[0][0], acc[1][0], lane);
+#pragma unroll
+    for (int r = 0; r < ROWS; ++r) total[r][0] = lane_value(t, r);
+  } else {
+#pragma unroll
+    for (int r = 0; r < ROWS; ++r)
+#pragma unroll
+      for (int b = 0; b < MB; ++b) total[r][b] = wave_sum(acc[r][b]);
+  }
   if constexpr (ROWS % 2 == 0) {
     if (fuse.pair_silu) {
       // rows (2i, 2i+1) hold (gate_i, up_i): out[., i] = silu(gate) * up, n/2 outputs per row
@@ -758,8 +799,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 4))) voi
         const uint32_t row = row0 + 2 * p, col = row >> 1;
 #pragma unroll
         for (int b = 0; b < MB; ++b) {
-          float gate = wave_sum(acc[2 * p][b]) * inv[b];
-          float up = wave_sum(acc[2 * p + 1][b]) * inv[b];
+          float gate = total[2 * p][b] * inv[b];
+          float up = total[2 * p + 1][b] * inv[b];
           if (lane == (p * MB + b) % kWave && row + 1 < n && (uint32_t)b < m) {
             if (bias) {
               gate += to_f32<XT>(bias[row]);
@@ -792,8 +833,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 4))) voi
 #pragma unroll
       for (int p = 0; p < ROWS / 2; ++p) {
         const uint32_t row = row0 + 2 * p, pair = row >> 1;
-        float x0 = wave_sum(acc[2 * p][0]) * inv[0];
-        float x1 = wave_sum(acc[2 * p + 1][0]) * inv[0];
+        float x0 = total[2 * p][0] * inv[0];
+        float x1 = total[2 * p + 1][0] * inv[0];
         if (lane != p % kWave || row + 1 >= n) continue;
         if (bias) {
           x0 += to_f32<XT>(bias[row]);
@@ -837,10 +878,10 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 4))) voi
   for (int r = 0; r < ROWS; ++r) {
 #pragma unroll
     for (int b = 0; b < MB; ++b) {
-      const float total = wave_sum(acc[r][b]) * inv[b];
+      const float sum = total[r][b] * inv[b];
       const uint32_t row = row0 + r;
       if (lane == (r * MB + b) % kWave && row < n && (uint32_t)b < m) {
-        float value = total + (bias ? to_f32<XT>(bias[row]) : 0.f);
+        float value = sum + (bias ? to_f32<XT>(bias[row]) : 0.f);
         if (residual) value += to_f32<XT>(residual[(size_t)b * n + row]);
         out[(size_t)b * n + row] = from_f32<XT>(value);
       }
