@@ -195,26 +195,40 @@ __global__ __launch_bounds__(kArgmaxThreads) void argmax_kernel(const XT* __rest
       }
     }
   }
-  for (int off = 32; off > 0; off >>= 1) {
-    const float ov = __shfl_xor(best, off, kWave);
-    const uint32_t oi = (uint32_t)__shfl_xor((int)at, off, kWave);
+  // Any tree gives the same pair.  Inside a 16-lane row the partners come through DPP (lane ^ 1,
+  // lane ^ 2, rotations by 4 and 8), the rows 16 and 32 lanes apart through the LDS crossbar.
+  auto take = [&](float ov, uint32_t oi) {
     if (beats(ov, oi, best, at)) {
       best = ov;
       at = oi;
     }
-  }
+  };
+  auto fold_row = [&]() {
+#define KRM_ARGMAX_DPP(CTRL)                                                                      \
+  take(__builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, best),   \
+                                                            CTRL, 0xf, 0xf, true)),              \
+       (uint32_t)__builtin_amdgcn_update_dpp(0, (int)at, CTRL, 0xf, 0xf, true))
+    KRM_ARGMAX_DPP(0xB1);   // quad_perm [1,0,3,2]
+    KRM_ARGMAX_DPP(0x4E);   // quad_perm [2,3,0,1]
+    KRM_ARGMAX_DPP(0x124);  // row_ror:4
+    KRM_ARGMAX_DPP(0x128);  // row_ror:8
+#undef KRM_ARGMAX_DPP
+  };
+  fold_row();
+  for (int off = 16; off <= 32; off <<= 1)
+    take(__shfl_xor(best, off, kWave), (uint32_t)__shfl_xor((int)at, off, kWave));
   if ((threadIdx.x & 63) == 0) {
     s_val[threadIdx.x >> 6] = best;
     s_idx[threadIdx.x >> 6] = at;
   }
   __syncthreads();
-  if (threadIdx.x == 0) {
-    for (int w = 1; w < kArgmaxThreads / kWave; ++w)
-      if (beats(s_val[w], s_idx[w], best, at)) {
-        best = s_val[w];
-        at = s_idx[w];
-      }
-    out[blockIdx.x] = (int32_t)at;
+  if (threadIdx.x < kWave) {  // the 16 wave results, one per lane of the first row
+    static_assert(kArgmaxThreads / kWave == 16, "one 16-lane row holds the wave results");
+    const int w = threadIdx.x & 15;
+    best = s_val[w];
+    at = s_idx[w];
+    fold_row();
+    if (threadIdx.x == 0) out[blockIdx.x] = (int32_t)at;
   }
 }
 
