@@ -26,61 +26,129 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
-# HBM bytes per config-0 GEMV launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled
-# by an 8 MiB copy kernel's readings (profiles/gemv_i4_config0_pmc_traffic.txt).
-GEMV_PMC_TRAFFIC_BYTES = 8_816_800
 USE_GRAPHS = True       # --no-graph: plain launches (rocprofv3's kernel trace crashes on graph launches)
+REPLAYS = 50            # timed replays of a recorded graph; the median is reported
+EVICT_BYTES = 512 << 20  # streamed between timed replays: twice the 256 MB Infinity Cache
+PROFILES = os.path.join(ROOT, "profiles")
 
 
 def log(msg: str) -> None:
     print(msg, file=sys.stderr, flush=True)
 
 
-def timed(ctx, fn, steps: int, warmup: int, period: int = 64) -> float:
-    """Milliseconds for exactly `steps` calls of fn(i), HIP events on the context's stream.
+def pmc_traffic_bytes(summary: str):
+    """HBM bytes per launch that a rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE summary under
+    profiles/ states on its `traffic_bytes_per_launch = N (kernel NAME)` line; None without it."""
+    try:
+        for line in open(os.path.join(PROFILES, summary)):
+            if line.startswith("traffic_bytes_per_launch"):
+                value = line.split("=", 1)[1].split()[0]
+                return int(value.replace(",", ""))
+    except OSError:
+        pass
+    return None
 
-    The calls are recorded once (`period` consecutive steps = one graph) and replayed, the way
-    a decode loop replays its recorded token step, so the host's launch cost is not what is
-    measured; a remainder of steps % period is issued as plain calls."""
-    if not USE_GRAPHS:
-        for i in range(warmup):
-            fn(i)
-        ctx.sync()
-        start, stop = ctx.event(), ctx.event()
-        start.record()
-        for i in range(steps):
-            fn(i)
-        stop.record()
-        ms = start.elapsed_ms(stop)
-        ctx.sync()
-        start.destroy()
-        stop.destroy()
-        return ms
-    with ctx.record() as rec:
-        for i in range(period):
-            fn(i)
-    graph = rec.graph
-    for _ in range(max(1, warmup // period)):
+
+class Timer:
+    """Times recorded launch sequences on one context.
+
+    `steps` calls fn(0..steps-1) are recorded into ONE graph (the way a decode loop records its
+    token step) and the graph is replayed REPLAYS times; every replay is bracketed by HIP events
+    on the launch stream and preceded by untimed work that (a) streams EVICT_BYTES through the
+    caches, so that no replay finds what the one before left there, and (b) keeps the device
+    busy while the host queues the start event and the graph, so that the events bracket device
+    time only.  The median replay is reported."""
+
+    def __init__(self, ctx, ka):
+        self.ctx, self.ka = ctx, ka
+        self.evict = ctx.alloc(EVICT_BYTES)
+        self.start, self.stop = ctx.event(), ctx.event()
+        self.evict_pass_ms = None
+
+    def close(self) -> None:
+        self.evict.free()
+        self.start.destroy()
+        self.stop.destroy()
+
+    def evict_pass(self) -> None:
+        self.ctx.probe_launch(self.ka.PROBE_READ, self.evict, EVICT_BYTES, grid=4096, block=256)
+
+    def _calibrate(self) -> None:
+        if self.evict_pass_ms is not None:
+            return
+        for _ in range(3):
+            self.evict_pass()
+        self.ctx.sync()
+        self.start.record()
+        for _ in range(4):
+            self.evict_pass()
+        self.stop.record()
+        self.evict_pass_ms = self.start.elapsed_ms(self.stop) / 4
+
+    def run(self, fn, steps: int, warmup: int, *, after_evict=None, branches: int = 1,
+            replays: int = REPLAYS) -> dict:
+        """{"ms": median ms of one pass of `steps` calls, "ms_min", "ms_max", "mode", ...}.
+        `after_evict` (optional) queues untimed calls behind the eviction (e.g. to warm the
+        caches again for a cache-resident figure)."""
+        ctx = self.ctx
+        if not USE_GRAPHS:
+            for i in range(warmup):
+                fn(i)
+            ctx.sync()
+            self.start.record()
+            for i in range(steps):
+                fn(i)
+            self.stop.record()
+            ms = self.start.elapsed_ms(self.stop)
+            ctx.sync()
+            return {"ms": ms, "ms_min": ms, "ms_max": ms, "mode": "plain launches", "replays": 1,
+                    "timed_s": ms * 1e-3}
+        self._calibrate()
+        with ctx.record() as rec:
+            if branches > 1:
+                for b in range(1, branches):
+                    rec.branch(b)   # every side branch forks before the first launch
+            for i in range(steps):
+                if branches > 1:
+                    rec.branch(i % branches)
+                fn(i)
+        graph = rec.graph
+        # host cost of queueing one replay, measured while the device is busy
+        for _ in range(4):
+            self.evict_pass()
+        t0 = time.perf_counter()
         graph.launch()
-    ctx.sync()
-    start, stop = ctx.event(), ctx.event()
-    start.record()
-    for _ in range(steps // period):
-        graph.launch()
-    for i in range(steps % period):
-        fn(i)
-    stop.record()
-    ms = start.elapsed_ms(stop)
-    ctx.sync()
-    start.destroy()
-    stop.destroy()
-    graph.destroy()
-    return ms
+        host_ms = (time.perf_counter() - t0) * 1e3
+        for _ in range(max(0, warmup // max(1, steps))):
+            graph.launch()
+        ctx.sync()
+        passes = 2 + int(1.5 * host_ms / self.evict_pass_ms)
+        samples = []
+        for _ in range(replays):
+            for _ in range(passes):
+                self.evict_pass()
+            if after_evict is not None:
+                after_evict()
+            self.start.record()
+            graph.launch()
+            self.stop.record()
+            samples.append(self.start.elapsed_ms(self.stop))
+        ctx.sync()
+        graph.destroy()
+        samples.sort()
+        return {"ms": samples[len(samples) // 2], "ms_min": samples[0], "ms_max": samples[-1],
+                "mode": "hipGraph replay" if branches == 1 else
+                        f"hipGraph replay, {branches} parallel branches",
+                "replays": replays, "timed_s": sum(samples) * 1e-3,
+                "evict_passes_between_replays": passes}
 
 
-def bench_gemv(ctx, ka, rng, steps: int, warmup: int, m: int, n: int, k: int, g: int,
-               copies: int):
-    """Returns (ms_total_rotating, ms_total_resident, algorithmic bytes per call)."""
+def bench_gemv(timer: Timer, rng, steps: int, warmup: int, m: int, n: int, k: int, g: int,
+               copies: int, *, extras: bool = False):
+    """Config-0 / config-3 GEMV over `copies` rotating weight buffers.  Returns the Timer result
+    of the serial rotating run plus, with `extras`, the cache-resident run, the run on four
+    parallel graph branches and the two floors (empty kernel, pure read) taken the same way."""
+    ctx, ka = timer.ctx, timer.ka
     row_bytes = k // 2
     weights, scales = [], []
     for _ in range(copies):
@@ -90,25 +158,44 @@ def bench_gemv(ctx, ka, rng, steps: int, warmup: int, m: int, n: int, k: int, g:
         weights.append(ctx.upload(packed))
         scales.append(ctx.upload(sc))
     x = ctx.upload(rng.normal(size=(m, k)).astype(np.float16))
-    out = ctx.alloc(m * n * 2)
+    outs = [ctx.alloc(m * n * 2) for _ in range(4)]
 
     def step(i: int) -> None:
         j = i % copies
-        ctx.linear_i4(x, weights[j], scales[j], None, out, m, n, k, g, ka.F16, ka.F16)
+        ctx.linear_i4(x, weights[j], scales[j], None, outs[0], m, n, k, g, ka.F16, ka.F16)
+
+    def step_branch(i: int) -> None:  # independent launches: own weights, own output per branch
+        j = i % copies
+        ctx.linear_i4(x, weights[j], scales[j], None, outs[i % 4], m, n, k, g, ka.F16, ka.F16)
 
     def step_resident(i: int) -> None:
-        ctx.linear_i4(x, weights[0], scales[0], None, out, m, n, k, g, ka.F16, ka.F16)
+        ctx.linear_i4(x, weights[0], scales[0], None, outs[0], m, n, k, g, ka.F16, ka.F16)
 
-    ms_rot = timed(ctx, step, steps, warmup, copies)
-    ms_res = timed(ctx, step_resident, steps, warmup, copies)
-    for b in weights + scales + [x, out]:
+    grid = (n + 3) // 4  # the GEMV's own grid: one wave a row, four waves a workgroup
+
+    def step_empty(i: int) -> None:
+        ctx.probe_launch(ka.PROBE_EMPTY, grid=grid, block=256)
+
+    def step_read(i: int) -> None:
+        ctx.probe_launch(ka.PROBE_READ, weights[i % copies], n * row_bytes, grid=grid, block=256)
+
+    res = {"rotating": timer.run(step, steps, warmup)}
+    if extras:
+        res["resident"] = timer.run(step_resident, steps, warmup,
+                                    after_evict=lambda: [step_resident(0) for _ in range(3)])
+        res["overlapped"] = timer.run(step_branch, steps, warmup, branches=4)
+        res["empty"] = timer.run(step_empty, steps, warmup)
+        res["read"] = timer.run(step_read, steps, warmup)
+    for b in weights + scales + [x] + outs:
         b.free()
-    algo = n * row_bytes + n * (k // g) * 2 + m * k * 2 + m * n * 2
-    return ms_rot, ms_res, algo
+    res["algo"] = n * row_bytes + n * (k // g) * 2 + m * k * 2 + m * n * 2
+    res["read_bytes"] = n * row_bytes
+    return res
 
 
-def bench_attention(ctx, ka, rng, steps: int, warmup: int, copies: int):
+def bench_attention(timer: Timer, rng, steps: int, warmup: int, copies: int):
     """benchmark config 2: B=1, H=32, Hkv=8, D=128, 4095 cached rows + this step's row, fp16."""
+    ctx, ka = timer.ctx, timer.ka
     heads, kv_heads, depth, past, cap = 32, 8, 128, 4095, 4096
     slots = []
     for _ in range(copies):
@@ -128,18 +215,83 @@ def bench_attention(ctx, ka, rng, steps: int, warmup: int, copies: int):
                             chunk_rows=1, depth=depth, capacity=cap, window=0, half_scale=half,
                             past=past, query=1, io_dtype=ka.F16, kv_dtype=ka.F16, workspace=ws)
 
-    ms = timed(ctx, step, steps, warmup, copies)
+    res = timer.run(step, steps, warmup)
     for pair in slots:
         pair[0].free()
         pair[1].free()
     for b in (q, ik, iv, out, ws):
         b.free()
     algo = 2 * kv_heads * (past + 1) * depth * 2 + 2 * heads * depth * 2
-    return ms, algo
+    return res["ms"] / steps, algo
 
 
-def bench_gemm(ctx, ka, rng, steps: int, warmup: int, m: int, n: int, k: int, g: int):
+def bench_ragged(timer: Timer, rng, steps: int, warmup: int):
+    """benchmark config 3's attention: 16 sequences with KV lengths ~ U{128..4096} (seeded),
+    packed along the slot's row axis, heads as config 2, fp16.  One varlen launch against the
+    same 16 sequences as 16 single-sequence launches; bytes = sum_i 2 * Hkv * L_i * D * 2."""
+    ctx, ka = timer.ctx, timer.ka
+    heads, kv_heads, depth, nseq = 32, 8, 128, 16
+    lengths = np.random.default_rng(3).integers(128, 4097, size=nseq)
+    cu = np.concatenate([[0], np.cumsum(lengths)]).astype(np.int32)
+    total = int(cu[-1])
+    copies = 6  # 6 x 2 x 8 x total x 128 x 2 B: well over the Infinity Cache
+    slots = [(ctx.upload(rng.normal(size=(kv_heads, total, depth)).astype(np.float16)),
+              ctx.upload(rng.normal(size=(kv_heads, total, depth)).astype(np.float16)))
+             for _ in range(copies)]
+    q = ctx.upload(rng.normal(size=(nseq, heads, depth)).astype(np.float16))
+    ik = ctx.upload(rng.normal(size=(nseq, kv_heads, depth)).astype(np.float16))
+    iv = ctx.upload(rng.normal(size=(nseq, kv_heads, depth)).astype(np.float16))
+    out = ctx.alloc(nseq * heads * depth * 2)
+    half = float(np.float32(np.sqrt(1.0 / np.sqrt(float(depth)))))
+    ws = ctx.alloc(ctx.attention_varlen_workspace(nseq, heads, kv_heads, depth, total))
+    cu_dev = ctx.upload(cu)
+    plan = ctx.alloc(ctx.attention_varlen_plan_bytes(nseq))
+    max_splits = ctx.attention_varlen_max_splits(nseq, depth, ka.F16, total)
+    ctx.attention_varlen_plan(cu_dev, plan, nseq=nseq, depth=depth, kv_dtype=ka.F16,
+                              total_rows=total, max_splits=max_splits)
+
+    def step(i: int) -> None:
+        sk, sv = slots[i % copies]
+        ctx.attention_varlen_planned(q, ik, iv, sk, sv, out, plan, nseq=nseq, heads=heads,
+                                     kv_heads=kv_heads, depth=depth, total_rows=total,
+                                     max_splits=max_splits, half_scale=half, io_dtype=ka.F16,
+                                     kv_dtype=ka.F16, workspace=ws)
+
+    one_ws = ctx.alloc(ctx.attention_state_workspace(1, heads, kv_heads, 1, depth, 0, 4096))
+    eb = 2
+
+    def step_singles(i: int) -> None:
+        # the same sequences one at a time: sequence s is the packed slot seen from its first
+        # row on, with capacity = total rows (the distance between the planes of the packed slot)
+        sk, sv = slots[i % copies]
+        for sidx in range(nseq):
+            base = int(cu[sidx]) * depth * eb
+            ctx.attention_state(q.offset(sidx * heads * depth * eb),
+                                ik.offset(sidx * kv_heads * depth * eb),
+                                iv.offset(sidx * kv_heads * depth * eb),
+                                sk.address + base, sv.address + base,
+                                out.offset(sidx * heads * depth * eb), batch=1, heads=heads,
+                                kv_heads=kv_heads, chunk_rows=1, depth=depth,
+                                capacity=total, window=0, half_scale=half,
+                                past=int(lengths[sidx]), query=1, io_dtype=ka.F16,
+                                kv_dtype=ka.F16, workspace=one_ws)
+
+    one = timer.run(step, steps, warmup)
+    singles = timer.run(step_singles, max(4, steps // 8), max(1, warmup // 8), replays=20)
+    for pair in slots:
+        pair[0].free()
+        pair[1].free()
+    for b in (q, ik, iv, out, ws, cu_dev, plan, one_ws):
+        b.free()
+    algo = int(sum(2 * kv_heads * int(L) * depth * 2 for L in lengths)) + 2 * nseq * heads * depth * 2
+    return one["ms"] / steps, singles["ms"] / max(4, steps // 8), algo, [int(L) for L in lengths]
+
+
+def bench_gemm(timer: Timer, rng, steps: int, warmup: int, m: int, n: int, k: int, g: int,
+               compute=None):
     """benchmark config 1: prefill GEMM on the matrix cores, fp16 activations and output."""
+    ctx, ka = timer.ctx, timer.ka
+    compute = ka.COMPUTE_F16 if compute is None else compute
     copies = 4
     weights, scales = [], []
     for _ in range(copies):
@@ -152,20 +304,20 @@ def bench_gemm(ctx, ka, rng, steps: int, warmup: int, m: int, n: int, k: int, g:
 
     def step(i: int) -> None:
         j = i % copies
-        ctx.linear_i4(x, weights[j], scales[j], None, out, m, n, k, g, ka.F16, ka.F16,
-                      ka.COMPUTE_F16)
+        ctx.linear_i4(x, weights[j], scales[j], None, out, m, n, k, g, ka.F16, ka.F16, compute)
 
-    ms = timed(ctx, step, steps, warmup, copies)
+    res = timer.run(step, steps, warmup, replays=20)
     for b in weights + scales + [x, out]:
         b.free()
-    return ms / steps, 2.0 * m * n * k
+    return res["ms"] / steps, 2.0 * m * n * k
 
 
-def bench_w4a8(ctx, ka, rng, steps: int, warmup: int, m: int, n: int, k: int, g: int,
+def bench_w4a8(timer: Timer, rng, steps: int, warmup: int, m: int, n: int, k: int, g: int,
                copies: int):
     """w4a8 `linear` (int8 activations x int4 weights, integer dot products): one step = the
     activation quantiser + the product, f32 x in, f32 out, fp16 group scales.
     Returns (ms per step, ms per step of the product alone)."""
+    ctx, ka = timer.ctx, timer.ka
     weights, scales = [], []
     for _ in range(copies):
         weights.append(ctx.upload(rng.integers(0, 256, size=n * k // 2, dtype=np.uint8)))
@@ -185,8 +337,9 @@ def bench_w4a8(ctx, ka, rng, steps: int, warmup: int, m: int, n: int, k: int, g:
         j = i % copies
         ctx.linear_w4a8(xq, xs, weights[j], scales[j], None, out, m, n, k, g, ka.F16)
 
-    ms = timed(ctx, step, steps, warmup, copies)
-    ms_product = timed(ctx, product, steps, warmup, copies)
+    reps = 20 if m > 16 else REPLAYS
+    ms = timer.run(step, steps, warmup, replays=reps)["ms"]
+    ms_product = timer.run(product, steps, warmup, replays=reps)["ms"]
     for b in weights + scales + [x, xq, xs, out]:
         b.free()
     return ms / steps, ms_product / steps
@@ -313,17 +466,21 @@ def cpu_decode_baseline(g: int, tokens: int = 3):
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=2000)
-    ap.add_argument("--warmup", type=int, default=200)
+    ap.add_argument("--steps", type=int, default=256)
+    ap.add_argument("--warmup", type=int, default=256)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-graph", action="store_true",
                     help="issue plain launches instead of replaying recorded graphs")
-    ap.add_argument("--only", default="", help="gemv | gemv16 | gemm | attention | w4a8 | model | traffic: run only that part besides the "
-                         "headline GEMV")
+    ap.add_argument("--only", default="",
+                    help="gemv | gemv16 | gemm | attention | ragged | w4a8 | model | traffic: run "
+                         "only that part besides the headline GEMV")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build measures one GPU only (--gpus 1); no multi-GPU figure is "
               "produced in this run", file=sys.stderr)
+        return 2
+    if args.steps < 1 or args.warmup < 0:
+        print("bench.py: --steps must be >= 1 and --warmup >= 0", file=sys.stderr)
         return 2
 
     import karume_amd as ka
@@ -331,37 +488,61 @@ def main() -> int:
     global USE_GRAPHS
     USE_GRAPHS = not args.no_graph
     ctx = ka.acquire_gpu(int(os.environ.get("LOCAL_RANK", "0")))
+    timer = Timer(ctx, ka)
     rng = np.random.default_rng(20261125)
     m, n, k, g = 1, 4096, 4096, 128
     copies = 64  # 64 x (8 MiB + 256 KiB) = 528 MiB of weights in rotation
-    log(f"[bench] GEMV M={m} K={k} N={n} g={g}, {copies} weight copies")
-    ms_rot, ms_res, algo = bench_gemv(ctx, ka, rng, args.steps, args.warmup, m, n, k, g, copies)
-    per_call_us = ms_rot * 1e3 / args.steps
+    steps, warmup = args.steps, args.warmup
+    log(f"[bench] GEMV M={m} K={k} N={n} g={g}, {copies} weight copies, {steps} steps per replay")
+    gv = bench_gemv(timer, rng, steps, warmup, m, n, k, g, copies, extras=USE_GRAPHS)
+    algo = gv["algo"]
+    rot = gv["rotating"]
+    per_call_us = rot["ms"] * 1e3 / steps
     gbs = algo / (per_call_us * 1e-6) / 1e9
-    gbs_res = algo / (ms_res * 1e3 / args.steps * 1e-6) / 1e9
     result = {
         "metric": "q-GEMV HBM GB/s (int4 g128, M=1, K=N=4096)",
         "value": round(gbs, 1),
         "unit": "GB/s",
         "n_gpus": 1,
-        "steps": args.steps,
-        "warmup": args.warmup,
-        "ms_per_step": ms_rot / args.steps,
+        "steps": steps,
+        "warmup": warmup,
+        "ms_per_step": rot["ms"] / steps,
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
         "dtype": "f32",
         "data": "synthetic",
-        "launch_mode": "hipGraph replay" if USE_GRAPHS else "plain launches",
+        "launch_mode": rot["mode"],
+        "replays": rot["replays"],
+        "timing": "median over the replays of one recorded graph of `steps` launches; HIP events "
+                  "on the launch stream around each replay; 512 MiB streamed (untimed) before "
+                  "each replay",
+        "timed_region_s": round(rot["timed_s"], 6),
         "config": {"workload": "config 0: int4 g128 GEMV M=1 K=4096 N=4096, fp16 x/scales/out, "
                                "f32 accumulate, 64 rotating weight buffers (528 MiB)"},
         "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS,
-                     "unit": "GB/s", "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": GEMV_PMC_TRAFFIC_BYTES,
+                     "unit": "GB/s", "frac": round(gbs / HBM_PEAK_GBS, 4),
+                     "traffic": pmc_traffic_bytes("gemv_i4_config0_pmc_traffic.txt"),
                      "kernel": "gemv_i4_kernel", "algorithmic_bytes_per_launch": algo,
-                     "us_per_launch": round(per_call_us, 3)},
+                     "us_per_launch": round(per_call_us, 3),
+                     "us_per_launch_min": round(rot["ms_min"] * 1e3 / steps, 3),
+                     "us_per_launch_max": round(rot["ms_max"] * 1e3 / steps, 3)},
         "pct_of_hbm_peak": round(100 * gbs / HBM_PEAK_GBS, 2),
-        "gemv_cache_resident_gbs": round(gbs_res, 1),
     }
+    if USE_GRAPHS:
+        us = lambda key: gv[key]["ms"] * 1e3 / steps  # noqa: E731
+        result["gemv_cache_resident_gbs"] = round(algo / us("resident") / 1e3, 1)
+        result["gemv_overlapped_gbs"] = round(algo / us("overlapped") / 1e3, 1)
+        result["gemv_overlapped_us"] = round(us("overlapped"), 3)
+        result["gemv_overlapped_mode"] = gv["overlapped"]["mode"]
+        result["floor"] = {
+            "empty_kernel_us": round(us("empty"), 3),
+            "pure_read_us": round(us("read"), 3),
+            "pure_read_bytes": gv["read_bytes"],
+            "pure_read_gbs": round(gv["read_bytes"] / us("read") / 1e3, 1),
+            "grid": f"{(n + 3) // 4} x 256 threads (the GEMV's own)",
+            "achieved_over_pure_read": round(us("read") / per_call_us, 3),
+        }
     if args.only == "traffic":
         # For `rocprofv3 --pmc FETCH_SIZE` / `--pmc WRITE_SIZE`: a plain 8 MiB copy (known
         # traffic: 8 MiB read + 8 MiB written) beside the GEMV, a few launches of each.
@@ -370,48 +551,65 @@ def main() -> int:
             ctx.copy(dst, src, 8 << 20)
         ctx.sync()
         # a few launches of the other hot kernels, for the same counters
-        bench_attention(ctx, ka, rng, 8, 2, 4)
-        bench_gemm(ctx, ka, rng, 4, 2, 512, 11008, 4096, g)
-        bench_gemm(ctx, ka, rng, 4, 2, 512, 4096, 11008, g)
-    steps2 = max(50, args.steps // 4)
+        bench_attention(timer, rng, 8, 2, 4)
+        bench_ragged(timer, rng, 8, 2)
+        bench_gemm(timer, rng, 4, 2, 512, 11008, 4096, g)
+        bench_gemm(timer, rng, 4, 2, 512, 4096, 11008, g)
+    steps2 = max(16, steps // 4)
+    warm2 = max(16, warmup // 4)
     if args.only in ("", "gemv16"):
         log("[bench] GEMV M=16 (config 3)")
-        ms16, _res16, algo16 = bench_gemv(ctx, ka, rng, steps2, max(10, args.warmup // 4), 16, n,
-                                          k, g, copies)
-        result["gemv_m16_gbs"] = round(algo16 / (ms16 / steps2 * 1e-3) / 1e9, 1)
-        result["gemv_m16_us"] = round(ms16 / steps2 * 1e3, 3)
+        g16 = bench_gemv(timer, rng, steps2, warm2, 16, n, k, g, copies)
+        us16 = g16["rotating"]["ms"] * 1e3 / steps2
+        result["gemv_m16_gbs"] = round(g16["algo"] / us16 / 1e3, 1)
+        result["gemv_m16_us"] = round(us16, 3)
     if args.only in ("", "attention"):
         log("[bench] decode attention (config 2)")
-        ms_att, algo_att = bench_attention(ctx, ka, rng, steps2, max(10, args.warmup // 4), 20)
-        att_gbs = algo_att / (ms_att / steps2 * 1e-3) / 1e9
+        ms_att, algo_att = bench_attention(timer, rng, steps2, warm2, 20)
+        att_gbs = algo_att / (ms_att * 1e-3) / 1e9
         result["attention_decode_gbs"] = round(att_gbs, 1)
-        result["attention_decode_us"] = round(ms_att / steps2 * 1e3, 3)
+        result["attention_decode_us"] = round(ms_att * 1e3, 3)
         result["attention_decode_pct_of_hbm_peak"] = round(100 * att_gbs / HBM_PEAK_GBS, 2)
+    if args.only in ("", "ragged"):
+        log("[bench] ragged decode attention, 16 sequences (config 3)")
+        ms_one, ms_16, algo_r, lens = bench_ragged(timer, rng, steps2, warm2)
+        result["attention_ragged"] = {
+            "kv_lengths": lens, "algorithmic_bytes": algo_r,
+            "one_launch_us": round(ms_one * 1e3, 3),
+            "one_launch_gbs": round(algo_r / (ms_one * 1e-3) / 1e9, 1),
+            "one_launch_pct_of_hbm_peak": round(100 * algo_r / (ms_one * 1e-3) / 8e12, 2),
+            "sixteen_launches_us": round(ms_16 * 1e3, 3),
+            "sixteen_launches_gbs": round(algo_r / (ms_16 * 1e-3) / 1e9, 1),
+        }
     if args.only in ("", "gemm"):
         for name, (gn, gk) in {"up": (11008, 4096), "down": (4096, 11008)}.items():
             log(f"[bench] prefill GEMM M=512 K={gk} N={gn} (config 1, {name}-projection)")
-            # 400 warm-up launches (30 ms): a shorter run still sees the clocks ramping up from
-            # idle (100 launches from idle measure 81 us each, 2000 measure 68 us)
-            ms_g, flops = bench_gemm(ctx, ka, rng, 400, 400, 512, gn, gk, g)
+            # graphs of 100 launches (7 ms each), 20 replays behind 100 warm-up launches: the
+            # clocks come up from idle over tens of milliseconds
+            ms_g, flops = bench_gemm(timer, rng, 100, 200, 512, gn, gk, g)
             result[f"gemm_{name}_tflops"] = round(flops / (ms_g * 1e-3) / 1e12, 1)
             result[f"gemm_{name}_us"] = round(ms_g * 1e3, 2)
             result[f"gemm_{name}_pct_of_f16_mfma_peak"] = round(
                 100 * flops / (ms_g * 1e-3) / 2.5e15, 2)
+            ms_g, flops = bench_gemm(timer, rng, 20, 40, 512, gn, gk, g, compute=ka.COMPUTE_F32)
+            result[f"gemm_{name}_f32class_us"] = round(ms_g * 1e3, 2)
+            result[f"gemm_{name}_f32class_tflops"] = round(flops / (ms_g * 1e-3) / 1e12, 1)
     if args.only in ("", "w4a8"):
         log("[bench] w4a8 linear: M=1 GEMV and M=512 up/down-projections")
-        ms_q, ms_p = bench_w4a8(ctx, ka, rng, steps2, max(10, args.warmup // 4), 1, n, k, g, copies)
+        ms_q, ms_p = bench_w4a8(timer, rng, steps2, warm2, 1, n, k, g, copies)
         w4_bytes = n * k // 2 + n * (k // g) * 2 + k + 4 + n * 4
         result["w4a8_gemv_us"] = round(ms_q * 1e3, 3)
         result["w4a8_gemv_product_us"] = round(ms_p * 1e3, 3)
         result["w4a8_gemv_product_gbs"] = round(w4_bytes / (ms_p * 1e-3) / 1e9, 1)
         for name, (gn, gk) in {"up": (11008, 4096), "down": (4096, 11008)}.items():
-            ms_q, ms_p = bench_w4a8(ctx, ka, rng, 400, 400, 512, gn, gk, g, 4)
+            ms_q, ms_p = bench_w4a8(timer, rng, 100, 200, 512, gn, gk, g, 4)
             ops = 2.0 * 512 * gn * gk
             result[f"w4a8_gemm_{name}_us"] = round(ms_q * 1e3, 2)
             result[f"w4a8_gemm_{name}_product_us"] = round(ms_p * 1e3, 2)
             result[f"w4a8_gemm_{name}_product_tops"] = round(ops / (ms_p * 1e-3) / 1e12, 1)
             result[f"w4a8_gemm_{name}_pct_of_i8_mfma_peak"] = round(
                 100 * ops / (ms_p * 1e-3) / 5.0e15, 2)
+    timer.close()
     if args.only in ("", "model"):
         # f32 activations: with this random init (|N(0,0.02)| scales on uniform codes) the
         # residual stream passes 65504 after a few layers, so fp16 activations are not usable

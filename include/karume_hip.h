@@ -51,8 +51,12 @@ typedef struct krm_event krm_event;
 /* `linear` arithmetic, the reference's SessionOptions.linearCompute
  * (packages/runtime/src/runtime/session-types.ts:127-195):
  *   KRM_COMPUTE_F32  — f32 products and f32 accumulation for every M (the reference default);
- *   KRM_COMPUTE_F16  — rows M > 16 go to the fp16 MFMA GEMM (x rounded to fp16, integer
- *                      weight codes exact in fp16, group scale applied to f32 partial sums).
+ *   KRM_COMPUTE_F16  — rows M > 16 go to the fp16 MFMA GEMM: x rounded to fp16, every weight
+ *                      rounded once to fp16((u - 8) * scale), fp16 x fp16 products accumulated
+ *                      in f32.  The per-weight rounding bounds the error of an output by about
+ *                      2^-11 * sqrt(k) * rms(x * w) (the reference rejects f16 compute with i4
+ *                      weights, packages/runtime/src/kernels/gemm.ts:1204-1209, so this form
+ *                      has no same-numerics counterpart there).
  * M <= 16 always runs the bandwidth-bound GEMV with f32 accumulation. */
 #define KRM_COMPUTE_F32 0
 #define KRM_COMPUTE_F16 1
@@ -95,6 +99,15 @@ int32_t krm_event_record(krm_ctx* ctx, krm_event* ev);
 /* Waits for `stop`, then writes the milliseconds between the two recorded events. */
 int32_t krm_event_elapsed_ms(krm_ctx* ctx, krm_event* start, krm_event* stop, float* ms);
 int32_t krm_event_destroy(krm_ctx* ctx, krm_event* ev);
+/* Measurement floors for a launch of `grid` workgroups of `block` threads on the context's
+ * stream (diagnostics like the timestamp queries above; no op of the reference):
+ *   KRM_PROBE_EMPTY — a kernel that does nothing (what a launch of that grid costs);
+ *   KRM_PROBE_READ  — every thread streams its share of `bytes` at `src` with 16-byte loads
+ *                     and stores nothing (what reading that much costs). */
+#define KRM_PROBE_EMPTY 0
+#define KRM_PROBE_READ 1
+int32_t krm_probe_launch(krm_ctx* ctx, int32_t kind, krm_buf src, size_t bytes, uint32_t grid,
+                         uint32_t block);
 
 /* ---- recorded launch sequences (the reference bakes a step's dispatch recipes once and
  *      replays them: executeBakedPlan, packages/runtime/src/runtime/recipe.ts:357-394) ------
@@ -104,6 +117,14 @@ int32_t krm_event_destroy(krm_ctx* ctx, krm_event* ev);
  * device (upload, download, free, sync, krm_attention_varlen) are rejected while recording. */
 typedef struct krm_graph krm_graph;
 int32_t krm_graph_begin(krm_ctx* ctx);
+/* While recording: the ops that follow go to parallel branch `branch` (0 = the main branch,
+ * 1..3 = side branches).  A side branch forks from the main branch at its first selection
+ * (it depends on what the main branch held at that moment) and every side branch joins the
+ * main branch in krm_graph_end.  Ops on different branches must not depend on one another;
+ * the device may run them at the same time (the recipes of one step that the reference
+ * submits in one command buffer without barriers between independent dispatches,
+ * packages/runtime/src/runtime/recipe.ts:385-394). */
+int32_t krm_graph_branch(krm_ctx* ctx, uint32_t branch);
 int32_t krm_graph_end(krm_ctx* ctx, krm_graph** out);
 int32_t krm_graph_launch(krm_ctx* ctx, krm_graph* graph);
 int32_t krm_graph_destroy(krm_ctx* ctx, krm_graph* graph);
@@ -214,7 +235,9 @@ int32_t krm_lengths_log_token(krm_ctx* ctx, krm_buf lengths, krm_buf token_i32,
  * the end of a recorded one-row decode step, which leaves the next step's position behind. */
 int32_t krm_lengths_step_end(krm_ctx* ctx, krm_buf lengths, krm_buf token_i32,
                              krm_buf history_i32, uint32_t history_len, krm_buf positions_i32);
-/* krm_attention_state with device lengths; `max_past` sizes the launch and the workspace. */
+/* krm_attention_state with device lengths; `max_past` sizes the launch and the workspace.  A
+ * replay whose device-side pastLength needs more column splits than `max_past` did raises the
+ * fault word and writes nothing (neither `out` nor the workspace nor the arrival counters). */
 int32_t krm_attention_state_lengths(krm_ctx* ctx, krm_buf q, krm_buf ins_k, krm_buf ins_v,
                                     krm_buf slot_k, krm_buf slot_v, krm_buf out, uint32_t batch,
                                     uint32_t heads, uint32_t kv_heads, uint32_t chunk_rows,
@@ -249,6 +272,31 @@ int32_t krm_attention_varlen(krm_ctx* ctx, krm_buf q, krm_buf ins_k, krm_buf ins
                              uint32_t kv_heads, uint32_t depth, uint64_t total_rows,
                              float half_scale, int32_t io_dtype, int32_t kv_dtype,
                              krm_buf workspace, size_t workspace_bytes);
+
+/* The same ragged step with its tables built on the device, so that the whole step can be
+ * recorded (krm_graph_*) and replayed while the sequences grow (no counterpart in the
+ * reference, as above).  `cu_seqlens_i32` is a DEVICE array of nseq+1 row offsets.
+ * krm_attention_varlen_plan turns it into the launch tables in `plan`
+ * (krm_attention_varlen_plan_bytes bytes: cu_rows[nseq+1], split_prefix[nseq+1], fault); one
+ * plan serves every layer of a step.  Offsets that are negative, not ascending, beyond
+ * total_rows, or that need more than `max_splits` column splits set plan's fault word (the
+ * last int32 of the tables, index 2*(nseq+1)) to 1 and make the attention launch a no-op.
+ * krm_attention_varlen_planned launches `max_splits` column splits (the bound
+ * krm_attention_varlen_max_splits returns: total_rows / split columns + nseq) and reads the
+ * tables on the device; results are bit-identical to krm_attention_varlen and to
+ * krm_attention_state on each sequence alone.  `workspace` as for krm_attention_varlen. */
+int32_t krm_attention_varlen_plan_bytes(uint32_t nseq, size_t* bytes);
+int32_t krm_attention_varlen_max_splits(uint32_t nseq, uint32_t depth, int32_t kv_dtype,
+                                        uint64_t total_rows, uint32_t* max_splits);
+int32_t krm_attention_varlen_plan(krm_ctx* ctx, krm_buf cu_seqlens_i32, krm_buf plan,
+                                  uint32_t nseq, uint32_t depth, int32_t kv_dtype,
+                                  uint64_t total_rows, uint32_t max_splits);
+int32_t krm_attention_varlen_planned(krm_ctx* ctx, krm_buf q, krm_buf ins_k, krm_buf ins_v,
+                                     krm_buf slot_k, krm_buf slot_v, krm_buf out, krm_buf plan,
+                                     uint32_t nseq, uint32_t heads, uint32_t kv_heads,
+                                     uint32_t depth, uint64_t total_rows, uint32_t max_splits,
+                                     float half_scale, int32_t io_dtype, int32_t kv_dtype,
+                                     krm_buf workspace, size_t workspace_bytes);
 
 /* ---- decoder-layer glue ops (f32 arithmetic; activations f32 or fp16) ------------------------
  * The ops a Llama-style layer runs around the linears and the attention in the decode graph

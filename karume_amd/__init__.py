@@ -9,7 +9,8 @@ from .format_i4 import I4Error, check_int4, group_scale_shape, pack_int4
 from .format_model import (ContainerError, IrError, KarumeModel, PackedInt4, SafetensorsError,
                            i4_resident_initializers, open_model, packed_int4,
                            parse_safetensors, tensor_bytes)
-from .runtime import (COMPUTE_F16, COMPUTE_F32, EPILOGUE_NONE, EPILOGUE_SILU_PAIRS, F16, F32, DeviceBuffer, ExecutionError,
+from .runtime import (COMPUTE_F16, COMPUTE_F32, EPILOGUE_NONE, EPILOGUE_SILU_PAIRS, F16, F32,
+                      PROBE_EMPTY, PROBE_READ, DeviceBuffer, ExecutionError,
                       GpuContext, GpuDeviceLostError, GpuEvent, GpuGraph, GpuOutOfMemoryError,
                       GpuValidationError, KarumeError, acquire_gpu, dtype_code, version)
 
@@ -22,7 +23,8 @@ __all__ = [
     "I4Error", "check_int4", "group_scale_shape", "pack_int4",
     "ContainerError", "IrError", "KarumeModel", "PackedInt4", "SafetensorsError",
     "i4_resident_initializers", "open_model", "packed_int4", "parse_safetensors", "tensor_bytes",
-    "COMPUTE_F16", "COMPUTE_F32", "EPILOGUE_NONE", "EPILOGUE_SILU_PAIRS", "F16", "F32", "DeviceBuffer", "ExecutionError", "GpuContext",
+    "COMPUTE_F16", "COMPUTE_F32", "EPILOGUE_NONE", "EPILOGUE_SILU_PAIRS", "F16", "F32",
+    "PROBE_EMPTY", "PROBE_READ", "DeviceBuffer", "ExecutionError", "GpuContext",
     "GpuDeviceLostError", "GpuEvent", "GpuGraph", "GpuOutOfMemoryError", "GpuValidationError", "KarumeError",
     "acquire_gpu", "dtype_code", "version",
 ]

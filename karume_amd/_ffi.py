@@ -36,7 +36,9 @@ PROTOTYPES = {
     "krm_event_record": (i32, [c_ctx, c_evt]),
     "krm_event_elapsed_ms": (i32, [c_ctx, c_evt, c_evt, C.POINTER(C.c_float)]),
     "krm_event_destroy": (i32, [c_ctx, c_evt]),
+    "krm_probe_launch": (i32, [c_ctx, i32, c_buf, size_t, u32, u32]),
     "krm_graph_begin": (i32, [c_ctx]),
+    "krm_graph_branch": (i32, [c_ctx, u32]),
     "krm_graph_end": (i32, [c_ctx, C.POINTER(C.c_void_p)]),
     "krm_graph_launch": (i32, [c_ctx, C.c_void_p]),
     "krm_graph_destroy": (i32, [c_ctx, C.c_void_p]),
@@ -58,6 +60,12 @@ PROTOTYPES = {
     "krm_attention_varlen": (i32, [c_ctx, c_buf, c_buf, c_buf, c_buf, c_buf, c_buf,
                                    C.POINTER(i32), u32, u32, u32, u32, u64, C.c_float, i32, i32,
                                    c_buf, size_t]),
+    "krm_attention_varlen_plan_bytes": (i32, [u32, C.POINTER(size_t)]),
+    "krm_attention_varlen_max_splits": (i32, [u32, u32, i32, u64, C.POINTER(u32)]),
+    "krm_attention_varlen_plan": (i32, [c_ctx, c_buf, c_buf, u32, u32, i32, u64, u32]),
+    "krm_attention_varlen_planned": (i32, [c_ctx, c_buf, c_buf, c_buf, c_buf, c_buf, c_buf, c_buf,
+                                           u32, u32, u32, u32, u64, u32, C.c_float, i32, i32,
+                                           c_buf, size_t]),
     "krm_lengths_set": (i32, [c_ctx, c_buf, u32, u32]),
     "krm_lengths_advance": (i32, [c_ctx, c_buf]),
     "krm_lengths_positions": (i32, [c_ctx, c_buf, c_buf, u32]),

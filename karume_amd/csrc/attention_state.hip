@@ -407,6 +407,7 @@ void attention_decode_kernel(
     first_split = (uint32_t)a.split_prefix[seq];
     nsplit = (uint32_t)a.split_prefix[seq + 1] - first_split;
     split = blockIdx.x - first_split;
+    if (split >= nsplit) return;  // a grid sized for the most splits the batch may need
     row_base = (uint32_t)a.cu_rows[seq];
     past = (uint32_t)a.cu_rows[seq + 1] - row_base;
   } else {
@@ -417,6 +418,14 @@ void attention_decode_kernel(
     row_base = 0;
     nsplit = decode_splits(past - window_low(a.window, past), kChunkCols);
     split = blockIdx.x;
+    // The grid and the workspace were sized on the host for the longest past the launch may
+    // see.  A replay whose device-side past needs more splits than that would never complete a
+    // ticket round and would index partials beyond the workspace: raise the fault word and
+    // leave everything untouched instead.
+    if (nsplit > gridDim.x) {
+      if (a.lengths && blockIdx.x == 0 && blockIdx.y == 0 && tid == 0) a.lengths[2] = 1u;
+      return;
+    }
     if (split >= nsplit) return;  // the grid is sized for the longest past it may see
     first_split = seq * nsplit;
   }
@@ -753,7 +762,15 @@ struct DecodeLaunch {
   float* ws_acc;
   DecodeArgs args;
   uint32_t grid_x, grid_z;     // splits (or total splits), batch
+  uint32_t ticket_slots = kTicketSlots;  // counters behind args.tickets
+  bool clear_tickets = false;  // zero the counters this launch uses before it runs
 };
+
+// Fill kernel for arrival counters (a kernel, not a memset, so that a caller may record it).
+__global__ void clear_tickets_kernel(uint32_t* tickets, uint32_t count) {
+  const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < count) tickets[(size_t)i * kTicketStride] = 0u;
+}
 
 template <typename XT, typename ST, int R, int LPR, bool RAGGED>
 int32_t launch_decode(krm_ctx* ctx, const DecodeLaunch& L) {
@@ -805,11 +822,15 @@ int32_t decode_dispatch(krm_ctx* ctx, DecodeLaunch& L, uint32_t repeat, uint32_t
 
   L.args.repeat = repeat;
   L.args.head_groups = repeat / per_block;
-  if ((uint64_t)L.args.kv_heads * L.args.head_groups > 65535 ||
-      (uint64_t)L.args.nseq * L.args.kv_heads * L.args.head_groups > kTicketSlots)
+  const uint64_t counters = (uint64_t)L.args.nseq * L.args.kv_heads * L.args.head_groups;
+  if ((uint64_t)L.args.kv_heads * L.args.head_groups > 65535 || counters > L.ticket_slots)
     return fail(ctx, KRM_ERR_VALIDATION, "decode attention: B * H = %llu exceeds %u",
-                (unsigned long long)L.args.nseq * L.args.kv_heads * L.args.head_groups,
-                kTicketSlots);
+                (unsigned long long)counters, L.ticket_slots);
+  if (L.clear_tickets) {
+    clear_tickets_kernel<<<dim3(((uint32_t)counters + 255) / 256), dim3(256), 0, ctx->stream>>>(
+        L.args.tickets, (uint32_t)counters);
+    KRM_TRY(launched(ctx, "clear_tickets_kernel"));
+  }
   if (io_dtype == KRM_F16 && kv_dtype == KRM_F16)
     return decode_by_depth<__half, __half, RAGGED>(ctx, L, per_block, lpr);
   if (io_dtype == KRM_F32 && kv_dtype == KRM_F32)
@@ -869,13 +890,16 @@ int32_t krm_attention_state_workspace(uint32_t batch, uint32_t heads, uint32_t k
 
 // `lengths` == 0: past / query are this run's values.  Otherwise they are read on the device
 // and `past` is the largest pastLength the launch has to be sized for.
+// `tickets` == nullptr: the context's arrival counters.  Otherwise counters supplied by the
+// caller (`ticket_slots` of them, kTicketStride words apart), which this call clears first.
 static int32_t attention_state_impl(krm_ctx* ctx, krm_buf q, krm_buf ins_k, krm_buf ins_v,
                                     krm_buf slot_k, krm_buf slot_v, krm_buf out, uint32_t batch,
                                     uint32_t heads, uint32_t kv_heads, uint32_t chunk_rows,
                                     uint32_t depth, uint32_t capacity, uint32_t window,
                                     float half_scale, uint32_t past, uint32_t query,
                                     krm_buf lengths, int32_t io_dtype, int32_t kv_dtype,
-                                    krm_buf workspace, size_t workspace_bytes) {
+                                    krm_buf workspace, size_t workspace_bytes,
+                                    uint32_t* tickets = nullptr, uint32_t ticket_slots = 0) {
   KRM_TRY(enter(ctx));
   const bool dyn = lengths != 0;
   KRM_REQUIRE(ctx, aligned(lengths, 4), "krm_attention_state: misaligned lengths buffer");
@@ -935,7 +959,9 @@ static int32_t attention_state_impl(krm_ctx* ctx, krm_buf q, krm_buf ins_k, krm_
     L.args.nseq = batch;
     L.grid_x = nsplit;
     L.grid_z = batch;
-    L.args.tickets = ctx->tickets;
+    L.args.tickets = tickets ? tickets : ctx->tickets;
+    L.ticket_slots = tickets ? ticket_slots : kTicketSlots;
+    L.clear_tickets = tickets != nullptr;
     L.args.lengths = ptr<uint32_t>(lengths);
     L.args.capacity = capacity;
     if (nsplit > 1) {
@@ -1085,6 +1111,132 @@ int32_t krm_attention_varlen(krm_ctx* ctx, krm_buf q, krm_buf ins_k, krm_buf ins
   L.ws_ml = ptr<float>(workspace + table_bytes);
   L.ws_acc = L.ws_ml + ml_floats;
   L.grid_x = (uint32_t)splits;
+  L.grid_z = 1;
+  L.args.tickets = ctx->tickets;
+  return decode_dispatch<true>(ctx, L, repeat, lpr, io_dtype, kv_dtype);
+}
+
+}  // extern "C"
+
+// ---- ragged batch whose tables are built on the device -------------------------------------
+
+// plan layout (int32): cu_rows[nseq + 1], split_prefix[nseq + 1], fault
+__global__ void varlen_plan_kernel(const int32_t* __restrict__ cu_seqlens, int32_t* __restrict__ plan,
+                                   uint32_t nseq, uint32_t chunk_columns, uint64_t total_rows,
+                                   uint32_t max_splits) {
+  if (blockIdx.x != 0 || threadIdx.x != 0) return;
+  int32_t* cu = plan;
+  int32_t* prefix = plan + nseq + 1;
+  int32_t* fault = plan + 2 * (nseq + 1);
+  bool ok = cu_seqlens[0] >= 0;
+  uint64_t splits = 0;
+  cu[0] = cu_seqlens[0];
+  for (uint32_t i = 1; i <= nseq; ++i) {
+    const int32_t lo = cu_seqlens[i - 1], hi = cu_seqlens[i];
+    cu[i] = hi;
+    ok = ok && hi >= lo;
+    prefix[i - 1] = (int32_t)splits;
+    splits += ok ? decode_splits((uint64_t)(hi - lo), chunk_columns) : 0u;
+  }
+  ok = ok && (uint64_t)cu_seqlens[nseq] <= total_rows && splits <= max_splits;
+  prefix[nseq] = (int32_t)splits;
+  if (!ok)  // no workgroup of the attention launch finds a split: nothing is read or written
+    for (uint32_t i = 0; i <= nseq; ++i) prefix[i] = 0;
+  *fault = ok ? 0 : 1;
+}
+
+extern "C" {
+
+int32_t krm_attention_varlen_plan_bytes(uint32_t nseq, size_t* bytes) {
+  if (!bytes) return fail(nullptr, KRM_ERR_VALIDATION, "krm_attention_varlen_plan_bytes: NULL");
+  *bytes = ((2 * ((size_t)nseq + 1) + 1) * sizeof(int32_t) + 63) & ~(size_t)63;
+  return KRM_OK;
+}
+
+int32_t krm_attention_varlen_max_splits(uint32_t nseq, uint32_t depth, int32_t kv_dtype,
+                                        uint64_t total_rows, uint32_t* max_splits) {
+  if (!max_splits) return fail(nullptr, KRM_ERR_VALIDATION, "krm_attention_varlen_max_splits: NULL");
+  if (!valid_dtype(kv_dtype))
+    return fail(nullptr, KRM_ERR_VALIDATION, "krm_attention_varlen_max_splits: kv_dtype %d", kv_dtype);
+  const uint32_t lpr = decode_lanes_per_row(depth, kv_dtype);
+  if (!lpr)
+    return fail(nullptr, KRM_ERR_VALIDATION,
+                "krm_attention_varlen_max_splits: D = %u is not covered by the decode kernel", depth);
+  // every sequence rounds its split count up
+  const uint64_t splits = total_rows / decode_split_columns(lpr) + nseq;
+  if (splits > 0x7fffffffull)
+    return fail(nullptr, KRM_ERR_VALIDATION, "krm_attention_varlen_max_splits: too many splits");
+  *max_splits = (uint32_t)splits;
+  return KRM_OK;
+}
+
+int32_t krm_attention_varlen_plan(krm_ctx* ctx, krm_buf cu_seqlens_i32, krm_buf plan,
+                                  uint32_t nseq, uint32_t depth, int32_t kv_dtype,
+                                  uint64_t total_rows, uint32_t max_splits) {
+  KRM_TRY(enter(ctx));
+  KRM_REQUIRE(ctx, valid_dtype(kv_dtype), "krm_attention_varlen_plan: kv_dtype %d", kv_dtype);
+  KRM_REQUIRE(ctx, nseq >= 1 && total_rows <= 0x7fffffffull,
+              "krm_attention_varlen_plan: nseq must be positive and total_rows < 2^31");
+  const uint32_t lpr = decode_lanes_per_row(depth, kv_dtype);
+  KRM_REQUIRE(ctx, lpr, "krm_attention_varlen_plan: D = %u with this slot dtype is not covered",
+              depth);
+  KRM_REQUIRE(ctx, cu_seqlens_i32 && plan && aligned(cu_seqlens_i32, 4) && aligned(plan, 4),
+              "krm_attention_varlen_plan: NULL or misaligned buffer");
+  varlen_plan_kernel<<<dim3(1), dim3(64), 0, ctx->stream>>>(
+      ptr<const int32_t>(cu_seqlens_i32), ptr<int32_t>(plan), nseq, decode_split_columns(lpr),
+      total_rows, max_splits);
+  return launched(ctx, "varlen_plan_kernel");
+}
+
+int32_t krm_attention_varlen_planned(krm_ctx* ctx, krm_buf q, krm_buf ins_k, krm_buf ins_v,
+                                     krm_buf slot_k, krm_buf slot_v, krm_buf out, krm_buf plan,
+                                     uint32_t nseq, uint32_t heads, uint32_t kv_heads,
+                                     uint32_t depth, uint64_t total_rows, uint32_t max_splits,
+                                     float half_scale, int32_t io_dtype, int32_t kv_dtype,
+                                     krm_buf workspace, size_t workspace_bytes) {
+  KRM_TRY(enter(ctx));
+  KRM_REQUIRE(ctx, valid_dtype(io_dtype) && valid_dtype(kv_dtype),
+              "krm_attention_varlen_planned: io_dtype %d / kv_dtype %d", io_dtype, kv_dtype);
+  KRM_REQUIRE(ctx, nseq >= 1 && heads >= 1 && kv_heads >= 1 && depth >= 1 && max_splits >= 1,
+              "krm_attention_varlen_planned: nseq / H / Hkv / D / max_splits must be positive");
+  KRM_REQUIRE(ctx, heads % kv_heads == 0,
+              "krm_attention_varlen_planned: H = %u is not a multiple of Hkv = %u", heads, kv_heads);
+  KRM_REQUIRE(ctx, std::isfinite(half_scale), "krm_attention_varlen_planned: scale is not finite");
+  KRM_REQUIRE(ctx, total_rows <= 0x7fffffffull && max_splits <= 0x7fffffffu,
+              "krm_attention_varlen_planned: total_rows or max_splits too large");
+  KRM_REQUIRE(ctx, heads <= 65535 && (uint64_t)nseq * heads <= kTicketSlots,
+              "krm_attention_varlen_planned: nseq * H = %llu exceeds %u",
+              (unsigned long long)nseq * heads, kTicketSlots);
+  const uint32_t repeat = heads / kv_heads;
+  const uint32_t lpr = decode_lanes_per_row(depth, kv_dtype);
+  KRM_REQUIRE(ctx, lpr && decode_repeat_ok(repeat),
+              "krm_attention_varlen_planned: D = %u with this slot dtype or H/Hkv = %u is not "
+              "covered by the split-K decode kernel", depth, repeat);
+  KRM_REQUIRE(ctx, q && ins_k && ins_v && slot_k && slot_v && out && workspace && plan,
+              "krm_attention_varlen_planned: NULL buffer");
+  KRM_REQUIRE(ctx, aligned(slot_k, 16) && aligned(slot_v, 16) && aligned(workspace, 16) &&
+                       aligned(q, 16) && aligned(plan, 4),
+              "krm_attention_varlen_planned: q, slots and workspace must be 16-byte aligned");
+  const size_t ml_floats = ((size_t)max_splits * heads * 2 + 3) & ~(size_t)3;
+  const size_t need = (ml_floats + (size_t)max_splits * heads * depth) * sizeof(float);
+  KRM_REQUIRE(ctx, workspace_bytes >= need,
+              "krm_attention_varlen_planned: workspace of %zu bytes, %zu needed", workspace_bytes,
+              need);
+  DecodeLaunch L{};
+  L.q = q; L.ins_k = ins_k; L.ins_v = ins_v; L.slot_k = slot_k; L.slot_v = slot_v; L.out = out;
+  L.args.heads = heads;
+  L.args.kv_heads = kv_heads;
+  L.args.window = 0;
+  L.args.past = 0;
+  L.args.slot_batch_stride = 0;
+  L.args.slot_plane_stride = total_rows * depth;
+  L.args.scale = half_scale;
+  L.args.nseq = nseq;
+  L.args.cu_rows = ptr<const int32_t>(plan);
+  L.args.split_prefix = L.args.cu_rows + nseq + 1;
+  L.ws_ml = ptr<float>(workspace);
+  L.ws_acc = L.ws_ml + ml_floats;
+  L.grid_x = max_splits;
   L.grid_z = 1;
   L.args.tickets = ctx->tickets;
   return decode_dispatch<true>(ctx, L, repeat, lpr, io_dtype, kv_dtype);

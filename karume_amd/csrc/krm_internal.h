@@ -26,6 +26,14 @@ struct krm_ctx {
   // allocated with the context so that launches can be recorded into graphs.
   float* gemm_partials = nullptr;
   bool recording = false;  // between krm_graph_begin and krm_graph_end
+  // Parallel branches of a recording (krm_graph_branch): `stream` is the stream launches go
+  // to, which is `main_stream` except while a side branch is selected.  Side streams are
+  // created on first use (default priority) and live as long as the context.
+  hipStream_t main_stream = nullptr;
+  static constexpr int kMaxBranches = 4;
+  hipStream_t branch_stream[kMaxBranches] = {nullptr, nullptr, nullptr, nullptr};
+  hipEvent_t branch_event[kMaxBranches] = {nullptr, nullptr, nullptr, nullptr};
+  bool branch_forked[kMaxBranches] = {false, false, false, false};
   char error[512] = {0};
 };
 

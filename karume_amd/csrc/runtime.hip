@@ -76,6 +76,7 @@ int32_t krm_ctx_create_on_stream(int32_t device, void* hip_stream, krm_ctx** out
   ctx->device = device;
   ctx->num_cus = prop.multiProcessorCount;
   ctx->stream = static_cast<hipStream_t>(hip_stream);
+  ctx->main_stream = ctx->stream;
   ctx->owns_stream = false;
   ctx->pinned_bytes = 1 << 20;
   hipError_t st = hipHostMalloc(&ctx->pinned, ctx->pinned_bytes, hipHostMallocDefault);
@@ -114,6 +115,7 @@ int32_t krm_ctx_create(int32_t device, krm_ctx** out) {
     *out = nullptr;
     return hip_status(nullptr, st, "hipStreamCreateWithFlags");
   }
+  ctx->main_stream = ctx->stream;
   ctx->owns_stream = true;
   return KRM_OK;
 }
@@ -121,7 +123,13 @@ int32_t krm_ctx_create(int32_t device, krm_ctx** out) {
 int32_t krm_ctx_destroy(krm_ctx* ctx) {
   if (!ctx) return KRM_OK;
   (void)hipSetDevice(ctx->device);
+  ctx->stream = ctx->main_stream;
   (void)hipStreamSynchronize(ctx->stream);
+  for (int i = 1; i < krm_ctx::kMaxBranches; ++i) {
+    if (ctx->branch_stream[i]) (void)hipStreamDestroy(ctx->branch_stream[i]);
+    if (ctx->branch_event[i]) (void)hipEventDestroy(ctx->branch_event[i]);
+  }
+  if (ctx->branch_event[0]) (void)hipEventDestroy(ctx->branch_event[0]);
   if (ctx->owns_stream) (void)hipStreamDestroy(ctx->stream);
   if (ctx->pinned) (void)hipHostFree(ctx->pinned);
   if (ctx->tickets) (void)hipFree(ctx->tickets);
@@ -235,13 +243,56 @@ int32_t krm_graph_begin(krm_ctx* ctx) {
   return KRM_OK;
 }
 
+int32_t krm_graph_branch(krm_ctx* ctx, uint32_t branch) {
+  KRM_TRY(enter(ctx));
+  KRM_REQUIRE(ctx, ctx->recording, "krm_graph_branch: no recording in progress");
+  KRM_REQUIRE(ctx, branch < (uint32_t)krm_ctx::kMaxBranches, "krm_graph_branch: branch %u of %d",
+              branch, krm_ctx::kMaxBranches);
+  if (branch == 0) {
+    ctx->stream = ctx->main_stream;
+    return KRM_OK;
+  }
+  if (!ctx->branch_stream[branch]) {
+    // default priority, like every stream of this library
+    KRM_TRY(hip_status(ctx, hipStreamCreateWithFlags(&ctx->branch_stream[branch],
+                                                     hipStreamNonBlocking),
+                       "hipStreamCreateWithFlags(branch)"));
+    KRM_TRY(hip_status(ctx, hipEventCreateWithFlags(&ctx->branch_event[branch],
+                                                    hipEventDisableTiming),
+                       "hipEventCreate(branch)"));
+  }
+  if (!ctx->branch_event[0])
+    KRM_TRY(hip_status(ctx, hipEventCreateWithFlags(&ctx->branch_event[0], hipEventDisableTiming),
+                       "hipEventCreate(fork)"));
+  if (!ctx->branch_forked[branch]) {
+    // fork: the side stream joins the capture behind what the main branch holds so far
+    KRM_TRY(hip_status(ctx, hipEventRecord(ctx->branch_event[0], ctx->main_stream),
+                       "hipEventRecord(fork)"));
+    KRM_TRY(hip_status(ctx, hipStreamWaitEvent(ctx->branch_stream[branch], ctx->branch_event[0], 0),
+                       "hipStreamWaitEvent(fork)"));
+    ctx->branch_forked[branch] = true;
+  }
+  ctx->stream = ctx->branch_stream[branch];
+  return KRM_OK;
+}
+
 int32_t krm_graph_end(krm_ctx* ctx, krm_graph** out) {
   KRM_TRY(enter(ctx));
   KRM_REQUIRE(ctx, out != nullptr, "krm_graph_end: out is NULL");
   KRM_REQUIRE(ctx, ctx->recording, "krm_graph_end: no recording in progress");
   ctx->recording = false;
+  ctx->stream = ctx->main_stream;
+  hipError_t st = hipSuccess;
+  // join: the main branch waits for every side branch before the recording closes
+  for (int i = 1; i < krm_ctx::kMaxBranches; ++i) {
+    if (!ctx->branch_forked[i]) continue;
+    ctx->branch_forked[i] = false;
+    if (st == hipSuccess) st = hipEventRecord(ctx->branch_event[i], ctx->branch_stream[i]);
+    if (st == hipSuccess) st = hipStreamWaitEvent(ctx->main_stream, ctx->branch_event[i], 0);
+  }
   krm_graph* g = new krm_graph();
-  hipError_t st = hipStreamEndCapture(ctx->stream, &g->graph);
+  hipError_t end = hipStreamEndCapture(ctx->main_stream, &g->graph);
+  if (st == hipSuccess) st = end;
   if (st == hipSuccess) st = hipGraphInstantiate(&g->exec, g->graph, nullptr, nullptr, 0);
   if (st != hipSuccess) {
     if (g->graph) (void)hipGraphDestroy(g->graph);
@@ -267,6 +318,42 @@ int32_t krm_graph_destroy(krm_ctx* ctx, krm_graph* graph) {
   if (graph->graph) (void)hipGraphDestroy(graph->graph);
   delete graph;
   return KRM_OK;
+}
+
+// Measurement floors: what a launch of a given grid costs when it does nothing, and when it
+// only streams `bytes` with 16-byte loads (every thread folds what it read into one word that
+// is stored only if it equals a value the data never has, so the loads stay).
+__global__ void krm_probe_empty_kernel() {}
+
+__global__ void krm_probe_read_kernel(const uint4* __restrict__ src, size_t pieces,
+                                      uint32_t* __restrict__ sink) {
+  size_t i = blockIdx.x * (size_t)blockDim.x + threadIdx.x;
+  const size_t stride = (size_t)gridDim.x * blockDim.x;
+  uint32_t fold = 0;
+  for (; i < pieces; i += stride) {
+    const uint4 v = src[i];
+    fold |= (v.x ^ v.y) + (v.z ^ v.w);
+  }
+  if (fold == 0x9E3779B9u && sink) sink[0] = fold;
+}
+
+int32_t krm_probe_launch(krm_ctx* ctx, int32_t kind, krm_buf src, size_t bytes, uint32_t grid,
+                         uint32_t block) {
+  KRM_TRY(enter(ctx));
+  KRM_REQUIRE(ctx, kind == KRM_PROBE_EMPTY || kind == KRM_PROBE_READ, "krm_probe_launch: kind %d",
+              kind);
+  KRM_REQUIRE(ctx, grid >= 1 && grid <= 0x7fffffffu && block >= 64 && block <= 1024 &&
+                       block % 64 == 0,
+              "krm_probe_launch: grid %u x block %u", grid, block);
+  if (kind == KRM_PROBE_EMPTY) {
+    krm_probe_empty_kernel<<<dim3(grid), dim3(block), 0, ctx->stream>>>();
+    return launched(ctx, "krm_probe_empty_kernel");
+  }
+  KRM_REQUIRE(ctx, src && src % 16 == 0 && bytes % 16 == 0 && bytes > 0,
+              "krm_probe_launch: the read probe needs a 16-byte aligned buffer and size");
+  krm_probe_read_kernel<<<dim3(grid), dim3(block), 0, ctx->stream>>>(
+      ptr<const uint4>(src), bytes / 16, ctx->tickets + (size_t)(kTicketSlots - 1) * kTicketStride);
+  return launched(ctx, "krm_probe_read_kernel");
 }
 
 int32_t krm_event_create(krm_ctx* ctx, krm_event** out) {

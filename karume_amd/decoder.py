@@ -189,6 +189,23 @@ class LlamaDecoderSession:
         self.workspace: Optional[DeviceBuffer] = None
         self.logits_shape = (1, c.vocab)
 
+    def close(self) -> None:
+        """Free every device buffer of the session (weights, tables, scratch activations)."""
+        for entry in self.layers:
+            for value in entry.values():
+                if isinstance(value, _DeviceLinear):
+                    value.w.free()
+                    value.s.free()
+                else:
+                    value.free()
+        for buf in list(self.buf.values()) + [self.embedding, self.final_norm, self.lm_head.w,
+                                              self.lm_head.s, self.rope_cos, self.rope_sin]:
+            buf.free()
+        if self.workspace is not None:
+            self.workspace.free()
+            self.workspace = None
+        self.layers, self.buf = [], {}
+
     # -- GreedySession surface ---------------------------------------------------------------
     def create_generation_context(self, *, capacity: int, chunk_length: int) -> GenerationContext:
         if chunk_length != self.chunk_length:

@@ -98,6 +98,11 @@ class GenerationContext:
     def rewind(self, position: int) -> None:
         """Forget everything at and after `position` (full contexts only,
         generation-context.ts:486-512)."""
+        if self.disposed:
+            raise GenerationContextError("the generation context was disposed")
+        if self.poisoned:
+            raise GenerationContextError(
+                "the generation context is poisoned by a failed run; create a new one")
         if self.window:
             raise ExecutionError("a sliding-window context cannot be rewound")
         if position < 0 or position > self.past:
@@ -118,22 +123,28 @@ class GreedySession(Protocol):
 
     def create_generation_context(self, *, capacity: int, chunk_length: int): ...
 
-    def run(self, input_ids: np.ndarray, position_ids: np.ndarray, last_row: int, *, context,
-            query_length: int) -> np.ndarray: ...
+    def run(self, input_ids: np.ndarray, position_ids: np.ndarray, last_row: Optional[int], *,
+            context, query_length: int) -> np.ndarray: ...
 
 
 def generate_greedy(session: GreedySession, *, prompt: Sequence[int], max_new_tokens: int,
-                    chunk_length: int, max_position: int, capacity: Optional[int] = None
-                    ) -> List[int]:
+                    chunk_length: int, max_position: int, capacity: Optional[int] = None,
+                    last_row: bool = True) -> List[int]:
     """Greedy continuation of `prompt` (packages/models/src/generation/greedy.ts:196-259).
 
-    `session.run` receives i32 ids/positions of shape [1, M] (pad rows zero), the index of the
-    last valid row, and returns the argmax token as an i32 array of shape [1, 1, 1]."""
+    `session.run` receives i32 ids/positions of shape [1, M] (pad rows zero) and, with
+    `last_row` (the token-only exit, the reference's default asset form), the index of the last
+    valid row; it then returns the argmax token as an i32 array of shape [1, 1, 1].  Without
+    `last_row` the session is handed None there and returns the argmax of every row,
+    [1, M, 1], of which the last valid row is read (greedy.ts:228-236).  Entry checks run
+    before the context is created; the context is disposed exactly once, also on failure."""
+    _assert_positive_integer(len(prompt), "prompt length")
     chunks = plan_prefill_chunks(len(prompt), chunk_length)
     _assert_positive_integer(max_new_tokens, "maxNewTokens")
     _assert_positive_integer(max_position, "maxPosition")
     for index, token in enumerate(prompt):
-        if not isinstance(token, (int, np.integer)) or token < 0 or token > 0x7FFFFFFF:
+        if (not isinstance(token, (int, np.integer)) or isinstance(token, bool) or token < 0
+                or token > 0x7FFFFFFF):
             raise ValueError(f"prompt[{index}] {token!r} is not an integer in 0..2147483647")
     last_position = len(prompt) + max_new_tokens - 2
     if last_position >= max_position:
@@ -150,23 +161,29 @@ def generate_greedy(session: GreedySession, *, prompt: Sequence[int], max_new_to
             n = chunk.query_length
             ids[0, :n] = prompt[chunk.position:chunk.position + n]
             positions[0, :n] = np.arange(chunk.position, chunk.position + n)
-            out = session.run(ids, positions, n - 1, context=context, query_length=n)
-            token = _read_token(out)
+            out = session.run(ids, positions, n - 1 if last_row else None, context=context,
+                              query_length=n)
+            token = (_read_token(out, 1, 0) if last_row
+                     else _read_token(out, chunk_length, n - 1))
         generated = [token]
         for index in range(max_new_tokens - 1):
             out = session.run(np.array([[generated[index]]], dtype=np.int32),
-                              np.array([[len(prompt) + index]], dtype=np.int32), 0,
-                              context=context, query_length=1)
-            generated.append(_read_token(out))
+                              np.array([[len(prompt) + index]], dtype=np.int32),
+                              0 if last_row else None, context=context, query_length=1)
+            generated.append(_read_token(out, 1, 0))
         return generated
     finally:
         context.dispose()
 
 
-def _read_token(out) -> int:
+def _read_token(out, rows: int, row: int) -> int:
+    """One row of the argmax output; dtype and shape are checked so that a wrong output (the
+    logits, the other exit form) fails instead of yielding tokens (greedy.ts:171-188)."""
+    if out is None:
+        raise ValueError("the run returned no token output")
     arr = np.asarray(out)
     if arr.dtype != np.int32:
         raise TypeError(f"the token output is {arr.dtype}, not int32")
-    if arr.shape != (1, 1, 1):
-        raise ValueError(f"the token output has shape {list(arr.shape)}, not [1, 1, 1]")
-    return int(arr[0, 0, 0])
+    if arr.shape != (1, rows, 1):
+        raise ValueError(f"the token output has shape {list(arr.shape)}, not [1, {rows}, 1]")
+    return int(arr[0, row, 0])

@@ -18,6 +18,8 @@ F32 = 0
 F16 = 1
 COMPUTE_F32 = 0
 COMPUTE_F16 = 1
+PROBE_EMPTY = 0
+PROBE_READ = 1
 EPILOGUE_NONE = 0
 EPILOGUE_SILU_PAIRS = 1
 
@@ -152,6 +154,11 @@ class _Recording:
         self.ctx = ctx
         self.graph: Optional[GpuGraph] = None
 
+    def branch(self, index: int) -> None:
+        """The ops that follow go to parallel branch `index` (0 = main, 1..3 = side branches
+        that fork from the main branch here and join it when the recording ends)."""
+        self.ctx._check(self.ctx._lib.krm_graph_branch(self.ctx._handle, index))
+
     def __enter__(self) -> "_Recording":
         self.ctx._check(self.ctx._lib.krm_graph_begin(self.ctx._handle))
         return self
@@ -235,6 +242,13 @@ class GpuContext:
 
     def copy(self, dst: BufferLike, src: BufferLike, nbytes: int) -> None:
         self._check(self._lib.krm_buf_copy(self._handle, _addr(dst), _addr(src), nbytes))
+
+    def probe_launch(self, kind: int, src: BufferLike = None, nbytes: int = 0, grid: int = 1,
+                     block: int = 256) -> None:
+        """Measurement floors: PROBE_EMPTY launches a kernel that does nothing, PROBE_READ one
+        that streams `nbytes` at `src` with 16-byte loads."""
+        self._check(self._lib.krm_probe_launch(self._handle, kind, _addr(src), nbytes, grid,
+                                               block))
 
     def borrow(self, address: int, nbytes: int) -> DeviceBuffer:
         """Wrap device memory owned by someone else (for example a torch tensor's data_ptr)."""
@@ -327,6 +341,37 @@ class GpuContext:
             depth, total_rows, float(half_scale), io_dtype, kv_dtype, _addr(workspace),
             workspace_bytes))
 
+    def attention_varlen_plan_bytes(self, nseq: int) -> int:
+        nbytes = C.c_size_t()
+        self._check(self._lib.krm_attention_varlen_plan_bytes(nseq, C.byref(nbytes)))
+        return int(nbytes.value)
+
+    def attention_varlen_max_splits(self, nseq: int, depth: int, kv_dtype: int,
+                                    total_rows: int) -> int:
+        splits = C.c_uint32()
+        self._check(self._lib.krm_attention_varlen_max_splits(nseq, depth, kv_dtype, total_rows,
+                                                              C.byref(splits)))
+        return int(splits.value)
+
+    def attention_varlen_plan(self, cu_seqlens: BufferLike, plan: BufferLike, *, nseq: int,
+                              depth: int, kv_dtype: int, total_rows: int, max_splits: int) -> None:
+        """Launch tables of a ragged step from a DEVICE cu_seqlens array (recordable)."""
+        self._check(self._lib.krm_attention_varlen_plan(
+            self._handle, _addr(cu_seqlens), _addr(plan), nseq, depth, kv_dtype, total_rows,
+            max_splits))
+
+    def attention_varlen_planned(self, q: BufferLike, ins_k: BufferLike, ins_v: BufferLike,
+                                 slot_k: BufferLike, slot_v: BufferLike, out: BufferLike,
+                                 plan: BufferLike, *, nseq: int, heads: int, kv_heads: int,
+                                 depth: int, total_rows: int, max_splits: int, half_scale: float,
+                                 io_dtype: int = F32, kv_dtype: int = F32,
+                                 workspace: BufferLike = None, workspace_bytes: int = 0) -> None:
+        if isinstance(workspace, DeviceBuffer) and not workspace_bytes:
+            workspace_bytes = workspace.nbytes
+        self._check(self._lib.krm_attention_varlen_planned(
+            self._handle, _addr(q), _addr(ins_k), _addr(ins_v), _addr(slot_k), _addr(slot_v),
+            _addr(out), _addr(plan), nseq, heads, kv_heads, depth, total_rows, max_splits,
+            float(half_scale), io_dtype, kv_dtype, _addr(workspace), workspace_bytes))
 
     # -- run-time lengths on the device ----------------------------------------------------------
     def lengths_set(self, lengths: BufferLike, past: int, query: int) -> None:

@@ -216,11 +216,12 @@ def synthetic_int4(rng: np.random.Generator, n: int, k: int, group: int, scale_f
 
 # ---------------------------------------------------------------------------- decoder oracle
 
-def oracle_decoder_logits(weights, ids) -> np.ndarray:
+def oracle_decoder_logits(weights, ids, rows=None) -> np.ndarray:
     """Full re-forward WITHOUT a KV cache over the whole id sequence (the way the reference
     derives its greedy goldens, tools/export-recipes/_shared/decode_series.py:51-73): every op
     is the CPU oracle's; attention is one causal pass (P = 0, Q = M = T).  Returns logits [T, V]
-    in float32."""
+    in float32, or [len(rows), V] for the listed positions only (the lm_head is the largest
+    linear; a long sequence needs it on few rows)."""
     c = weights.config
     ids = np.asarray(ids, dtype=np.int32)
     t = ids.size
@@ -249,6 +250,8 @@ def oracle_decoder_logits(weights, ids) -> np.ndarray:
         xn = oracle.rms_norm(h, lw["ffn_norm"], c.rms_eps)
         act = oracle.silu_mul(lin(xn, lw["gate"]), lin(xn, lw["up"]))
         h = (h + lin(act, lw["down"])).astype(np.float32)
+    if rows is not None:
+        h = np.ascontiguousarray(h[np.asarray(rows, dtype=np.int64)])
     xn = oracle.rms_norm(h, weights.final_norm, c.rms_eps)
     return lin(xn, weights.lm_head)
 

@@ -140,6 +140,46 @@ def test_decode_with_device_lengths_equals_scalar_form(gpu_ctx, case, io, kv):
         b.free()
 
 
+@pytest.mark.parametrize("max_past,device_past", [(600, 900), (100, 700)])
+def test_replay_beyond_the_sized_past_raises_the_fault_word(gpu_ctx, max_past, device_past):
+    """A launch sized for `max_past` (5 splits, or a single split without a workspace) meets a
+    device-side pastLength that needs more splits: the fault word is raised, `out` keeps its
+    bytes, and the arrival counters stay clean — the same launch with a legal pastLength
+    afterwards still equals the scalar form bitwise.  Every workgroup exits normally."""
+    case = StateCase("guard", 1, 8, 2, 1, 128, 1024, 0, device_past, 1)
+    x = random_state_inputs(case, seed=11, f16_values=True)
+    io = kv = np.float16
+    bufs = {k: gpu_ctx.upload(np.ascontiguousarray(v, dtype=np.float16)) for k, v in x.items()}
+    sentinel = np.full(case.heads * case.depth, 123.0, dtype=io)
+    out = gpu_ctx.upload(sentinel)
+    ws = gpu_ctx.alloc(max(16, gpu_ctx.attention_state_workspace(
+        1, case.heads, case.kv_heads, 1, case.depth, 0, max_past, 1)))
+    lengths = gpu_ctx.zeros(16)
+
+    def launch():
+        gpu_ctx.attention_state_lengths(
+            bufs["q"], bufs["ins_k"], bufs["ins_v"], bufs["slot_k"], bufs["slot_v"], out,
+            batch=1, heads=case.heads, kv_heads=case.kv_heads, chunk_rows=1, depth=case.depth,
+            capacity=case.capacity, window=0, half_scale=oracle.half_scale(case.depth),
+            lengths=lengths, max_past=max_past, io_dtype=ka.F16, kv_dtype=ka.F16,
+            workspace=ws if max_past > 512 else None)
+
+    gpu_ctx.lengths_set(lengths, device_past, 1)
+    launch()
+    state = lengths.download(np.uint32, (4,))
+    assert state[2] == 1 and state[0] == device_past
+    assert out.download(io, sentinel.shape).tobytes() == sentinel.tobytes()
+    # a legal pastLength through the same launch shape afterwards
+    legal = StateCase("legal", 1, 8, 2, 1, 128, 1024, 0, max_past, 1)
+    want = run_attention(gpu_ctx, legal, x, io=io, kv=kv)
+    gpu_ctx.lengths_set(lengths, max_past, 1)
+    launch()
+    assert lengths.download(np.uint32, (4,))[2] == 0
+    assert out.download(io, want.shape).tobytes() == want.tobytes()
+    for b in list(bufs.values()) + [out, ws, lengths]:
+        b.free()
+
+
 def test_config2_decode_attention(gpu_ctx):
     """benchmark config 2: B=1, H=32, Hkv=8, D=128, 4095 slot rows + this step's row, fp16."""
     case = StateCase("config 2", 1, 32, 8, 1, 128, 4096, 0, 4095, 1)
@@ -403,4 +443,84 @@ def test_varlen_edges(gpu_ctx):
                                  [0, 5, 3], heads=heads, kv_heads=kv_heads, depth=depth,
                                  total_rows=total, half_scale=0.3, workspace=ws)
     for b in list(d.values()) + [out, ws]:
+        b.free()
+
+
+def test_varlen_planned_on_the_device_is_recordable(gpu_ctx):
+    """The ragged step with its tables built on the device: equals the host-table form bitwise;
+    recorded once and replayed while the sequences grow (the offsets are rewritten between the
+    replays, with eager work and synchronisations in between) every replay equals the eager
+    host-table result of the same lengths; offsets that are not ascending raise the plan's
+    fault word and leave `out` untouched."""
+    heads, kv_heads, depth, nseq = 8, 2, 128, 5
+    capacity_rows = [700, 300, 900, 140, 20]           # rows each sequence owns in the slot
+    starts = np.concatenate([[0], np.cumsum(capacity_rows)]).astype(np.int64)
+    total = int(starts[-1])
+    rng = np.random.default_rng(17)
+    f16 = lambda a: a.astype(np.float16)  # noqa: E731
+    slot_k, slot_v = (f16(rng.normal(size=(kv_heads, total, depth))) for _ in range(2))
+    q, ins_k, ins_v = (f16(rng.normal(size=(nseq, h, depth))) for h in (heads, kv_heads, kv_heads))
+    d = {name: gpu_ctx.upload(arr) for name, arr in
+         dict(q=q, ins_k=ins_k, ins_v=ins_v, slot_k=slot_k, slot_v=slot_v).items()}
+    half = oracle.half_scale(depth)
+    out, out_host = gpu_ctx.alloc(q.nbytes), gpu_ctx.alloc(q.nbytes)
+    ws = gpu_ctx.alloc(gpu_ctx.attention_varlen_workspace(nseq, heads, kv_heads, depth, total))
+    ws_host = gpu_ctx.alloc(gpu_ctx.attention_varlen_workspace(nseq, heads, kv_heads, depth, total))
+    plan = gpu_ctx.alloc(gpu_ctx.attention_varlen_plan_bytes(nseq))
+    max_splits = gpu_ctx.attention_varlen_max_splits(nseq, depth, ka.F16, total)
+    assert max_splits == total // 128 + nseq
+    cu_dev = gpu_ctx.alloc(4 * (nseq + 1))
+    common = dict(heads=heads, kv_heads=kv_heads, depth=depth, total_rows=total, half_scale=half,
+                  io_dtype=ka.F16, kv_dtype=ka.F16)
+
+    # each replay sees other (ascending) offsets: sequence i holds fill * capacity_rows[i] rows
+    def offsets(fill):
+        cu = np.zeros(nseq + 1, dtype=np.int32)
+        for i in range(nseq):
+            cu[i + 1] = cu[i] + int(capacity_rows[i] * fill)
+        return cu
+
+    with gpu_ctx.record() as rec:
+        gpu_ctx.attention_varlen_plan(cu_dev, plan, nseq=nseq, depth=depth, kv_dtype=ka.F16,
+                                      total_rows=total, max_splits=max_splits)
+        gpu_ctx.attention_varlen_planned(d["q"], d["ins_k"], d["ins_v"], d["slot_k"], d["slot_v"],
+                                         out, plan, nseq=nseq, max_splits=max_splits,
+                                         workspace=ws, **common)
+    for fill in (0.25, 0.6, 1.0, 0.4):
+        cu = offsets(fill)
+        cu_dev.upload(cu)
+        out.upload(np.full(q.size, 77.0, dtype=np.float16))
+        rec.graph.launch()
+        got = out.download(np.float16, q.shape)
+        assert plan.download(np.int32, (2 * (nseq + 1) + 1,))[-1] == 0
+        gpu_ctx.attention_varlen(d["q"], d["ins_k"], d["ins_v"], d["slot_k"], d["slot_v"],
+                                 out_host, cu, workspace=ws_host, **common)
+        want = out_host.download(np.float16, q.shape)
+        assert got.tobytes() == want.tobytes(), fill
+    rec.graph.destroy()
+
+    # offsets that break the contract: fault word, no store
+    for bad in ([0, 50, 40, 60, 70, 80], [0, 10, 20, 30, 40, total + 1], [-1, 10, 20, 30, 40, 50]):
+        cu_dev.upload(np.array(bad, dtype=np.int32))
+        sentinel = np.full(q.size, 55.0, dtype=np.float16)
+        out.upload(sentinel)
+        gpu_ctx.attention_varlen_plan(cu_dev, plan, nseq=nseq, depth=depth, kv_dtype=ka.F16,
+                                      total_rows=total, max_splits=max_splits)
+        gpu_ctx.attention_varlen_planned(d["q"], d["ins_k"], d["ins_v"], d["slot_k"], d["slot_v"],
+                                         out, plan, nseq=nseq, max_splits=max_splits,
+                                         workspace=ws, **common)
+        assert plan.download(np.int32, (2 * (nseq + 1) + 1,))[-1] == 1, bad
+        assert out.download(np.float16, (q.size,)).tobytes() == sentinel.tobytes(), bad
+    # a legal plan afterwards still works (the counters were left clean)
+    cu = offsets(1.0)
+    cu_dev.upload(cu)
+    gpu_ctx.attention_varlen_plan(cu_dev, plan, nseq=nseq, depth=depth, kv_dtype=ka.F16,
+                                  total_rows=total, max_splits=max_splits)
+    gpu_ctx.attention_varlen_planned(d["q"], d["ins_k"], d["ins_v"], d["slot_k"], d["slot_v"],
+                                     out, plan, nseq=nseq, max_splits=max_splits, workspace=ws,
+                                     **common)
+    gpu_ctx.attention_varlen(d["q"], d["ins_k"], d["ins_v"], d["slot_k"], d["slot_v"], out_host,
+                             cu, workspace=ws_host, **common)
+    assert out.download(np.float16, q.shape).tobytes() == out_host.download(np.float16, q.shape).tobytes()
+    for b in list(d.values()) + [out, out_host, ws, ws_host, plan, cu_dev]:
         b.free()

@@ -232,19 +232,6 @@ def test_transpose(gpu_ctx):
     assert np.array_equal(out.download(np.float32, (5, 3, 4)), x.transpose(1, 0, 2))
 
 
-def test_plan_prefill_chunks_and_greedy_input_checks():
-    # packages/models/tests/generation_greedy_test.ts (chunk planning and entry checks)
-    chunks = plan_prefill_chunks(10, 4)
-    assert [(c.position, c.query_length) for c in chunks] == [(0, 4), (4, 4), (8, 2)]
-    assert [(c.position, c.query_length) for c in plan_prefill_chunks(4, 4)] == [(0, 4)]
-    with pytest.raises(ValueError):
-        plan_prefill_chunks(0, 4)
-    with pytest.raises(ValueError):
-        generate_greedy(None, prompt=[1, 2], max_new_tokens=10, chunk_length=4, max_position=8)
-    with pytest.raises(ValueError):
-        generate_greedy(None, prompt=[1, -2], max_new_tokens=1, chunk_length=4, max_position=8)
-
-
 SMALL = LlamaConfig(layers=2, d_model=256, ffn=384, heads=8, kv_heads=2, head_dim=32, vocab=512,
                     group_size=128, max_position=64)
 

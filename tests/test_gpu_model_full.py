@@ -1,0 +1,76 @@
+"""Benchmark config 4 at its real shape: the 1.1B-shape int4 decoder (22 layers, d_model 2048,
+FFN 5632, 32 heads / 4 KV heads of 64, vocab 32000, int4 g128 + fp16 scales, random init of the
+benchmark's distributions), teacher-forced: a 128-token prompt in one prefill chunk, then 16
+one-row decode steps, each run's last-row logits against the CPU oracle's full re-forward
+without a KV cache (how the reference derives its greedy goldens,
+tools/export-recipes/_shared/decode_series.py:51-73).
+
+Tolerance.  The random init lets the residual stream grow by about 2e4 per layer, so logits are
+of the order 1e5..1e6 and an absolute gate means nothing across seeds; the gate is relative to
+the largest |logit| of the row.  f32 arithmetic (KRM_COMPUTE_F32 prefill, the reference's
+default linearCompute): gate 4e-6 (TO-MEASURE).  fp16-operand prefill
+(KRM_COMPUTE_F16, what bench.py times): gate 1.2e-3 (TO-MEASURE).  The token of a row
+must equal the oracle's argmax wherever the oracle's top-1/top-2 margin exceeds twice the gate.
+"""
+import time
+
+import numpy as np
+import pytest
+
+import helpers
+import karume_amd as ka
+from karume_amd.decoder import LlamaConfig, LlamaDecoderSession, random_weights
+
+pytestmark = pytest.mark.gpu
+
+PROMPT, DECODE = 128, 16
+
+
+@pytest.fixture(scope="module")
+def full_model():
+    config = LlamaConfig()
+    weights = random_weights(config, seed=4)
+    ids = np.random.default_rng(44).integers(0, config.vocab, size=PROMPT + DECODE).astype(np.int32)
+    rows = list(range(PROMPT - 1, PROMPT + DECODE))
+    t0 = time.perf_counter()
+    want = helpers.oracle_decoder_logits(weights, ids, rows=rows)
+    print(f"[config 4] oracle re-forward of {ids.size} rows: {time.perf_counter() - t0:.1f} s",
+          flush=True)
+    return config, weights, ids, want
+
+
+@pytest.mark.parametrize("label,compute,gate", [("f32", ka.COMPUTE_F32, 4e-6),
+                                                ("f16-operand prefill", ka.COMPUTE_F16, 1.2e-3)])
+def test_full_size_teacher_forced_logits(gpu_ctx, full_model, label, compute, gate):
+    config, weights, ids, want = full_model
+    session = LlamaDecoderSession(gpu_ctx, weights, io_dtype=ka.F32, kv_dtype=ka.F32,
+                                  chunk_length=PROMPT, prefill_compute=compute)
+    ctx = session.create_generation_context(capacity=config.max_position, chunk_length=PROMPT)
+    worst, checked_tokens, disagreements = 0.0, 0, 0
+
+    def check(token, logits, want_row):
+        nonlocal worst, checked_tokens, disagreements
+        scale = float(np.max(np.abs(want_row)))
+        err = float(np.max(np.abs(logits.astype(np.float64) - want_row))) / scale
+        worst = max(worst, err)
+        top = np.sort(want_row)
+        if (top[-1] - top[-2]) / scale > 2 * gate:
+            checked_tokens += 1
+            disagreements += int(token[0, 0, 0]) != int(np.argmax(want_row))
+
+    pos = np.arange(PROMPT, dtype=np.int32)[None]
+    token, logits = session.run(ids[None, :PROMPT], pos, PROMPT - 1, context=ctx,
+                                query_length=PROMPT, want_logits=True)
+    check(token, logits[0], want[0])
+    for step in range(DECODE):
+        p = PROMPT + step
+        token, logits = session.run(ids[p:p + 1][None], np.array([[p]], dtype=np.int32), 0,
+                                    context=ctx, query_length=1, want_logits=True)
+        check(token, logits[0], want[1 + step])
+    print(f"[config 4, {label}] worst |logit error| / max|logit| over {1 + DECODE} rows: "
+          f"{worst:.3e}; {checked_tokens} tokens checked, {disagreements} disagree", flush=True)
+    assert ctx.past == PROMPT + DECODE
+    assert worst <= gate, worst
+    assert disagreements == 0 and checked_tokens >= 1
+    ctx.dispose()
+    session.close()

@@ -213,10 +213,13 @@ def test_append_ring_mutation_is_visible():
     assert good[0, 1].tolist() == [77, 77] and good[0, 2].tolist() == [77, 77]
 
 
-def run_chain(window: int, capacity: int, steps, heads=4, kv_heads=2, depth=8, widen=0):
+def run_chain(window: int, capacity: int, steps, heads=4, kv_heads=2, depth=8, widen=0,
+              with_slots=False):
     """Prefill -> decode chain carried on the host: each step reads the slots, then appends
     (packages/runtime/tests/gpu_state_execution_test.ts:152-212).  Returns the outputs of the
-    valid rows of every step and the full K/V history that was fed in."""
+    valid rows of every step and the full K/V history that was fed in (and the final slots
+    with `with_slots`).  Only the valid rows are drawn from the generator, so two chains whose
+    steps differ in pad rows alone see the same values."""
     rng = np.random.default_rng(5)
     r = heads // kv_heads
     slot_k = np.zeros((1, kv_heads, capacity, depth), dtype=np.float32)
@@ -224,11 +227,12 @@ def run_chain(window: int, capacity: int, steps, heads=4, kv_heads=2, depth=8, w
     past = 0
     outs, qs, ks, vs = [], [], [], []
     for chunk_rows, query in steps:
-        q = rng.normal(size=(1, heads, chunk_rows, depth)).astype(np.float32)
-        k = rng.normal(size=(1, kv_heads, chunk_rows, depth)).astype(np.float32)
-        v = rng.normal(size=(1, kv_heads, chunk_rows, depth)).astype(np.float32)
-        k[:, :, query:] = 9.0   # pad rows carry poison
-        v[:, :, query:] = 400.0
+        q = np.full((1, heads, chunk_rows, depth), 0.5, dtype=np.float32)
+        k = np.full((1, kv_heads, chunk_rows, depth), 9.0, dtype=np.float32)    # pad rows carry
+        v = np.full((1, kv_heads, chunk_rows, depth), 400.0, dtype=np.float32)  # poison
+        q[:, :, :query] = rng.normal(size=(1, heads, query, depth))
+        k[:, :, :query] = rng.normal(size=(1, kv_heads, query, depth))
+        v[:, :, :query] = rng.normal(size=(1, kv_heads, query, depth))
         out = oracle.state_attention(q, k, v, slot_k, slot_v, batch=1, heads=heads,
                                      kv_heads=kv_heads, chunk_rows=chunk_rows, depth=depth,
                                      capacity=capacity, window=window + widen if window else 0,
@@ -243,7 +247,8 @@ def run_chain(window: int, capacity: int, steps, heads=4, kv_heads=2, depth=8, w
         vs.append(v[:, :, :query])
         past += query
     cat = lambda parts: np.concatenate(parts, axis=2)  # noqa: E731
-    return cat(outs), cat(qs), np.repeat(cat(ks), r, axis=1), np.repeat(cat(vs), r, axis=1)
+    result = (cat(outs), cat(qs), np.repeat(cat(ks), r, axis=1), np.repeat(cat(vs), r, axis=1))
+    return result + (slot_k, slot_v) if with_slots else result
 
 
 @pytest.mark.parametrize("window,capacity", [(0, 32), (5, 5), (5, 8)])
@@ -268,9 +273,13 @@ def test_capacity_and_pad_rows_do_not_change_results():
     (packages/runtime/tests/gpu_state_acceptance_test.ts:586-708,780-833)."""
     steps_pad = [(8, 5), (1, 1), (1, 1)]
     steps_tight = [(5, 5), (1, 1), (1, 1)]
-    small, *_ = run_chain(0, 8, steps_pad)
+    small, *_, small_k, small_v = run_chain(0, 8, steps_pad, with_slots=True)
     large, *_ = run_chain(0, 4096, steps_pad)
-    tight, *_ = run_chain(0, 8, steps_tight)
+    tight, *_, tight_k, tight_v = run_chain(0, 8, steps_tight, with_slots=True)
     assert np.array_equal(small.view(np.uint32), large.view(np.uint32))
-    # the chain draws q/k/v per step with the chunk's shape, so compare the first step only
-    assert np.array_equal(small[:, :, :5].shape, tight[:, :, :5].shape)
+    # pad rows change neither the valid rows' outputs nor a byte of the KV slots
+    assert small.shape == tight.shape == (1, 4, 7, 8)
+    assert np.array_equal(small.view(np.uint32), tight.view(np.uint32))
+    assert np.array_equal(small_k.view(np.uint32), tight_k.view(np.uint32))
+    assert np.array_equal(small_v.view(np.uint32), tight_v.view(np.uint32))
+    assert not np.any(small_k == 9.0) and not np.any(small_v == 400.0)
