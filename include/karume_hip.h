@@ -103,7 +103,9 @@ int32_t krm_event_destroy(krm_ctx* ctx, krm_event* ev);
  * stream (diagnostics like the timestamp queries above; no op of the reference):
  *   KRM_PROBE_EMPTY — a kernel that does nothing (what a launch of that grid costs);
  *   KRM_PROBE_READ  — every thread streams its share of `bytes` at `src` with 16-byte loads
- *                     and stores nothing (what reading that much costs). */
+ *                     and stores nothing (what reading that much costs); up to eight loads a
+ *                     thread are requested before any is used, so a grid that covers `bytes`
+ *                     in one pass pays one memory round trip. */
 #define KRM_PROBE_EMPTY 0
 #define KRM_PROBE_READ 1
 int32_t krm_probe_launch(krm_ctx* ctx, int32_t kind, krm_buf src, size_t bytes, uint32_t grid,

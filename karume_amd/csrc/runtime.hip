@@ -325,14 +325,23 @@ int32_t krm_graph_destroy(krm_ctx* ctx, krm_graph* graph) {
 // is stored only if it equals a value the data never has, so the loads stay).
 __global__ void krm_probe_empty_kernel() {}
 
+// PER 16-byte loads per thread are requested before any is used (one memory round trip for
+// the whole launch when the grid covers `pieces` in one pass); larger buffers take more passes.
+template <int PER>
 __global__ void krm_probe_read_kernel(const uint4* __restrict__ src, size_t pieces,
                                       uint32_t* __restrict__ sink) {
-  size_t i = blockIdx.x * (size_t)blockDim.x + threadIdx.x;
-  const size_t stride = (size_t)gridDim.x * blockDim.x;
+  const size_t threads = (size_t)gridDim.x * blockDim.x;
+  const size_t tid = blockIdx.x * (size_t)blockDim.x + threadIdx.x;
   uint32_t fold = 0;
-  for (; i < pieces; i += stride) {
-    const uint4 v = src[i];
-    fold |= (v.x ^ v.y) + (v.z ^ v.w);
+  for (size_t base = 0; base < pieces; base += threads * PER) {
+    uint4 v[PER];
+#pragma unroll
+    for (int j = 0; j < PER; ++j) {
+      const size_t i = base + (size_t)j * threads + tid;  // a wave reads 1 KiB in a row
+      v[j] = src[i < pieces ? i : 0];
+    }
+#pragma unroll
+    for (int j = 0; j < PER; ++j) fold |= (v[j].x ^ v[j].y) + (v[j].z ^ v[j].w);
   }
   if (fold == 0x9E3779B9u && sink) sink[0] = fold;
 }
@@ -351,8 +360,17 @@ int32_t krm_probe_launch(krm_ctx* ctx, int32_t kind, krm_buf src, size_t bytes, 
   }
   KRM_REQUIRE(ctx, src && src % 16 == 0 && bytes % 16 == 0 && bytes > 0,
               "krm_probe_launch: the read probe needs a 16-byte aligned buffer and size");
-  krm_probe_read_kernel<<<dim3(grid), dim3(block), 0, ctx->stream>>>(
-      ptr<const uint4>(src), bytes / 16, ctx->tickets + (size_t)(kTicketSlots - 1) * kTicketStride);
+  const size_t pieces = bytes / 16, threads = (size_t)grid * block;
+  uint32_t* sink = ctx->tickets + (size_t)(kTicketSlots - 1) * kTicketStride;
+  const size_t per = (pieces + threads - 1) / threads;
+  if (per <= 1)
+    krm_probe_read_kernel<1><<<dim3(grid), dim3(block), 0, ctx->stream>>>(ptr<const uint4>(src), pieces, sink);
+  else if (per <= 2)
+    krm_probe_read_kernel<2><<<dim3(grid), dim3(block), 0, ctx->stream>>>(ptr<const uint4>(src), pieces, sink);
+  else if (per <= 4)
+    krm_probe_read_kernel<4><<<dim3(grid), dim3(block), 0, ctx->stream>>>(ptr<const uint4>(src), pieces, sink);
+  else
+    krm_probe_read_kernel<8><<<dim3(grid), dim3(block), 0, ctx->stream>>>(ptr<const uint4>(src), pieces, sink);
   return launched(ctx, "krm_probe_read_kernel");
 }
 

@@ -8,8 +8,8 @@ tools/export-recipes/_shared/decode_series.py:51-73).
 Tolerance.  The random init lets the residual stream grow by about 2e4 per layer, so logits are
 of the order 1e5..1e6 and an absolute gate means nothing across seeds; the gate is relative to
 the largest |logit| of the row.  f32 arithmetic (KRM_COMPUTE_F32 prefill, the reference's
-default linearCompute): gate 4e-6 (TO-MEASURE).  fp16-operand prefill
-(KRM_COMPUTE_F16, what bench.py times): gate 1.2e-3 (TO-MEASURE).  The token of a row
+default linearCompute): worst measured 1.64e-7, gate 3.5e-7.  fp16-operand prefill
+(KRM_COMPUTE_F16, what bench.py times): worst measured 5.69e-5, gate 1.2e-4.  The token of a row
 must equal the oracle's argmax wherever the oracle's top-1/top-2 margin exceeds twice the gate.
 """
 import time
@@ -39,8 +39,8 @@ def full_model():
     return config, weights, ids, want
 
 
-@pytest.mark.parametrize("label,compute,gate", [("f32", ka.COMPUTE_F32, 4e-6),
-                                                ("f16-operand prefill", ka.COMPUTE_F16, 1.2e-3)])
+@pytest.mark.parametrize("label,compute,gate", [("f32", ka.COMPUTE_F32, 3.5e-7),
+                                                ("f16-operand prefill", ka.COMPUTE_F16, 1.2e-4)])
 def test_full_size_teacher_forced_logits(gpu_ctx, full_model, label, compute, gate):
     config, weights, ids, want = full_model
     session = LlamaDecoderSession(gpu_ctx, weights, io_dtype=ka.F32, kv_dtype=ka.F32,
