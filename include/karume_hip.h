@@ -200,6 +200,23 @@ int32_t krm_attention_state(krm_ctx* ctx, krm_buf q, krm_buf ins_k, krm_buf ins_
                             float half_scale, uint32_t past, uint32_t query, int32_t io_dtype,
                             int32_t kv_dtype, krm_buf workspace, size_t workspace_bytes);
 
+/* krm_attention_state for callers that cannot allocate device memory or hand in a workspace:
+ * code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.  It has
+ * no counterpart in the reference.  Same arguments, checks and results (bit for bit) as
+ * krm_attention_state, minus the workspace: split partials and arrival counters live in a
+ * 4 MiB array that is part of the library's device code (every GPU the library runs on holds
+ * its copy until the process ends).  It calls no allocating routine.  Limits: the call's split
+ * partials (krm_attention_state_workspace bytes) must fit 4 MiB - 64 KiB and it may use at most
+ * 512 arrival counters (B * Hkv * head groups); beyond that it returns KRM_ERR_VALIDATION and
+ * krm_attention_state with a workspace is the call to make.  All calls on one GPU share the
+ * array, whatever their context: calls that overlap on one GPU race. */
+int32_t krm_attention_state_noalloc(krm_ctx* ctx, krm_buf q, krm_buf ins_k, krm_buf ins_v,
+                                    krm_buf slot_k, krm_buf slot_v, krm_buf out, uint32_t batch,
+                                    uint32_t heads, uint32_t kv_heads, uint32_t chunk_rows,
+                                    uint32_t depth, uint32_t capacity, uint32_t window,
+                                    float half_scale, uint32_t past, uint32_t query,
+                                    int32_t io_dtype, int32_t kv_dtype);
+
 /* ---- state_append (packages/runtime/src/kernels/state-append.ts:47-96,120-173;
  *      builder packages/runtime/src/runtime/recipe-builder.ts:2011-2048) --------------------
  * Copies the first `query` rows of x[kv_planes, M, D] (x_dtype) into

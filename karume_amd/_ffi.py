@@ -55,6 +55,9 @@ PROTOTYPES = {
     "krm_attention_state": (i32, [c_ctx, c_buf, c_buf, c_buf, c_buf, c_buf, c_buf, u32, u32, u32,
                                   u32, u32, u32, u32, C.c_float, u32, u32, i32, i32, c_buf,
                                   size_t]),
+    "krm_attention_state_noalloc": (i32, [c_ctx, c_buf, c_buf, c_buf, c_buf, c_buf, c_buf, u32,
+                                          u32, u32, u32, u32, u32, u32, C.c_float, u32, u32, i32,
+                                          i32]),
     "krm_state_append": (i32, [c_ctx, c_buf, c_buf, u32, u32, u32, u32, u32, u32, u32, i32, i32]),
     "krm_attention_varlen_workspace": (i32, [u32, u32, u32, u32, u64, C.POINTER(size_t)]),
     "krm_attention_varlen": (i32, [c_ctx, c_buf, c_buf, c_buf, c_buf, c_buf, c_buf,

@@ -1243,3 +1243,71 @@ int32_t krm_attention_varlen_planned(krm_ctx* ctx, krm_buf q, krm_buf ins_k, krm
 }
 
 }  // extern "C"
+// ---- the decode attention for callers that cannot allocate ----------------------------------
+//
+// Split partials and arrival counters live in one file-scope device array instead of a
+// caller-supplied workspace and the context's counters.  Each GPU holds its own copy of the
+// array at its own address; the address is looked up once per device and that pointer — never
+// the array's name, which in host code is only a stand-in — is what kernels and fills receive.
+namespace {
+
+constexpr size_t kStaticTicketSlots = 512;
+constexpr size_t kStaticTicketBytes = kStaticTicketSlots * kTicketStride * sizeof(uint32_t);
+constexpr size_t kStaticScratchBytes = 4u << 20;  // counters + split partials, per GPU
+constexpr int kMaxDevices = 64;
+
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
+unsigned char* g_scratch_ptr[kMaxDevices] = {};
+
+// Device address of this device's copy of `scratch` (the context's device is current).
+int32_t static_scratch(krm_ctx* ctx, unsigned char** out) {
+  KRM_REQUIRE(ctx, ctx->device >= 0 && ctx->device < kMaxDevices,
+              "krm_attention_state_noalloc: device %d is outside 0..%d", ctx->device,
+              kMaxDevices - 1);
+  unsigned char* p = __atomic_load_n(&g_scratch_ptr[ctx->device], __ATOMIC_ACQUIRE);
+  if (!p) {
+    void* address = nullptr;
+    KRM_TRY(hip_status(ctx, hipGetSymbolAddress(&address, HIP_SYMBOL(scratch)),
+                       "hipGetSymbolAddress(scratch)"));
+    KRM_REQUIRE(ctx, address != nullptr, "krm_attention_state_noalloc: scratch has no address");
+    p = static_cast<unsigned char*>(address);
+    __atomic_store_n(&g_scratch_ptr[ctx->device], p, __ATOMIC_RELEASE);
+  }
+  *out = p;
+  return KRM_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int32_t krm_attention_state_noalloc(krm_ctx* ctx, krm_buf q, krm_buf ins_k, krm_buf ins_v,
+                                    krm_buf slot_k, krm_buf slot_v, krm_buf out, uint32_t batch,
+                                    uint32_t heads, uint32_t kv_heads, uint32_t chunk_rows,
+                                    uint32_t depth, uint32_t capacity, uint32_t window,
+                                    float half_scale, uint32_t past, uint32_t query,
+                                    int32_t io_dtype, int32_t kv_dtype) {
+  KRM_TRY(enter(ctx));
+  unsigned char* base = nullptr;
+  KRM_TRY(static_scratch(ctx, &base));
+  // the same sizing rule as krm_attention_state_workspace, against the fixed array
+  size_t need = 0;
+  KRM_TRY(krm_attention_state_workspace(batch, heads, kv_heads, chunk_rows, depth, window, past,
+                                        query, &need));
+  const size_t room = kStaticScratchBytes - kStaticTicketBytes;
+  if (need > room)
+    return fail(ctx, KRM_ERR_VALIDATION,
+                "krm_attention_state_noalloc: this call needs %zu bytes of split partials, the "
+                "built-in scratch holds %zu (use krm_attention_state with a workspace)",
+                need, room);
+  return attention_state_impl(ctx, q, ins_k, ins_v, slot_k, slot_v, out, batch, heads, kv_heads,
+                              chunk_rows, depth, capacity, window, half_scale, past, query, 0,
+                              io_dtype, kv_dtype,
+                              static_cast<krm_buf>(reinterpret_cast<uintptr_t>(
+                                  base + kStaticTicketBytes)),
+                              room, reinterpret_cast<uint32_t*>(base),
+                              (uint32_t)kStaticTicketSlots);
+}
+
+}  // extern "C"

@@ -312,6 +312,19 @@ class GpuContext:
             float(half_scale), past, query, io_dtype, kv_dtype, _addr(workspace),
             workspace_bytes))
 
+    def attention_state_noalloc(self, q: BufferLike, ins_k: BufferLike, ins_v: BufferLike,
+                                slot_k: BufferLike, slot_v: BufferLike, out: BufferLike, *,
+                                batch: int, heads: int, kv_heads: int, chunk_rows: int,
+                                depth: int, capacity: int, window: int, half_scale: float,
+                                past: int, query: int, io_dtype: int = F32,
+                                kv_dtype: int = F32) -> None:
+        """attention_state without a workspace: partials and counters in the library's own
+        device array (for callers that cannot allocate); rejects calls beyond its fixed size."""
+        self._check(self._lib.krm_attention_state_noalloc(
+            self._handle, _addr(q), _addr(ins_k), _addr(ins_v), _addr(slot_k), _addr(slot_v),
+            _addr(out), batch, heads, kv_heads, chunk_rows, depth, capacity, window,
+            float(half_scale), past, query, io_dtype, kv_dtype))
+
     def state_append(self, x: BufferLike, slot: BufferLike, *, kv_planes: int, chunk_rows: int,
                      depth: int, capacity: int, window: int, past: int, query: int,
                      x_dtype: int = F32, slot_dtype: int = F32) -> None:
