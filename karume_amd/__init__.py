@@ -14,6 +14,7 @@ from .runtime import (COMPUTE_F16, COMPUTE_F32, EPILOGUE_NONE, EPILOGUE_SILU_PAI
                       GpuContext, GpuDeviceLostError, GpuEvent, GpuGraph, GpuOutOfMemoryError,
                       GpuValidationError, KarumeError, acquire_gpu, dtype_code, version)
 
+from .decoder_loader import GraphShapeError, decoder_weights_from_model
 from .generation import (GenerationContext, GenerationContextError, PrefillChunk,
                          generate_greedy, plan_prefill_chunks)
 
@@ -21,6 +22,7 @@ __all__ = [
     "GenerationContext", "GenerationContextError", "PrefillChunk", "generate_greedy",
     "plan_prefill_chunks",
     "I4Error", "check_int4", "group_scale_shape", "pack_int4",
+    "GraphShapeError", "decoder_weights_from_model",
     "ContainerError", "IrError", "KarumeModel", "PackedInt4", "SafetensorsError",
     "i4_resident_initializers", "open_model", "packed_int4", "parse_safetensors", "tensor_bytes",
     "COMPUTE_F16", "COMPUTE_F32", "EPILOGUE_NONE", "EPILOGUE_SILU_PAIRS", "F16", "F32",

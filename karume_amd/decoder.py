@@ -65,6 +65,14 @@ class DecoderWeights:
     rope_cos: np.ndarray = None                # [max_position, head_dim] float32
     rope_sin: np.ndarray = None
 
+    @staticmethod
+    def from_model(model) -> "DecoderWeights":
+        """Weights of a model file (karume_amd.open_model) whose graph is the Llama-style
+        states-form decode graph; see karume_amd.decoder_loader."""
+        from .decoder_loader import decoder_weights_from_model
+
+        return decoder_weights_from_model(model)
+
 
 def rope_tables(config: LlamaConfig):
     """cos / sin rows for positions 0..max_position-1, half-split convention (the two halves of
@@ -106,7 +114,10 @@ class _DeviceLinear:
     def __init__(self, gpu: GpuContext, lin: Int4Linear):
         self.n, self.k = lin.n, lin.k
         self.w = gpu.upload(lin.packed)
-        self.s = gpu.upload(lin.scales)
+        # fp16 scales (the benchmark configs) or f32 scales (the IR's companion tensors)
+        self.scale_dtype = F16 if lin.scales.dtype == np.float16 else F32
+        self.s = gpu.upload(np.ascontiguousarray(
+            lin.scales, dtype=np.float16 if self.scale_dtype == F16 else np.float32))
 
 
 def _stack_rows(*lins: Int4Linear) -> Int4Linear:
@@ -251,7 +262,7 @@ class LlamaDecoderSession:
     def _linear(self, x, lin: _DeviceLinear, out, m: int) -> None:
         compute = self.prefill_compute if m > 16 else COMPUTE_F32
         self.gpu.linear_i4(x, lin.w, lin.s, None, out, m, lin.n, lin.k, self.config.group_size,
-                           self.io_dtype, F16, compute)
+                           self.io_dtype, lin.scale_dtype, compute)
 
     def _forward(self, context: GenerationContext, m: int, past: int, query: int, last_row: int,
                  lengths: Optional[DeviceBuffer], ids: Optional[DeviceBuffer] = None) -> None:
@@ -328,7 +339,7 @@ class LlamaDecoderSession:
 
     def _fused(self, x, lin: _DeviceLinear, out, **kw) -> None:
         self.gpu.linear_i4_fused(x, lin.w, lin.s, out, 1, lin.n, lin.k, self.config.group_size,
-                                 io_dtype=self.io_dtype, scale_dtype=F16, **kw)
+                                 io_dtype=self.io_dtype, scale_dtype=lin.scale_dtype, **kw)
 
     def _forward_fused_row(self, context: GenerationContext, past: int,
                            lengths: Optional[DeviceBuffer]) -> None:
@@ -351,7 +362,7 @@ class LlamaDecoderSession:
                          table_rows=c.max_position, capacity=context.capacity,
                          window=context.window, past=past, lengths=lengths,
                          norm_weight=lw["attn_norm"], norm_eps=c.rms_eps, io_dtype=io,
-                         scale_dtype=F16, kv_dtype=self.kv_dtype)
+                         scale_dtype=lin.scale_dtype, kv_dtype=self.kv_dtype)
             if lengths is None:
                 g.attention_state(q_r, k_r, v_row, context.slots_k[li], context.slots_v[li],
                                   b["att"], batch=1, heads=c.heads, kv_heads=c.kv_heads,

@@ -376,3 +376,41 @@ def test_lengths_step_end_equals_the_three_launches(gpu_ctx):
                          pos.download(np.int32, (4,)).tolist()))
         assert outs[0] == outs[1]
         assert outs[1][0][0] == (41 if fault else 42) and outs[1][1][2] == 777
+
+
+def test_session_from_a_model_file_equals_session_from_arrays(gpu_ctx):
+    """A decoder written out as a Karume model file (safetensors + karume_ir graph in the decode
+    recipe's node order), read back with open_model / DecoderWeights.from_model, prefills and
+    decodes to the same logits bits and tokens as the session built from the arrays (the file
+    carries f32 scale companions, the arrays fp16 ones: the same numbers)."""
+    from karume_amd.decoder import DecoderWeights
+    from model_file import decoder_model_file
+
+    weights = random_weights(SMALL, seed=21)
+    loaded = DecoderWeights.from_model(ka.open_model(decoder_model_file(weights)))
+    assert loaded.config == SMALL
+    ids = np.random.default_rng(8).integers(0, SMALL.vocab, size=13).astype(np.int32)
+    results = []
+    for w in (weights, loaded):
+        session = LlamaDecoderSession(gpu_ctx, w, io_dtype=ka.F32, kv_dtype=ka.F32, chunk_length=8)
+        ctx = session.create_generation_context(capacity=SMALL.max_position, chunk_length=8)
+        rows = []
+        for chunk in plan_prefill_chunks(11, 8):
+            n = chunk.query_length
+            cid, cpos = np.zeros((1, 8), dtype=np.int32), np.zeros((1, 8), dtype=np.int32)
+            cid[0, :n] = ids[chunk.position:chunk.position + n]
+            cpos[0, :n] = np.arange(chunk.position, chunk.position + n)
+            rows.append(session.run(cid, cpos, n - 1, context=ctx, query_length=n,
+                                    want_logits=True))
+        for pos in (11, 12):
+            rows.append(session.run(ids[pos:pos + 1][None], np.array([[pos]], dtype=np.int32), 0,
+                                    context=ctx, query_length=1, want_logits=True))
+        tokens = session.decode_tokens(ctx, int(rows[-1][0][0, 0, 0]), 5)
+        results.append((rows, tokens))
+        ctx.dispose()
+        session.close()
+    (rows_a, tokens_a), (rows_b, tokens_b) = results
+    assert tokens_a == tokens_b
+    for (tok_a, log_a), (tok_b, log_b) in zip(rows_a, rows_b):
+        assert np.array_equal(tok_a, tok_b)
+        assert log_a.tobytes() == log_b.tobytes()
