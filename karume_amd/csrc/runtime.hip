@@ -54,6 +54,32 @@ int32_t launched(krm_ctx* ctx, const char* kernel) {
 
 using namespace krm;
 
+// Measurement floors: what a launch of a given grid costs when it does nothing, and when it
+// only streams `bytes` with 16-byte loads (every thread folds what it read into one word that
+// is stored only if it equals a value the data never has, so the loads stay).
+__global__ void krm_probe_empty_kernel() {}
+
+// PER 16-byte loads per thread are requested before any is used (one memory round trip for
+// the whole launch when the grid covers `pieces` in one pass); larger buffers take more passes.
+template <int PER>
+__global__ void krm_probe_read_kernel(const uint4* __restrict__ src, size_t pieces,
+                                      uint32_t* __restrict__ sink) {
+  const size_t threads = (size_t)gridDim.x * blockDim.x;
+  const size_t tid = blockIdx.x * (size_t)blockDim.x + threadIdx.x;
+  uint32_t fold = 0;
+  for (size_t base = 0; base < pieces; base += threads * PER) {
+    uint4 v[PER];
+#pragma unroll
+    for (int j = 0; j < PER; ++j) {
+      const size_t i = base + (size_t)j * threads + tid;  // a wave reads 1 KiB in a row
+      v[j] = src[i < pieces ? i : 0];
+    }
+#pragma unroll
+    for (int j = 0; j < PER; ++j) fold |= (v[j].x ^ v[j].y) + (v[j].z ^ v[j].w);
+  }
+  if (fold == 0x9E3779B9u && sink) sink[0] = fold;
+}
+
 extern "C" {
 
 const char* krm_version(void) { return "karume-hip 0.1 gfx950"; }
@@ -318,32 +344,6 @@ int32_t krm_graph_destroy(krm_ctx* ctx, krm_graph* graph) {
   if (graph->graph) (void)hipGraphDestroy(graph->graph);
   delete graph;
   return KRM_OK;
-}
-
-// Measurement floors: what a launch of a given grid costs when it does nothing, and when it
-// only streams `bytes` with 16-byte loads (every thread folds what it read into one word that
-// is stored only if it equals a value the data never has, so the loads stay).
-__global__ void krm_probe_empty_kernel() {}
-
-// PER 16-byte loads per thread are requested before any is used (one memory round trip for
-// the whole launch when the grid covers `pieces` in one pass); larger buffers take more passes.
-template <int PER>
-__global__ void krm_probe_read_kernel(const uint4* __restrict__ src, size_t pieces,
-                                      uint32_t* __restrict__ sink) {
-  const size_t threads = (size_t)gridDim.x * blockDim.x;
-  const size_t tid = blockIdx.x * (size_t)blockDim.x + threadIdx.x;
-  uint32_t fold = 0;
-  for (size_t base = 0; base < pieces; base += threads * PER) {
-    uint4 v[PER];
-#pragma unroll
-    for (int j = 0; j < PER; ++j) {
-      const size_t i = base + (size_t)j * threads + tid;  // a wave reads 1 KiB in a row
-      v[j] = src[i < pieces ? i : 0];
-    }
-#pragma unroll
-    for (int j = 0; j < PER; ++j) fold |= (v[j].x ^ v[j].y) + (v[j].z ^ v[j].w);
-  }
-  if (fold == 0x9E3779B9u && sink) sink[0] = fold;
 }
 
 int32_t krm_probe_launch(krm_ctx* ctx, int32_t kind, krm_buf src, size_t bytes, uint32_t grid,
