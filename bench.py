@@ -186,11 +186,30 @@ def bench_gemv(timer: Timer, rng, steps: int, warmup: int, m: int, n: int, k: in
         res["overlapped"] = timer.run(step_branch, steps, warmup, branches=4)
         res["empty"] = timer.run(step_empty, steps, warmup)
         res["read"] = timer.run(step_read, steps, warmup)
+        res["read_overlapped"] = timer.run(step_read, steps, warmup, branches=4)
     for b in weights + scales + [x] + outs:
         b.free()
     res["algo"] = n * row_bytes + n * (k // g) * 2 + m * k * 2 + m * n * 2
     res["read_bytes"] = n * row_bytes
     return res
+
+
+def bench_exchange(timer: Timer, entries: int = 2048, phases: int = 2000):
+    """Microseconds per all-to-all hand-over of a vector between the 256 workgroups of one
+    persistent launch (krm_probe_exchange): what a single-launch decode step would pay at each
+    op boundary, to set beside floor.empty_kernel_us, the cost of a kernel boundary."""
+    ctx = timer.ctx
+    work = ctx.alloc(2 * entries * 4 + 1040)
+    best = None
+    for _ in range(3):
+        timer.start.record()
+        ctx.probe_exchange(work, entries, phases)
+        timer.stop.record()
+        ms = timer.start.elapsed_ms(timer.stop)
+        best = ms if best is None else min(best, ms)
+    fault = int(work.download(np.uint32, (1,), byte_offset=2 * entries * 4 + 1024)[0])
+    work.free()
+    return best * 1e3 / phases, fault
 
 
 def bench_attention(timer: Timer, rng, steps: int, warmup: int, copies: int):
@@ -542,7 +561,20 @@ def main() -> int:
             "pure_read_gbs": round(gv["read_bytes"] / us("read") / 1e3, 1),
             "grid": f"{(n + 3) // 4} x 256 threads (the GEMV's own)",
             "achieved_over_pure_read": round(us("read") / per_call_us, 3),
+            # the same read probe on four parallel graph branches: what overlapped launches of
+            # this size can reach at all (to set beside gemv_overlapped_us)
+            "pure_read_overlapped_us": round(us("read_overlapped"), 3),
+            "pure_read_overlapped_gbs": round(gv["read_bytes"] / us("read_overlapped") / 1e3, 1),
         }
+        ex_us, ex_fault = bench_exchange(timer)
+        result["floor"]["in_kernel_exchange_us"] = round(ex_us, 3)
+        result["floor"]["in_kernel_exchange_fault"] = ex_fault
+        log("[bench] GEMV M=1 K=4096 N=65536 (128 MiB of weights per launch)")
+        big = bench_gemv(timer, rng, max(8, steps // 16), max(8, warmup // 16), 1, 65536, k, g, 5)
+        big_us = big["rotating"]["ms"] * 1e3 / max(8, steps // 16)
+        result["gemv_n65536_us"] = round(big_us, 2)
+        result["gemv_n65536_gbs"] = round(big["algo"] / big_us / 1e3, 1)
+        result["gemv_n65536_pct_of_hbm_peak"] = round(100 * big["algo"] / big_us / 1e3 / 8000, 2)
     if args.only == "traffic":
         # For `rocprofv3 --pmc FETCH_SIZE` / `--pmc WRITE_SIZE`: a plain 8 MiB copy (known
         # traffic: 8 MiB read + 8 MiB written) beside the GEMV, a few launches of each.

@@ -25,6 +25,12 @@ export const KARUME_HIP_SYMBOLS = {
   krm_event_elapsed_ms: { parameters: ["pointer", "pointer", "pointer", "buffer"], result: "i32" },
   krm_event_destroy: { parameters: ["pointer", "pointer"], result: "i32" },
   krm_probe_launch: { parameters: ["pointer", "i32", "u64", "usize", "u32", "u32"], result: "i32" },
+  krm_probe_exchange: {
+    parameters: [
+      "pointer", "u64", "usize", "u32", "u32", "u32"
+    ],
+    result: "i32",
+  },
   krm_graph_begin: { parameters: ["pointer"], result: "i32" },
   krm_graph_branch: { parameters: ["pointer", "u32"], result: "i32" },
   krm_graph_end: { parameters: ["pointer", "buffer"], result: "i32" },

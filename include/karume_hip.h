@@ -111,6 +111,16 @@ int32_t krm_event_destroy(krm_ctx* ctx, krm_event* ev);
 int32_t krm_probe_launch(krm_ctx* ctx, int32_t kind, krm_buf src, size_t bytes, uint32_t grid,
                          uint32_t block);
 
+/* What an all-to-all hand-over of a vector of `entries` floats (2048, 4096 or 8192) costs
+ * between the 256 workgroups of ONE persistent launch, `phases` times in a row: flags polled
+ * and the vector read with agent-scope loads, results written with agent-scope stores (the
+ * step a single-launch decode would pay at every op boundary).  `work` is scratch of at least
+ * 2 * entries * 4 + 1040 bytes that the call clears; its last word written (offset
+ * 2 * entries * 4 + 1024) is a fault flag: 1 if a poll exceeded `spin_limit` rounds (every wait
+ * is bounded; the launch always ends).  Time it with events; no op of the reference. */
+int32_t krm_probe_exchange(krm_ctx* ctx, krm_buf work, size_t work_bytes, uint32_t entries,
+                           uint32_t phases, uint32_t spin_limit);
+
 /* ---- recorded launch sequences (the reference bakes a step's dispatch recipes once and
  *      replays them: executeBakedPlan, packages/runtime/src/runtime/recipe.ts:357-394) ------
  * Between krm_graph_begin and krm_graph_end the op entry points record instead of running

@@ -80,6 +80,94 @@ __global__ void krm_probe_read_kernel(const uint4* __restrict__ src, size_t piec
   if (fold == 0x9E3779B9u && sink) sink[0] = fold;
 }
 
+// What one all-to-all hand-over of a vector between the workgroups of ONE launch costs — the
+// step a persistent decode kernel would pay where today's decode step ends one kernel and
+// starts the next.  Every workgroup owns n / grid entries of the vector.  Phase p: wave 0 polls
+// the producers' flags (agent-scope 16-byte loads, four flags a lane) until all have reached p,
+// loads the vector (agent-scope 16-byte loads, all in flight) into LDS, barrier; the other
+// waves compute this workgroup's entries from LDS (a few adds: stand-in work), barrier; wave 0
+// stores the entries with agent-scope stores, waits for their acknowledgement and stores its
+// flag p + 1.  Vectors are double-buffered by phase parity.  Every wait is bounded: a poll that
+// exceeds `spin_limit` rounds raises the fault word and the workgroup leaves.
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+__device__ inline void probe_load_agent_b128(u32x4_t& v, const void* p) {
+  asm volatile("global_load_dwordx4 %0, %1, off sc1" : "=v"(v) : "v"(p) : "memory");
+}
+__device__ inline void probe_wait_loads(u32x4_t& a) {
+  asm volatile("s_waitcnt vmcnt(0)" : "+v"(a)::"memory");  // ties the register to the wait
+}
+
+template <int N>
+__global__ __launch_bounds__(576) void krm_probe_exchange_kernel(float* vec, uint32_t* flags,
+                                                                 uint32_t* fault, uint32_t phases,
+                                                                 uint32_t spin_limit) {
+  __shared__ __attribute__((aligned(16))) float s_x[N];
+  __shared__ float s_out[64];
+  __shared__ int s_ok;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const uint32_t nwg = gridDim.x;
+  const uint32_t per_wg = N / nwg;
+  constexpr int kPieces = N / 4, kPerLane = (kPieces + 63) / 64;
+  if (threadIdx.x == 0) s_ok = 1;
+  __syncthreads();
+  for (uint32_t p = 0; p < phases; ++p) {
+    float* cur = vec + (size_t)(p & 1) * N;
+    float* nxt = vec + (size_t)((p + 1) & 1) * N;
+    if (wave == 0) {
+      bool ok = true;
+      if (p > 0) {
+        uint32_t spins = 0;
+        while (true) {
+          u32x4_t f;
+          probe_load_agent_b128(f, flags + ((uint32_t)lane * 4 < nwg ? lane * 4 : 0));
+          probe_wait_loads(f);
+          const bool mine = (uint32_t)lane * 4 >= nwg ||
+                            (f.x >= p && f.y >= p && f.z >= p && f.w >= p);
+          if (__all(mine)) break;
+          if (++spins > spin_limit) { ok = false; break; }
+        }
+      }
+      if (!ok && lane == 0) { *fault = 1u; s_ok = 0; }
+      u32x4_t v[kPerLane];
+#pragma unroll
+      for (int j = 0; j < kPerLane; ++j) {
+        const int piece = j * 64 + lane;
+        probe_load_agent_b128(v[j], cur + 4 * (piece < kPieces ? piece : 0));
+      }
+#pragma unroll
+      for (int j = 0; j < kPerLane; ++j) probe_wait_loads(v[j]);
+#pragma unroll
+      for (int j = 0; j < kPerLane; ++j) {
+        const int piece = j * 64 + lane;
+        if (piece < kPieces)
+          *reinterpret_cast<float4*>(&s_x[4 * piece]) =
+              p > 0 ? make_float4(__uint_as_float(v[j].x), __uint_as_float(v[j].y),
+                                  __uint_as_float(v[j].z), __uint_as_float(v[j].w))
+                    : make_float4(1.f, 1.f, 1.f, 1.f);
+      }
+    }
+    __syncthreads();
+    if (!s_ok) break;
+    if (wave > 0) {
+      const uint32_t t = threadIdx.x - 64;
+      if (t < per_wg) {
+        float sum = 0.f;
+        for (int j = 0; j < 8; ++j) sum += s_x[(t * 37 + j * 101 + blockIdx.x) % N];
+        s_out[t] = sum * 0.125f;
+      }
+    }
+    __syncthreads();
+    if (wave == 0) {
+      if ((uint32_t)lane < per_wg)
+        __hip_atomic_store(&nxt[blockIdx.x * per_wg + lane], s_out[lane], __ATOMIC_RELAXED,
+                           __HIP_MEMORY_SCOPE_AGENT);
+      __builtin_amdgcn_s_waitcnt(0);  // the stores are acknowledged
+      if (lane == 0)
+        __hip_atomic_store(&flags[blockIdx.x], p + 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+  }
+}
+
 extern "C" {
 
 const char* krm_version(void) { return "karume-hip 0.1 gfx950"; }
@@ -372,6 +460,32 @@ int32_t krm_probe_launch(krm_ctx* ctx, int32_t kind, krm_buf src, size_t bytes, 
   else
     krm_probe_read_kernel<8><<<dim3(grid), dim3(block), 0, ctx->stream>>>(ptr<const uint4>(src), pieces, sink);
   return launched(ctx, "krm_probe_read_kernel");
+}
+
+int32_t krm_probe_exchange(krm_ctx* ctx, krm_buf work, size_t work_bytes, uint32_t entries,
+                           uint32_t phases, uint32_t spin_limit) {
+  KRM_TRY(enter(ctx));
+  KRM_REQUIRE(ctx, entries == 2048 || entries == 4096 || entries == 8192,
+              "krm_probe_exchange: entries %u (2048, 4096 or 8192)", entries);
+  KRM_REQUIRE(ctx, phases >= 1 && spin_limit >= 1, "krm_probe_exchange: phases / spin_limit");
+  // one workgroup per CU, all resident: 256 of them (a multiple of 4 that divides `entries`)
+  const uint32_t grid = 256;
+  KRM_REQUIRE(ctx, (uint32_t)ctx->num_cus >= grid,
+              "krm_probe_exchange: %d CUs cannot hold %u resident workgroups", ctx->num_cus, grid);
+  const size_t need = (size_t)2 * entries * sizeof(float) + (size_t)grid * 4 + 16;
+  KRM_REQUIRE(ctx, work && work % 16 == 0 && work_bytes >= need,
+              "krm_probe_exchange: work buffer of %zu bytes, %zu needed", work_bytes, need);
+  KRM_TRY(krm_buf_zero(ctx, work, 0, need));
+  float* vec = ptr<float>(work);
+  uint32_t* flags = reinterpret_cast<uint32_t*>(vec + 2 * (size_t)entries);
+  uint32_t* fault = flags + grid;
+  if (entries == 2048)
+    krm_probe_exchange_kernel<2048><<<dim3(grid), dim3(576), 0, ctx->stream>>>(vec, flags, fault, phases, spin_limit);
+  else if (entries == 4096)
+    krm_probe_exchange_kernel<4096><<<dim3(grid), dim3(576), 0, ctx->stream>>>(vec, flags, fault, phases, spin_limit);
+  else
+    krm_probe_exchange_kernel<8192><<<dim3(grid), dim3(576), 0, ctx->stream>>>(vec, flags, fault, phases, spin_limit);
+  return launched(ctx, "krm_probe_exchange_kernel");
 }
 
 int32_t krm_event_create(krm_ctx* ctx, krm_event** out) {

@@ -250,6 +250,12 @@ class GpuContext:
         self._check(self._lib.krm_probe_launch(self._handle, kind, _addr(src), nbytes, grid,
                                                block))
 
+    def probe_exchange(self, work: DeviceBuffer, entries: int, phases: int,
+                       spin_limit: int = 1 << 16) -> None:
+        """`phases` all-to-all hand-overs of a vector between the workgroups of one launch."""
+        self._check(self._lib.krm_probe_exchange(self._handle, _addr(work), work.nbytes, entries,
+                                                 phases, spin_limit))
+
     def borrow(self, address: int, nbytes: int) -> DeviceBuffer:
         """Wrap device memory owned by someone else (for example a torch tensor's data_ptr)."""
         return DeviceBuffer(self, address, nbytes, owned=False)

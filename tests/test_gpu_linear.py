@@ -307,3 +307,23 @@ def test_linear_from_a_model_file(gpu_ctx):
     got = run_linear(gpu_ctx, x, weight.packed, weight.scales, bias, n, k, g)
     ok, fails, max_abs, worst = oracle.allclose(got, want, atol=1e-5, rtol=1e-3)
     assert ok, (fails, max_abs, worst)
+
+
+def test_probe_exchange_is_bounded_and_clean(gpu_ctx):
+    """The in-kernel hand-over probe: with a generous spin limit every poll succeeds (fault 0);
+    with a limit of one round some poll gives up, the fault word is raised or not, and the launch
+    ends either way — no wait in it is unbounded."""
+    entries = 2048
+    work = gpu_ctx.alloc(2 * entries * 4 + 1040)
+    gpu_ctx.probe_exchange(work, entries, 200)
+    gpu_ctx.sync()
+    assert work.download(np.uint32, (1,), byte_offset=2 * entries * 4 + 1024)[0] == 0
+    gpu_ctx.probe_exchange(work, entries, 200, spin_limit=1)
+    gpu_ctx.sync()
+    assert work.download(np.uint32, (1,), byte_offset=2 * entries * 4 + 1024)[0] in (0, 1)
+    gpu_ctx.probe_exchange(work, entries, 50)     # clean again after a faulted run
+    gpu_ctx.sync()
+    assert work.download(np.uint32, (1,), byte_offset=2 * entries * 4 + 1024)[0] == 0
+    with pytest.raises(ka.GpuValidationError):
+        gpu_ctx.probe_exchange(work, 1000, 10)
+    work.free()
