@@ -307,10 +307,13 @@ def bench_ragged(timer: Timer, rng, steps: int, warmup: int):
 
 
 def bench_gemm(timer: Timer, rng, steps: int, warmup: int, m: int, n: int, k: int, g: int,
-               compute=None):
-    """benchmark config 1: prefill GEMM on the matrix cores, fp16 activations and output."""
+               f32_class: bool = False):
+    """benchmark config 1: prefill GEMM on the matrix cores.  Default: fp16 activations and
+    output, KRM_COMPUTE_F16.  `f32_class`: f32 activations and output with KRM_COMPUTE_F32 (the
+    reference's default linearCompute): activations split into fp16 hi + lo, two MFMAs a step."""
     ctx, ka = timer.ctx, timer.ka
-    compute = ka.COMPUTE_F16 if compute is None else compute
+    compute = ka.COMPUTE_F32 if f32_class else ka.COMPUTE_F16
+    io, io_np, eb = (ka.F32, np.float32, 4) if f32_class else (ka.F16, np.float16, 2)
     copies = 4
     weights, scales = [], []
     for _ in range(copies):
@@ -318,12 +321,12 @@ def bench_gemm(timer: Timer, rng, steps: int, warmup: int, m: int, n: int, k: in
         scales.append(ctx.upload(np.maximum(
             np.abs(rng.normal(0, 0.02, size=(n, k // g))).astype(np.float16),
             np.float16(6.104e-05))))
-    x = ctx.upload(rng.normal(size=(m, k)).astype(np.float16))
-    out = ctx.alloc(m * n * 2)
+    x = ctx.upload(rng.normal(size=(m, k)).astype(io_np))
+    out = ctx.alloc(m * n * eb)
 
     def step(i: int) -> None:
         j = i % copies
-        ctx.linear_i4(x, weights[j], scales[j], None, out, m, n, k, g, ka.F16, ka.F16, compute)
+        ctx.linear_i4(x, weights[j], scales[j], None, out, m, n, k, g, io, ka.F16, compute)
 
     res = timer.run(step, steps, warmup, replays=20)
     for b in weights + scales + [x, out]:
@@ -623,7 +626,7 @@ def main() -> int:
             result[f"gemm_{name}_us"] = round(ms_g * 1e3, 2)
             result[f"gemm_{name}_pct_of_f16_mfma_peak"] = round(
                 100 * flops / (ms_g * 1e-3) / 2.5e15, 2)
-            ms_g, flops = bench_gemm(timer, rng, 20, 40, 512, gn, gk, g, compute=ka.COMPUTE_F32)
+            ms_g, flops = bench_gemm(timer, rng, 50, 100, 512, gn, gk, g, f32_class=True)
             result[f"gemm_{name}_f32class_us"] = round(ms_g * 1e3, 2)
             result[f"gemm_{name}_f32class_tflops"] = round(flops / (ms_g * 1e-3) / 1e12, 1)
     if args.only in ("", "w4a8"):

@@ -49,15 +49,22 @@ typedef struct krm_event krm_event;
 #define KRM_F16 1
 
 /* `linear` arithmetic, the reference's SessionOptions.linearCompute
- * (packages/runtime/src/runtime/session-types.ts:127-195):
- *   KRM_COMPUTE_F32  — f32 products and f32 accumulation for every M (the reference default);
- *   KRM_COMPUTE_F16  — rows M > 16 go to the fp16 MFMA GEMM: x rounded to fp16, every weight
- *                      rounded once to fp16((u - 8) * scale), fp16 x fp16 products accumulated
- *                      in f32.  The per-weight rounding bounds the error of an output by about
- *                      2^-11 * sqrt(k) * rms(x * w) (the reference rejects f16 compute with i4
- *                      weights, packages/runtime/src/kernels/gemm.ts:1204-1209, so this form
- *                      has no same-numerics counterpart there).
- * M <= 16 always runs the bandwidth-bound GEMV with f32 accumulation. */
+ * (packages/runtime/src/runtime/session-types.ts:127-195).  M <= 16 always runs the
+ * bandwidth-bound GEMV (exact products, f32 accumulation).  For M > 16:
+ *   KRM_COMPUTE_F32  — f32-class results for every M (the reference default).  f32 activations
+ *                      on large shapes run on the matrix cores: x * 2^e = hi + lo (two fp16,
+ *                      22 bits, e per row), weights as the exact integers (u - 8), products
+ *                      exact, f32 sums, the group scale applied to the f32 sum of each group;
+ *                      gated at the GEMV's tolerance.  fp16 activations need no split.  Other
+ *                      shapes take the GEMV over blocks of 16 rows.
+ *   KRM_COMPUTE_F16  — f32 activations are rounded to fp16 once.  Large shapes (the (tile,
+ *                      stage) units of 64 x 512 tiles cover every CU at least twice, group >= 64,
+ *                      k % 32 == 0): exact integer weights as above, so with fp16 activations
+ *                      the result is of f32 class.  Smaller shapes: every weight rounded once
+ *                      to fp16((u - 8) * scale), which bounds an output's error by about
+ *                      2^-11 * sqrt(k) * rms(x * w).  (The reference rejects f16 compute with
+ *                      i4 weights, packages/runtime/src/kernels/gemm.ts:1204-1209: no
+ *                      same-numerics counterpart there.) */
 #define KRM_COMPUTE_F32 0
 #define KRM_COMPUTE_F16 1
 

@@ -52,6 +52,14 @@ __device__ inline uint32_t scale_bits<float>(const float* s, size_t i) {
   return reinterpret_cast<const uint32_t*>(s)[i];
 }
 template <typename ST>
+__device__ inline float load_scale_f32(const ST* s, size_t i);
+template <>
+__device__ inline float load_scale_f32<__half>(const __half* s, size_t i) {
+  return __half2float(s[i]);
+}
+template <>
+__device__ inline float load_scale_f32<float>(const float* s, size_t i) { return s[i]; }
+template <typename ST>
 __device__ inline _Float16 scale_from_bits(uint32_t bits);
 template <>
 __device__ inline _Float16 scale_from_bits<__half>(uint32_t bits) {
@@ -899,6 +907,380 @@ void gemm_i4_f16_dealt_kernel(const XT* __restrict__ x, const uint8_t* __restric
   }
 }
 
+// ------------------------------------------------ exact integer operands, 64 x 512 tiles
+//
+// The weights enter the matrix cores as the exact integers (u - 8) in fp16 and the group scale
+// multiplies the f32 sum of a group afterwards — the arithmetic of the GEMV, on MFMA.  Two
+// activation forms:
+//   kOperandF16  x is rounded to fp16 once (exact when it already is fp16): one MFMA a step;
+//   kOperandSplit  f32 x is split as x * 2^e = hi + lo, both fp16, |x * 2^e - (hi + lo)| <=
+//                2^-23 |x * 2^e| (e per row, chosen so that the row's largest magnitude lands in
+//                [2^13, 2^14): no overflow, and small entries keep an absolute resolution of
+//                2^-38 of the row's maximum): two MFMAs a step, products exact, f32 sums —
+//                the class of the reference's default f32 `linear`, on the matrix cores.
+// Tile 64 x 512, eight waves side by side (wave = 64 rows x 64 columns = 2 x 2 MFMA tiles), so
+// every weight word is turned into integers exactly once per workgroup (in the 128 x 256 tile
+// above the two waves of a column strip each do it).  Per MFMA step the wave holds the sums of
+// the current scale group in `acc`; at a group's end total = fma(acc, scale[column], total)
+// (the C layout keeps the column in lane % 32, so the scale is one value per lane and column
+// tile).  Stages, LDS layout, the (tile, stage) deal over the CUs and the ordered merge of the
+// partials are those of the kernel above.
+constexpr int kOperandF16 = 0, kOperandSplit = 1;
+
+// 8 codes of a word -> 8 fp16 integers (u - 8), order (c0,c4,c1,c5,c2,c6,c3,c7).
+__device__ inline uint4 ints_word(uint32_t word) {
+  const uint32_t magic = 0x64006400u;  // (1024, 1024)
+  const half2_t off_lo = {(_Float16)1032.0f, (_Float16)1032.0f};
+  const half2_t sixteenth = {(_Float16)0.0625f, (_Float16)0.0625f};
+  const half2_t off_hi = {(_Float16)-72.0f, (_Float16)-72.0f};
+  const uint32_t upper = word >> 8;
+  const half2_t q0 = __builtin_bit_cast(half2_t, and_or(word, 0x000F000Fu, magic)) - off_lo;
+  const half2_t q1 = __builtin_elementwise_fma(
+      __builtin_bit_cast(half2_t, and_or(word, 0x00F000F0u, magic)), sixteenth, off_hi);
+  const half2_t q2 = __builtin_bit_cast(half2_t, and_or(upper, 0x000F000Fu, magic)) - off_lo;
+  const half2_t q3 = __builtin_elementwise_fma(
+      __builtin_bit_cast(half2_t, and_or(upper, 0x00F000F0u, magic)), sixteenth, off_hi);
+  return make_uint4(__builtin_bit_cast(uint32_t, q0), __builtin_bit_cast(uint32_t, q1),
+                    __builtin_bit_cast(uint32_t, q2), __builtin_bit_cast(uint32_t, q3));
+}
+
+// x * scale = hi + lo for eight f32 activations, both halves in the paired order.
+__device__ inline void split_paired(const uint4& a, const uint4& b, float scale, uint4& hi,
+                                    uint4& lo) {
+  const float v[8] = {__uint_as_float(a.x), __uint_as_float(a.y), __uint_as_float(a.z),
+                      __uint_as_float(a.w), __uint_as_float(b.x), __uint_as_float(b.y),
+                      __uint_as_float(b.z), __uint_as_float(b.w)};
+  _Float16 h[8], l[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const float xs = v[i] * scale;             // exact: a power of two
+    h[i] = (_Float16)xs;                       // round to nearest even
+    l[i] = (_Float16)(xs - (float)h[i]);       // the difference is exact in f32
+  }
+  auto pack = [](_Float16 p, _Float16 q) {
+    const half2_t t = {p, q};
+    return __builtin_bit_cast(uint32_t, t);
+  };
+  hi = make_uint4(pack(h[0], h[4]), pack(h[1], h[5]), pack(h[2], h[6]), pack(h[3], h[7]));
+  lo = make_uint4(pack(l[0], l[4]), pack(l[1], l[5]), pack(l[2], l[6]), pack(l[3], l[7]));
+}
+
+// Row scales of the split form: scale[2r] = 2^e with max|x[r, :]| * 2^e in [2^13, 2^14),
+// scale[2r + 1] = 2^-e.  A row of zeros (or whose maximum is not finite) gets 1 / 1: what is
+// not finite stays so through the product.
+__global__ __launch_bounds__(256) void row_scale_kernel(const float* __restrict__ x,
+                                                        float* __restrict__ row_scale, uint32_t k) {
+  __shared__ uint32_t s_max[4];
+  const float* row = x + (size_t)blockIdx.x * k;
+  uint32_t top = 0;  // largest |x| as raw bits (monotonic for non-negative floats; NaN on top)
+  const uint32_t pieces = k >> 2;
+  for (uint32_t i = threadIdx.x; i < pieces; i += 256) {
+    const uint4 v = reinterpret_cast<const uint4*>(row)[i];
+    top = max(max(top, v.x & 0x7fffffffu), max(v.y & 0x7fffffffu, max(v.z & 0x7fffffffu, v.w & 0x7fffffffu)));
+  }
+  for (uint32_t i = (pieces << 2) + threadIdx.x; i < k; i += 256)
+    top = max(top, __float_as_uint(row[i]) & 0x7fffffffu);
+  for (int off = 32; off > 0; off >>= 1) top = max(top, (uint32_t)__shfl_xor((int)top, off, kWave));
+  if ((threadIdx.x & 63) == 0) s_max[threadIdx.x >> 6] = top;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    top = max(max(s_max[0], s_max[1]), max(s_max[2], s_max[3]));
+    const uint32_t biased = top >> 23;  // exponent of the maximum
+    uint32_t up = 127u, down = 127u;    // 2^0
+    if (top != 0 && biased != 255u) {
+      // e = 13 - (biased - 127), kept inside the normal range of both 2^e and 2^-e
+      int e = 13 - ((int)biased - 127);
+      e = e > 126 ? 126 : (e < -126 ? -126 : e);
+      up = (uint32_t)(127 + e);
+      down = (uint32_t)(127 - e);
+    }
+    row_scale[2 * (size_t)blockIdx.x] = __uint_as_float(up << 23);
+    row_scale[2 * (size_t)blockIdx.x + 1] = __uint_as_float(down << 23);
+  }
+}
+
+template <typename XT, typename ST, int OPERAND>
+__global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2)))
+void gemm_i4_exact_kernel(const XT* __restrict__ x, const uint8_t* __restrict__ w,
+                          const ST* __restrict__ scales, const XT* __restrict__ bias,
+                          XT* __restrict__ out, uint32_t m, uint32_t n, uint32_t k,
+                          uint32_t group_shift, uint32_t m_blocks, UnitDeal deal,
+                          const float* __restrict__ row_scale) {
+  constexpr int MT = 2, WN = 2, T = 512;
+  constexpr int BM = 64, BN = 512;
+  constexpr int NA = OPERAND == kOperandSplit ? 2 : 1;  // copies of the x tile (hi, lo)
+  constexpr int kStage = 128;
+  constexpr int kRowA = kStage * 2 + 16;
+  constexpr int kRowB = kStage / 2 + 16;
+  constexpr int kAUnits = BM * (kStage / 8) / T;   // 2
+  constexpr int kBUnits = BN * (kStage / 32) / T;  // 4
+  static_assert((size_t)BM * BN == kPartialFloats, "the partial slots hold one tile");
+  static_assert(OPERAND == kOperandF16 || sizeof(XT) == 4, "only f32 activations are split");
+  __shared__ __align__(16) uint8_t s_a[2][NA][BM * kRowA];
+  __shared__ __align__(16) uint8_t s_b[2][BN * kRowB];
+  __shared__ float s_s[2][BN][2];
+  __shared__ float s_inv[BM];
+  __shared__ uint32_t s_ticket;
+
+  const int tid = threadIdx.x, lane = tid & 63, wn = tid >> 6;
+  const int frag_row = lane & 31, frag_h = lane >> 5;
+  const uint32_t groups = k >> group_shift;
+  const bool half_stage_groups = group_shift == 6;  // 64 codes a group: two groups a stage
+  const uint32_t spt = deal.stages_per_tile;
+  const uint32_t arow0 = tid >> 4, aunit = (tid & 15u) * 8u;
+  const uint32_t brow0 = tid >> 2, bunit = (tid & 3u) * 16u;
+  const uint32_t a_base = (uint32_t)(frag_row * kRowA + 64 * frag_h);
+  const uint32_t b_base = (uint32_t)((wn * 64 + frag_row) * kRowB + 16 * frag_h);
+
+  uint32_t v = blockIdx.x;
+  if ((gridDim.x & 7u) == 0) v = (blockIdx.x & 7u) * (gridDim.x >> 3) + (blockIdx.x >> 3);
+  const uint32_t my_begin = deal_begin(deal, v);
+  uint32_t left = deal.units_lo + (v < deal.extra ? 1u : 0u);
+
+  while (left > 0) {
+    const uint32_t range_end = my_begin + left;
+    const uint32_t tile = (range_end - 1u) / spt;
+    const uint32_t tile_first = tile * spt;
+    const uint32_t s0 = my_begin > tile_first ? my_begin - tile_first : 0u;
+    const uint32_t s1 = range_end - tile_first;
+    const uint32_t nb = tile / m_blocks, mb = tile - nb * m_blocks;
+    const uint32_t m0 = mb * BM, n0 = nb * BN;
+    const ST* ssrc = scales + (size_t)min(n0 + (uint32_t)tid, n - 1) * groups;
+
+    float rs[kAUnits];  // 2^e of the rows this thread stages
+#pragma unroll
+    for (int i = 0; i < kAUnits; ++i) rs[i] = 1.0f;
+    if constexpr (OPERAND == kOperandSplit) {
+#pragma unroll
+      for (int i = 0; i < kAUnits; ++i)
+        rs[i] = row_scale[2 * (size_t)min(m0 + arow0 + 32u * i, m - 1)];
+      if (tid < BM) s_inv[tid] = row_scale[2 * (size_t)min(m0 + (uint32_t)tid, m - 1) + 1];
+    }
+
+    struct Staged {
+      Acts8<XT> a[kAUnits];
+      uint4 b[kBUnits];
+    };
+    auto load_stage = [&](uint32_t stage, Staged& d) {
+      const uint32_t a_at = stage * kStage + aunit, b_at = stage * (kStage / 2) + bunit;
+      const uint32_t a_off = a_at < k ? a_at : 0u, b_off = b_at < (k >> 1) ? b_at : 0u;
+#pragma unroll
+      for (int i = 0; i < kAUnits; ++i)
+        d.a[i].load(x + (size_t)min(m0 + arow0 + 32u * i, m - 1) * k + a_off);
+#pragma unroll
+      for (int i = 0; i < kBUnits; ++i)
+        d.b[i] = *reinterpret_cast<const uint4*>(
+            w + (size_t)min(n0 + brow0 + 128u * i, n - 1) * (k >> 1) + b_off);
+    };
+    auto park_stage = [&](uint32_t stage, int buf, Staged& d) {
+      const uint32_t keep = stage * kStage + aunit < k ? 0xFFFFFFFFu : 0u;
+#pragma unroll
+      for (int i = 0; i < kAUnits; ++i) {
+        const uint32_t at = (arow0 + 32u * i) * kRowA + aunit * 2u;
+        if constexpr (OPERAND == kOperandSplit) {
+          uint4 hi, lo;
+          split_paired(d.a[i].a, d.a[i].b, rs[i], hi, lo);
+          hi.x &= keep; hi.y &= keep; hi.z &= keep; hi.w &= keep;  // past K: zeros
+          lo.x &= keep; lo.y &= keep; lo.z &= keep; lo.w &= keep;
+          *reinterpret_cast<uint4*>(&s_a[buf][0][at]) = hi;
+          *reinterpret_cast<uint4*>(&s_a[buf][NA - 1][at]) = lo;
+        } else {
+          uint4 pv = d.a[i].paired();
+          pv.x &= keep; pv.y &= keep; pv.z &= keep; pv.w &= keep;
+          *reinterpret_cast<uint4*>(&s_a[buf][0][at]) = pv;
+        }
+      }
+#pragma unroll
+      for (int i = 0; i < kBUnits; ++i)
+        *reinterpret_cast<uint4*>(&s_b[buf][(brow0 + 128u * i) * kRowB + bunit]) = d.b[i];
+      const uint32_t c0 = stage * kStage, c1 = stage * kStage + 64u;
+      s_s[buf][tid][0] = load_scale_f32<ST>(ssrc, (c0 < k ? c0 : 0u) >> group_shift);
+      s_s[buf][tid][1] = load_scale_f32<ST>(ssrc, (c1 < k ? c1 : 0u) >> group_shift);
+    };
+
+    float16_t total[MT][WN], acc[MT][WN];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+      for (int nt = 0; nt < WN; ++nt)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) total[mt][nt][r] = acc[mt][nt][r] = 0.f;
+
+    Staged staged;
+    load_stage(s0, staged);
+    park_stage(s0, 0, staged);
+    __syncthreads();
+
+    auto run_stage = [&](uint32_t stage, int buf) {
+      load_stage(stage + 1, staged);
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int c = 0; c < 2; ++c) {
+        uint4 braw[WN];
+        float ws[WN];
+#pragma unroll
+        for (int nt = 0; nt < WN; ++nt) {
+          braw[nt] = *reinterpret_cast<const uint4*>(&s_b[buf][b_base + nt * 32 * kRowB + 32 * c]);
+          ws[nt] = s_s[buf][wn * 64 + nt * 32 + frag_row][c];
+        }
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          half8_t a[NA][MT];
+#pragma unroll
+          for (int copy = 0; copy < NA; ++copy)
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt)
+              a[copy][mt] = *reinterpret_cast<const half8_t*>(
+                  &s_a[buf][copy][a_base + mt * 32 * kRowA + 128 * c + 16 * j]);
+#pragma unroll
+          for (int nt = 0; nt < WN; ++nt) {
+            const uint32_t word = j == 0 ? braw[nt].x : j == 1 ? braw[nt].y : j == 2 ? braw[nt].z
+                                                                                    : braw[nt].w;
+            const half8_t b = __builtin_bit_cast(half8_t, ints_word(word));
+            __builtin_amdgcn_s_setprio(1);
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) {
+#pragma unroll
+              for (int copy = 0; copy < NA; ++copy)
+                acc[mt][nt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[copy][mt], b, acc[mt][nt], 0, 0, 0);
+            }
+            __builtin_amdgcn_s_setprio(0);
+          }
+        }
+        if (c == 1 || half_stage_groups) {  // the scale group ends here
+#pragma unroll
+          for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+            for (int nt = 0; nt < WN; ++nt)
+#pragma unroll
+              for (int r = 0; r < 16; ++r) {
+                total[mt][nt][r] = fmaf(acc[mt][nt][r], ws[nt], total[mt][nt][r]);
+                acc[mt][nt][r] = 0.f;
+              }
+        }
+      }
+      park_stage(stage + 1, buf ^ 1, staged);
+      __syncthreads();
+    };
+    for (uint32_t stage = s0; stage < s1; stage += 2) {
+      run_stage(stage, 0);
+      if (stage + 1 < s1) run_stage(stage + 1, 1);
+    }
+
+    auto store_block = [&](int mt, int nt, const float16_t& sum) {
+      const uint32_t col = n0 + wn * 64 + nt * 32 + frag_row;
+      const float b = (bias && col < n) ? bias_f32<XT>(bias, col) : 0.f;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const uint32_t local = mt * 32 + 8 * (r / 4) + 4 * frag_h + (r % 4);
+        const uint32_t row = m0 + local;
+        float value = sum[r];
+        if constexpr (OPERAND == kOperandSplit) value *= s_inv[local];  // exact: a power of two
+        if (row < m && col < n) store_out<XT>(out, (size_t)row * n + col, value + b);
+      }
+    };
+
+    if (s0 == 0 && s1 == spt) {
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+        for (int nt = 0; nt < WN; ++nt) store_block(mt, nt, total[mt][nt]);
+    } else {
+      const uint32_t tile_begin = tile * spt;
+      auto slot_of = [&](uint32_t u) {
+        return 2u * u + (deal_begin(deal, u) <= tile_begin ? 1u : 0u);
+      };
+      uint32_t* ticket = deal.tickets + (size_t)tile * kTicketStride;
+      const uint32_t first = deal_owner(deal, tile_begin), last = deal_owner(deal, tile_begin + spt - 1u);
+      if (tid == 0)
+        s_ticket = __hip_atomic_load(ticket, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      __syncthreads();
+      bool merge = s_ticket == last - first;
+      __syncthreads();
+      if (!merge) {
+        float4_t* mine =
+            reinterpret_cast<float4_t*>(deal.partials + (size_t)slot_of(v) * kPartialFloats);
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+          for (int nt = 0; nt < WN; ++nt)
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+              const float4_t piece = {total[mt][nt][4 * q], total[mt][nt][4 * q + 1],
+                                      total[mt][nt][4 * q + 2], total[mt][nt][4 * q + 3]};
+              publish4(mine + (size_t)(((mt * WN + nt) * 4 + q) * T + tid), piece);
+            }
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();
+        if (tid == 0)
+          s_ticket = __hip_atomic_fetch_add(ticket, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __syncthreads();
+        merge = s_ticket == last - first;
+      }
+      if (merge) {
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+          float16_t sum[WN];
+          for (uint32_t u = first; u <= last; ++u) {
+            float16_t part[WN];
+#pragma unroll
+            for (int nt = 0; nt < WN; ++nt) part[nt] = total[mt][nt];
+            if (u != v) {
+              const float4_t* src =
+                  reinterpret_cast<const float4_t*>(deal.partials + (size_t)slot_of(u) * kPartialFloats) +
+                  (size_t)(mt * WN * 4 * T + tid);
+              float4_t p[8];
+#pragma unroll
+              for (int i = 0; i < 8; ++i) p[i] = observe4(src + (size_t)i * T);
+              landed(p);
+#pragma unroll
+              for (int nt = 0; nt < WN; ++nt)
+#pragma unroll
+                for (int q = 0; q < 4; ++q)
+#pragma unroll
+                  for (int i = 0; i < 4; ++i) part[nt][4 * q + i] = p[nt * 4 + q][i];
+            }
+#pragma unroll
+            for (int nt = 0; nt < WN; ++nt) {
+              if (u == first) {
+                sum[nt] = part[nt];
+              } else {
+#pragma unroll
+                for (int r = 0; r < 16; ++r) sum[nt][r] += part[nt][r];
+              }
+            }
+          }
+#pragma unroll
+          for (int nt = 0; nt < WN; ++nt) store_block(mt, nt, sum[nt]);
+        }
+        if (tid == 0)
+          __hip_atomic_store(ticket, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      }
+    }
+    __syncthreads();  // s_inv and the LDS tiles are rewritten by the next tile of the range
+    left -= s1 - s0;
+  }
+}
+
+// The deal of the 64 x 512 tiles: one workgroup per CU, every workgroup at least two stages.
+bool plan_exact_deal(krm_ctx* ctx, uint32_t m, uint32_t n, uint32_t k, uint32_t& grid,
+                     UnitDeal& deal) {
+  const uint64_t cus = (uint64_t)ctx->num_cus;
+  const uint64_t tiles = (uint64_t)((m + 63) / 64) * ((n + 511) / 512);
+  const uint32_t spt = (k + 127) / 128;
+  const uint64_t units = tiles * spt;
+  if (tiles > kTicketSlots || units > 0x7fffffffull || units < 2 * cus) return false;
+  if (tiles * 8 < cus) return false;  // a tile shared by more than eight workgroups
+  if (!ctx->gemm_partials) return false;
+  grid = (uint32_t)cus;
+  deal.stages_per_tile = spt;
+  deal.units_lo = (uint32_t)(units / cus);
+  deal.extra = (uint32_t)(units % cus);
+  deal.partials = ctx->gemm_partials;
+  deal.tickets = ctx->tickets;
+  return true;
+}
+
 // Workgroups, units and scratch of a dealt launch; false when the shape is not worth it.
 bool plan_deal(krm_ctx* ctx, uint32_t m, uint32_t n, uint32_t k, uint32_t& grid, UnitDeal& deal) {
   const uint64_t cus = (uint64_t)ctx->num_cus;
@@ -1017,9 +1399,54 @@ int32_t pick_tile(krm_ctx* ctx, krm_buf x, krm_buf w, krm_buf scales, krm_buf bi
   return launch<XT, ST, 1, 1, 64, 1, 1>(ctx, x, w, scales, bias, out, m, n, k, group_shift);
 }
 
+template <typename XT, typename ST, int OPERAND>
+int32_t launch_exact(krm_ctx* ctx, krm_buf x, krm_buf w, krm_buf scales, krm_buf bias, krm_buf out,
+                     uint32_t m, uint32_t n, uint32_t k, uint32_t group_shift, uint32_t grid,
+                     const UnitDeal& deal) {
+  if constexpr (OPERAND == kOperandSplit) {
+    row_scale_kernel<<<dim3(m), dim3(256), 0, ctx->stream>>>(ptr<const float>(x), ctx->row_scales, k);
+    KRM_TRY(launched(ctx, "row_scale_kernel"));
+  }
+  gemm_i4_exact_kernel<XT, ST, OPERAND><<<dim3(grid), dim3(512), 0, ctx->stream>>>(
+      ptr<const XT>(x), ptr<const uint8_t>(w), ptr<const ST>(scales), ptr<const XT>(bias),
+      ptr<XT>(out), m, n, k, group_shift, (m + 63) / 64, deal, ctx->row_scales);
+  return launched(ctx, "gemm_i4_exact_kernel");
+}
+
 }  // namespace
 
 namespace krm {
+
+// The exact-integer-operand GEMM for shapes whose (tile, stage) units cover the chip; sets
+// *handled = false (and launches nothing) for every other shape.
+int32_t linear_i4_gemm_exact(krm_ctx* ctx, krm_buf x, krm_buf w, krm_buf scales, krm_buf bias,
+                             krm_buf out, uint32_t m, uint32_t n, uint32_t k, uint32_t group,
+                             int32_t io_dtype, int32_t scale_dtype, int32_t compute,
+                             bool* handled) {
+  *handled = false;
+  const bool split = compute == KRM_COMPUTE_F32 && io_dtype == KRM_F32;
+  if (group < 64 || k % 32 != 0 || !aligned(w, 16) || !aligned(x, 16)) return KRM_OK;
+  if (split && (m > kMaxSplitRows || !ctx->row_scales)) return KRM_OK;
+  uint32_t grid = 0;
+  UnitDeal deal{};
+  if (!plan_exact_deal(ctx, m, n, k, grid, deal)) return KRM_OK;
+  uint32_t group_shift = 0;
+  while ((1u << group_shift) < group) ++group_shift;
+  *handled = true;
+#define KRM_EXACT(XT, ST, OP) \
+  return launch_exact<XT, ST, OP>(ctx, x, w, scales, bias, out, m, n, k, group_shift, grid, deal)
+  if (io_dtype == KRM_F16) {
+    if (scale_dtype == KRM_F16) KRM_EXACT(__half, __half, kOperandF16);
+    KRM_EXACT(__half, float, kOperandF16);
+  }
+  if (split) {
+    if (scale_dtype == KRM_F16) KRM_EXACT(float, __half, kOperandSplit);
+    KRM_EXACT(float, float, kOperandSplit);
+  }
+  if (scale_dtype == KRM_F16) KRM_EXACT(float, __half, kOperandF16);
+  KRM_EXACT(float, float, kOperandF16);
+#undef KRM_EXACT
+}
 
 int32_t linear_i4_gemm_f16(krm_ctx* ctx, krm_buf x, krm_buf w, krm_buf scales, krm_buf bias,
                            krm_buf out, uint32_t m, uint32_t n, uint32_t k, uint32_t group,

@@ -25,6 +25,9 @@ struct krm_ctx {
   // Scratch of the unit-dealt GEMM: two 128 x 256 f32 partials per CU (64 MiB on 256 CUs),
   // allocated with the context so that launches can be recorded into graphs.
   float* gemm_partials = nullptr;
+  // Per-row scales {2^e, 2^-e} of the f32-class prefill GEMM (kMaxSplitRows rows), written by
+  // a pre-pass of every such launch.
+  float* row_scales = nullptr;
   bool recording = false;  // between krm_graph_begin and krm_graph_end
   // Parallel branches of a recording (krm_graph_branch): `stream` is the stream launches go
   // to, which is `main_stream` except while a side branch is selected.  Side streams are
@@ -55,6 +58,7 @@ constexpr uint32_t kTicketSlots = 1u << 16;
 // decode step, counting on 16 neighbouring words, spent 5.8 us queueing there.
 constexpr uint32_t kTicketStride = 32;
 constexpr size_t kGemmPartialBytes = 128u * 256u * sizeof(float);
+constexpr uint32_t kMaxSplitRows = 1u << 16;
 
 // Records the message on the context (or on the context-less slot) and returns `code`.
 int32_t fail(krm_ctx* ctx, int32_t code, const char* fmt, ...);

@@ -1031,7 +1031,11 @@ int32_t linear_i4_gemv(krm_ctx* ctx, krm_buf x, krm_buf w, krm_buf scales, krm_b
                        GemvFusion{});
 }
 
-// fp16 MFMA GEMM for M > 16 (gemm_i4.hip).
+// MFMA GEMMs for M > 16 (gemm_i4.hip): exact integer weights (large shapes), fp16 weights.
+int32_t linear_i4_gemm_exact(krm_ctx* ctx, krm_buf x, krm_buf w, krm_buf scales, krm_buf bias,
+                             krm_buf out, uint32_t m, uint32_t n, uint32_t k, uint32_t group,
+                             int32_t io_dtype, int32_t scale_dtype, int32_t compute,
+                             bool* handled);
 int32_t linear_i4_gemm_f16(krm_ctx* ctx, krm_buf x, krm_buf w, krm_buf scales, krm_buf bias,
                            krm_buf out, uint32_t m, uint32_t n, uint32_t k, uint32_t group,
                            int32_t io_dtype, int32_t scale_dtype);
@@ -1061,6 +1065,10 @@ int32_t krm_linear_i4(krm_ctx* ctx, krm_buf x, krm_buf w, krm_buf scales, krm_bu
               "krm_linear_i4: x must be 16-byte aligned, w 4-byte aligned");
   if (m <= 16)
     return linear_i4_gemv(ctx, x, w, scales, bias, out, m, n, k, group, io_dtype, scale_dtype);
+  bool handled = false;
+  KRM_TRY(linear_i4_gemm_exact(ctx, x, w, scales, bias, out, m, n, k, group, io_dtype,
+                               scale_dtype, compute, &handled));
+  if (handled) return KRM_OK;
   if (compute == KRM_COMPUTE_F16)
     return linear_i4_gemm_f16(ctx, x, w, scales, bias, out, m, n, k, group, io_dtype,
                               scale_dtype);

@@ -204,8 +204,12 @@ int32_t krm_ctx_create_on_stream(int32_t device, void* hip_stream, krm_ctx** out
   if (st == hipSuccess)
     st = hipMalloc(reinterpret_cast<void**>(&ctx->gemm_partials),
                    (size_t)2 * ctx->num_cus * kGemmPartialBytes);
+  if (st == hipSuccess)
+    st = hipMalloc(reinterpret_cast<void**>(&ctx->row_scales),
+                   (size_t)kMaxSplitRows * 2 * sizeof(float));
   if (st == hipSuccess) st = hipDeviceSynchronize();
   if (st != hipSuccess) {
+    if (ctx->row_scales) (void)hipFree(ctx->row_scales);
     if (ctx->gemm_partials) (void)hipFree(ctx->gemm_partials);
     if (ctx->tickets) (void)hipFree(ctx->tickets);
     (void)hipHostFree(ctx->pinned);
@@ -222,6 +226,7 @@ int32_t krm_ctx_create(int32_t device, krm_ctx** out) {
   // Default priority on purpose: mixed stream priorities are not used anywhere.
   hipError_t st = hipStreamCreateWithFlags(&ctx->stream, hipStreamNonBlocking);
   if (st != hipSuccess) {
+    (void)hipFree(ctx->row_scales);
     (void)hipFree(ctx->gemm_partials);
     (void)hipFree(ctx->tickets);
     (void)hipHostFree(ctx->pinned);
@@ -248,6 +253,7 @@ int32_t krm_ctx_destroy(krm_ctx* ctx) {
   if (ctx->pinned) (void)hipHostFree(ctx->pinned);
   if (ctx->tickets) (void)hipFree(ctx->tickets);
   if (ctx->gemm_partials) (void)hipFree(ctx->gemm_partials);
+  if (ctx->row_scales) (void)hipFree(ctx->row_scales);
   delete ctx;
   return KRM_OK;
 }

@@ -1,13 +1,17 @@
-"""GPU parity of the fp16 MFMA GEMM path of `linear` (M > 16, KRM_COMPUTE_F16) against the CPU
-oracle.
+"""GPU parity of the MFMA GEMM paths of `linear` (M > 16) against the CPU oracle.
 
-Numerics of this path (stated in the kernel): x is rounded to fp16 (exact when it already is),
-each weight is dequantised to fp16 as fp16((u-8) * scale) — one fp16 rounding, relative error
-<= 2^-11 — and products are accumulated in f32.  With K terms of typical size t the error of an
-output behaves like sqrt(K) * t * 2^-11 / sqrt(3); the tests scale their tolerance with the
-RMS of the oracle's output:  |got - want| <= 2e-3 * rms(want) + 1e-3 * |want|  (measured worst
-case about a third of that).  When every scale is a power of two the dequantised weights are
-exact and the gate tightens to f32-accumulation level (atol 3e-5 * rms, measured ~5e-6).
+Two numerics classes (stated in the kernels):
+* exact-operand kernel (large shapes; KRM_COMPUTE_F16, and KRM_COMPUTE_F32 with the f32
+  activations split into fp16 hi + lo): weights enter as exact integers, the group scale
+  multiplies f32 group sums — gated at the GEMV's tolerance (`row_gate`: atol 3e-5 times the
+  row's largest |x|, rtol 1e-5).
+* fp16-weight kernels (smaller shapes under KRM_COMPUTE_F16): x rounded to fp16, each weight
+  dequantised to fp16 as fp16((u-8) * scale) — one fp16 rounding, relative error <= 2^-11 — and
+  products accumulated in f32.  With K terms of typical size t the error of an output behaves
+  like sqrt(K) * t * 2^-11 / sqrt(3); those tests scale their tolerance with the RMS of the
+  oracle's output:  |got - want| <= 2e-3 * rms(want) + 1e-3 * |want|  (measured worst case about
+  a third of that).  When every scale is a power of two the dequantised weights are exact and
+  the gate tightens to f32-accumulation level (atol 3e-5 * rms, measured ~5e-6).
 """
 import numpy as np
 import pytest
@@ -137,3 +141,84 @@ def test_gemm_f32_mode_stays_on_f32_arithmetic(gpu_ctx):
     got = run_linear(gpu_ctx, x, packed, scale, bias, n, k, g, compute=ka.COMPUTE_F32)
     ok, fails, max_abs, worst = oracle.allclose(got, want, atol=3e-5, rtol=1e-5)
     assert ok, (fails, max_abs, worst)
+
+
+def row_gate(x):
+    """Absolute tolerance per output row of the exact-operand forms: the GEMV's gate
+    (atol 3e-5 for activations of unit size, rtol 1e-5) scaled with the row's largest |x|."""
+    top = np.max(np.abs(np.where(np.isfinite(x), x, 0.0)), axis=1, keepdims=True)
+    return 3e-5 * np.maximum(top, 1e-30)
+
+
+@pytest.mark.parametrize("m,n,k,g", [(512, 11008, 4096, 128), (512, 4096, 11008, 128)])
+def test_config1_f32_class_runs_on_the_matrix_cores_within_the_gemv_gate(gpu_ctx, m, n, k, g):
+    """KRM_COMPUTE_F32 with f32 activations at benchmark config 1's shapes: the activations are
+    split into fp16 hi + lo (22 bits, scaled per row), the weights enter as exact integers, the
+    group scale multiplies f32 group sums.  Rows of very different magnitude (1e5, 1e-6, beyond
+    the fp16 range in both directions), a row of zeros and values that are not
+    fp16-representable; 160 sampled columns against the f64 oracle at the GEMV's gate."""
+    rng = np.random.default_rng(n * 3 + k)
+    packed, _q, scale = helpers.synthetic_int4(rng, n, k, g)
+    x = rng.normal(size=(m, k)).astype(np.float32)
+    x[3] *= 1e5
+    x[4] *= 3e7
+    x[5] *= 1e-6
+    x[6] *= 1e-30
+    x[7] = 0.0
+    x[8, ::2] *= 1e-4          # wide dynamic range inside one row
+    bias = rng.normal(size=n).astype(np.float32)
+    got = run_linear(gpu_ctx, x, packed, scale, bias, n, k, g, compute=ka.COMPUTE_F32)
+    cols = np.unique(np.concatenate([[0, 1, 63, 64, 511, 512, n - 513, n - 65, n - 2, n - 1],
+                                     rng.choice(n, size=150, replace=False)]))
+    want = sampled_oracle(x, packed, scale.astype(np.float32), bias, n, k, g, cols)
+    err = np.abs(got[:, cols].astype(np.float64) - want)
+    bound = row_gate(x) + 1e-5 * np.abs(want)
+    assert np.all(err <= bound), float(np.max(err / bound))
+    assert np.all(got[7] == bias)      # the row of zeros: exactly the bias
+
+
+@pytest.mark.parametrize("io", [np.float16, np.float32])
+def test_config1_f16_operands_are_exact_integers_times_fp16_x(gpu_ctx, io):
+    """KRM_COMPUTE_F16 at config 1's up-projection: with fp16-representable activations every
+    product is exact and the group scale multiplies f32 sums, so the result meets the GEMV's
+    gate (the per-weight fp16 rounding of the small-shape kernels is gone here)."""
+    m, n, k, g = 512, 11008, 4096, 128
+    rng = np.random.default_rng(91)
+    packed, _q, scale = helpers.synthetic_int4(rng, n, k, g)
+    x = rng.normal(size=(m, k)).astype(np.float16)
+    bias = rng.normal(size=n).astype(np.float16)
+    got = run_linear(gpu_ctx, x.astype(io), packed, scale, bias.astype(io), n, k, g,
+                     compute=ka.COMPUTE_F16)
+    cols = np.unique(rng.choice(n, size=128, replace=False))
+    want = sampled_oracle(x.astype(np.float32), packed, scale.astype(np.float32),
+                          bias.astype(np.float32), n, k, g, cols)
+    err = np.abs(got[:, cols].astype(np.float64) - want)
+    bound = row_gate(x.astype(np.float32)) + 1e-5 * np.abs(want)
+    if io == np.float16:                # the output rounding: half an fp16 ulp of |want|
+        bound = bound + 2.0 ** -11 * np.abs(want) + 1e-7
+    assert np.all(err <= bound), float(np.max(err / bound))
+
+
+def test_f32_class_gemm_edges_and_non_finite_rows(gpu_ctx):
+    """Ragged M, N and K (K ends inside a 128-code stage, two scale groups a stage), f32 scales,
+    and rows holding Inf / NaN: those rows come out non-finite where the oracle's do, every
+    other row meets the gate."""
+    m, n, k, g = 300, 13349, 2624, 64
+    rng = np.random.default_rng(12)
+    q = rng.integers(-8, 8, size=(n, k), dtype=np.int8)
+    scale = np.abs(rng.normal(0, 0.02, size=(n, k // g))).astype(np.float32) + 1e-4
+    packed = oracle.pack_i4(q)
+    x = rng.normal(size=(m, k)).astype(np.float32)
+    x[11, 5] = np.inf
+    x[12, 2000] = np.nan
+    bias = rng.normal(size=n).astype(np.float32)
+    got = run_linear(gpu_ctx, x, packed, scale, bias, n, k, g, compute=ka.COMPUTE_F32)
+    cols = np.unique(np.concatenate([[0, 511, 512, n - 1], rng.choice(n, size=60, replace=False)]))
+    want = sampled_oracle(x, packed, scale, bias, n, k, g, cols)
+    finite = np.ones(m, dtype=bool)
+    finite[[11, 12]] = False
+    err = np.abs(got[finite][:, cols].astype(np.float64) - want[finite])
+    bound = row_gate(x[finite]) + 1e-5 * np.abs(want[finite])
+    assert np.all(err <= bound), float(np.max(err / bound))
+    assert not np.any(np.isfinite(got[[11, 12]][:, cols]))
+    assert not np.any(np.isfinite(want[[11, 12]]))
