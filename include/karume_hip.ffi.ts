@@ -56,6 +56,13 @@ export const KARUME_HIP_SYMBOLS = {
     ],
     result: "i32",
   },
+  krm_linear_i4_rows: {
+    parameters: [
+      "pointer", "u64", "u64", "u64", "u64", "u64", "u64", "u32", "u32", "u32", "u32", "i32",
+      "i32", "i32", "i32"
+    ],
+    result: "i32",
+  },
   krm_attention_state_workspace: {
     parameters: [
       "u32", "u32", "u32", "u32", "u32", "u32", "u32", "u32", "buffer"
@@ -154,6 +161,13 @@ export const KARUME_HIP_SYMBOLS = {
     parameters: [
       "pointer", "u64", "u64", "u64", "u64", "u64", "u64", "u64", "u32", "u32", "u32", "u32",
       "u32", "u32", "u32", "u64", "i32", "i32"
+    ],
+    result: "i32",
+  },
+  krm_prefill_qkv: {
+    parameters: [
+      "pointer", "u64", "u64", "u64", "u64", "u64", "u64", "u64", "u64", "u64", "u64", "u32",
+      "u32", "u32", "u32", "u32", "u32", "u32", "i32", "i32", "i32"
     ],
     result: "i32",
   },

@@ -188,6 +188,24 @@ int32_t krm_linear_i4_fused(krm_ctx* ctx, krm_buf x, krm_buf norm_weight_f32, fl
                             krm_buf out, uint32_t m, uint32_t n, uint32_t k, uint32_t group,
                             int32_t io_dtype, int32_t scale_dtype, int32_t epilogue);
 
+/* The same op for a chunk of rows (prefill; any m >= 1) with the epilogues of the fused form,
+ * on the matrix cores: weights enter as the exact integers (u - 8), the group scale multiplies
+ * the f32 sum of a group; KRM_COMPUTE_F16 rounds x to fp16 once, KRM_COMPUTE_F32 with f32 x
+ * splits it into fp16 hi + lo (as krm_linear_i4 does for large shapes).
+ *   residual != 0           : out = linear(...) + residual   ([m, n_out], io_dtype; `out` may be
+ *                             the residual buffer itself: an element is read and written by
+ *                             one thread)
+ *   KRM_EPILOGUE_SILU_PAIRS : rows (2i, 2i+1) of w = (gate_i, up_i), out[m, i] = silu(gate) * up,
+ *                             n_out = n / 2; gate and up are not rounded to io_dtype in between
+ * Covers group_size >= 64, k % 32 == 0, 16-byte aligned x and w; anything else is rejected
+ * (krm_linear_i4 + krm_silu_mul + krm_add remain).  A pure function of the shape and dtypes.
+ * Fuses packages/runtime/src/kernels/linear.ts:34-64 with the elementwise add / silu-mul that
+ * follow it in a decoder layer (packages/runtime/src/runtime/fusion.ts). */
+int32_t krm_linear_i4_rows(krm_ctx* ctx, krm_buf x, krm_buf w, krm_buf scales, krm_buf bias,
+                           krm_buf residual, krm_buf out, uint32_t m, uint32_t n, uint32_t k,
+                           uint32_t group, int32_t io_dtype, int32_t scale_dtype, int32_t compute,
+                           int32_t epilogue);
+
 /* ---- states-form attention (Params 10 words + Lengths{past,query} + bindings:
  *      packages/runtime/src/kernels/state-attention.ts:169-180,190-193,284-294,476-487;
  *      builder packages/runtime/src/runtime/recipe-builder.ts:1856-2002;
@@ -384,6 +402,23 @@ int32_t krm_decode_qkv(krm_ctx* ctx, krm_buf x, krm_buf norm_weight_f32, float n
                        uint32_t k, uint32_t group, uint32_t table_rows, uint32_t capacity,
                        uint32_t window, uint32_t past, krm_buf lengths, int32_t io_dtype,
                        int32_t scale_dtype, int32_t kv_dtype);
+/* The attention inputs of a chunk of m rows in one launch: the fused [q; k; v] projection
+ * (weights laid out as for krm_decode_qkv: q and k rows interleaved per head as
+ * (0, D/2, 1, D/2 + 1, ...), v natural; arithmetic of krm_linear_i4_rows), each value rounded
+ * to io_dtype as a separate linear would store it, half-split RoPE of q and k by
+ * positions[row] (roundings of krm_rope_half; a position outside the table gives NaN), and the
+ * head-major layouts the attention reads:
+ *   q_out [H, m, D]   k_out [Hkv, m, D]   v_out [Hkv, m, D]      (io_dtype)
+ * The state appends stay separate calls (after the attention, as docs/ir-v1.md:345-348 orders
+ * them).  Same coverage limits as krm_linear_i4_rows.
+ * Fuses packages/runtime/src/kernels/linear.ts:34-64, packages/runtime/src/kernels/rope.ts:5-20,
+ * 52-80 and the permute nodes of tools/export-recipes/minicpm5/export_decode.py:14-35. */
+int32_t krm_prefill_qkv(krm_ctx* ctx, krm_buf x, krm_buf w, krm_buf scales, krm_buf bias,
+                        krm_buf positions_i32, krm_buf cos_table_f32, krm_buf sin_table_f32,
+                        krm_buf q_out, krm_buf k_out, krm_buf v_out, uint32_t m, uint32_t heads,
+                        uint32_t kv_heads, uint32_t depth, uint32_t k, uint32_t group,
+                        uint32_t table_rows, int32_t io_dtype, int32_t scale_dtype,
+                        int32_t compute);
 /* ---- w4a8: `linear` with int4 weights on integer dot products (the reference's opt-in
  *      SessionOptions.linearCompute "i8a8" with int4-resident weights,
  *      packages/runtime/src/runtime/recipe-builder.ts:1320-1341,1407-1488;

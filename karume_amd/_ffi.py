@@ -48,6 +48,10 @@ PROTOTYPES = {
                             i32, i32]),
     "krm_linear_i4_fused": (i32, [c_ctx, c_buf, c_buf, C.c_float, c_buf, c_buf, c_buf, c_buf,
                                   c_buf, u32, u32, u32, u32, i32, i32, i32]),
+    "krm_linear_i4_rows": (i32, [c_ctx, c_buf, c_buf, c_buf, c_buf, c_buf, c_buf, u32, u32, u32,
+                                 u32, i32, i32, i32, i32]),
+    "krm_prefill_qkv": (i32, [c_ctx, c_buf, c_buf, c_buf, c_buf, c_buf, c_buf, c_buf, c_buf, c_buf,
+                              c_buf, u32, u32, u32, u32, u32, u32, u32, i32, i32, i32]),
     "krm_quantize_rows": (i32, [c_ctx, c_buf, c_buf, c_buf, u32, u32]),
     "krm_linear_w4a8": (i32, [c_ctx, c_buf, c_buf, c_buf, c_buf, c_buf, c_buf, u32, u32, u32, u32,
                               i32]),

@@ -1399,6 +1399,356 @@ int32_t pick_tile(krm_ctx* ctx, krm_buf x, krm_buf w, krm_buf scales, krm_buf bi
   return launch<XT, ST, 1, 1, 64, 1, 1>(ctx, x, w, scales, bias, out, m, n, k, group_shift);
 }
 
+// ------------------------------------------------ exact integer operands, few rows
+//
+// The same arithmetic for products too small for the 64 x 512 deal (a prefill chunk of a few
+// hundred rows): tile 32 x 32 (or 32 x 64) per workgroup, and the eight waves of a workgroup
+// split K between them instead of the columns, so (M / 32) (N / 32) workgroups each walk K / 8
+// per wave.  Such a product is bound by what a CU's vector memory path takes per workgroup,
+// which counts cache lines per load: every load here covers whole rows, 16 bytes a lane.
+// A wave's slice is walked 128 codes at a time:
+//   x     32 rows x 128 codes, turned into fp16 (or hi + lo) and parked in the wave's own LDS
+//         area in natural order; no other wave reads it, so the K loop has no barrier;
+//   w     32 (64) rows x 64 bytes, parked as they are; a lane reads the word of its column and
+//         MFMA step back, turns it into integers and puts them in natural order (four byte
+//         permutes a word);
+//   two chunks are in flight: a K of 2048 is requested whole before anything is used.
+// At the end the eight waves' sums meet in LDS and are added in wave order; the epilogue (bias,
+// residual, gate/up pairs, RoPE of a fused [q; k; v] projection) works on column pairs there.
+template <typename XT>
+__device__ inline float round_io(float v);
+template <>
+__device__ inline float round_io<float>(float v) { return v; }
+template <>
+__device__ inline float round_io<__half>(float v) { return __half2float(__float2half_rn(v)); }
+
+// Columns (col, col + 1) of output row `row`, summed: bias, then what the call asked for.
+template <typename XT>
+__device__ inline void finish_pair(float v0, float v1, uint32_t row, uint32_t col, uint32_t m,
+                                   uint32_t n, const XT* __restrict__ bias, XT* __restrict__ out,
+                                   const RowsFusion& fuse) {
+  const XT* residual = static_cast<const XT*>(fuse.residual);
+  const bool two = col + 1 < n;
+  if (bias) {
+    v0 += bias_f32<XT>(bias, col);
+    if (two) v1 += bias_f32<XT>(bias, col + 1);
+  }
+  if (fuse.mode == 1) {
+    // (gate, up) -> silu(gate) * up, the roundings of the decode row's epilogue
+    const float t = __builtin_amdgcn_exp2f(-fabsf(v0) * 1.4426950408889634f);
+    const float r = __builtin_amdgcn_rcpf(1.0f + t);
+    const float sig = v0 < 0.f ? t * r : r;
+    float value = __fmul_rn(__fmul_rn(v0, sig), v1);
+    const size_t at = (size_t)row * (n >> 1) + (col >> 1);
+    if (residual) value += bias_f32<XT>(residual, at);
+    store_out<XT>(out, at, value);
+  } else if (fuse.mode == 2) {
+    // what a separate linear would have stored, then the rotation of krm_rope_half
+    const float x0 = round_io<XT>(v0), x1 = round_io<XT>(v1);
+    const uint32_t half = fuse.depth >> 1, pair = col >> 1;
+    const uint32_t rope_pairs = (fuse.heads + fuse.kv_heads) * half;
+    if (pair < rope_pairs) {
+      const uint32_t head = pair / half, j = pair - head * half;
+      const int32_t pos = fuse.positions[row];
+      float o0 = NAN, o1 = NAN;  // a position outside the table is never a valid rotation
+      if (pos >= 0 && (uint32_t)pos < fuse.table_rows) {
+        const size_t t = (size_t)pos * fuse.depth + j;
+        o0 = __fadd_rn(__fmul_rn(x0, fuse.cos_table[t]), __fmul_rn(-x1, fuse.sin_table[t]));
+        o1 = __fadd_rn(__fmul_rn(x1, fuse.cos_table[t + half]),
+                       __fmul_rn(x0, fuse.sin_table[t + half]));
+      }
+      XT* dst = head < fuse.heads
+                    ? static_cast<XT*>(fuse.q_out) + ((size_t)head * m + row) * fuse.depth
+                    : static_cast<XT*>(fuse.k_out) +
+                          ((size_t)(head - fuse.heads) * m + row) * fuse.depth;
+      store_out<XT>(dst, j, o0);
+      store_out<XT>(dst, j + half, o1);
+    } else {
+      const uint32_t e = (pair - rope_pairs) * 2u;  // the v section keeps its natural order
+      const uint32_t plane = e / fuse.depth, d = e - plane * fuse.depth;
+      XT* dst = static_cast<XT*>(fuse.v_out) + ((size_t)plane * m + row) * fuse.depth;
+      store_out<XT>(dst, d, x0);
+      store_out<XT>(dst, d + 1, x1);
+    }
+  } else {
+    const size_t at = (size_t)row * n + col;
+    if (residual) {
+      v0 += bias_f32<XT>(residual, at);
+      if (two) v1 += bias_f32<XT>(residual, at + 1);
+    }
+    store_out<XT>(out, at, v0);
+    if (two) store_out<XT>(out, at + 1, v1);
+  }
+}
+
+// 8 codes of a word -> 8 fp16 integers (u - 8) in their natural order c0..c7.
+__device__ inline uint4 ints_word_natural(uint32_t word) {
+  const uint4 q = ints_word(word);  // (c0,c4), (c1,c5), (c2,c6), (c3,c7)
+  return make_uint4(__builtin_amdgcn_perm(q.y, q.x, 0x05040100u),   // (c0, c1)
+                    __builtin_amdgcn_perm(q.w, q.z, 0x05040100u),   // (c2, c3)
+                    __builtin_amdgcn_perm(q.y, q.x, 0x07060302u),   // (c4, c5)
+                    __builtin_amdgcn_perm(q.w, q.z, 0x07060302u));  // (c6, c7)
+}
+
+// One row piece of x as it arrives (16 bytes: 4 f32 or 8 fp16) and as it is parked (fp16, natural
+// order; the split form parks hi and lo).
+template <typename XT, int OPERAND>
+struct RowPiece;
+template <int OPERAND>
+struct RowPiece<float, OPERAND> {
+  static constexpr int kCodes = 4;
+  uint4 raw;
+  __device__ inline void park(uint8_t* hi_at, uint8_t* lo_at, float scale, uint32_t keep) const {
+    const float v[4] = {__uint_as_float(raw.x), __uint_as_float(raw.y), __uint_as_float(raw.z),
+                        __uint_as_float(raw.w)};
+    _Float16 h[4], l[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      if constexpr (OPERAND == kOperandSplit) {
+        const float xs = v[i] * scale;        // exact: a power of two
+        h[i] = (_Float16)xs;                  // round to nearest even
+        l[i] = (_Float16)(xs - (float)h[i]);  // the difference is exact in f32
+      } else {
+        h[i] = (_Float16)v[i];
+      }
+    }
+    auto pack = [](_Float16 p, _Float16 q) {
+      const half2_t t = {p, q};
+      return __builtin_bit_cast(uint32_t, t);
+    };
+    *reinterpret_cast<uint2*>(hi_at) = make_uint2(pack(h[0], h[1]) & keep, pack(h[2], h[3]) & keep);
+    if constexpr (OPERAND == kOperandSplit)
+      *reinterpret_cast<uint2*>(lo_at) =
+          make_uint2(pack(l[0], l[1]) & keep, pack(l[2], l[3]) & keep);
+  }
+};
+template <int OPERAND>
+struct RowPiece<__half, OPERAND> {
+  static constexpr int kCodes = 8;
+  uint4 raw;
+  __device__ inline void park(uint8_t* hi_at, uint8_t*, float, uint32_t keep) const {
+    *reinterpret_cast<uint4*>(hi_at) =
+        make_uint4(raw.x & keep, raw.y & keep, raw.z & keep, raw.w & keep);
+  }
+};
+
+template <typename XT, typename ST, int OPERAND, int WN>
+__global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2)))
+void gemm_i4_rows_kernel(const XT* __restrict__ x, const uint8_t* __restrict__ w,
+                         const ST* __restrict__ scales, const XT* __restrict__ bias,
+                         XT* __restrict__ out, uint32_t m, uint32_t n, uint32_t k,
+                         uint32_t group_shift, uint32_t m_blocks,
+                         const float* __restrict__ row_scale, RowsFusion fuse) {
+  constexpr int BM = 32, BN = 32 * WN, kWaves = 8;
+  constexpr int NA = OPERAND == kOperandSplit ? 2 : 1;
+  constexpr int kChunk = 128;
+  constexpr int kRowA = kChunk * 2 + 16;          // bytes of a parked x row
+  constexpr int kPlane = BM * kRowA;
+  constexpr int kRowB = kChunk / 2 + 16;          // bytes of a parked weight row
+  constexpr int kWords = BN * kRowB;
+  constexpr int kSumBytes = BM * BN * 4;
+  constexpr int kStageBytes = NA * kPlane + kWords;
+  constexpr int kWaveBytes = kStageBytes > kSumBytes ? kStageBytes : kSumBytes;
+  constexpr int kPieceCodes = RowPiece<XT, OPERAND>::kCodes;
+  constexpr int kLanesPerRow = kChunk / kPieceCodes;          // 32 (f32) or 16 (fp16)
+  constexpr int kRowsPerLoad = 64 / kLanesPerRow;             // 2 or 4
+  constexpr int kActLoads = BM / kRowsPerLoad;                // 16 or 8
+  constexpr int kWordLoads = BN / 16;                         // 16 rows x 4 pieces a load
+  static_assert(OPERAND == kOperandF16 || sizeof(XT) == 4, "only f32 activations are split");
+  __shared__ __align__(16) uint8_t s_wave[kWaves][kWaveBytes];
+  __shared__ float s_inv[BM], s_up[BM];
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int frag_row = lane & 31, frag_h = lane >> 5;
+  const uint32_t groups = k >> group_shift;
+  const bool half_groups = group_shift == 6;  // 64 codes a group: two groups a chunk
+  const uint32_t nb = blockIdx.x / m_blocks, mb = blockIdx.x - nb * m_blocks;
+  const uint32_t m0 = mb * BM, n0 = nb * BN;
+  const uint32_t chunks = (k + kChunk - 1) / kChunk;
+  const uint32_t c_begin = (uint32_t)wave * chunks / kWaves;
+  const uint32_t c_end = ((uint32_t)wave + 1u) * chunks / kWaves;
+  uint8_t* mine = s_wave[wave];
+  uint8_t* my_words = mine + NA * kPlane;
+
+  // staging: whole rows, 16 bytes a lane (coalesced), kRowsPerLoad rows a load
+  const uint32_t a_piece = lane % kLanesPerRow, a_row = lane / kLanesPerRow;
+  const uint32_t b_piece = lane & 3u, b_row = lane >> 2;
+  // (element offsets in 32 bits — the launcher checks that x and w are that small — and the
+  // row scales in LDS: the registers are wanted for two chunks in flight)
+  const uint32_t x_row0 = m0 + a_row;
+  if constexpr (OPERAND == kOperandSplit) {
+    if (tid < BM) {
+      const size_t row = min(m0 + (uint32_t)tid, m - 1);
+      s_up[tid] = row_scale[2 * row];
+      s_inv[tid] = row_scale[2 * row + 1];
+    }
+    __syncthreads();
+  }
+  uint32_t wrow[kWordLoads];
+#pragma unroll
+  for (int i = 0; i < kWordLoads; ++i) wrow[i] = min(n0 + 16u * i + b_row, n - 1) * (k >> 1);
+  const ST* srow[WN];
+#pragma unroll
+  for (int nt = 0; nt < WN; ++nt)
+    srow[nt] = scales + (size_t)min(n0 + 32u * nt + (uint32_t)frag_row, n - 1) * groups;
+
+  struct Staged {
+    RowPiece<XT, OPERAND> a[kActLoads];
+    uint4 b[kWordLoads];
+    float ws[WN][2];  // the scales of the chunk's first and second 64 codes
+  };
+  auto load_chunk = [&](uint32_t c, Staged& d) {
+    const uint32_t at = c * kChunk + a_piece * kPieceCodes;
+    const uint32_t off = at < k ? at : 0u;
+#pragma unroll
+    for (int i = 0; i < kActLoads; ++i)
+      d.a[i].raw = *reinterpret_cast<const uint4*>(
+          x + ((size_t)(min(x_row0 + (uint32_t)(kRowsPerLoad * i), m - 1) * k) + off));
+    const uint32_t bat = c * (kChunk / 2) + b_piece * 16u;
+    const uint32_t boff = bat < (k >> 1) ? bat : 0u;
+#pragma unroll
+    for (int i = 0; i < kWordLoads; ++i)
+      d.b[i] = *reinterpret_cast<const uint4*>(w + ((size_t)wrow[i] + boff));
+    const uint32_t c0 = c * kChunk < k ? c * kChunk : 0u;
+    const uint32_t c1 = c * kChunk + 64u < k ? c * kChunk + 64u : c0;
+#pragma unroll
+    for (int nt = 0; nt < WN; ++nt) {
+      d.ws[nt][0] = load_scale_f32<ST>(srow[nt], c0 >> group_shift);
+      d.ws[nt][1] = load_scale_f32<ST>(srow[nt], c1 >> group_shift);
+    }
+  };
+  auto park_chunk = [&](uint32_t c, const Staged& d) {
+    const uint32_t keep = c * kChunk + a_piece * kPieceCodes < k ? 0xFFFFFFFFu : 0u;  // past K: 0
+#pragma unroll
+    for (int i = 0; i < kActLoads; ++i) {
+      const uint32_t at = (kRowsPerLoad * i + a_row) * kRowA + a_piece * (kPieceCodes * 2);
+      float up = 1.0f;
+      if constexpr (OPERAND == kOperandSplit) up = s_up[kRowsPerLoad * i + a_row];
+      d.a[i].park(mine + at, mine + kPlane + at, up, keep);
+    }
+#pragma unroll
+    for (int i = 0; i < kWordLoads; ++i)
+      *reinterpret_cast<uint4*>(my_words + (16 * i + b_row) * kRowB + b_piece * 16u) = d.b[i];
+  };
+  // The parked rows are written and read by the same wave only: what orders them is the LDS
+  // queue of the wave, and the compiler is told not to move accesses across this point.
+  auto wave_sync = [] {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+  };
+
+  float16_t total[WN], acc[WN];
+#pragma unroll
+  for (int nt = 0; nt < WN; ++nt)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) total[nt][r] = acc[nt][r] = 0.f;
+  auto flush = [&](const float (&ws)[WN][2], int which) {
+#pragma unroll
+    for (int nt = 0; nt < WN; ++nt)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        total[nt][r] = fmaf(acc[nt][r], ws[nt][which], total[nt][r]);
+        acc[nt][r] = 0.f;
+      }
+  };
+
+  // kDepth chunks in flight (two where the registers allow: a K of 2048 is then requested whole
+  // before anything is used)
+  constexpr int kDepth = (sizeof(XT) == 2 || (WN == 1 && OPERAND == kOperandF16)) ? 2 : 1;
+  Staged staged[kDepth];
+#pragma unroll
+  for (int d = 0; d < kDepth; ++d)
+    if (c_begin + d < c_end) load_chunk(c_begin + d, staged[d]);
+  auto run_chunk = [&](uint32_t c, int cur) {
+    park_chunk(c, staged[cur]);
+    float ws[WN][2];
+#pragma unroll
+    for (int nt = 0; nt < WN; ++nt) {
+      ws[nt][0] = staged[cur].ws[nt][0];
+      ws[nt][1] = staged[cur].ws[nt][1];
+    }
+    if (c + kDepth < c_end) load_chunk(c + kDepth, staged[cur]);
+    wave_sync();
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {  // step j: codes 16 j + 8 h .. + 7 of the chunk
+      half8_t a[NA];
+#pragma unroll
+      for (int copy = 0; copy < NA; ++copy)
+        a[copy] = *reinterpret_cast<const half8_t*>(mine + copy * kPlane + frag_row * kRowA +
+                                                    32 * j + 16 * frag_h);
+#pragma unroll
+      for (int nt = 0; nt < WN; ++nt) {
+        const uint32_t word = *reinterpret_cast<const uint32_t*>(
+            my_words + (32 * nt + frag_row) * kRowB + 8 * j + 4 * frag_h);
+        const half8_t b = __builtin_bit_cast(half8_t, ints_word_natural(word));
+#pragma unroll
+        for (int copy = 0; copy < NA; ++copy)
+          acc[nt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[copy], b, acc[nt], 0, 0, 0);
+      }
+      if (j == 3 && half_groups) flush(ws, 0);
+    }
+    wave_sync();
+    // the scale group ends with this chunk, or the wave's slice does
+    if (half_groups || (((c + 1) * kChunk) & ((1u << group_shift) - 1u)) == 0u || c + 1 == c_end)
+      flush(ws, 1);
+  };
+  for (uint32_t c = c_begin; c < c_end; c += kDepth) {
+    run_chunk(c, 0);
+    if constexpr (kDepth == 2) {
+      if (c + 1 < c_end) run_chunk(c + 1, 1);
+    }
+  }
+
+  // the wave's sums, [row][column] in its own area
+  float* sums = reinterpret_cast<float*>(mine);
+#pragma unroll
+  for (int nt = 0; nt < WN; ++nt)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const int local = 8 * (r / 4) + 4 * frag_h + (r % 4);
+      sums[local * BN + nt * 32 + frag_row] = total[nt][r];
+    }
+  __syncthreads();
+
+  constexpr int kPairs = BM * BN / 2;
+#pragma unroll
+  for (int i = 0; i < kPairs / 512; ++i) {
+    const int p = tid + 512 * i;
+    const int local = p / (BN / 2), cp = p - local * (BN / 2);
+    const uint32_t row = m0 + local, col = n0 + 2u * cp;
+    float v0 = 0.f, v1 = 0.f;
+#pragma unroll
+    for (int wv = 0; wv < kWaves; ++wv) {  // wave order: a fixed sum
+      const float2 part =
+          *reinterpret_cast<const float2*>(s_wave[wv] + (size_t)(local * BN + 2 * cp) * 4);
+      v0 += part.x;
+      v1 += part.y;
+    }
+    if (row >= m || col >= n) continue;
+    if constexpr (OPERAND == kOperandSplit) {  // exact: a power of two
+      v0 *= s_inv[local];
+      v1 *= s_inv[local];
+    }
+    finish_pair<XT>(v0, v1, row, col, m, n, bias, out, fuse);
+  }
+}
+
+template <typename XT, typename ST, int OPERAND, int WN>
+int32_t launch_rows(krm_ctx* ctx, krm_buf x, krm_buf w, krm_buf scales, krm_buf bias, krm_buf out,
+                    uint32_t m, uint32_t n, uint32_t k, uint32_t group_shift,
+                    const RowsFusion& fuse) {
+  if constexpr (OPERAND == kOperandSplit) {
+    row_scale_kernel<<<dim3(m), dim3(256), 0, ctx->stream>>>(ptr<const float>(x), ctx->row_scales, k);
+    KRM_TRY(launched(ctx, "row_scale_kernel"));
+  }
+  const uint32_t m_blocks = (m + 31) / 32, n_blocks = (n + 32 * WN - 1) / (32 * WN);
+  gemm_i4_rows_kernel<XT, ST, OPERAND, WN><<<dim3(m_blocks * n_blocks), dim3(512), 0, ctx->stream>>>(
+      ptr<const XT>(x), ptr<const uint8_t>(w), ptr<const ST>(scales), ptr<const XT>(bias),
+      ptr<XT>(out), m, n, k, group_shift, m_blocks, ctx->row_scales, fuse);
+  return launched(ctx, "gemm_i4_rows_kernel");
+}
+
 template <typename XT, typename ST, int OPERAND>
 int32_t launch_exact(krm_ctx* ctx, krm_buf x, krm_buf w, krm_buf scales, krm_buf bias, krm_buf out,
                      uint32_t m, uint32_t n, uint32_t k, uint32_t group_shift, uint32_t grid,
@@ -1446,6 +1796,45 @@ int32_t linear_i4_gemm_exact(krm_ctx* ctx, krm_buf x, krm_buf w, krm_buf scales,
   if (scale_dtype == KRM_F16) KRM_EXACT(float, __half, kOperandF16);
   KRM_EXACT(float, float, kOperandF16);
 #undef KRM_EXACT
+}
+
+// The few-row form of the same arithmetic, with its epilogues; any shape with a group of at
+// least 64 codes, K a multiple of 32 and 16-byte aligned rows.  *handled = false (nothing
+// launched) otherwise.
+int32_t linear_i4_gemm_rows(krm_ctx* ctx, krm_buf x, krm_buf w, krm_buf scales, krm_buf bias,
+                            krm_buf out, uint32_t m, uint32_t n, uint32_t k, uint32_t group,
+                            int32_t io_dtype, int32_t scale_dtype, int32_t compute,
+                            const RowsFusion& fuse, bool* handled) {
+  *handled = false;
+  const bool split = compute == KRM_COMPUTE_F32 && io_dtype == KRM_F32;
+  if (group < 64 || k % 32 != 0 || !aligned(w, 16) || !aligned(x, 16)) return KRM_OK;
+  if (split && (m > kMaxSplitRows || !ctx->row_scales)) return KRM_OK;
+  const uint64_t m_blocks = (m + 31) / 32;
+  if (m_blocks * ((n + 31) / 32) > 0x7fffffffull) return KRM_OK;
+  if ((uint64_t)m * k > 0xffffffffull || (uint64_t)n * (k >> 1) > 0xffffffffull) return KRM_OK;
+  uint32_t group_shift = 0;
+  while ((1u << group_shift) < group) ++group_shift;
+  *handled = true;
+  // 64 columns a workgroup once 32 would need more than one round of workgroups: fewer reads of
+  // x for the same weights
+  const bool wide = m_blocks * ((n + 31) / 32) > (uint64_t)ctx->num_cus;
+#define KRM_ROWS(XT, ST, OP)                                                                      \
+  return wide ? launch_rows<XT, ST, OP, 2>(ctx, x, w, scales, bias, out, m, n, k, group_shift, fuse) \
+              : launch_rows<XT, ST, OP, 1>(ctx, x, w, scales, bias, out, m, n, k, group_shift, fuse)
+  if (io_dtype == KRM_F16) {
+    if (scale_dtype == KRM_F16) KRM_ROWS(__half, __half, kOperandF16);
+    KRM_ROWS(__half, float, kOperandF16);
+  }
+  if (split) {  // (hi and lo planes of eight waves leave no LDS for 64 columns)
+    if (scale_dtype == KRM_F16)
+      return launch_rows<float, __half, kOperandSplit, 1>(ctx, x, w, scales, bias, out, m, n, k,
+                                                          group_shift, fuse);
+    return launch_rows<float, float, kOperandSplit, 1>(ctx, x, w, scales, bias, out, m, n, k,
+                                                       group_shift, fuse);
+  }
+  if (scale_dtype == KRM_F16) KRM_ROWS(float, __half, kOperandF16);
+  KRM_ROWS(float, float, kOperandF16);
+#undef KRM_ROWS
 }
 
 int32_t linear_i4_gemm_f16(krm_ctx* ctx, krm_buf x, krm_buf w, krm_buf scales, krm_buf bias,

@@ -85,6 +85,22 @@ inline T* ptr(krm_buf address) {
   return reinterpret_cast<T*>(static_cast<uintptr_t>(address));
 }
 
+// What the few-row MFMA GEMM (gemm_i4.hip) does with a finished sum besides storing it.
+struct RowsFusion {
+  const void* residual = nullptr;  // [m, n_out] added to the result (the activation type)
+  // 0: plain; 1: columns (2i, 2i+1) = (gate_i, up_i), out[., i] = silu(gate) * up;
+  // 2: a fused [q; k; v] projection whose q and k columns are interleaved per head as
+  //    (0, D/2, 1, D/2 + 1, ...): half-split RoPE by positions[row], results head-major
+  int mode = 0;
+  const int32_t* positions = nullptr;
+  const float* cos_table = nullptr;
+  const float* sin_table = nullptr;
+  void* q_out = nullptr;  // [H, m, D]
+  void* k_out = nullptr;  // [Hkv, m, D]
+  void* v_out = nullptr;  // [Hkv, m, D]
+  uint32_t heads = 0, kv_heads = 0, depth = 0, table_rows = 0;
+};
+
 }  // namespace krm
 
 #define KRM_TRY(expr)                  \

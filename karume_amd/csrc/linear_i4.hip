@@ -1036,6 +1036,10 @@ int32_t linear_i4_gemm_exact(krm_ctx* ctx, krm_buf x, krm_buf w, krm_buf scales,
                              krm_buf out, uint32_t m, uint32_t n, uint32_t k, uint32_t group,
                              int32_t io_dtype, int32_t scale_dtype, int32_t compute,
                              bool* handled);
+int32_t linear_i4_gemm_rows(krm_ctx* ctx, krm_buf x, krm_buf w, krm_buf scales, krm_buf bias,
+                            krm_buf out, uint32_t m, uint32_t n, uint32_t k, uint32_t group,
+                            int32_t io_dtype, int32_t scale_dtype, int32_t compute,
+                            const RowsFusion& fuse, bool* handled);
 int32_t linear_i4_gemm_f16(krm_ctx* ctx, krm_buf x, krm_buf w, krm_buf scales, krm_buf bias,
                            krm_buf out, uint32_t m, uint32_t n, uint32_t k, uint32_t group,
                            int32_t io_dtype, int32_t scale_dtype);
@@ -1068,6 +1072,9 @@ int32_t krm_linear_i4(krm_ctx* ctx, krm_buf x, krm_buf w, krm_buf scales, krm_bu
   bool handled = false;
   KRM_TRY(linear_i4_gemm_exact(ctx, x, w, scales, bias, out, m, n, k, group, io_dtype,
                                scale_dtype, compute, &handled));
+  if (handled) return KRM_OK;
+  KRM_TRY(linear_i4_gemm_rows(ctx, x, w, scales, bias, out, m, n, k, group, io_dtype, scale_dtype,
+                              compute, RowsFusion{}, &handled));
   if (handled) return KRM_OK;
   if (compute == KRM_COMPUTE_F16)
     return linear_i4_gemm_f16(ctx, x, w, scales, bias, out, m, n, k, group, io_dtype,
@@ -1114,6 +1121,91 @@ int32_t krm_linear_i4_fused(krm_ctx* ctx, krm_buf x, krm_buf norm_weight_f32, fl
   fuse.residual = ptr<const void>(residual);
   fuse.pair_silu = epilogue == KRM_EPILOGUE_SILU_PAIRS ? 1u : 0u;
   return gemv_dispatch(ctx, x, w, scales, bias, out, m, n, k, group, io_dtype, scale_dtype, fuse);
+}
+
+int32_t krm_linear_i4_rows(krm_ctx* ctx, krm_buf x, krm_buf w, krm_buf scales, krm_buf bias,
+                           krm_buf residual, krm_buf out, uint32_t m, uint32_t n, uint32_t k,
+                           uint32_t group, int32_t io_dtype, int32_t scale_dtype, int32_t compute,
+                           int32_t epilogue) {
+  KRM_TRY(enter(ctx));
+  KRM_REQUIRE(ctx, valid_dtype(io_dtype) && valid_dtype(scale_dtype),
+              "krm_linear_i4_rows: io_dtype %d / scale_dtype %d", io_dtype, scale_dtype);
+  KRM_REQUIRE(ctx, compute == KRM_COMPUTE_F32 || compute == KRM_COMPUTE_F16,
+              "krm_linear_i4_rows: compute %d", compute);
+  KRM_REQUIRE(ctx, epilogue == KRM_EPILOGUE_NONE || epilogue == KRM_EPILOGUE_SILU_PAIRS,
+              "krm_linear_i4_rows: epilogue %d", epilogue);
+  KRM_REQUIRE(ctx, is_pow2(group) && group >= 16 && k >= 1 && k % group == 0,
+              "krm_linear_i4_rows: group_size %u must be a power of two >= 16 dividing k = %u",
+              group, k);
+  KRM_REQUIRE(ctx, epilogue != KRM_EPILOGUE_SILU_PAIRS || n % 2 == 0,
+              "krm_linear_i4_rows: the gate/up epilogue needs an even n, got %u", n);
+  if (m == 0 || n == 0) return KRM_OK;
+  KRM_REQUIRE(ctx, x && w && scales && out, "krm_linear_i4_rows: NULL buffer");
+  KRM_REQUIRE(ctx, aligned(out, dtype_bytes(io_dtype)) && aligned(residual, dtype_bytes(io_dtype)) &&
+                       aligned(bias, dtype_bytes(io_dtype)) &&
+                       aligned(scales, dtype_bytes(scale_dtype)),
+              "krm_linear_i4_rows: misaligned buffer");
+  RowsFusion fuse{};
+  fuse.residual = ptr<const void>(residual);
+  fuse.mode = epilogue == KRM_EPILOGUE_SILU_PAIRS ? 1 : 0;
+  bool handled = false;
+  KRM_TRY(linear_i4_gemm_rows(ctx, x, w, scales, bias, out, m, n, k, group, io_dtype, scale_dtype,
+                              compute, fuse, &handled));
+  if (handled) return KRM_OK;
+  return fail(ctx, KRM_ERR_VALIDATION,
+              "krm_linear_i4_rows: covers group_size >= 64, k %% 32 == 0 and 16-byte aligned x and "
+              "w (group %u, k %u); use krm_linear_i4 and the separate ops", group, k);
+}
+
+int32_t krm_prefill_qkv(krm_ctx* ctx, krm_buf x, krm_buf w, krm_buf scales, krm_buf bias,
+                        krm_buf positions_i32, krm_buf cos_table_f32, krm_buf sin_table_f32,
+                        krm_buf q_out, krm_buf k_out, krm_buf v_out, uint32_t m, uint32_t heads,
+                        uint32_t kv_heads, uint32_t depth, uint32_t k, uint32_t group,
+                        uint32_t table_rows, int32_t io_dtype, int32_t scale_dtype,
+                        int32_t compute) {
+  KRM_TRY(enter(ctx));
+  KRM_REQUIRE(ctx, valid_dtype(io_dtype) && valid_dtype(scale_dtype),
+              "krm_prefill_qkv: io_dtype %d / scale_dtype %d", io_dtype, scale_dtype);
+  KRM_REQUIRE(ctx, compute == KRM_COMPUTE_F32 || compute == KRM_COMPUTE_F16,
+              "krm_prefill_qkv: compute %d", compute);
+  KRM_REQUIRE(ctx, is_pow2(group) && group >= 16 && k >= 1 && k % group == 0,
+              "krm_prefill_qkv: group_size %u must be a power of two >= 16 dividing k = %u", group,
+              k);
+  KRM_REQUIRE(ctx, heads >= 1 && kv_heads >= 1 && depth >= 2 && depth % 2 == 0 && table_rows >= 1,
+              "krm_prefill_qkv: H / Hkv / D / table rows (%u / %u / %u / %u)", heads, kv_heads,
+              depth, table_rows);
+  KRM_REQUIRE(ctx, ((uint64_t)heads + 2ull * kv_heads) * depth <= 0x7fffffffull,
+              "krm_prefill_qkv: the row is too long");
+  if (m == 0) return KRM_OK;
+  KRM_REQUIRE(ctx, x && w && scales && positions_i32 && cos_table_f32 && sin_table_f32 && q_out &&
+                       k_out && v_out,
+              "krm_prefill_qkv: NULL buffer");
+  KRM_REQUIRE(ctx, aligned(q_out, dtype_bytes(io_dtype)) && aligned(k_out, dtype_bytes(io_dtype)) &&
+                       aligned(v_out, dtype_bytes(io_dtype)) &&
+                       aligned(bias, dtype_bytes(io_dtype)) &&
+                       aligned(scales, dtype_bytes(scale_dtype)) && aligned(positions_i32, 4) &&
+                       aligned(cos_table_f32, 4) && aligned(sin_table_f32, 4),
+              "krm_prefill_qkv: misaligned buffer");
+  RowsFusion fuse{};
+  fuse.mode = 2;
+  fuse.positions = ptr<const int32_t>(positions_i32);
+  fuse.cos_table = ptr<const float>(cos_table_f32);
+  fuse.sin_table = ptr<const float>(sin_table_f32);
+  fuse.q_out = ptr<void>(q_out);
+  fuse.k_out = ptr<void>(k_out);
+  fuse.v_out = ptr<void>(v_out);
+  fuse.heads = heads;
+  fuse.kv_heads = kv_heads;
+  fuse.depth = depth;
+  fuse.table_rows = table_rows;
+  const uint32_t n = (heads + 2 * kv_heads) * depth;
+  bool handled = false;
+  KRM_TRY(linear_i4_gemm_rows(ctx, x, w, scales, bias, q_out, m, n, k, group, io_dtype, scale_dtype,
+                              compute, fuse, &handled));
+  if (handled) return KRM_OK;
+  return fail(ctx, KRM_ERR_VALIDATION,
+              "krm_prefill_qkv: covers group_size >= 64, k %% 32 == 0 and 16-byte aligned x and w "
+              "(group %u, k %u); use krm_linear_i4, krm_rope_half and krm_transpose_01", group, k);
 }
 
 int32_t krm_decode_qkv(krm_ctx* ctx, krm_buf x, krm_buf norm_weight_f32, float norm_eps,

@@ -273,6 +273,10 @@ class LlamaDecoderSession:
         if m == 1 and self.fuse_decode:
             self._forward_fused_row(context, past, lengths)
             return
+        if m > 16 and self.fuse_decode and self._rows_form_covers():
+            self._forward_rows(context, m, past, query, lengths)
+            self._head(last_row)
+            return
         for li, lw in enumerate(self.layers):
             g.rms_norm(b["h"], lw["attn_norm"], b["xn"], m, d, c.rms_eps, io)
             self._linear(b["xn"], lw["q"], b["q"], m)
@@ -325,11 +329,77 @@ class LlamaDecoderSession:
             g.silu_mul(b["g"], b["u"], b["act"], m * c.ffn, io)
             self._linear(b["act"], lw["down"], b["dn"], m)
             g.add(b["h"], b["dn"], b["h"], m * d, io)
-        # token-only exit: the head runs on the last valid row only
-        row = b["h"].offset(last_row * d * self.eb)
-        g.rms_norm(row, self.final_norm, b["xn"], 1, d, c.rms_eps, io)
+        self._head(last_row)
+
+    def _head(self, last_row: int) -> None:
+        """Token-only exit: the head runs on the last valid row only."""
+        g, c, b, io = self.gpu, self.config, self.buf, self.io_dtype
+        row = b["h"].offset(last_row * c.d_model * self.eb)
+        g.rms_norm(row, self.final_norm, b["xn"], 1, c.d_model, c.rms_eps, io)
         self._linear(b["xn"], self.lm_head, b["logits"], 1)
         g.argmax(b["logits"], b["token"], 1, c.vocab, io)
+
+    def _rows_form_covers(self) -> bool:
+        """The chunk-of-rows launches need groups of 64 codes or more and K a multiple of 32."""
+        c = self.config
+        return (c.group_size >= 64 and c.d_model % 32 == 0 and c.ffn % 32 == 0
+                and (c.heads * c.head_dim) % 32 == 0)
+
+    def _forward_rows(self, context: GenerationContext, m: int, past: int, query: int,
+                      lengths: Optional[DeviceBuffer]) -> None:
+        """A chunk of m > 16 rows, 10 launches a layer: the [q; k; v] projection writes roped,
+        head-major q / k / v, the o and down projections add the residual in place, the gate/up
+        projection applies silu * up."""
+        from .runtime import EPILOGUE_SILU_PAIRS
+        g, c, b, io = self.gpu, self.config, self.buf, self.io_dtype
+        d, group, compute = c.d_model, c.group_size, self.prefill_compute
+        spec = dict(chunk_rows=m, depth=c.head_dim, capacity=context.capacity,
+                    window=context.window)
+        for li, lw in enumerate(self.layers):
+            g.rms_norm(b["h"], lw["attn_norm"], b["xn"], m, d, c.rms_eps, io)
+            lin = lw["qkv"]
+            g.prefill_qkv(b["xn"], lin.w, lin.s, b["pos"], self.rope_cos, self.rope_sin, b["qr"],
+                          b["kr"], b["vt"], m=m, heads=c.heads, kv_heads=c.kv_heads,
+                          depth=c.head_dim, k=d, group=group, table_rows=c.max_position,
+                          io_dtype=io, scale_dtype=lin.scale_dtype, compute=compute)
+            if lengths is None:
+                g.attention_state(b["qr"], b["kr"], b["vt"], context.slots_k[li],
+                                  context.slots_v[li], b["att"], batch=1, heads=c.heads,
+                                  kv_heads=c.kv_heads, half_scale=c.half_scale, past=past,
+                                  query=query, io_dtype=io, kv_dtype=self.kv_dtype,
+                                  workspace=self.workspace, **spec)
+                # readers first, then the appends (docs/ir-v1.md:345-348)
+                g.state_append(b["kr"], context.slots_k[li], kv_planes=c.kv_heads, past=past,
+                               query=query, x_dtype=io, slot_dtype=self.kv_dtype, **spec)
+                g.state_append(b["vt"], context.slots_v[li], kv_planes=c.kv_heads, past=past,
+                               query=query, x_dtype=io, slot_dtype=self.kv_dtype, **spec)
+            else:
+                g.attention_state_lengths(b["qr"], b["kr"], b["vt"], context.slots_k[li],
+                                          context.slots_v[li], b["att"], batch=1, heads=c.heads,
+                                          kv_heads=c.kv_heads, half_scale=c.half_scale,
+                                          lengths=lengths, max_past=context.capacity - 1,
+                                          io_dtype=io, kv_dtype=self.kv_dtype,
+                                          workspace=self.workspace, **spec)
+                g.state_append_lengths(b["kr"], context.slots_k[li], kv_planes=c.kv_heads,
+                                       lengths=lengths, x_dtype=io, slot_dtype=self.kv_dtype,
+                                       **spec)
+                g.state_append_lengths(b["vt"], context.slots_v[li], kv_planes=c.kv_heads,
+                                       lengths=lengths, x_dtype=io, slot_dtype=self.kv_dtype,
+                                       **spec)
+            g.transpose_01(b["att"], b["att2"], c.heads, m, c.head_dim, io)
+            lin = lw["o"]
+            g.linear_i4_rows(b["att2"], lin.w, lin.s, b["h"], m, lin.n, lin.k, group,
+                             residual=b["h"], io_dtype=io, scale_dtype=lin.scale_dtype,
+                             compute=compute)
+            g.rms_norm(b["h"], lw["ffn_norm"], b["xn"], m, d, c.rms_eps, io)
+            lin = lw["gate_up"]
+            g.linear_i4_rows(b["xn"], lin.w, lin.s, b["act"], m, lin.n, lin.k, group,
+                             io_dtype=io, scale_dtype=lin.scale_dtype, compute=compute,
+                             epilogue=EPILOGUE_SILU_PAIRS)
+            lin = lw["down"]
+            g.linear_i4_rows(b["act"], lin.w, lin.s, b["h"], m, lin.n, lin.k, group,
+                             residual=b["h"], io_dtype=io, scale_dtype=lin.scale_dtype,
+                             compute=compute)
 
     def _replay_max_past(self, context: GenerationContext) -> int:
         """Largest pastLength the recorded step will be replayed with: sizes the attention

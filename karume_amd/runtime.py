@@ -481,6 +481,31 @@ class GpuContext:
             _addr(slot_v), heads, kv_heads, depth, k, group, table_rows, capacity, window, past,
             _addr(lengths) if lengths is not None else 0, io_dtype, scale_dtype, kv_dtype))
 
+    def linear_i4_rows(self, x: BufferLike, w: BufferLike, scales: BufferLike, out: BufferLike,
+                       m: int, n: int, k: int, group: int, *, bias: Optional[BufferLike] = None,
+                       residual: Optional[BufferLike] = None, io_dtype: int = F32,
+                       scale_dtype: int = F32, compute: int = COMPUTE_F32,
+                       epilogue: int = EPILOGUE_NONE) -> None:
+        """`linear` for a chunk of rows on the matrix cores, with the residual add or the
+        gate/up silu-mul folded in."""
+        self._check(self._lib.krm_linear_i4_rows(
+            self._handle, _addr(x), _addr(w), _addr(scales),
+            _addr(bias) if bias is not None else 0, _addr(residual) if residual is not None else 0,
+            _addr(out), m, n, k, group, io_dtype, scale_dtype, compute, epilogue))
+
+    def prefill_qkv(self, x: BufferLike, w: BufferLike, scales: BufferLike, positions: BufferLike,
+                    cos_table: BufferLike, sin_table: BufferLike, q_out: BufferLike,
+                    k_out: BufferLike, v_out: BufferLike, *, m: int, heads: int, kv_heads: int,
+                    depth: int, k: int, group: int, table_rows: int,
+                    bias: Optional[BufferLike] = None, io_dtype: int = F32, scale_dtype: int = F32,
+                    compute: int = COMPUTE_F32) -> None:
+        """Fused [q; k; v] projection of m rows + RoPE of q and k, written head-major."""
+        self._check(self._lib.krm_prefill_qkv(
+            self._handle, _addr(x), _addr(w), _addr(scales),
+            _addr(bias) if bias is not None else 0, _addr(positions), _addr(cos_table),
+            _addr(sin_table), _addr(q_out), _addr(k_out), _addr(v_out), m, heads, kv_heads, depth,
+            k, group, table_rows, io_dtype, scale_dtype, compute))
+
     def transpose_01(self, x: BufferLike, out: BufferLike, a: int, b: int, d: int,
                      io_dtype: int = F32) -> None:
         self._check(self._lib.krm_transpose_01(self._handle, _addr(x), _addr(out), a, b, d,

@@ -222,3 +222,119 @@ def test_f32_class_gemm_edges_and_non_finite_rows(gpu_ctx):
     assert np.all(err <= bound), float(np.max(err / bound))
     assert not np.any(np.isfinite(got[[11, 12]][:, cols]))
     assert not np.any(np.isfinite(want[[11, 12]]))
+
+
+# ---------------------------------------------------------------- few rows (a prefill chunk)
+
+def run_rows(ctx, x, packed, scale, bias, n, k, group, compute, residual=None,
+             epilogue=ka.EPILOGUE_NONE):
+    x = np.ascontiguousarray(x)
+    m = x.shape[0]
+    n_out = n // 2 if epilogue == ka.EPILOGUE_SILU_PAIRS else n
+    dx, dw, ds = ctx.upload(x), ctx.upload(packed), ctx.upload(np.ascontiguousarray(scale))
+    db = ctx.upload(np.ascontiguousarray(bias, dtype=x.dtype)) if bias is not None else None
+    dr = ctx.upload(np.ascontiguousarray(residual, dtype=x.dtype)) if residual is not None else None
+    out = ctx.alloc(max(m * n_out * x.itemsize, 16))
+    ctx.linear_i4_rows(dx, dw, ds, out, m, n, k, group, bias=db, residual=dr,
+                       io_dtype=ka.dtype_code(x.dtype), scale_dtype=ka.dtype_code(scale.dtype),
+                       compute=compute, epilogue=epilogue)
+    got = out.download(x.dtype, (m, n_out))
+    for b in (dx, dw, ds, out, db, dr):
+        if b is not None:
+            b.free()
+    return got
+
+
+ROWS_SHAPES = [(128, 2560, 2048, 128),   # a 128-row chunk of the benchmark decoder: [q; k; v]
+               (128, 2048, 5632, 128),   # its down-projection: 44 groups over 8 waves
+               (40, 512, 1024, 128), (100, 129, 320, 64), (257, 96, 4096, 256),
+               (17, 33, 192, 64),        # fewer 64-code chunks than waves
+               (1, 64, 2048, 128)]
+
+
+@pytest.mark.parametrize("m,n,k,g", ROWS_SHAPES)
+@pytest.mark.parametrize("mode", ["f32", "f16 on f32", "f16"])
+def test_few_row_products_meet_the_gemv_gate(gpu_ctx, m, n, k, g, mode):
+    """Shapes too small for the 64 x 512 deal run on the few-row kernel (eight waves split K):
+    exact integer weights and f32 group sums, so the f32 class (x split hi + lo) and the fp16
+    class (x rounded to fp16 once: the oracle is given the rounded x) both meet the GEMV's
+    gate.  Ragged M, N, K, a single row and a K shorter than eight chunks included."""
+    rng = np.random.default_rng(m * 7 + n + k)
+    packed, _q, scale = helpers.synthetic_int4(rng, n, k, g)
+    x = rng.normal(size=(m, k)).astype(np.float32)
+    x[0] *= 300.0
+    if m > 2:
+        x[2] *= 1e-3
+    bias = rng.normal(size=n).astype(np.float32)
+    if mode == "f32":
+        got = run_rows(gpu_ctx, x, packed, scale, bias, n, k, g, ka.COMPUTE_F32)
+        seen = x
+    elif mode == "f16 on f32":
+        got = run_rows(gpu_ctx, x, packed, scale, bias, n, k, g, ka.COMPUTE_F16)
+        seen = x.astype(np.float16).astype(np.float32)
+    else:
+        got = run_rows(gpu_ctx, x.astype(np.float16), packed, scale, bias, n, k, g,
+                       ka.COMPUTE_F16)
+        seen = x.astype(np.float16).astype(np.float32)
+        bias = bias.astype(np.float16).astype(np.float32)
+    if m > 16 and mode != "f16":   # krm_linear_i4 takes the same kernel for these shapes
+        compute = ka.COMPUTE_F32 if mode == "f32" else ka.COMPUTE_F16
+        same = run_linear(gpu_ctx, x, packed, scale, bias, n, k, g, compute=compute)
+        assert np.array_equal(got.view(np.uint32), same.view(np.uint32))
+    want = oracle.linear_i4(seen, packed, scale.astype(np.float32), bias, n, k, g)
+    err = np.abs(got.astype(np.float64) - want)
+    bound = row_gate(seen) + 1e-5 * np.abs(want)
+    if mode == "f16":
+        bound = bound + 2.0 ** -11 * np.abs(want) + 1e-7
+    assert np.all(err <= bound), float(np.max(err / bound))
+
+
+def test_few_row_epilogues_against_the_oracle_and_the_separate_ops(gpu_ctx):
+    """residual add and the gate/up pairs folded into the few-row kernel: equal to the plain
+    call followed by the oracle's add / silu-mul within one rounding of the stored type, and
+    the oracle's own chain within the gate."""
+    rng = np.random.default_rng(404)
+    m, n, k, g = 96, 1408, 2048, 128
+    packed, _q, scale = helpers.synthetic_int4(rng, n, k, g)
+    x = rng.normal(size=(m, k)).astype(np.float32)
+    bias = rng.normal(size=n).astype(np.float32)
+    residual = rng.normal(size=(m, n)).astype(np.float32)
+    plain = run_rows(gpu_ctx, x, packed, scale, bias, n, k, g, ka.COMPUTE_F32)
+    via_linear = run_linear(gpu_ctx, x, packed, scale, bias, n, k, g, compute=ka.COMPUTE_F32)
+    assert np.array_equal(plain.view(np.uint32), via_linear.view(np.uint32))
+    with_res = run_rows(gpu_ctx, x, packed, scale, bias, n, k, g, ka.COMPUTE_F32, residual=residual)
+    assert np.array_equal(with_res.view(np.uint32), (plain + residual).view(np.uint32))
+    # pairs: rows (2i, 2i+1) of w are (gate_i, up_i)
+    paired = run_rows(gpu_ctx, x, packed, scale, bias, n, k, g, ka.COMPUTE_F32,
+                      epilogue=ka.EPILOGUE_SILU_PAIRS)
+    want = oracle.linear_i4(x, packed, scale.astype(np.float32), bias, n, k, g)
+    chain = oracle.silu_mul(want[:, 0::2].astype(np.float32), want[:, 1::2].astype(np.float32))
+    scale_of = np.abs(want[:, 0::2]) * np.abs(want[:, 1::2]) + np.abs(want[:, 1::2]) + 1.0
+    assert np.all(np.abs(paired.astype(np.float64) - chain) <= 1e-4 * scale_of)
+    separate = oracle.silu_mul(plain[:, 0::2].copy(), plain[:, 1::2].copy())
+    assert np.all(np.abs(paired - separate) <= 4e-6 * scale_of)
+    # fp16 storage, the wide (64-column) tiles: n / 32 x m / 64 workgroups beyond two a CU
+    m, n, k, g = 128, 11264, 2048, 128
+    packed, _q, scale = helpers.synthetic_int4(rng, n, k, g)
+    x = rng.normal(size=(m, k)).astype(np.float16)
+    paired = run_rows(gpu_ctx, x, packed, scale, None, n, k, g, ka.COMPUTE_F16,
+                      epilogue=ka.EPILOGUE_SILU_PAIRS)
+    cols = np.unique(rng.choice(n // 2, size=96, replace=False))
+    rows = np.stack([2 * cols, 2 * cols + 1], axis=1).reshape(-1)
+    want = sampled_oracle(x.astype(np.float32), packed, scale.astype(np.float32),
+                          np.zeros(n, dtype=np.float32), n, k, g, rows)
+    chain = oracle.silu_mul(want[:, 0::2].astype(np.float32), want[:, 1::2].astype(np.float32))
+    err = np.abs(paired[:, cols].astype(np.float64) - chain)
+    assert np.all(err <= 1e-3 * np.abs(chain) + 1e-3), float(err.max())
+
+
+def test_few_row_kernel_rejects_what_it_does_not_cover(gpu_ctx):
+    rng = np.random.default_rng(1)
+    packed, _q, scale = helpers.synthetic_int4(rng, 64, 64, 16)
+    x = rng.normal(size=(20, 64)).astype(np.float32)
+    with pytest.raises(ka.GpuValidationError, match="group_size >= 64"):
+        run_rows(gpu_ctx, x, packed, scale, None, 64, 64, 16, ka.COMPUTE_F32)
+    with pytest.raises(ka.GpuValidationError, match="even n"):
+        packed, _q, scale = helpers.synthetic_int4(rng, 33, 128, 64)
+        run_rows(gpu_ctx, rng.normal(size=(20, 128)).astype(np.float32), packed, scale, None, 33,
+                 128, 64, ka.COMPUTE_F32, epilogue=ka.EPILOGUE_SILU_PAIRS)
