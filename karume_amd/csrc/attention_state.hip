@@ -174,6 +174,234 @@ __global__ __launch_bounds__(kThreads) void attention_generic_kernel(
   }
 }
 
+// ------------------------------------------------------------------- chunks of rows, MFMA
+//
+// A chunk of M > 1 rows with D = 64 or 128 (a prefill step): workgroup = (plane z, 32 query
+// rows), four waves; the key columns the 32 rows can see are walked in blocks of 32 and wave w
+// takes blocks w, w + 4, ...  All arithmetic is f32 (v_mfma_f32_32x32x2_f32: f32 products, f32
+// sums), the operand roundings are the generic kernel's: q * scale and k * scale are rounded
+// before the product.
+//   S^T = K Q^T    A = the K block (row = key), B = Q^T (column = query row): a lane ends up
+//                  with 16 scores of ONE query row (lane % 32), so the running maximum and sum
+//                  of the online softmax are per lane, plus one exchange between the two
+//                  half-waves;
+//   O^T += V^T P^T the scores a lane holds (keys 8 (i / 4) + 4 (lane / 32) + i % 4, i < 16) are
+//                  exactly a B operand if MFMA step i is given those keys, so the probabilities
+//                  never move; V^T is the A operand, read from the parked V block with the
+//                  same key per step.  The result again has the query row in lane % 32.
+// K and V blocks are parked in the wave's own LDS area (coalesced 16-byte loads; a block may
+// straddle the state slot and this step's rows).  The four waves' (max, sum, O) are merged in
+// LDS at the end; rows >= query are written as +0.
+typedef float float16v_t __attribute__((ext_vector_type(16)));
+
+template <typename T>
+__device__ inline float4 load4_f32(const T* p);
+template <>
+__device__ inline float4 load4_f32<float>(const float* p) {
+  return *reinterpret_cast<const float4*>(p);
+}
+template <>
+__device__ inline float4 load4_f32<__half>(const __half* p) {
+  const uint2 raw = *reinterpret_cast<const uint2*>(p);
+  const __half2 a = __builtin_bit_cast(__half2, raw.x), b = __builtin_bit_cast(__half2, raw.y);
+  return make_float4(__low2float(a), __high2float(a), __low2float(b), __high2float(b));
+}
+
+template <typename XT, typename ST, int D>
+__global__ __launch_bounds__(256) void attention_rows_kernel(
+    const XT* __restrict__ q, const XT* __restrict__ ins_k, const XT* __restrict__ ins_v,
+    const ST* __restrict__ slot_k, const ST* __restrict__ slot_v, XT* __restrict__ out,
+    GenericArgs a, uint32_t row_major) {
+  constexpr int kRow = D + 4;                 // floats of a parked row
+  constexpr int NT = D / 32;
+  constexpr int kHalf = D / 2;                // dims a half-wave walks
+  constexpr int kPieces = D / 4;              // 4-element pieces of a row
+  constexpr int kRowsPerLoad = 64 / kPieces;
+  constexpr int kLoads = 32 / kRowsPerLoad;
+  __shared__ __align__(16) float s_k[4][32 * kRow];
+  __shared__ __align__(16) float s_v[4][32 * kRow];
+  __shared__ float s_m[4][32], s_l[4][32];
+
+  const uint32_t z = blockIdx.x, row0 = blockIdx.y * 32u;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int r = lane & 31, h = lane >> 5;
+  uint32_t past = a.past, query = a.query;
+  if (!device_lengths(a.lengths, a.chunk_rows, a.capacity, a.window, past, query)) return;
+
+  auto out_index = [&](uint32_t row, uint32_t d) -> size_t {
+    if (row_major) {  // [B, M, H, D]
+      const uint32_t b = z / a.heads, head = z - b * a.heads;
+      return (((size_t)b * a.chunk_rows + row) * a.heads + head) * D + d;
+    }
+    return ((size_t)z * a.chunk_rows + row) * D + d;
+  };
+  if (row0 >= query) {  // a block of pad rows: exact zeros, nothing is read
+    for (uint32_t i = tid; i < 32u * D; i += 256u) {
+      const uint32_t row = row0 + i / D;
+      if (row < a.chunk_rows) st_f32<XT>(out, out_index(row, i % D), 0.0f);
+    }
+    return;
+  }
+  const uint32_t kv_plane = z / (a.heads / a.kv_heads);
+
+  // Q block -> LDS (scaled), then each lane's B operands: Q[r][h * D/2 + s]
+  for (uint32_t i = tid; i < 32u * kPieces; i += 256u) {
+    const uint32_t rr = i / kPieces, piece = i - rr * kPieces;
+    const uint32_t row = min(row0 + rr, a.chunk_rows - 1);
+    float4 v = load4_f32<XT>(q + ((size_t)z * a.chunk_rows + row) * D + 4 * piece);
+    v.x *= a.scale; v.y *= a.scale; v.z *= a.scale; v.w *= a.scale;
+    *reinterpret_cast<float4*>(&s_k[0][rr * kRow + 4 * piece]) = v;
+  }
+  __syncthreads();
+  float qf[kHalf];
+#pragma unroll
+  for (int i = 0; i < kHalf / 4; ++i) {
+    const float4 v = *reinterpret_cast<const float4*>(&s_k[0][r * kRow + h * kHalf + 4 * i]);
+    qf[4 * i] = v.x; qf[4 * i + 1] = v.y; qf[4 * i + 2] = v.z; qf[4 * i + 3] = v.w;
+  }
+  __syncthreads();
+
+  // columns the block's rows can see: [c_lo, limit_hi]
+  const uint32_t last_row = min(row0 + 31u, query - 1u);
+  const uint64_t limit_hi = (uint64_t)past + last_row;
+  const uint64_t c_lo = window_low(a.window, (uint64_t)past + row0);
+  const uint32_t blocks = (uint32_t)((limit_hi - c_lo) / 32u) + 1u;
+  const uint64_t my_limit = (uint64_t)past + row0 + (uint32_t)r;
+  const uint64_t my_low = window_low(a.window, my_limit);
+
+  float* mk = s_k[wave];
+  float* mv = s_v[wave];
+  auto wave_sync = [] {  // the areas are the wave's own: its LDS queue orders them
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+  };
+
+  float run_m = -INFINITY, run_l = 0.f;
+  float16v_t acc[NT];
+#pragma unroll
+  for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) acc[nt][i] = 0.f;
+
+  for (uint32_t kb = (uint32_t)wave; kb < blocks; kb += 4u) {
+    const uint64_t c0 = c_lo + (uint64_t)kb * 32u;
+    // park the K (scaled) and V rows of the block
+    float4 kraw[kLoads], vraw[kLoads];
+#pragma unroll
+    for (int j = 0; j < kLoads; ++j) {
+      const uint32_t key = j * kRowsPerLoad + lane / kPieces, piece = lane % kPieces;
+      uint64_t c = c0 + key;
+      c = c < limit_hi ? c : limit_hi;  // beyond the last column: any valid row, masked below
+      if (c < past) {
+        const uint64_t prow = a.window ? c % a.window : c;
+        const size_t at = ((size_t)kv_plane * a.capacity + prow) * D + 4 * piece;
+        kraw[j] = load4_f32<ST>(slot_k + at);
+        vraw[j] = load4_f32<ST>(slot_v + at);
+      } else {
+        const size_t at = ((size_t)kv_plane * a.chunk_rows + (size_t)(c - past)) * D + 4 * piece;
+        kraw[j] = load4_f32<XT>(ins_k + at);
+        vraw[j] = load4_f32<XT>(ins_v + at);
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < kLoads; ++j) {
+      const uint32_t key = j * kRowsPerLoad + lane / kPieces, piece = lane % kPieces;
+      float4 kv = kraw[j];
+      kv.x *= a.scale; kv.y *= a.scale; kv.z *= a.scale; kv.w *= a.scale;
+      *reinterpret_cast<float4*>(&mk[key * kRow + 4 * piece]) = kv;
+      *reinterpret_cast<float4*>(&mv[key * kRow + 4 * piece]) = vraw[j];
+    }
+    wave_sync();
+
+    // S^T[key][query row]: A = K[key = r][h * D/2 + s], B = Q^T
+    float16v_t st;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) st[i] = 0.f;
+#pragma unroll
+    for (int i = 0; i < kHalf / 4; ++i) {
+      const float4 kf = *reinterpret_cast<const float4*>(&mk[r * kRow + h * kHalf + 4 * i]);
+      st = __builtin_amdgcn_mfma_f32_32x32x2f32(kf.x, qf[4 * i], st, 0, 0, 0);
+      st = __builtin_amdgcn_mfma_f32_32x32x2f32(kf.y, qf[4 * i + 1], st, 0, 0, 0);
+      st = __builtin_amdgcn_mfma_f32_32x32x2f32(kf.z, qf[4 * i + 2], st, 0, 0, 0);
+      st = __builtin_amdgcn_mfma_f32_32x32x2f32(kf.w, qf[4 * i + 3], st, 0, 0, 0);
+    }
+    // this lane: query row r, keys 8 (i / 4) + 4 h + i % 4
+    float block_max = -INFINITY;
+    bool valid[16];
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      const uint64_t c = c0 + (uint32_t)(8 * (i / 4) + 4 * h + (i % 4));
+      valid[i] = c <= my_limit && c >= my_low;
+      block_max = fmaxf(block_max, valid[i] ? st[i] : -INFINITY);
+    }
+    block_max = fmaxf(block_max, __shfl_xor(block_max, 32, kWave));
+    const float new_m = fmaxf(run_m, block_max);
+    const float ref = new_m == -INFINITY ? 0.f : new_m;  // nothing seen yet: exp(-inf - 0) = 0
+    const float alpha = expf(run_m - ref);
+    float p[16], sum = 0.f;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      p[i] = valid[i] ? expf(st[i] - ref) : 0.f;
+      sum += p[i];
+    }
+    run_l = run_l * alpha + sum;
+    run_m = new_m;
+    // O^T[d][query row] = alpha * O^T + V^T P^T: step i carries the keys of register i
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) {
+#pragma unroll
+      for (int i = 0; i < 16; ++i) acc[nt][i] *= alpha;
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        const float vf = mv[(8 * (i / 4) + 4 * h + (i % 4)) * kRow + 32 * nt + r];
+        acc[nt] = __builtin_amdgcn_mfma_f32_32x32x2f32(vf, p[i], acc[nt], 0, 0, 0);
+      }
+    }
+    wave_sync();  // the block's rows have been read: the next block may be parked
+  }
+
+  // the wave's state: (max, sum) per query row and O[row][d] in its own area
+  run_l += __shfl_xor(run_l, 32, kWave);
+  if (h == 0) {
+    s_m[wave][r] = run_m;
+    s_l[wave][r] = run_l;
+  }
+#pragma unroll
+  for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+    for (int g = 0; g < 4; ++g)  // registers 4g..4g+3: dims 32 nt + 8 g + 4 h + 0..3
+      *reinterpret_cast<float4*>(&mk[r * kRow + 32 * nt + 8 * g + 4 * h]) =
+          make_float4(acc[nt][4 * g], acc[nt][4 * g + 1], acc[nt][4 * g + 2], acc[nt][4 * g + 3]);
+  __syncthreads();
+
+  // merge of the four waves, wave order; 8 threads a row
+  {
+    constexpr int kPer = D / 8;
+    const uint32_t rr = tid >> 3, d0 = (tid & 7u) * kPer;
+    const uint32_t row = row0 + rr;
+    float top = s_m[0][rr];
+#pragma unroll
+    for (int wv = 1; wv < 4; ++wv) top = fmaxf(top, s_m[wv][rr]);  // finite: the own column
+    float wgt[4], total_l = 0.f;
+#pragma unroll
+    for (int wv = 0; wv < 4; ++wv) {
+      wgt[wv] = expf(s_m[wv][rr] - top);
+      total_l = fmaf(wgt[wv], s_l[wv][rr], total_l);
+    }
+    const float inv = 1.0f / total_l;
+    if (row < a.chunk_rows) {
+#pragma unroll
+      for (int e = 0; e < kPer; ++e) {
+        float o = 0.f;
+#pragma unroll
+        for (int wv = 0; wv < 4; ++wv) o = fmaf(wgt[wv], s_k[wv][rr * kRow + d0 + e], o);
+        st_f32<XT>(out, out_index(row, d0 + e), row < query ? o * inv : 0.0f);
+      }
+    }
+  }
+}
+
 // ------------------------------------------------------------------------------ decode
 
 typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
@@ -862,6 +1090,20 @@ int32_t launch_generic(krm_ctx* ctx, krm_buf q, krm_buf ins_k, krm_buf ins_v, kr
   return launched(ctx, "attention_generic_kernel");
 }
 
+template <typename XT, typename ST>
+int32_t launch_rows(krm_ctx* ctx, krm_buf q, krm_buf ins_k, krm_buf ins_v, krm_buf slot_k,
+                    krm_buf slot_v, krm_buf out, uint32_t batch, const GenericArgs& a,
+                    uint32_t row_major) {
+  const dim3 grid(batch * a.heads, (a.chunk_rows + 31) / 32);
+#define KRM_ROWS_ATTENTION(DEPTH)                                                              \
+  attention_rows_kernel<XT, ST, DEPTH><<<grid, dim3(kThreads), 0, ctx->stream>>>(             \
+      ptr<const XT>(q), ptr<const XT>(ins_k), ptr<const XT>(ins_v), ptr<const ST>(slot_k),     \
+      ptr<const ST>(slot_v), ptr<XT>(out), a, row_major)
+  if (a.depth == 64) KRM_ROWS_ATTENTION(64); else KRM_ROWS_ATTENTION(128);
+#undef KRM_ROWS_ATTENTION
+  return launched(ctx, "attention_rows_kernel");
+}
+
 // smallest split any dtype uses for this head dim (f32 rows span the most lanes)
 uint32_t min_split_columns(uint32_t depth) {
   uint32_t lpr = decode_lanes_per_row(depth, KRM_F32);
@@ -981,6 +1223,18 @@ static int32_t attention_state_impl(krm_ctx* ctx, krm_buf q, krm_buf ins_k, krm_
 
   GenericArgs a{heads, kv_heads, chunk_rows, depth, capacity, window, past, query, half_scale,
                 ptr<uint32_t>(lengths)};
+  // chunks of rows with the usual head dims: the MFMA form
+  if (chunk_rows > 1 && (depth == 64 || depth == 128) && aligned(q, 16) && aligned(ins_k, 16) &&
+      aligned(ins_v, 16) && aligned(slot_k, 16) && aligned(slot_v, 16) &&
+      (uint64_t)batch * heads <= 0x7fffffffull && (chunk_rows + 31) / 32 <= 65535) {
+    if (io_dtype == KRM_F32 && kv_dtype == KRM_F32)
+      return launch_rows<float, float>(ctx, q, ins_k, ins_v, slot_k, slot_v, out, batch, a, 0);
+    if (io_dtype == KRM_F16 && kv_dtype == KRM_F16)
+      return launch_rows<__half, __half>(ctx, q, ins_k, ins_v, slot_k, slot_v, out, batch, a, 0);
+    if (io_dtype == KRM_F32 && kv_dtype == KRM_F16)
+      return launch_rows<float, __half>(ctx, q, ins_k, ins_v, slot_k, slot_v, out, batch, a, 0);
+    return launch_rows<__half, float>(ctx, q, ins_k, ins_v, slot_k, slot_v, out, batch, a, 0);
+  }
   if (io_dtype == KRM_F32 && kv_dtype == KRM_F32)
     return launch_generic<float, float>(ctx, q, ins_k, ins_v, slot_k, slot_v, out, batch, a);
   if (io_dtype == KRM_F16 && kv_dtype == KRM_F16)

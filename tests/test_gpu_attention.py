@@ -106,6 +106,73 @@ def test_decode_split_k(gpu_ctx, case, io, kv):
         assert np.all(err <= ulp), float(np.max(err))
 
 
+ROWS_CASES = [
+    # chunks of rows with D = 64 / 128: the matrix-core form (32 query rows a workgroup, key
+    # blocks of 32 dealt to four waves)
+    StateCase("rows D64 M128 P0 r8 (decoder prefill)", 1, 32, 4, 128, 64, 256, 0, 0, 128),
+    StateCase("rows D64 M40 Q33 P100 pad + slot/ins straddle", 2, 8, 2, 40, 64, 192, 0, 100, 33),
+    StateCase("rows D128 M64 P31 r1", 1, 4, 4, 64, 128, 128, 0, 31, 64),
+    StateCase("rows D128 M33 Q2 P0", 1, 2, 1, 33, 128, 64, 0, 0, 2),
+    StateCase("rows D64 sliding W48 P200 wrap", 2, 4, 2, 70, 64, 48, 48, 200, 70),
+    StateCase("rows D64 sliding W16 M64 Q50 gt W", 1, 4, 4, 64, 64, 16, 16, 7, 50),
+    StateCase("rows D128 sliding W100 C128 P1000", 1, 8, 2, 35, 128, 128, 100, 1000, 20),
+    StateCase("rows D64 M2 Q1 P5", 1, 4, 2, 2, 64, 16, 0, 5, 1),
+]
+
+
+@pytest.mark.parametrize("case", ROWS_CASES, ids=lambda c: c.name)
+@pytest.mark.parametrize("io,kv", [(np.float32, np.float32), (np.float16, np.float16),
+                                   (np.float32, np.float16)])
+def test_chunks_of_rows_on_the_matrix_cores(gpu_ctx, case, io, kv):
+    """M > 1 with D = 64 / 128 (f32 MFMA, online softmax per lane): the reference's gate for
+    f32 output (atol 5e-6, rtol 0); for fp16 output the same gate plus one fp16 ulp of the
+    oracle's value (the rounding of the stored result); pad rows exact +0; poison in every slot
+    row that must not be read and in the ins pad rows."""
+    x = random_state_inputs(case, seed=case.past + case.depth + case.chunk_rows, f16_values=True)
+    x["ins_k"][:, :, case.query:] = 9.0
+    x["ins_v"][:, :, case.query:] = 400.0
+    want = oracle_state_attention(case, x)
+    got = run_attention(gpu_ctx, case, x, io=io, kv=kv)
+    pad = got[:, :, case.query:, :]
+    assert np.all(pad == 0.0) and not np.any(np.signbit(pad))
+    if io == np.float32:
+        ok, fails, max_abs, worst = oracle.allclose(got, want, atol=STATE_ATOL, rtol=0)
+        assert ok, (fails, max_abs, worst)
+    else:
+        want16 = want.astype(np.float16)
+        ulp = np.abs(np.nextafter(want16, np.float16(np.inf)).astype(np.float32)
+                     - want16.astype(np.float32))
+        err = np.abs(got.astype(np.float32) - want16.astype(np.float32))
+        assert np.all(err <= ulp + STATE_ATOL), float(np.max(err - ulp))
+
+
+def test_chunks_of_rows_with_device_lengths_and_mutation_witness(gpu_ctx):
+    """The device-lengths form of a chunk equals the scalar form bit for bit, and a dropped
+    window bound, a ring taken modulo the capacity, or an ignored kv repeat (the oracle's
+    mutations) would each be seen at this gate."""
+    case = StateCase("rows D64 sliding W40 C48 P200 Q33", 2, 8, 2, 40, 64, 48, 40, 200, 33)
+    x = random_state_inputs(case, seed=5, f16_values=False)
+    got = run_attention(gpu_ctx, case, x)
+    want = oracle_state_attention(case, x)
+    ok, fails, max_abs, worst = oracle.allclose(got, want, atol=STATE_ATOL, rtol=0)
+    assert ok, (fails, max_abs, worst)
+    for mutation in (oracle.MUT_DROP_LOWER_BOUND, oracle.MUT_RING_MOD_CAPACITY,
+                     oracle.MUT_IGNORE_KV_REPEAT):
+        wrong = oracle_state_attention(case, x, mutation=mutation)
+        assert not oracle.allclose(got, wrong, atol=STATE_ATOL, rtol=0)[0], mutation
+    bufs = {k: gpu_ctx.upload(np.ascontiguousarray(v, dtype=np.float32)) for k, v in x.items()}
+    out = gpu_ctx.upload(np.full(got.size, 7.0, dtype=np.float32))
+    lengths = gpu_ctx.zeros(16)
+    gpu_ctx.lengths_set(lengths, case.past, case.query)
+    spec = {k: v for k, v in case.kwargs().items() if k not in ("past", "query")}
+    gpu_ctx.attention_state_lengths(bufs["q"], bufs["ins_k"], bufs["ins_v"], bufs["slot_k"],
+                                    bufs["slot_v"], out, half_scale=oracle.half_scale(case.depth),
+                                    lengths=lengths, max_past=case.capacity - 1, **spec)
+    again = out.download(np.float32, got.shape)
+    assert np.array_equal(again.view(np.uint32), got.view(np.uint32))
+    assert lengths.download(np.uint32, (4,))[2] == 0
+
+
 @pytest.mark.parametrize("case", DECODE_CASES, ids=lambda c: c.name)
 @pytest.mark.parametrize("io,kv", [(np.float32, np.float32), (np.float16, np.float16)])
 def test_decode_with_device_lengths_equals_scalar_form(gpu_ctx, case, io, kv):
