@@ -334,6 +334,54 @@ def bench_gemm(timer: Timer, rng, steps: int, warmup: int, m: int, n: int, k: in
     return res["ms"] / steps, 2.0 * m * n * k
 
 
+def bench_prefill_chunk(timer: Timer, rng, steps: int, warmup: int, g: int):
+    """A 128-row prefill chunk of the config-4 decoder, kernel by kernel: the four few-row
+    products of a layer (f32 activations as the model runs them, KRM_COMPUTE_F16; the f32 class
+    beside it) and the chunk's attention (32 heads, 4 kv heads, D = 64, past 0).  us per launch."""
+    ctx, ka = timer.ctx, timer.ka
+    m, d, ffn, heads, kv_heads, depth = 128, 2048, 5632, 32, 4, 64
+    out = {}
+    shapes = {"qkv": (heads * depth + 2 * kv_heads * depth, d), "o": (d, heads * depth),
+              "gate_up": (2 * ffn, d), "down": (d, ffn)}
+    copies = 8
+    for name, (n, k) in shapes.items():
+        weights = [ctx.upload(rng.integers(0, 256, size=n * k // 2, dtype=np.uint8))
+                   for _ in range(copies)]
+        scales = [ctx.upload(np.maximum(
+            np.abs(rng.normal(0, 0.02, size=(n, k // g))).astype(np.float16),
+            np.float16(6.104e-05))) for _ in range(copies)]
+        x = ctx.upload(rng.normal(size=(m, k)).astype(np.float32))
+        y = ctx.alloc(m * n * 4)
+        epilogue = ka.EPILOGUE_SILU_PAIRS if name == "gate_up" else ka.EPILOGUE_NONE
+        for label, compute in (("us", ka.COMPUTE_F16), ("f32class_us", ka.COMPUTE_F32)):
+            def step(i: int) -> None:
+                j = i % copies
+                ctx.linear_i4_rows(x, weights[j], scales[j], y, m, n, k, g, io_dtype=ka.F32,
+                                   scale_dtype=ka.F16, compute=compute, epilogue=epilogue)
+            res = timer.run(step, steps, warmup, replays=20)
+            out[f"{name}_{label}"] = round(res["ms"] / steps * 1e3, 2)
+        out[f"{name}_tflops"] = round(2.0 * m * n * k / (out[f"{name}_us"] * 1e-6) / 1e12, 1)
+        for b in weights + scales + [x, y]:
+            b.free()
+    capacity = 2048
+    q = ctx.upload(rng.normal(size=(heads, m, depth)).astype(np.float32))
+    ik = ctx.upload(rng.normal(size=(kv_heads, m, depth)).astype(np.float32))
+    iv = ctx.upload(rng.normal(size=(kv_heads, m, depth)).astype(np.float32))
+    slots = [ctx.upload(rng.normal(size=(kv_heads, capacity, depth)).astype(np.float32))
+             for _ in range(2)]
+    att = ctx.alloc(heads * m * depth * 4)
+    for label, past in (("attention_past0_us", 0), ("attention_past1024_us", 1024)):
+        def step(i: int) -> None:
+            ctx.attention_state(q, ik, iv, slots[0], slots[1], att, batch=1, heads=heads,
+                                kv_heads=kv_heads, chunk_rows=m, depth=depth, capacity=capacity,
+                                window=0, half_scale=float(depth ** -0.25), past=past, query=m)
+        res = timer.run(step, steps, warmup, replays=20)
+        out[label] = round(res["ms"] / steps * 1e3, 2)
+    for b in [q, ik, iv, att] + slots:
+        b.free()
+    return out
+
+
 def bench_w4a8(timer: Timer, rng, steps: int, warmup: int, m: int, n: int, k: int, g: int,
                copies: int):
     """w4a8 `linear` (int8 activations x int4 weights, integer dot products): one step = the
@@ -494,7 +542,7 @@ def main() -> int:
     ap.add_argument("--no-graph", action="store_true",
                     help="issue plain launches instead of replaying recorded graphs")
     ap.add_argument("--only", default="",
-                    help="gemv | gemv16 | gemm | attention | ragged | w4a8 | model | traffic: run "
+                    help="gemv | gemv16 | gemm | attention | ragged | prefill | w4a8 | model | traffic: run "
                          "only that part besides the headline GEMV")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -590,6 +638,7 @@ def main() -> int:
         bench_ragged(timer, rng, 8, 2)
         bench_gemm(timer, rng, 4, 2, 512, 11008, 4096, g)
         bench_gemm(timer, rng, 4, 2, 512, 4096, 11008, g)
+        bench_prefill_chunk(timer, rng, 4, 2, g)
     steps2 = max(16, steps // 4)
     warm2 = max(16, warmup // 4)
     if args.only in ("", "gemv16"):
@@ -629,6 +678,9 @@ def main() -> int:
             ms_g, flops = bench_gemm(timer, rng, 50, 100, 512, gn, gk, g, f32_class=True)
             result[f"gemm_{name}_f32class_us"] = round(ms_g * 1e3, 2)
             result[f"gemm_{name}_f32class_tflops"] = round(flops / (ms_g * 1e-3) / 1e12, 1)
+    if args.only in ("", "prefill"):
+        log("[bench] 128-row prefill chunk of the config-4 decoder, kernel by kernel")
+        result["prefill_chunk_m128"] = bench_prefill_chunk(timer, rng, 64, 64, g)
     if args.only in ("", "w4a8"):
         log("[bench] w4a8 linear: M=1 GEMV and M=512 up/down-projections")
         ms_q, ms_p = bench_w4a8(timer, rng, steps2, warm2, 1, n, k, g, copies)

@@ -1537,7 +1537,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2)))
 void gemm_i4_rows_kernel(const XT* __restrict__ x, const uint8_t* __restrict__ w,
                          const ST* __restrict__ scales, const XT* __restrict__ bias,
                          XT* __restrict__ out, uint32_t m, uint32_t n, uint32_t k,
-                         uint32_t group_shift, uint32_t m_blocks,
+                         uint32_t group_shift, uint32_t m_blocks, uint32_t tiles,
                          const float* __restrict__ row_scale, RowsFusion fuse) {
   constexpr int BM = 32, BN = 32 * WN, kWaves = 8;
   constexpr int NA = OPERAND == kOperandSplit ? 2 : 1;
@@ -1562,7 +1562,12 @@ void gemm_i4_rows_kernel(const XT* __restrict__ x, const uint8_t* __restrict__ w
   const int frag_row = lane & 31, frag_h = lane >> 5;
   const uint32_t groups = k >> group_shift;
   const bool half_groups = group_shift == 6;  // 64 codes a group: two groups a chunk
-  const uint32_t nb = blockIdx.x / m_blocks, mb = blockIdx.x - nb * m_blocks;
+  // blockIdx & 7 is the XCD: each XCD takes a contiguous range of tiles, the row tiles of a
+  // column tile next to each other, so the weights of a column tile come from memory once
+  const uint32_t per_xcd = (tiles + 7u) >> 3;
+  const uint32_t tile = (blockIdx.x & 7u) * per_xcd + (blockIdx.x >> 3);
+  if (tile >= tiles) return;
+  const uint32_t nb = tile / m_blocks, mb = tile - nb * m_blocks;
   const uint32_t m0 = mb * BM, n0 = nb * BN;
   const uint32_t chunks = (k + kChunk - 1) / kChunk;
   const uint32_t c_begin = (uint32_t)wave * chunks / kWaves;
@@ -1743,9 +1748,11 @@ int32_t launch_rows(krm_ctx* ctx, krm_buf x, krm_buf w, krm_buf scales, krm_buf 
     KRM_TRY(launched(ctx, "row_scale_kernel"));
   }
   const uint32_t m_blocks = (m + 31) / 32, n_blocks = (n + 32 * WN - 1) / (32 * WN);
-  gemm_i4_rows_kernel<XT, ST, OPERAND, WN><<<dim3(m_blocks * n_blocks), dim3(512), 0, ctx->stream>>>(
-      ptr<const XT>(x), ptr<const uint8_t>(w), ptr<const ST>(scales), ptr<const XT>(bias),
-      ptr<XT>(out), m, n, k, group_shift, m_blocks, ctx->row_scales, fuse);
+  const uint32_t tiles = m_blocks * n_blocks;
+  gemm_i4_rows_kernel<XT, ST, OPERAND, WN>
+      <<<dim3(((tiles + 7) / 8) * 8), dim3(512), 0, ctx->stream>>>(
+          ptr<const XT>(x), ptr<const uint8_t>(w), ptr<const ST>(scales), ptr<const XT>(bias),
+          ptr<XT>(out), m, n, k, group_shift, m_blocks, tiles, ctx->row_scales, fuse);
   return launched(ctx, "gemm_i4_rows_kernel");
 }
 
