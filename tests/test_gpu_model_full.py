@@ -9,7 +9,8 @@ Tolerance.  The random init lets the residual stream grow by about 2e4 per layer
 of the order 1e5..1e6 and an absolute gate means nothing across seeds; the gate is relative to
 the largest |logit| of the row.  f32 arithmetic (KRM_COMPUTE_F32 prefill, the reference's
 default linearCompute): worst measured 1.64e-7, gate 3.5e-7.  fp16-operand prefill
-(KRM_COMPUTE_F16, what bench.py times): worst measured 5.69e-5, gate 1.2e-4.  The token of a row
+(KRM_COMPUTE_F16, what bench.py times: x rounded to fp16 at every product of the chunk): worst
+measured 6.34e-5, gate 1.2e-4.  The token of a row
 must equal the oracle's argmax wherever the oracle's top-1/top-2 margin exceeds twice the gate.
 """
 import time
