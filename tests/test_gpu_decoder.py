@@ -414,3 +414,60 @@ def test_session_from_a_model_file_equals_session_from_arrays(gpu_ctx):
     for (tok_a, log_a), (tok_b, log_b) in zip(rows_a, rows_b):
         assert np.array_equal(tok_a, tok_b)
         assert log_a.tobytes() == log_b.tobytes()
+
+
+@pytest.mark.parametrize("io,compute,m", [(ka.F32, ka.COMPUTE_F32, 40), (ka.F32, ka.COMPUTE_F16, 128),
+                                          (ka.F16, ka.COMPUTE_F16, 33), (ka.F32, ka.COMPUTE_F32, 5)])
+def test_prefill_qkv_equals_linear_rope_transpose(gpu_ctx, io, compute, m):
+    """krm_prefill_qkv (fused [q;k;v] projection of a chunk on pair-interleaved rows + RoPE,
+    head-major) writes the same bits as krm_linear_i4_rows on the natural rows followed by
+    krm_rope_half (to head-major) for q and k and krm_transpose_01 for v; a position outside
+    the table gives NaN in that row of q and k only."""
+    from karume_amd.decoder import Int4Linear, _rope_pair_rows, _stack_rows
+    rng = np.random.default_rng(100 + m)
+    heads, kv_heads, d, table, k, group = 8, 2, 64, 200, 512, 128
+    io_np = np.float32 if io == ka.F32 else np.float16
+    eb = np.dtype(io_np).itemsize
+    hq, hk = heads * d, kv_heads * d
+    n = hq + 2 * hk
+    packed, _codes, scales = helpers.synthetic_int4(rng, n, k, group)
+    packed = packed.reshape(n, k // 2)
+    x = rng.normal(size=(m, k)).astype(io_np)
+    ang = rng.normal(size=(table, d))
+    cos, sin = np.cos(ang).astype(np.float32), np.sin(ang).astype(np.float32)
+    pos = rng.integers(0, table, size=m).astype(np.int32)
+    pos[m // 2] = table + 3                       # outside the table
+    dx, dc, ds, dp = map(gpu_ctx.upload, (x, cos, sin, pos))
+
+    def linear(lo, hi):
+        out = gpu_ctx.alloc(m * (hi - lo) * eb)
+        gpu_ctx.linear_i4_rows(dx, gpu_ctx.upload(packed[lo:hi]), gpu_ctx.upload(scales[lo:hi]), out,
+                               m, hi - lo, k, group, io_dtype=io, scale_dtype=ka.F16,
+                               compute=compute)
+        return out
+    q, kk, v = linear(0, hq), linear(hq, hq + hk), linear(hq + hk, n)
+    want_q, want_k, want_v = (gpu_ctx.alloc(m * hq * eb), gpu_ctx.alloc(m * hk * eb),
+                              gpu_ctx.alloc(m * hk * eb))
+    gpu_ctx.rope_half(q, dp, dc, ds, want_q, m, heads, d, table, True, io)
+    gpu_ctx.rope_half(kk, dp, dc, ds, want_k, m, kv_heads, d, table, True, io)
+    gpu_ctx.transpose_01(v, want_v, m, kv_heads, d, io)
+
+    def part(lo, hi):
+        return Int4Linear(hi - lo, k, packed[lo:hi], scales[lo:hi])
+    fused = _stack_rows(_rope_pair_rows(part(0, hq), d), _rope_pair_rows(part(hq, hq + hk), d),
+                        part(hq + hk, n))
+    got_q, got_k, got_v = (gpu_ctx.zeros(m * hq * eb), gpu_ctx.zeros(m * hk * eb),
+                           gpu_ctx.zeros(m * hk * eb))
+    gpu_ctx.prefill_qkv(dx, gpu_ctx.upload(fused.packed), gpu_ctx.upload(fused.scales), dp, dc, ds,
+                        got_q, got_k, got_v, m=m, heads=heads, kv_heads=kv_heads, depth=d, k=k,
+                        group=group, table_rows=table, io_dtype=io, scale_dtype=ka.F16,
+                        compute=compute)
+    bits = np.uint32 if io == ka.F32 else np.uint16
+    for got, want, planes in ((got_q, want_q, heads), (got_k, want_k, kv_heads),
+                              (got_v, want_v, kv_heads)):
+        a = got.download(io_np, (planes, m, d))
+        b = want.download(io_np, (planes, m, d))
+        assert np.array_equal(a.view(bits), b.view(bits))
+    q_host = got_q.download(io_np, (heads, m, d))
+    assert np.all(np.isnan(q_host[:, m // 2])) and not np.any(np.isnan(np.delete(q_host, m // 2, 1)))
+    assert not np.any(np.isnan(got_v.download(io_np, (kv_heads, m, d))))
