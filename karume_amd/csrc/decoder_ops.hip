@@ -179,6 +179,37 @@ __global__ __launch_bounds__(kArgmaxThreads) void argmax_kernel(const XT* __rest
   const size_t base = (size_t)blockIdx.x * dim;
   float best = -INFINITY;
   uint32_t at = dim;  // sentinel: any real element beats it on the index comparison
+  // f32 rows of whole 16-byte pieces: four elements a load (a quarter of the load instructions —
+  // one workgroup's vector-memory path is what a 128 KB row costs)
+  if constexpr (sizeof(XT) == 4) {
+    if ((dim & 3u) == 0 && (((uintptr_t)(x + base)) & 15u) == 0) {
+      const uint32_t pieces = dim >> 2;
+      const float4* src = reinterpret_cast<const float4*>(x + base);
+      constexpr int kWide = 8;
+      for (uint32_t p0 = threadIdx.x; p0 < pieces; p0 += kArgmaxThreads * kWide) {
+        float4 v[kWide];
+#pragma unroll
+        for (int u = 0; u < kWide; ++u) {
+          const uint32_t p = p0 + u * kArgmaxThreads;
+          v[u] = src[p < pieces ? p : p0];
+        }
+#pragma unroll
+        for (int u = 0; u < kWide; ++u) {
+          const uint32_t p = p0 + u * kArgmaxThreads;
+          if (p < pieces) {
+            const float e[4] = {v[u].x, v[u].y, v[u].z, v[u].w};
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+              if (beats(e[j], 4 * p + j, best, at)) {
+                best = e[j];
+                at = 4 * p + j;
+              }
+          }
+        }
+      }
+      dim = 0;  // the scalar walk below has nothing left
+    }
+  }
   for (uint32_t i0 = threadIdx.x; i0 < dim; i0 += kArgmaxThreads * kArgmaxUnroll) {
     float v[kArgmaxUnroll];
 #pragma unroll
