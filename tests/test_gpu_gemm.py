@@ -338,3 +338,22 @@ def test_few_row_kernel_rejects_what_it_does_not_cover(gpu_ctx):
         packed, _q, scale = helpers.synthetic_int4(rng, 33, 128, 64)
         run_rows(gpu_ctx, rng.normal(size=(20, 128)).astype(np.float32), packed, scale, None, 33,
                  128, 64, ka.COMPUTE_F32, epilogue=ka.EPILOGUE_SILU_PAIRS)
+
+
+@pytest.mark.parametrize("compute", [ka.COMPUTE_F32, ka.COMPUTE_F16])
+def test_few_row_results_do_not_depend_on_the_batch(gpu_ctx, compute):
+    """In the reference an output row has the same bits whatever M is
+    (packages/runtime/tests/gpu_gemm_skinny_test.ts:11-15,156-198).  The few-row kernel keeps
+    that: a row's products, its split over the eight waves (a function of K) and the order of the
+    final sum do not depend on the other rows, on the row's place in the chunk, or on the tile
+    width chosen for the chunk (32 or 64 columns)."""
+    rng = np.random.default_rng(808)
+    n, k, g = 4224, 1024, 128      # 128 rows: 4 x 132 tiles > 256 CUs -> 64-column tiles
+    packed, _q, scale = helpers.synthetic_int4(rng, n, k, g)
+    x = rng.normal(size=(128, k)).astype(np.float32)
+    x[5] *= 1e4
+    bias = rng.normal(size=n).astype(np.float32)
+    whole = run_rows(gpu_ctx, x, packed, scale, bias, n, k, g, compute)
+    for rows in ([5], [0, 5, 77], list(range(40, 73))):   # 1, 3 and 33 rows: 32-column tiles
+        part = run_rows(gpu_ctx, x[rows], packed, scale, bias, n, k, g, compute)
+        assert np.array_equal(part.view(np.uint32), whole[rows].view(np.uint32)), rows
