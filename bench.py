@@ -498,7 +498,52 @@ def cpu_baseline(n: int, k: int, g: int, budget_s: float = 12.0):
         reps += 1
     dt = time.perf_counter() - t0
     result["w4a8_gemv_us"] = round(dt / reps * 1e6, 1)
+    torch_leg = torch_cpu_baseline(packed, scale, x, n, k, g, cores)
+    if torch_leg is not None:
+        result["torch_cpu"] = torch_leg
     return result
+
+
+def torch_cpu_baseline(packed, scale, x, n: int, k: int, g: int, cores: int):
+    """PyTorch-CPU lowering of the same two ops with library calls: F.linear on the dequantised
+    f32 weight (config 0) and scaled_dot_product_attention on config 2's shapes (f32, GQA expanded),
+    about 2 s each.  None when torch is not importable."""
+    try:
+        import torch
+        import torch.nn.functional as F
+    except Exception:
+        return None
+    from oracle import oracle
+    torch.set_num_threads(cores)
+    weight = torch.from_numpy(oracle.decode_i4(packed, [n, k], scale, [n, k // g], g))
+    xt = torch.from_numpy(x)
+    out = {"threads": cores}
+    with torch.no_grad():
+        F.linear(xt, weight)
+        reps, t0 = 0, time.perf_counter()
+        while time.perf_counter() - t0 < 2.0:
+            F.linear(xt, weight)
+            reps += 1
+        dt = (time.perf_counter() - t0) / reps
+        out["linear_f32_gemv_us"] = round(dt * 1e6, 1)
+        out["linear_f32_weight_gbs"] = round(n * k * 4 / dt / 1e9, 1)
+        heads, kv_heads, depth, length = 32, 8, 128, 4096
+        gen = torch.Generator().manual_seed(3)
+        q = torch.randn(1, heads, 1, depth, generator=gen)
+        kk = torch.randn(1, kv_heads, length, depth, generator=gen).repeat_interleave(
+            heads // kv_heads, dim=1)
+        vv = torch.randn(1, kv_heads, length, depth, generator=gen).repeat_interleave(
+            heads // kv_heads, dim=1)
+        F.scaled_dot_product_attention(q, kk, vv)
+        reps, t0 = 0, time.perf_counter()
+        while time.perf_counter() - t0 < 2.0:
+            F.scaled_dot_product_attention(q, kk, vv)
+            reps += 1
+        out["sdpa_config2_us"] = round((time.perf_counter() - t0) / reps * 1e6, 1)
+    out["sample"] = ("F.linear(x f32 [1,4096], dequantised W f32 [4096,4096]) and "
+                     "scaled_dot_product_attention(q [1,32,1,128], K/V [1,32,4096,128] f32), "
+                     "about 2 s each")
+    return out
 
 
 def cpu_decode_baseline(g: int, tokens: int = 3):
