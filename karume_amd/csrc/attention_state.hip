@@ -505,9 +505,19 @@ __host__ __device__ inline uint32_t decode_split_columns(uint32_t lanes_per_row)
 __host__ __device__ inline uint32_t decode_chunks(uint64_t slot_columns, uint32_t chunk_columns) {
   return (uint32_t)((slot_columns + chunk_columns - 1) / chunk_columns);
 }
+// Chunks a split of a long past walks.  Two (both requested before the first is scored) halve
+// the partials and help a launch that is bandwidth-bound — the 16-sequence ragged batch went
+// from 36.7 to 33.9 us — but a single 4096-column sequence then has 256 workgroups instead of
+// 512 and went from 10.1 to 12.6 us; the partition has to be the same function of a
+// sequence's columns in both launches (a sequence gives the same bits alone and in a batch),
+// so it stays at one.
+#ifndef KRM_SPLIT_CHUNKS
+#define KRM_SPLIT_CHUNKS 1
+#endif
+constexpr uint32_t kSplitChunks = KRM_SPLIT_CHUNKS;
 __host__ __device__ inline uint32_t decode_splits(uint64_t slot_columns, uint32_t chunk_columns) {
   const uint32_t chunks = decode_chunks(slot_columns, chunk_columns);
-  return chunks <= kSingleSplitChunks ? 1u : chunks;
+  return chunks <= kSingleSplitChunks ? 1u : (chunks + kSplitChunks - 1) / kSplitChunks;
 }
 
 constexpr float kLog2e = 1.4426950408889634f;
@@ -611,7 +621,7 @@ void attention_decode_kernel(
     early = a.lengths != nullptr && a.window == 0;
     if (early) {
       const size_t base = (size_t)blockIdx.z * a.slot_batch_stride + (size_t)hk * a.slot_plane_stride;
-      const uint32_t want = blockIdx.x * (uint32_t)kChunkCols;
+      const uint32_t want = blockIdx.x * (kSplitChunks * (uint32_t)kChunkCols);
       const uint32_t c_begin = want < a.capacity ? want : a.capacity - 1u;
       const uint32_t room = a.capacity - c_begin;
       request_rows(slot_k + base, slot_v + base, 0u, c_begin,
@@ -659,8 +669,9 @@ void attention_decode_kernel(
   }
   const uint32_t low = (uint32_t)window_low(a.window, past);  // limit of row 0 is `past`
   const uint32_t total_chunks = decode_chunks(past - low, kChunkCols);
-  const uint32_t my_chunks = nsplit == 1 ? total_chunks : 1u;
-  const uint32_t c_first = low + split * kChunkCols;  // < past
+  const uint32_t my_chunks =
+      nsplit == 1 ? total_chunks : min(kSplitChunks, total_chunks - split * kSplitChunks);
+  const uint32_t c_first = low + split * (kSplitChunks * kChunkCols);  // < past (split 0 alone)
   const bool last = split + 1 == nsplit;
 
   const size_t slot_base = (size_t)seq * a.slot_batch_stride + (size_t)hk * a.slot_plane_stride;
@@ -832,10 +843,18 @@ void attention_decode_kernel(
     }
   }
   if (!walked && my_chunks > 0) {
-    consume_chunk(0, rows0);
-    for (uint32_t chunk = 1; chunk < my_chunks; ++chunk) {
-      load_chunk(chunk, rows0);
-      consume_chunk(chunk, rows0);
+    if (kSplitChunks == 2 && nsplit > 1 && my_chunks == 2) {
+      // a split of a long past: both chunks requested before the first is scored
+      ChunkRows rows1;
+      load_chunk(1, rows1);
+      consume_chunk(0, rows0);
+      consume_chunk(1, rows1);
+    } else {
+      consume_chunk(0, rows0);
+      for (uint32_t chunk = 1; chunk < my_chunks; ++chunk) {
+        load_chunk(chunk, rows0);
+        consume_chunk(chunk, rows0);
+      }
     }
   }
   // this step's own column: one more row for group 0 of the last split (for every other lane
