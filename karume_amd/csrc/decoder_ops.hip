@@ -46,6 +46,28 @@ __global__ __launch_bounds__(kThreads) void rms_norm_kernel(const XT* __restrict
                                                            float eps) {
   __shared__ float scratch[kThreads / kWave];
   const size_t base = (size_t)blockIdx.x * dim;
+  constexpr int kKeep = 16;  // rows up to 4096 elements stay in registers: one trip to memory
+  if (dim <= (uint32_t)(kThreads * kKeep)) {
+    float v[kKeep], wv[kKeep];
+#pragma unroll
+    for (int j = 0; j < kKeep; ++j) {
+      const uint32_t i = threadIdx.x + j * kThreads;
+      v[j] = i < dim ? ld<XT>(x, base + i) : 0.f;
+      wv[j] = i < dim ? weight[i] : 0.f;
+    }
+    float squares = 0.f;  // the same elements in the same order as the loop below
+#pragma unroll
+    for (int j = 0; j < kKeep; ++j)
+      if (threadIdx.x + j * kThreads < dim) squares = fmaf(v[j], v[j], squares);
+    const float total = block_sum(squares, scratch);
+    const float inv = 1.0f / sqrtf(total / (float)dim + eps);
+#pragma unroll
+    for (int j = 0; j < kKeep; ++j) {
+      const uint32_t i = threadIdx.x + j * kThreads;
+      if (i < dim) st<XT>(out, base + i, v[j] * inv * wv[j]);
+    }
+    return;
+  }
   float squares = 0.f;
   for (uint32_t i = threadIdx.x; i < dim; i += kThreads) {
     const float v = ld<XT>(x, base + i);
