@@ -76,6 +76,13 @@ export const KARUME_HIP_SYMBOLS = {
     ],
     result: "i32",
   },
+  krm_attention_chunk: {
+    parameters: [
+      "pointer", "u64", "u64", "u64", "u64", "u64", "u64", "u32", "u32", "u32", "u32", "u32",
+      "u32", "u32", "f32", "u32", "u32", "u64", "i32", "i32", "u32"
+    ],
+    result: "i32",
+  },
   krm_attention_state_noalloc: {
     parameters: [
       "pointer", "u64", "u64", "u64", "u64", "u64", "u64", "u32", "u32", "u32", "u32", "u32",

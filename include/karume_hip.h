@@ -252,6 +252,28 @@ int32_t krm_attention_state_noalloc(krm_ctx* ctx, krm_buf q, krm_buf ins_k, krm_
                                     float half_scale, uint32_t past, uint32_t query,
                                     int32_t io_dtype, int32_t kv_dtype);
 
+/* The attention of a chunk of rows (a prefill step) with what a decoder layer does around it
+ * folded in; D = 64 or 128 and 16-byte aligned buffers, anything else is rejected (the three
+ * separate calls remain).  Arguments as krm_attention_state; `lengths` != 0 reads past / query
+ * on the device as krm_attention_state_lengths does.  No workspace.
+ *   KRM_CHUNK_OUT_ROW_MAJOR : `out` is [B, M, H, D] (what the o-projection reads) instead of
+ *                             [B, H, M, D] — the permute + reshape nodes behind the attention
+ *   KRM_CHUNK_APPEND        : the first `query` rows of ins_k / ins_v are also appended to the
+ *                             slots (krm_state_append's result, same roundings).  window == 0
+ *                             only: slot rows past.. are read by nobody in this launch, while a
+ *                             ring would overwrite rows it still reads (docs/ir-v1.md:345-348).
+ * Fuses packages/runtime/src/kernels/state-attention.ts:169-552 with
+ * packages/runtime/src/kernels/state-append.ts:47-96 and the permute of
+ * tools/export-recipes/minicpm5/export_decode.py:14-35. */
+#define KRM_CHUNK_OUT_ROW_MAJOR 1u
+#define KRM_CHUNK_APPEND 2u
+int32_t krm_attention_chunk(krm_ctx* ctx, krm_buf q, krm_buf ins_k, krm_buf ins_v, krm_buf slot_k,
+                            krm_buf slot_v, krm_buf out, uint32_t batch, uint32_t heads,
+                            uint32_t kv_heads, uint32_t chunk_rows, uint32_t depth,
+                            uint32_t capacity, uint32_t window, float half_scale, uint32_t past,
+                            uint32_t query, krm_buf lengths, int32_t io_dtype, int32_t kv_dtype,
+                            uint32_t flags);
+
 /* ---- state_append (packages/runtime/src/kernels/state-append.ts:47-96,120-173;
  *      builder packages/runtime/src/runtime/recipe-builder.ts:2011-2048) --------------------
  * Copies the first `query` rows of x[kv_planes, M, D] (x_dtype) into

@@ -60,6 +60,8 @@ PROTOTYPES = {
     "krm_attention_state": (i32, [c_ctx, c_buf, c_buf, c_buf, c_buf, c_buf, c_buf, u32, u32, u32,
                                   u32, u32, u32, u32, C.c_float, u32, u32, i32, i32, c_buf,
                                   size_t]),
+    "krm_attention_chunk": (i32, [c_ctx, c_buf, c_buf, c_buf, c_buf, c_buf, c_buf, u32, u32, u32,
+                                  u32, u32, u32, u32, C.c_float, u32, u32, c_buf, i32, i32, u32]),
     "krm_attention_state_noalloc": (i32, [c_ctx, c_buf, c_buf, c_buf, c_buf, c_buf, c_buf, u32,
                                           u32, u32, u32, u32, u32, u32, C.c_float, u32, u32, i32,
                                           i32]),

@@ -210,8 +210,8 @@ __device__ inline float4 load4_f32<__half>(const __half* p) {
 template <typename XT, typename ST, int D>
 __global__ __launch_bounds__(256) void attention_rows_kernel(
     const XT* __restrict__ q, const XT* __restrict__ ins_k, const XT* __restrict__ ins_v,
-    const ST* __restrict__ slot_k, const ST* __restrict__ slot_v, XT* __restrict__ out,
-    GenericArgs a, uint32_t row_major) {
+    ST* __restrict__ slot_k, ST* __restrict__ slot_v, XT* __restrict__ out,
+    GenericArgs a, uint32_t flags) {
   constexpr int kRow = D + 4;                 // floats of a parked row
   constexpr int NT = D / 32;
   constexpr int kHalf = D / 2;                // dims a half-wave walks
@@ -228,6 +228,7 @@ __global__ __launch_bounds__(256) void attention_rows_kernel(
   uint32_t past = a.past, query = a.query;
   if (!device_lengths(a.lengths, a.chunk_rows, a.capacity, a.window, past, query)) return;
 
+  const bool row_major = (flags & KRM_CHUNK_OUT_ROW_MAJOR) != 0;
   auto out_index = [&](uint32_t row, uint32_t d) -> size_t {
     if (row_major) {  // [B, M, H, D]
       const uint32_t b = z / a.heads, head = z - b * a.heads;
@@ -235,6 +236,24 @@ __global__ __launch_bounds__(256) void attention_rows_kernel(
     }
     return ((size_t)z * a.chunk_rows + row) * D + d;
   };
+  // The chunk's own K / V rows of this block go to the state slots here when asked for (the
+  // first query head of each kv plane does it).  Without a window no reader of this launch
+  // touches them: slot rows are read for columns < past only, these are rows past + row.
+  if ((flags & KRM_CHUNK_APPEND) && z % (a.heads / a.kv_heads) == 0) {
+    const uint32_t plane = z / (a.heads / a.kv_heads);
+    for (uint32_t i = tid; i < 32u * kPieces; i += 256u) {
+      const uint32_t rr = i / kPieces, piece = i - rr * kPieces;
+      const uint32_t row = row0 + rr;
+      if (row >= query) continue;
+      const size_t src = ((size_t)plane * a.chunk_rows + row) * D + 4 * piece;
+      const size_t dst = ((size_t)plane * a.capacity + past + row) * D + 4 * piece;
+      const float4 kv = load4_f32<XT>(ins_k + src), vv = load4_f32<XT>(ins_v + src);
+      st_f32<ST>(slot_k, dst, kv.x); st_f32<ST>(slot_k, dst + 1, kv.y);
+      st_f32<ST>(slot_k, dst + 2, kv.z); st_f32<ST>(slot_k, dst + 3, kv.w);
+      st_f32<ST>(slot_v, dst, vv.x); st_f32<ST>(slot_v, dst + 1, vv.y);
+      st_f32<ST>(slot_v, dst + 2, vv.z); st_f32<ST>(slot_v, dst + 3, vv.w);
+    }
+  }
   if (row0 >= query) {  // a block of pad rows: exact zeros, nothing is read
     for (uint32_t i = tid; i < 32u * D; i += 256u) {
       const uint32_t row = row0 + i / D;
@@ -1112,12 +1131,12 @@ int32_t launch_generic(krm_ctx* ctx, krm_buf q, krm_buf ins_k, krm_buf ins_v, kr
 template <typename XT, typename ST>
 int32_t launch_rows(krm_ctx* ctx, krm_buf q, krm_buf ins_k, krm_buf ins_v, krm_buf slot_k,
                     krm_buf slot_v, krm_buf out, uint32_t batch, const GenericArgs& a,
-                    uint32_t row_major) {
+                    uint32_t flags) {
   const dim3 grid(batch * a.heads, (a.chunk_rows + 31) / 32);
 #define KRM_ROWS_ATTENTION(DEPTH)                                                              \
   attention_rows_kernel<XT, ST, DEPTH><<<grid, dim3(kThreads), 0, ctx->stream>>>(             \
-      ptr<const XT>(q), ptr<const XT>(ins_k), ptr<const XT>(ins_v), ptr<const ST>(slot_k),     \
-      ptr<const ST>(slot_v), ptr<XT>(out), a, row_major)
+      ptr<const XT>(q), ptr<const XT>(ins_k), ptr<const XT>(ins_v), ptr<ST>(slot_k),           \
+      ptr<ST>(slot_v), ptr<XT>(out), a, flags)
   if (a.depth == 64) KRM_ROWS_ATTENTION(64); else KRM_ROWS_ATTENTION(128);
 #undef KRM_ROWS_ATTENTION
   return launched(ctx, "attention_rows_kernel");
@@ -1160,7 +1179,8 @@ static int32_t attention_state_impl(krm_ctx* ctx, krm_buf q, krm_buf ins_k, krm_
                                     float half_scale, uint32_t past, uint32_t query,
                                     krm_buf lengths, int32_t io_dtype, int32_t kv_dtype,
                                     krm_buf workspace, size_t workspace_bytes,
-                                    uint32_t* tickets = nullptr, uint32_t ticket_slots = 0) {
+                                    uint32_t* tickets = nullptr, uint32_t ticket_slots = 0,
+                                    uint32_t chunk_flags = 0, bool chunk_only = false) {
   KRM_TRY(enter(ctx));
   const bool dyn = lengths != 0;
   KRM_REQUIRE(ctx, aligned(lengths, 4), "krm_attention_state: misaligned lengths buffer");
@@ -1202,7 +1222,8 @@ static int32_t attention_state_impl(krm_ctx* ctx, krm_buf q, krm_buf ins_k, krm_
 
   const uint32_t repeat = heads / kv_heads;
   const uint32_t lpr = decode_lanes_per_row(depth, kv_dtype);
-  const bool fast = (dyn || query == 1) && chunk_rows == 1 && lpr && decode_repeat_ok(repeat) &&
+  const bool fast = !chunk_only && (dyn || query == 1) && chunk_rows == 1 && lpr &&
+                    decode_repeat_ok(repeat) &&
                     aligned(slot_k, 16) && aligned(slot_v, 16) && aligned(q, 16) && batch <= 65535 &&
                     heads <= 65535 && (uint64_t)batch * heads <= kTicketSlots;
   if (fast) {
@@ -1243,17 +1264,22 @@ static int32_t attention_state_impl(krm_ctx* ctx, krm_buf q, krm_buf ins_k, krm_
   GenericArgs a{heads, kv_heads, chunk_rows, depth, capacity, window, past, query, half_scale,
                 ptr<uint32_t>(lengths)};
   // chunks of rows with the usual head dims: the MFMA form
-  if (chunk_rows > 1 && (depth == 64 || depth == 128) && aligned(q, 16) && aligned(ins_k, 16) &&
-      aligned(ins_v, 16) && aligned(slot_k, 16) && aligned(slot_v, 16) &&
+  if ((chunk_rows > 1 || chunk_only) && (depth == 64 || depth == 128) && aligned(q, 16) &&
+      aligned(ins_k, 16) && aligned(ins_v, 16) && aligned(slot_k, 16) && aligned(slot_v, 16) &&
       (uint64_t)batch * heads <= 0x7fffffffull && (chunk_rows + 31) / 32 <= 65535) {
+    const uint32_t f = chunk_flags;
     if (io_dtype == KRM_F32 && kv_dtype == KRM_F32)
-      return launch_rows<float, float>(ctx, q, ins_k, ins_v, slot_k, slot_v, out, batch, a, 0);
+      return launch_rows<float, float>(ctx, q, ins_k, ins_v, slot_k, slot_v, out, batch, a, f);
     if (io_dtype == KRM_F16 && kv_dtype == KRM_F16)
-      return launch_rows<__half, __half>(ctx, q, ins_k, ins_v, slot_k, slot_v, out, batch, a, 0);
+      return launch_rows<__half, __half>(ctx, q, ins_k, ins_v, slot_k, slot_v, out, batch, a, f);
     if (io_dtype == KRM_F32 && kv_dtype == KRM_F16)
-      return launch_rows<float, __half>(ctx, q, ins_k, ins_v, slot_k, slot_v, out, batch, a, 0);
-    return launch_rows<__half, float>(ctx, q, ins_k, ins_v, slot_k, slot_v, out, batch, a, 0);
+      return launch_rows<float, __half>(ctx, q, ins_k, ins_v, slot_k, slot_v, out, batch, a, f);
+    return launch_rows<__half, float>(ctx, q, ins_k, ins_v, slot_k, slot_v, out, batch, a, f);
   }
+  if (chunk_only)
+    return fail(ctx, KRM_ERR_VALIDATION,
+                "krm_attention_chunk: covers D = 64 or 128 and 16-byte aligned buffers (D = %u); "
+                "use krm_attention_state, krm_state_append and krm_transpose_01", depth);
   if (io_dtype == KRM_F32 && kv_dtype == KRM_F32)
     return launch_generic<float, float>(ctx, q, ins_k, ins_v, slot_k, slot_v, out, batch, a);
   if (io_dtype == KRM_F16 && kv_dtype == KRM_F16)
@@ -1285,6 +1311,23 @@ int32_t krm_attention_state_lengths(krm_ctx* ctx, krm_buf q, krm_buf ins_k, krm_
   return attention_state_impl(ctx, q, ins_k, ins_v, slot_k, slot_v, out, batch, heads, kv_heads,
                               chunk_rows, depth, capacity, window, half_scale, max_past,
                               chunk_rows, lengths, io_dtype, kv_dtype, workspace, workspace_bytes);
+}
+
+int32_t krm_attention_chunk(krm_ctx* ctx, krm_buf q, krm_buf ins_k, krm_buf ins_v, krm_buf slot_k,
+                            krm_buf slot_v, krm_buf out, uint32_t batch, uint32_t heads,
+                            uint32_t kv_heads, uint32_t chunk_rows, uint32_t depth,
+                            uint32_t capacity, uint32_t window, float half_scale, uint32_t past,
+                            uint32_t query, krm_buf lengths, int32_t io_dtype, int32_t kv_dtype,
+                            uint32_t flags) {
+  KRM_REQUIRE(ctx, (flags & ~(uint32_t)(KRM_CHUNK_OUT_ROW_MAJOR | KRM_CHUNK_APPEND)) == 0,
+              "krm_attention_chunk: unknown flags 0x%x", flags);
+  KRM_REQUIRE(ctx, !(flags & KRM_CHUNK_APPEND) || window == 0,
+              "krm_attention_chunk: the fused append needs window == 0 (a ring overwrites rows "
+              "this launch still reads); call krm_state_append after the attention");
+  return attention_state_impl(ctx, q, ins_k, ins_v, slot_k, slot_v, out, batch, heads, kv_heads,
+                              chunk_rows, depth, capacity, window, half_scale,
+                              lengths ? capacity - 1 : past, lengths ? chunk_rows : query, lengths,
+                              io_dtype, kv_dtype, 0, 0, nullptr, 0, flags, true);
 }
 
 int32_t krm_attention_varlen_workspace(uint32_t nseq, uint32_t heads, uint32_t kv_heads,

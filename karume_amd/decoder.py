@@ -339,6 +339,17 @@ class LlamaDecoderSession:
         self._linear(b["xn"], self.lm_head, b["logits"], 1)
         g.argmax(b["logits"], b["token"], 1, c.vocab, io)
 
+    def _append_chunk(self, context: GenerationContext, li: int, past: int, query: int,
+                      lengths: Optional[DeviceBuffer], spec: dict) -> None:
+        g, c, b, io = self.gpu, self.config, self.buf, self.io_dtype
+        for src, slot in ((b["kr"], context.slots_k[li]), (b["vt"], context.slots_v[li])):
+            if lengths is None:
+                g.state_append(src, slot, kv_planes=c.kv_heads, past=past, query=query,
+                               x_dtype=io, slot_dtype=self.kv_dtype, **spec)
+            else:
+                g.state_append_lengths(src, slot, kv_planes=c.kv_heads, lengths=lengths,
+                                       x_dtype=io, slot_dtype=self.kv_dtype, **spec)
+
     def _rows_form_covers(self) -> bool:
         """The chunk-of-rows launches need groups of 64 codes or more and K a multiple of 32."""
         c = self.config
@@ -347,9 +358,10 @@ class LlamaDecoderSession:
 
     def _forward_rows(self, context: GenerationContext, m: int, past: int, query: int,
                       lengths: Optional[DeviceBuffer]) -> None:
-        """A chunk of m > 16 rows, 10 launches a layer: the [q; k; v] projection writes roped,
-        head-major q / k / v, the o and down projections add the residual in place, the gate/up
-        projection applies silu * up."""
+        """A chunk of m > 16 rows, 7 launches a layer: the [q; k; v] projection writes roped,
+        head-major q / k / v, the attention writes row-major and appends the chunk's K / V rows,
+        the o and down projections add the residual in place, the gate/up projection applies
+        silu * up."""
         from .runtime import EPILOGUE_SILU_PAIRS
         g, c, b, io = self.gpu, self.config, self.buf, self.io_dtype
         d, group, compute = c.d_model, c.group_size, self.prefill_compute
@@ -362,31 +374,34 @@ class LlamaDecoderSession:
                           b["kr"], b["vt"], m=m, heads=c.heads, kv_heads=c.kv_heads,
                           depth=c.head_dim, k=d, group=group, table_rows=c.max_position,
                           io_dtype=io, scale_dtype=lin.scale_dtype, compute=compute)
-            if lengths is None:
-                g.attention_state(b["qr"], b["kr"], b["vt"], context.slots_k[li],
-                                  context.slots_v[li], b["att"], batch=1, heads=c.heads,
+            if c.head_dim in (64, 128):
+                # attention + output permute (+ both appends when no window can wrap) in one launch
+                g.attention_chunk(b["qr"], b["kr"], b["vt"], context.slots_k[li],
+                                  context.slots_v[li], b["att2"], batch=1, heads=c.heads,
                                   kv_heads=c.kv_heads, half_scale=c.half_scale, past=past,
-                                  query=query, io_dtype=io, kv_dtype=self.kv_dtype,
-                                  workspace=self.workspace, **spec)
-                # readers first, then the appends (docs/ir-v1.md:345-348)
-                g.state_append(b["kr"], context.slots_k[li], kv_planes=c.kv_heads, past=past,
-                               query=query, x_dtype=io, slot_dtype=self.kv_dtype, **spec)
-                g.state_append(b["vt"], context.slots_v[li], kv_planes=c.kv_heads, past=past,
-                               query=query, x_dtype=io, slot_dtype=self.kv_dtype, **spec)
+                                  query=query, lengths=lengths, io_dtype=io,
+                                  kv_dtype=self.kv_dtype, row_major=True,
+                                  append=context.window == 0, **spec)
+                if context.window != 0:
+                    self._append_chunk(context, li, past, query, lengths, spec)
             else:
-                g.attention_state_lengths(b["qr"], b["kr"], b["vt"], context.slots_k[li],
-                                          context.slots_v[li], b["att"], batch=1, heads=c.heads,
-                                          kv_heads=c.kv_heads, half_scale=c.half_scale,
-                                          lengths=lengths, max_past=context.capacity - 1,
-                                          io_dtype=io, kv_dtype=self.kv_dtype,
-                                          workspace=self.workspace, **spec)
-                g.state_append_lengths(b["kr"], context.slots_k[li], kv_planes=c.kv_heads,
-                                       lengths=lengths, x_dtype=io, slot_dtype=self.kv_dtype,
-                                       **spec)
-                g.state_append_lengths(b["vt"], context.slots_v[li], kv_planes=c.kv_heads,
-                                       lengths=lengths, x_dtype=io, slot_dtype=self.kv_dtype,
-                                       **spec)
-            g.transpose_01(b["att"], b["att2"], c.heads, m, c.head_dim, io)
+                if lengths is None:
+                    g.attention_state(b["qr"], b["kr"], b["vt"], context.slots_k[li],
+                                      context.slots_v[li], b["att"], batch=1, heads=c.heads,
+                                      kv_heads=c.kv_heads, half_scale=c.half_scale, past=past,
+                                      query=query, io_dtype=io, kv_dtype=self.kv_dtype,
+                                      workspace=self.workspace, **spec)
+                else:
+                    g.attention_state_lengths(b["qr"], b["kr"], b["vt"], context.slots_k[li],
+                                              context.slots_v[li], b["att"], batch=1,
+                                              heads=c.heads, kv_heads=c.kv_heads,
+                                              half_scale=c.half_scale, lengths=lengths,
+                                              max_past=context.capacity - 1, io_dtype=io,
+                                              kv_dtype=self.kv_dtype, workspace=self.workspace,
+                                              **spec)
+                # readers first, then the appends (docs/ir-v1.md:345-348)
+                self._append_chunk(context, li, past, query, lengths, spec)
+                g.transpose_01(b["att"], b["att2"], c.heads, m, c.head_dim, io)
             lin = lw["o"]
             g.linear_i4_rows(b["att2"], lin.w, lin.s, b["h"], m, lin.n, lin.k, group,
                              residual=b["h"], io_dtype=io, scale_dtype=lin.scale_dtype,

@@ -21,6 +21,7 @@ COMPUTE_F16 = 1
 PROBE_EMPTY = 0
 PROBE_READ = 1
 EPILOGUE_NONE = 0
+CHUNK_OUT_ROW_MAJOR, CHUNK_APPEND = 1, 2
 EPILOGUE_SILU_PAIRS = 1
 
 _NP_DTYPE_CODE = {np.dtype(np.float32): F32, np.dtype(np.float16): F16}
@@ -317,6 +318,21 @@ class GpuContext:
             _addr(out), batch, heads, kv_heads, chunk_rows, depth, capacity, window,
             float(half_scale), past, query, io_dtype, kv_dtype, _addr(workspace),
             workspace_bytes))
+
+    def attention_chunk(self, q: BufferLike, ins_k: BufferLike, ins_v: BufferLike,
+                        slot_k: BufferLike, slot_v: BufferLike, out: BufferLike, *, batch: int,
+                        heads: int, kv_heads: int, chunk_rows: int, depth: int, capacity: int,
+                        window: int, half_scale: float, past: int = 0, query: int = 0,
+                        lengths: Optional[BufferLike] = None, io_dtype: int = F32,
+                        kv_dtype: int = F32, row_major: bool = False,
+                        append: bool = False) -> None:
+        """The attention of a chunk of rows with the output permute and the state appends
+        folded in (D = 64 / 128)."""
+        flags = (CHUNK_OUT_ROW_MAJOR if row_major else 0) | (CHUNK_APPEND if append else 0)
+        self._check(self._lib.krm_attention_chunk(
+            self._handle, _addr(q), _addr(ins_k), _addr(ins_v), _addr(slot_k), _addr(slot_v),
+            _addr(out), batch, heads, kv_heads, chunk_rows, depth, capacity, window,
+            float(half_scale), past, query, _addr(lengths), io_dtype, kv_dtype, flags))
 
     def attention_state_noalloc(self, q: BufferLike, ins_k: BufferLike, ins_v: BufferLike,
                                 slot_k: BufferLike, slot_v: BufferLike, out: BufferLike, *,

@@ -591,3 +591,61 @@ def test_varlen_planned_on_the_device_is_recordable(gpu_ctx):
     assert out.download(np.float16, q.shape).tobytes() == out_host.download(np.float16, q.shape).tobytes()
     for b in list(d.values()) + [out, out_host, ws, ws_host, plan, cu_dev]:
         b.free()
+
+
+@pytest.mark.parametrize("io,kv", [(np.float32, np.float32), (np.float16, np.float16),
+                                   (np.float32, np.float16)])
+@pytest.mark.parametrize("dyn", [False, True])
+def test_attention_chunk_equals_attention_transpose_and_appends(gpu_ctx, io, kv, dyn):
+    """krm_attention_chunk with the row-major output and the fused append writes the bits of
+    krm_attention_state + krm_transpose_01 + two krm_state_append (pad rows: zeros in the output,
+    nothing appended; every other slot row untouched); with a window the append is refused and
+    the row-major output alone still matches."""
+    case = StateCase("chunk D64 M40 Q33 P100", 2, 8, 2, 40, 64, 192, 0, 100, 33)
+    x = random_state_inputs(case, seed=77, f16_values=True)
+    b, h, hkv, m, d, c = (case.batch, case.heads, case.kv_heads, case.chunk_rows, case.depth,
+                          case.capacity)
+    io_code, kv_code = ka.dtype_code(io), ka.dtype_code(kv)
+
+    def upload():
+        return {k: gpu_ctx.upload(np.ascontiguousarray(v, dtype=io if k in ("q", "ins_k", "ins_v")
+                                                       else kv)) for k, v in x.items()}
+    ref = upload()
+    want_hm = gpu_ctx.upload(np.full(b * h * m * d, 5.0, dtype=io))
+    gpu_ctx.attention_state(ref["q"], ref["ins_k"], ref["ins_v"], ref["slot_k"], ref["slot_v"],
+                            want_hm, half_scale=oracle.half_scale(d), io_dtype=io_code,
+                            kv_dtype=kv_code, **case.kwargs())
+    spec = dict(kv_planes=b * hkv, chunk_rows=m, depth=d, capacity=c, window=0, x_dtype=io_code,
+                slot_dtype=kv_code)
+    gpu_ctx.state_append(ref["ins_k"], ref["slot_k"], past=case.past, query=case.query, **spec)
+    gpu_ctx.state_append(ref["ins_v"], ref["slot_v"], past=case.past, query=case.query, **spec)
+    want = want_hm.download(io, (b, h, m, d)).transpose(0, 2, 1, 3)
+
+    got = upload()
+    out = gpu_ctx.upload(np.full(b * h * m * d, 7.0, dtype=io))
+    lengths = None
+    if dyn:
+        lengths = gpu_ctx.zeros(16)
+        gpu_ctx.lengths_set(lengths, case.past, case.query)
+    geometry = {k: v for k, v in case.kwargs().items() if k not in ("past", "query")}
+    gpu_ctx.attention_chunk(got["q"], got["ins_k"], got["ins_v"], got["slot_k"], got["slot_v"],
+                            out, half_scale=oracle.half_scale(d), past=0 if dyn else case.past,
+                            query=0 if dyn else case.query, lengths=lengths, io_dtype=io_code,
+                            kv_dtype=kv_code, row_major=True, append=True, **geometry)
+    bits = np.uint32 if io == np.float32 else np.uint16
+    kbits = np.uint32 if kv == np.float32 else np.uint16
+    assert np.array_equal(out.download(io, (b, m, h, d)).view(bits), np.ascontiguousarray(want).view(bits))
+    for name in ("slot_k", "slot_v"):
+        assert np.array_equal(got[name].download(kv, (b, hkv, c, d)).view(kbits),
+                              ref[name].download(kv, (b, hkv, c, d)).view(kbits)), name
+    if dyn:
+        assert lengths.download(np.uint32, (4,))[2] == 0
+    with pytest.raises(ka.GpuValidationError, match="window == 0"):
+        gpu_ctx.attention_chunk(got["q"], got["ins_k"], got["ins_v"], got["slot_k"], got["slot_v"],
+                                out, half_scale=oracle.half_scale(d), past=case.past,
+                                query=case.query, io_dtype=io_code, kv_dtype=kv_code, append=True,
+                                **{**geometry, "window": 64})
+    with pytest.raises(ka.GpuValidationError, match="D = 64 or 128"):
+        gpu_ctx.attention_chunk(got["q"], got["ins_k"], got["ins_v"], got["slot_k"], got["slot_v"],
+                                out, half_scale=0.5, past=0, query=1, io_dtype=io_code,
+                                kv_dtype=kv_code, **{**geometry, "depth": 32})
