@@ -1099,6 +1099,9 @@ void gemm_i4_exact_kernel(const XT* __restrict__ x, const uint8_t* __restrict__ 
     };
 
     float16_t total[MT][WN], acc[MT][WN];
+    float16_t zero16;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) zero16[r] = 0.f;
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
@@ -1141,8 +1144,13 @@ void gemm_i4_exact_kernel(const XT* __restrict__ x, const uint8_t* __restrict__ 
 #pragma unroll
             for (int mt = 0; mt < MT; ++mt) {
 #pragma unroll
-              for (int copy = 0; copy < NA; ++copy)
-                acc[mt][nt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[copy][mt], b, acc[mt][nt], 0, 0, 0);
+              for (int copy = 0; copy < NA; ++copy) {
+                // the first product of a scale group starts from zero (an inline constant of
+                // the instruction: the sums are not cleared by VALU moves)
+                const bool opens = copy == 0 && j == 0 && (c == 0 || half_stage_groups);
+                acc[mt][nt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(
+                    a[copy][mt], b, opens ? zero16 : acc[mt][nt], 0, 0, 0);
+              }
             }
             __builtin_amdgcn_s_setprio(0);
           }
@@ -1153,10 +1161,8 @@ void gemm_i4_exact_kernel(const XT* __restrict__ x, const uint8_t* __restrict__ 
 #pragma unroll
             for (int nt = 0; nt < WN; ++nt)
 #pragma unroll
-              for (int r = 0; r < 16; ++r) {
+              for (int r = 0; r < 16; ++r)
                 total[mt][nt][r] = fmaf(acc[mt][nt][r], ws[nt], total[mt][nt][r]);
-                acc[mt][nt][r] = 0.f;
-              }
         }
       }
       park_stage(stage + 1, buf ^ 1, staged);
