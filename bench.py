@@ -28,6 +28,7 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
 USE_GRAPHS = True       # --no-graph: plain launches (rocprofv3's kernel trace crashes on graph launches)
 REPLAYS = 50            # timed replays of a recorded graph; the median is reported
+MIN_GRAPH_LAUNCHES = 256  # calls recorded into one graph at least (shorter sequences repeat)
 EVICT_BYTES = 512 << 20  # streamed between timed replays: twice the 256 MB Infinity Cache
 PROFILES = os.path.join(ROOT, "profiles")
 
@@ -57,7 +58,14 @@ class Timer:
     on the launch stream and preceded by untimed work that (a) streams EVICT_BYTES through the
     caches, so that no replay finds what the one before left there, and (b) keeps the device
     busy while the host queues the start event and the graph, so that the events bracket device
-    time only.  The median replay is reported."""
+    time only.  The median replay is reported.
+
+    Starting a graph costs the device about 10 us once per replay, whatever the graph holds
+    (measured: 5.00 / 4.67 / 4.53 us a launch with 20 / 64 / 256 launches recorded, the same with
+    an untimed lead-in of the same kernel).  A sequence shorter than MIN_GRAPH_LAUNCHES is
+    therefore recorded several times over into the one graph, with the call index running on so
+    that rotating buffers keep rotating, and the replay time is divided by the number of
+    repetitions: the figure is the time of `steps` calls in a long recorded run."""
 
     def __init__(self, ctx, ka):
         self.ctx, self.ka = ctx, ka
@@ -86,7 +94,7 @@ class Timer:
         self.evict_pass_ms = self.start.elapsed_ms(self.stop) / 4
 
     def run(self, fn, steps: int, warmup: int, *, after_evict=None, branches: int = 1,
-            replays: int = REPLAYS) -> dict:
+            replays: int = REPLAYS, min_launches: int = None) -> dict:
         """{"ms": median ms of one pass of `steps` calls, "ms_min", "ms_max", "mode", ...}.
         `after_evict` (optional) queues untimed calls behind the eviction (e.g. to warm the
         caches again for a cache-resident figure)."""
@@ -104,11 +112,14 @@ class Timer:
             return {"ms": ms, "ms_min": ms, "ms_max": ms, "mode": "plain launches", "replays": 1,
                     "timed_s": ms * 1e-3}
         self._calibrate()
+        if min_launches is None:
+            min_launches = MIN_GRAPH_LAUNCHES
+        repeats = max(1, -(-min_launches // steps))
         with ctx.record() as rec:
             if branches > 1:
                 for b in range(1, branches):
                     rec.branch(b)   # every side branch forks before the first launch
-            for i in range(steps):
+            for i in range(repeats * steps):
                 if branches > 1:
                     rec.branch(i % branches)
                 fn(i)
@@ -119,7 +130,7 @@ class Timer:
         t0 = time.perf_counter()
         graph.launch()
         host_ms = (time.perf_counter() - t0) * 1e3
-        for _ in range(max(0, warmup // max(1, steps))):
+        for _ in range(max(0, warmup // max(1, repeats * steps))):
             graph.launch()
         ctx.sync()
         passes = 2 + int(1.5 * host_ms / self.evict_pass_ms)
@@ -132,14 +143,15 @@ class Timer:
             self.start.record()
             graph.launch()
             self.stop.record()
-            samples.append(self.start.elapsed_ms(self.stop))
+            samples.append(self.start.elapsed_ms(self.stop) / repeats)
         ctx.sync()
         graph.destroy()
         samples.sort()
         return {"ms": samples[len(samples) // 2], "ms_min": samples[0], "ms_max": samples[-1],
                 "mode": "hipGraph replay" if branches == 1 else
                         f"hipGraph replay, {branches} parallel branches",
-                "replays": replays, "timed_s": sum(samples) * 1e-3,
+                "replays": replays, "timed_s": sum(samples) * repeats * 1e-3,
+                "calls_per_replay": repeats * steps,
                 "evict_passes_between_replays": passes}
 
 
@@ -629,9 +641,11 @@ def main() -> int:
         "data": "synthetic",
         "launch_mode": rot["mode"],
         "replays": rot["replays"],
-        "timing": "median over the replays of one recorded graph of `steps` launches; HIP events "
-                  "on the launch stream around each replay; 512 MiB streamed (untimed) before "
-                  "each replay",
+        "timing": "median over the replays of one recorded graph; the graph holds the `steps` "
+                  "launches, recorded again until it has at least 256 (calls_per_replay), and a "
+                  "replay's time is divided by that repetition count; HIP events on the launch "
+                  "stream around each replay; 512 MiB streamed (untimed) before each replay",
+        "calls_per_replay": rot.get("calls_per_replay", steps),
         "timed_region_s": round(rot["timed_s"], 6),
         "config": {"workload": "config 0: int4 g128 GEMV M=1 K=4096 N=4096, fp16 x/scales/out, "
                                "f32 accumulate, 64 rotating weight buffers (528 MiB)"},
