@@ -398,7 +398,8 @@ def bench_w4a8(timer: Timer, rng, steps: int, warmup: int, m: int, n: int, k: in
                copies: int):
     """w4a8 `linear` (int8 activations x int4 weights, integer dot products): one step = the
     activation quantiser + the product, f32 x in, f32 out, fp16 group scales.
-    Returns (ms per step, ms per step of the product alone)."""
+    Returns (ms per step, ms per step of the product alone, ms per step of the pair behind
+    krm_linear_w4a8_fused — one launch for few rows)."""
     ctx, ka = timer.ctx, timer.ka
     weights, scales = [], []
     for _ in range(copies):
@@ -419,12 +420,18 @@ def bench_w4a8(timer: Timer, rng, steps: int, warmup: int, m: int, n: int, k: in
         j = i % copies
         ctx.linear_w4a8(xq, xs, weights[j], scales[j], None, out, m, n, k, g, ka.F16)
 
+    def fused(i: int) -> None:
+        j = i % copies
+        ctx.linear_w4a8_fused(x, weights[j], scales[j], None, out, m, n, k, g, ka.F16, xq_i8=xq,
+                              xs_f32=xs)
+
     reps = 20 if m > 16 else REPLAYS
     ms = timer.run(step, steps, warmup, replays=reps)["ms"]
     ms_product = timer.run(product, steps, warmup, replays=reps)["ms"]
+    ms_fused = timer.run(fused, steps, warmup, replays=reps)["ms"] if m <= 8 else ms
     for b in weights + scales + [x, xq, xs, out]:
         b.free()
-    return ms / steps, ms_product / steps
+    return ms / steps, ms_product / steps, ms_fused / steps
 
 
 def bench_model(ctx, ka, io_dtype, kv_dtype, prompt_len: int = 128, new_tokens: int = 256):
@@ -742,13 +749,14 @@ def main() -> int:
         result["prefill_chunk_m128"] = bench_prefill_chunk(timer, rng, 64, 64, g)
     if args.only in ("", "w4a8"):
         log("[bench] w4a8 linear: M=1 GEMV and M=512 up/down-projections")
-        ms_q, ms_p = bench_w4a8(timer, rng, steps2, warm2, 1, n, k, g, copies)
+        ms_q, ms_p, ms_f = bench_w4a8(timer, rng, steps2, warm2, 1, n, k, g, copies)
+        result["w4a8_gemv_one_launch_us"] = round(ms_f * 1e3, 3)
         w4_bytes = n * k // 2 + n * (k // g) * 2 + k + 4 + n * 4
         result["w4a8_gemv_us"] = round(ms_q * 1e3, 3)
         result["w4a8_gemv_product_us"] = round(ms_p * 1e3, 3)
         result["w4a8_gemv_product_gbs"] = round(w4_bytes / (ms_p * 1e-3) / 1e9, 1)
         for name, (gn, gk) in {"up": (11008, 4096), "down": (4096, 11008)}.items():
-            ms_q, ms_p = bench_w4a8(timer, rng, 100, 200, 512, gn, gk, g, 4)
+            ms_q, ms_p, _ = bench_w4a8(timer, rng, 100, 200, 512, gn, gk, g, 4)
             ops = 2.0 * 512 * gn * gk
             result[f"w4a8_gemm_{name}_us"] = round(ms_q * 1e3, 2)
             result[f"w4a8_gemm_{name}_product_us"] = round(ms_p * 1e3, 2)

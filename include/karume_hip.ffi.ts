@@ -193,6 +193,12 @@ export const KARUME_HIP_SYMBOLS = {
     ],
     result: "i32",
   },
+  krm_linear_w4a8_fused: {
+    parameters: [
+      "pointer", "u64", "u64", "u64", "u64", "u64", "u64", "u64", "u32", "u32", "u32", "u32", "i32"
+    ],
+    result: "i32",
+  },
   krm_transpose_01: {
     parameters: [
       "pointer", "u64", "u64", "u32", "u32", "u32", "i32"

@@ -468,6 +468,18 @@ int32_t krm_quantize_rows(krm_ctx* ctx, krm_buf x_f32, krm_buf xq_i8, krm_buf xs
 int32_t krm_linear_w4a8(krm_ctx* ctx, krm_buf xq_i8, krm_buf xs_f32, krm_buf w, krm_buf scales,
                         krm_buf bias_f32, krm_buf out_f32, uint32_t m, uint32_t n, uint32_t k,
                         uint32_t group, int32_t scale_dtype);
+/* Steps 1 and 2 behind one call for f32 activations x [m, k] (the reference's builder emits
+ * the pair back to back with node-local xq / xs, recipe-builder.ts:1407-1488): the same result
+ * bit for bit.  For up to 8 rows with 32 <= group <= 2048 and rows-per-block * k <= 16384
+ * (blocks of 1, 2 or 4 rows: m = 1 up to k = 16384, m <= 2 up to 8192, else 4096) it is ONE
+ * launch — every workgroup quantises the block of x rows it multiplies, in LDS, while its
+ * weights are on their way — and xq / xs are not touched (0 is allowed).  Every other shape runs
+ * krm_quantize_rows + krm_linear_w4a8 through xq [m, k] int8 and xs [m] f32, which must then be
+ * given.  Argument rules are those of the two steps. */
+int32_t krm_linear_w4a8_fused(krm_ctx* ctx, krm_buf x_f32, krm_buf xq_i8, krm_buf xs_f32,
+                              krm_buf w, krm_buf scales, krm_buf bias_f32, krm_buf out_f32,
+                              uint32_t m, uint32_t n, uint32_t k, uint32_t group,
+                              int32_t scale_dtype);
 /* [a, b, d] -> [b, a, d] (the reshape + permute between linears and attention). */
 int32_t krm_transpose_01(krm_ctx* ctx, krm_buf x, krm_buf out, uint32_t a, uint32_t b, uint32_t d,
                          int32_t io_dtype);

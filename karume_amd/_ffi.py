@@ -55,6 +55,8 @@ PROTOTYPES = {
     "krm_quantize_rows": (i32, [c_ctx, c_buf, c_buf, c_buf, u32, u32]),
     "krm_linear_w4a8": (i32, [c_ctx, c_buf, c_buf, c_buf, c_buf, c_buf, c_buf, u32, u32, u32, u32,
                               i32]),
+    "krm_linear_w4a8_fused": (i32, [c_ctx, c_buf, c_buf, c_buf, c_buf, c_buf, c_buf, c_buf, u32,
+                                    u32, u32, u32, i32]),
     "krm_attention_state_workspace": (i32, [u32, u32, u32, u32, u32, u32, u32, u32,
                                             C.POINTER(size_t)]),
     "krm_attention_state": (i32, [c_ctx, c_buf, c_buf, c_buf, c_buf, c_buf, c_buf, u32, u32, u32,

@@ -56,12 +56,29 @@ __device__ inline bool is_nan_bits(float v) {
 // next to a rounding tie.
 constexpr int kQuantCache = 12;  // float4 per thread: rows of up to 12288 elements
 
-__device__ inline uint32_t quantize4(const float4& v, float s) {
+// x / s must be the correctly rounded quotient only where it decides the code: t = x * (1 / s)
+// (1 / s correctly rounded) lies within 2.3e-5 of it for |x / s| <= 127.5, so when t is further
+// than 2^-14 from every half-integer both round to the same integer and the product serves;
+// otherwise (and for a NaN) the lane divides.
+__device__ inline uint32_t quantize4(const float4& v, float s, float inv_s) {
   const float f[4] = {v.x, v.y, v.z, v.w};
+  float t[4];
+  bool near[4], any_near = false;
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    t[e] = f[e] * inv_s;
+    near[e] = !(fabsf(__builtin_amdgcn_fractf(fabsf(t[e])) - 0.5f) > 0x1p-14f);
+    any_near = any_near || near[e];
+  }
+  if (__builtin_amdgcn_ballot_w64(any_near) != 0) {  // wave-uniform and rare
+    asm volatile("" ::: "memory");  // keeps the divisions inside the branch
+#pragma unroll
+    for (int e = 0; e < 4; ++e) t[e] = near[e] ? f[e] / s : t[e];
+  }
   uint32_t packed = 0;
 #pragma unroll
   for (int e = 0; e < 4; ++e) {
-    float r = rintf(f[e] / s);
+    float r = rintf(t[e]);
     r = is_nan_bits(r) ? 0.f : fminf(fmaxf(r, -127.f), 127.f);
     packed |= ((uint32_t)(int32_t)r & 0xffu) << (8 * e);
   }
@@ -116,15 +133,16 @@ __global__ __launch_bounds__(256) void quantize_rows_kernel(const float* __restr
     float s = fmaxf(amax * (float)(1.0 / 127.0), kF32Tiny);
     if (row_nan) s = __uint_as_float(0x7fc00000u);
     if (threadIdx.x == 0) xs[row] = s;
+    const float inv_s = 1.0f / s;
     uint32_t* qr = xq + (size_t)row * quads;
     if (cached) {
 #pragma unroll
       for (int i = 0; i < kQuantCache; ++i) {
         const uint32_t at = threadIdx.x + 256u * i;
-        if (at < quads) qr[at] = quantize4(cache[i], s);
+        if (at < quads) qr[at] = quantize4(cache[i], s, inv_s);
       }
     } else {
-      for (uint32_t i = threadIdx.x; i < quads; i += 256) qr[i] = quantize4(xr[i], s);
+      for (uint32_t i = threadIdx.x; i < quads; i += 256) qr[i] = quantize4(xr[i], s, inv_s);
     }
     __syncthreads();  // s_max / s_nan are rewritten by the next row
   }
@@ -178,15 +196,31 @@ __global__ __launch_bounds__(256) void linear_w4a8_generic_kernel(
 // match and two v_dot4_i32_i8 add eight products.  The lanes of a group add their sums
 // (exact), the group totals and scales go through LDS to one lane per output, which runs the
 // ascending fma chain.
-template <typename ST, int MB>
+//  FUSED: `xin` is the f32 activations themselves and the quantiser runs in the prologue: every
+//  workgroup turns the whole block of x rows into int8 in LDS (the rows are needed whole by
+//  every output; quantising them again per workgroup costs less than a launch of its own, and
+//  it happens while the weights are on their way).  Same maximum, same scale, same correctly
+//  rounded quotients as quantize_rows_kernel, so the result is the two-launch result bit for
+//  bit.  The block's MB * K elements are held in registers between maximum and quotient, FUSE
+//  float4 per thread (a compile-time count of unconditional loads: the waits for them can then
+//  leave the weight requests behind them in flight): MB * K <= 256 * 4 * FUSE, FUSE <= 16.
+constexpr int kFuseCache = 16;
+
+template <typename ST, int MB, int FUSE>
 __global__ __launch_bounds__(256) void linear_w4a8_rows_kernel(
-    const uint32_t* __restrict__ xq, const float* __restrict__ xs, const uint32_t* __restrict__ w,
+    const void* __restrict__ xin, const float* __restrict__ xs, const uint32_t* __restrict__ w,
     const ST* __restrict__ scales, const float* __restrict__ bias, float* __restrict__ out,
     uint32_t m, uint32_t n, uint32_t k, uint32_t group_shift) {
   constexpr int ROWS = 2;
   constexpr int kStep = 64 * 32;
+  constexpr bool FUSED = FUSE > 0;
   __shared__ int32_t s_sum[4][ROWS * MB][64];
   __shared__ float s_ws[4][ROWS][64];
+  __shared__ float s_max[4][MB];
+  __shared__ uint32_t s_nan[4][MB];
+  __shared__ float s_xs[MB];
+  extern __shared__ __align__(16) uint32_t s_xq[];  // FUSED: MB rows of K int8
+  const uint32_t* xq = static_cast<const uint32_t*>(xin);
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const uint32_t row0 = (blockIdx.x * 4 + wave) * ROWS;
   const uint32_t b0 = blockIdx.y * MB;
@@ -213,20 +247,29 @@ __global__ __launch_bounds__(256) void linear_w4a8_rows_kernel(
     uint4 x[MB][2];
   };
   // requests only; lanes past the end of K re-read the row's start and are masked later
-  auto fetch = [&](uint32_t step, Step& d) {
+  auto fetch_x = [&](uint32_t step, Step& d) {
     const uint32_t k0 = step * kStep + lane * 32;
     const uint32_t kc = k0 < k ? k0 : 0u;
-    // activations first: they come from the cache, and loads return in order
 #pragma unroll
     for (int b = 0; b < MB; ++b) {
-      d.x[b][0] = *reinterpret_cast<const uint4*>(xrow[b] + (kc >> 2));
-      d.x[b][1] = *reinterpret_cast<const uint4*>(xrow[b] + (kc >> 2) + 4);
+      const uint32_t* row = FUSED ? s_xq + (size_t)b * (k >> 2) : xrow[b];
+      d.x[b][0] = *reinterpret_cast<const uint4*>(row + (kc >> 2));
+      d.x[b][1] = *reinterpret_cast<const uint4*>(row + (kc >> 2) + 4);
     }
+  };
+  auto fetch_w = [&](uint32_t step, Step& d) {
+    const uint32_t k0 = step * kStep + lane * 32;
+    const uint32_t kc = k0 < k ? k0 : 0u;
 #pragma unroll
     for (int r = 0; r < ROWS; ++r) {
       d.w[r] = *reinterpret_cast<const uint4*>(wrow[r] + (kc >> 3));
       d.s[r] = scale_f32<ST>(srow[r], kc >> group_shift);
     }
+  };
+  // activations first: they come from the cache, and loads return in order
+  auto fetch = [&](uint32_t step, Step& d) {
+    fetch_x(step, d);
+    fetch_w(step, d);
   };
 
   const int chain_r = lane / MB, chain_b = lane % MB;  // the output a chain lane owns
@@ -234,9 +277,102 @@ __global__ __launch_bounds__(256) void linear_w4a8_rows_kernel(
   float accf = 0.f;
 
   Step cur, nxt;
-  fetch(0, cur);
-  for (uint32_t step = 0; step < steps; ++step) {
-    fetch(step + 1 < steps ? step + 1 : step, nxt);  // unconditional: no wait inside a branch
+  if constexpr (FUSED) {
+    // x first (it comes from the cache and returns first), then the first step's weights; the
+    // quantiser below runs while those are on their way.
+    const float* xf = static_cast<const float*>(xin) + (size_t)b0 * k;
+    const uint32_t row_quads = k >> 2;
+    const uint32_t live_rows = m - b0 < (uint32_t)MB ? m - b0 : (uint32_t)MB;
+    const uint32_t quads = live_rows * row_quads;  // rows of the block lie back to back
+    float4 cache[FUSED ? FUSE : 1];
+#pragma unroll
+    for (int i = 0; i < FUSE; ++i) {
+      const uint32_t at = threadIdx.x + 256u * i;
+#if KRM_LAB == 2
+      cache[i] = make_float4(1.f + at, 2.f, 3.f, (float)quads);
+#else
+      cache[i] = reinterpret_cast<const float4*>(xf)[at < quads ? at : 0u];  // no branch
+#endif
+    }
+    fetch_w(0, cur);
+    fetch_w(steps > 1 ? 1u : 0u, nxt);
+    __builtin_amdgcn_sched_barrier(0);  // every request is out before the first x value is used
+    float amax[MB];
+    bool nan[MB];
+#pragma unroll
+    for (int b = 0; b < MB; ++b) {
+      amax[b] = 0.f;
+      nan[b] = false;
+    }
+#pragma unroll
+    for (int i = 0; i < FUSE; ++i) {
+      const uint32_t at = threadIdx.x + 256u * i;
+      const bool live = at < quads;
+      const uint32_t row = MB == 1 ? 0u : at / row_quads;
+      const float a[4] = {fabsf(cache[i].x), fabsf(cache[i].y), fabsf(cache[i].z),
+                          fabsf(cache[i].w)};
+      float top = 0.f;
+      bool bad = false;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        bad = bad || is_nan_bits(a[e]);
+        top = fmaxf(top, a[e]);  // ignores a NaN operand; the flag carries it
+      }
+#pragma unroll
+      for (int b = 0; b < MB; ++b) {
+        const bool mine = live && row == (uint32_t)b;
+        amax[b] = mine ? fmaxf(amax[b], top) : amax[b];
+        nan[b] = nan[b] || (mine && bad);
+      }
+    }
+#pragma unroll
+    for (int b = 0; b < MB; ++b) {
+#pragma unroll
+      for (int off = 32; off > 0; off >>= 1) amax[b] = fmaxf(amax[b], __shfl_xor(amax[b], off));
+      const bool wave_nan = __any(nan[b]);
+      if (lane == 0) {
+        s_max[wave][b] = amax[b];
+        s_nan[wave][b] = wave_nan ? 1u : 0u;
+      }
+    }
+    __syncthreads();
+    float scale_of[MB], inverse_of[MB];
+#pragma unroll
+    for (int b = 0; b < MB; ++b) {
+      const float top = fmaxf(fmaxf(s_max[0][b], s_max[1][b]), fmaxf(s_max[2][b], s_max[3][b]));
+      const bool row_nan = (s_nan[0][b] | s_nan[1][b] | s_nan[2][b] | s_nan[3][b]) != 0u;
+      float sc = fmaxf(top * (float)(1.0 / 127.0), kF32Tiny);
+      if (row_nan) sc = __uint_as_float(0x7fc00000u);
+      scale_of[b] = sc;
+      inverse_of[b] = 1.0f / sc;
+      if (threadIdx.x == 0) s_xs[b] = sc;
+    }
+#pragma unroll
+    for (int i = 0; i < FUSE; ++i) {
+      const uint32_t at = threadIdx.x + 256u * i;
+      if (at < quads) {
+        const uint32_t row = MB == 1 ? 0u : at / row_quads;
+        float sc = scale_of[0], inv = inverse_of[0];
+#pragma unroll
+        for (int b = 1; b < MB; ++b) {
+          sc = row == (uint32_t)b ? scale_of[b] : sc;
+          inv = row == (uint32_t)b ? inverse_of[b] : inv;
+        }
+#if KRM_LAB == 1
+        s_xq[at] = 0x01010101u + (uint32_t)(sc > 1e30f) + (uint32_t)(inv > 1e30f);
+#else
+        s_xq[at] = quantize4(cache[i], sc, inv);
+#endif
+      }
+    }
+    // rows of the block past M: zeros (their outputs are not stored)
+    for (uint32_t at = quads + threadIdx.x; at < (uint32_t)MB * row_quads; at += 256) s_xq[at] = 0u;
+    __syncthreads();
+    fetch_x(0, cur);
+  } else {
+    fetch(0, cur);
+  }
+  auto consume = [&](uint32_t step) {
     const bool active = step * kStep + lane * 32 < k;
     int32_t acc[ROWS][MB];
 #pragma unroll
@@ -295,11 +431,21 @@ __global__ __launch_bounds__(256) void linear_w4a8_rows_kernel(
     }
     __syncthreads();
     cur = nxt;
+  };
+  uint32_t step = 0;
+  if constexpr (FUSED) {  // the second step's weights were requested in front of the quantiser
+    fetch_x(steps > 1 ? 1u : 0u, nxt);
+    consume(0);
+    step = 1;
+  }
+  for (; step < steps; ++step) {
+    fetch(step + 1 < steps ? step + 1 : step, nxt);  // unconditional: no wait inside a branch
+    consume(step);
   }
   if (chain) {
     const uint32_t row = row0 + chain_r, xb = b0 + chain_b;
     if (row < n && xb < m)
-      out[(size_t)xb * n + row] = fmaf(accf, xs[xb], bias ? bias[row] : 0.f);
+      out[(size_t)xb * n + row] = fmaf(accf, FUSED ? s_xs[chain_b] : xs[xb], bias ? bias[row] : 0.f);
   }
 }
 
@@ -720,13 +866,13 @@ int32_t launch_w4a8(krm_ctx* ctx, krm_buf xq, krm_buf xs, krm_buf w, krm_buf sca
   if (rows_form) {
     const dim3 grid((n + 7) / 8, m <= 1 ? 1 : m <= 2 ? 1 : (m + 3) / 4);
     if (m <= 1)
-      hipLaunchKernelGGL((linear_w4a8_rows_kernel<ST, 1>), grid, dim3(256), 0, ctx->stream, pxq,
+      hipLaunchKernelGGL((linear_w4a8_rows_kernel<ST, 1, 0>), grid, dim3(256), 0, ctx->stream, pxq,
                          pxs, pw, ps, pb, po, m, n, k, shift);
     else if (m <= 2)
-      hipLaunchKernelGGL((linear_w4a8_rows_kernel<ST, 2>), grid, dim3(256), 0, ctx->stream, pxq,
+      hipLaunchKernelGGL((linear_w4a8_rows_kernel<ST, 2, 0>), grid, dim3(256), 0, ctx->stream, pxq,
                          pxs, pw, ps, pb, po, m, n, k, shift);
     else
-      hipLaunchKernelGGL((linear_w4a8_rows_kernel<ST, 4>), grid, dim3(256), 0, ctx->stream, pxq,
+      hipLaunchKernelGGL((linear_w4a8_rows_kernel<ST, 4, 0>), grid, dim3(256), 0, ctx->stream, pxq,
                          pxs, pw, ps, pb, po, m, n, k, shift);
     return launched(ctx, "linear_w4a8_rows_kernel");
   }
@@ -776,6 +922,41 @@ int32_t launch_w4a8(krm_ctx* ctx, krm_buf xq, krm_buf xs, krm_buf w, krm_buf sca
   return launched(ctx, "linear_w4a8_generic_kernel");
 }
 
+// The quantiser inside the product's launch; false when the shape is not covered.
+template <typename ST>
+bool launch_w4a8_fused(krm_ctx* ctx, krm_buf x, krm_buf w, krm_buf scales, krm_buf bias,
+                       krm_buf out, uint32_t m, uint32_t n, uint32_t k, uint32_t group) {
+  uint32_t shift = 0;
+  while ((1u << shift) < group) ++shift;
+  const uint32_t block = m <= 1 ? 1u : m <= 2 ? 2u : 4u;
+  if (!(group >= 32 && group <= 2048 && m <= 8 && aligned(x, 16) && aligned(w, 16) &&
+        (uint64_t)block * k <= 256ull * 4 * kFuseCache))
+    return false;
+  const dim3 grid((n + 7) / 8, (m + block - 1) / block);
+  const size_t lds = (size_t)block * k;
+  const void* px = ptr<const void>(x);
+  const uint32_t* pw = ptr<const uint32_t>(w);
+  const ST* ps = ptr<const ST>(scales);
+  const float* pb = ptr<const float>(bias);
+  float* po = ptr<float>(out);
+  const uint32_t per_thread = (uint32_t)(((uint64_t)block * k / 4 + 255) / 256);
+#define KRM_W4A8_FUSED(MB, FUSE)                                                               \
+  hipLaunchKernelGGL((linear_w4a8_rows_kernel<ST, MB, FUSE>), grid, dim3(256), lds,            \
+                     ctx->stream, px, nullptr, pw, ps, pb, po, m, n, k, shift)
+#define KRM_W4A8_FUSED_MB(MB)                      \
+  do {                                             \
+    if (per_thread <= 4) KRM_W4A8_FUSED(MB, 4);    \
+    else if (per_thread <= 8) KRM_W4A8_FUSED(MB, 8); \
+    else KRM_W4A8_FUSED(MB, 16);                   \
+  } while (0)
+  if (block == 1) KRM_W4A8_FUSED_MB(1);
+  else if (block == 2) KRM_W4A8_FUSED_MB(2);
+  else KRM_W4A8_FUSED_MB(4);
+#undef KRM_W4A8_FUSED_MB
+#undef KRM_W4A8_FUSED
+  return true;
+}
+
 }  // namespace
 
 extern "C" int32_t krm_quantize_rows(krm_ctx* ctx, krm_buf x, krm_buf xq, krm_buf xs,
@@ -816,4 +997,36 @@ extern "C" int32_t krm_linear_w4a8(krm_ctx* ctx, krm_buf xq, krm_buf xs, krm_buf
   if (scale_dtype == KRM_F16)
     return launch_w4a8<__half>(ctx, xq, xs, w, scales, bias, out, m, n, k, group);
   return launch_w4a8<float>(ctx, xq, xs, w, scales, bias, out, m, n, k, group);
+}
+
+extern "C" int32_t krm_linear_w4a8_fused(krm_ctx* ctx, krm_buf x, krm_buf xq, krm_buf xs,
+                                         krm_buf w, krm_buf scales, krm_buf bias, krm_buf out,
+                                         uint32_t m, uint32_t n, uint32_t k, uint32_t group,
+                                         int32_t scale_dtype) {
+  KRM_TRY(enter(ctx));
+  KRM_REQUIRE(ctx, krm::valid_dtype(scale_dtype), "linear w4a8: unknown scale dtype %d",
+              scale_dtype);
+  KRM_REQUIRE(ctx, k > 0 && k % 4 == 0, "linear w4a8: k must be a positive multiple of 4 (%u)", k);
+  KRM_REQUIRE(ctx, krm::is_pow2(group) && group >= 16,
+              "linear w4a8: group_size %u is not a power of two >= 16", group);
+  KRM_REQUIRE(ctx, k % group == 0, "linear w4a8: k=%u is not a multiple of group_size %u", k,
+              group);
+  KRM_REQUIRE(ctx, group <= kMaxGroup,
+              "linear w4a8: group_size %u exceeds the int32 reduction limit %u", group, kMaxGroup);
+  if (m == 0 || n == 0) return KRM_OK;
+  KRM_REQUIRE(ctx, x && w && scales && out, "linear w4a8: null buffer");
+  KRM_REQUIRE(ctx, krm::aligned(x, 16) && krm::aligned(w, 4) && krm::aligned(out, 4) &&
+                       krm::aligned(bias, 4) &&
+                       krm::aligned(scales, krm::dtype_bytes(scale_dtype)),
+              "linear w4a8: misaligned buffer");
+  const bool fused = scale_dtype == KRM_F16
+                         ? launch_w4a8_fused<__half>(ctx, x, w, scales, bias, out, m, n, k, group)
+                         : launch_w4a8_fused<float>(ctx, x, w, scales, bias, out, m, n, k, group);
+  if (fused) return krm::launched(ctx, "linear_w4a8_rows_kernel");
+  KRM_REQUIRE(ctx, xq && xs,
+              "linear w4a8 (fused): this shape (m=%u, k=%u, group=%u) takes the two-launch form, "
+              "which needs the xq and xs work buffers",
+              m, k, group);
+  KRM_TRY(krm_quantize_rows(ctx, x, xq, xs, m, k));
+  return krm_linear_w4a8(ctx, xq, xs, w, scales, bias, out, m, n, k, group, scale_dtype);
 }

@@ -296,6 +296,17 @@ class GpuContext:
                                               _addr(scales), _addr(bias_f32), _addr(out_f32), m, n,
                                               k, group, scale_dtype))
 
+    def linear_w4a8_fused(self, x_f32: BufferLike, w: BufferLike, scales: BufferLike,
+                          bias_f32: BufferLike, out_f32: BufferLike, m: int, n: int, k: int,
+                          group: int, scale_dtype: int = F32, *, xq_i8: BufferLike = None,
+                          xs_f32: BufferLike = None) -> None:
+        """quantize_rows + linear_w4a8 behind one call (one launch for few rows); xq / xs are the
+        work buffers of the shapes that take two launches."""
+        self._check(self._lib.krm_linear_w4a8_fused(self._handle, _addr(x_f32), _addr(xq_i8),
+                                                    _addr(xs_f32), _addr(w), _addr(scales),
+                                                    _addr(bias_f32), _addr(out_f32), m, n, k,
+                                                    group, scale_dtype))
+
     def attention_state_workspace(self, batch: int, heads: int, kv_heads: int, chunk_rows: int,
                                   depth: int, window: int, max_past: int, max_query: int = 1
                                   ) -> int:

@@ -98,6 +98,36 @@ def test_quantize_random_rows_bit_exact_without_a_tie_margin(gpu_ctx, rows, dim)
     assert_exact(q, want_q, "codes")
 
 
+def test_quantize_quotients_on_and_next_to_every_tie(gpu_ctx):
+    """Rows built so that x / s lands on, one ulp below and one ulp above each half-integer of
+    the code range (scales that are no power of two), plus rows in the subnormal range: the
+    quantiser takes a reciprocal product where that provably rounds like the quotient and the
+    division elsewhere — the codes must equal the oracle's everywhere."""
+    rng = np.random.default_rng(5)
+    rows = []
+    for top in (1.0, 3.0, 0.7310585975646973, 1234.5677490234375, 6.103515625e-05, 2.9e37,
+                1.3e-36):
+        s = np.float32(np.float32(top) * np.float32(1.0 / 127.0))
+        halves = (np.arange(-127, 127, dtype=np.float64) + 0.5)
+        centre = (halves * np.float64(s)).astype(np.float32)
+        row = np.concatenate([[np.float32(top)], centre, np.nextafter(centre, np.float32(np.inf)),
+                              np.nextafter(centre, np.float32(-np.inf)),
+                              np.nextafter(np.nextafter(centre, np.float32(np.inf)),
+                                           np.float32(np.inf))]).astype(np.float32)
+        row = row[np.abs(row) <= np.float32(top)]
+        rows.append(np.resize(row, 1024))
+    sub = rng.integers(-(1 << 22), 1 << 22, size=1024).astype(np.int32)   # subnormal bit patterns
+    rows.append((np.abs(sub).astype(np.uint32) | np.where(sub < 0, 1 << 31, 0).astype(np.uint32))
+                .view(np.float32))
+    rows.append(rows[-1] * np.float32(0.01))
+    x = np.stack(rows).astype(np.float32)
+    q, s = run_quantize(gpu_ctx, x)
+    want_q, want_s = oracle.quantize_rows(x, x.shape[1])
+    assert_exact(s, want_s, "scale")
+    assert_exact(q, want_q, "codes")
+    assert len(np.unique(want_q[0])) > 200  # the rows do walk the code range
+
+
 def test_quantize_rejections(gpu_ctx):
     buf = gpu_ctx.alloc(256)
     with pytest.raises(ka.GpuValidationError, match="multiple of 4"):
@@ -206,3 +236,83 @@ def test_w4a8_rejections(gpu_ctx):
     with pytest.raises(ka.GpuValidationError, match="int32 reduction limit"):
         gpu_ctx.linear_w4a8(*args, 1, 1, 1 << 22, 1 << 22)
     buf.free()
+
+
+# ---- the pair behind one call: the same bits from one launch ---------------------------------
+
+def run_w4a8_fused(ctx, x, packed, scale, bias, n, k, group, work=True):
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    scale = np.ascontiguousarray(scale)
+    m = x.shape[0]
+    dx, dw, dsc = ctx.upload(x), ctx.upload(packed), ctx.upload(scale)
+    db = ctx.upload(np.ascontiguousarray(bias, dtype=np.float32)) if bias is not None else None
+    dq = ctx.alloc(max(m * k, 16)) if work else None
+    dxs = ctx.alloc(max(m * 4, 16)) if work else None
+    out = ctx.alloc(max(m * n * 4, 16))
+    try:
+        ctx.linear_w4a8_fused(dx, dw, dsc, db, out, m, n, k, group, ka.dtype_code(scale.dtype),
+                              xq_i8=dq, xs_f32=dxs)
+        return out.download(np.float32, (m, n))
+    finally:
+        for b in (dx, dw, dsc, out, dq, dxs, db):
+            if b is not None:
+                b.free()
+
+
+FUSED_SHAPES = [  # (m, n, k, group, fp16 scales, bias, one launch)
+    (1, 4096, 4096, 128, True, False, True),     # the decode GEMV shape
+    (1, 130, 2048, 32, False, True, True),
+    (1, 64, 6144, 2048, True, True, True),
+    (1, 40, 11008, 64, True, True, True),        # partial last step, 11 quads a thread
+    (1, 24, 16384, 128, True, True, True),       # the longest single row of the one-launch form
+    (1, 24, 16512, 128, True, True, False),      # one group past it: two launches
+    (2, 70, 4096, 64, True, True, True),
+    (2, 70, 8192, 64, False, True, True),
+    (3, 50, 4096, 128, True, True, True),        # a block of four rows with one row unused
+    (4, 100, 1024, 128, False, True, True),      # K shorter than a step
+    (7, 33, 2048, 128, True, True, True),        # two blocks, the second ragged
+    (8, 16, 4096, 64, True, False, True),
+    (7, 33, 5632, 128, True, True, False),       # four rows of 5632 do not fit: two launches
+    (3, 21, 64, 16, False, True, False),         # groups of 16: two launches
+    (40, 300, 1024, 128, True, True, False),     # the matrix-core form
+]
+
+
+@pytest.mark.parametrize("m, n, k, group, scale_f16, with_bias, one_launch", FUSED_SHAPES)
+def test_w4a8_fused_call_equals_the_two_steps(gpu_ctx, m, n, k, group, scale_f16, with_bias,
+                                              one_launch):
+    rng = np.random.default_rng(m * 104729 + n * 31 + k + group)
+    packed, q, scale = helpers.synthetic_int4(rng, n, k, group, scale_f16)
+    x = (rng.normal(size=(m, k)) * rng.choice([1e-3, 1.0, 300.0], size=(m, 1))).astype(np.float32)
+    bias = rng.normal(size=n).astype(np.float32) if with_bias else None
+    want = oracle.linear_w4a8(x, packed, np.asarray(scale, dtype=np.float32), bias, n, k, group)
+    assert_exact(run_w4a8_fused(gpu_ctx, x, packed, scale, bias, n, k, group), want,
+                 (m, n, k, group))
+    assert_exact(run_w4a8(gpu_ctx, x, packed, scale, bias, n, k, group), want, "two steps")
+    if one_launch:  # needs no work buffers
+        assert_exact(run_w4a8_fused(gpu_ctx, x, packed, scale, bias, n, k, group, work=False),
+                     want, "no work buffers")
+    else:
+        with pytest.raises(ka.GpuValidationError, match="work buffers"):
+            run_w4a8_fused(gpu_ctx, x, packed, scale, bias, n, k, group, work=False)
+
+
+def test_w4a8_fused_call_special_rows_and_ties(gpu_ctx):
+    """A NaN row, a row of zeros, a row with an infinity and quotients on rounding ties."""
+    rng = np.random.default_rng(11)
+    n, k, group = 48, 1024, 128
+    packed, q, scale = helpers.synthetic_int4(rng, n, k, group)
+    x = rng.normal(size=(4, k)).astype(np.float32)
+    x[0, 17] = np.nan
+    x[1] = 0.0
+    x[2, 5] = np.inf
+    x[3] = rng.integers(-254, 255, size=k).astype(np.float32) * 0.5   # halves: ties everywhere
+    x[3, 0] = 127.0                                                   # scale exactly 1
+    want = oracle.linear_w4a8(x, packed, np.asarray(scale, dtype=np.float32), None, n, k, group)
+    got = run_w4a8_fused(gpu_ctx, x, packed, scale, None, n, k, group, work=False)
+    assert_exact(got, want, "special rows")
+    assert np.isnan(got[0]).all() and (got[1] == 0).all()
+    for row in range(4):  # each row alone (block of one) gives the same bits
+        alone = run_w4a8_fused(gpu_ctx, x[row:row + 1], packed, scale, None, n, k, group,
+                               work=False)
+        assert_exact(alone[0], want[row], ("alone", row))
