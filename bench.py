@@ -477,11 +477,26 @@ def bench_model(ctx, ka, io_dtype, kv_dtype, prompt_len: int = 128, new_tokens: 
         times.append((t_prefill - t_start, t_end - t_prefill))
         gen.dispose()
     prefill_s, decode_s = times[-1]
+    # the same prefill in the reference's default class (KRM_COMPUTE_F32: f32 x split hi + lo)
+    session.prefill_compute = ka.COMPUTE_F32
+    prefill_f32_s = None
+    for _ in range(2):
+        gen = session.create_generation_context(capacity=config.max_position,
+                                                chunk_length=prompt_len)
+        ids = prompt.reshape(1, prompt_len).copy()
+        pos = np.arange(prompt_len, dtype=np.int32).reshape(1, prompt_len)
+        ctx.sync()
+        t_start = time.perf_counter()
+        session.run(ids, pos, prompt_len - 1, context=gen, query_length=prompt_len)
+        prefill_f32_s = time.perf_counter() - t_start
+        gen.dispose()
     bytes_per_token = 517_210_112 + 16_162_816  # int4 weights + fp16 scales read per token
     return {
         "decode_tokens_per_s": round((new_tokens - 1) / decode_s, 1),
         "decode_ms_per_token": round(decode_s / (new_tokens - 1) * 1e3, 4),
         "prefill_ms": round(prefill_s * 1e3, 2),
+        "prefill_compute": "KRM_COMPUTE_F16 (f32 activations rounded to fp16 once per product)",
+        "prefill_f32class_ms": round(prefill_f32_s * 1e3, 2),
         "end_to_end_tokens_per_s": round(new_tokens / (prefill_s + decode_s), 1),
         "weight_gbs": round(bytes_per_token * (new_tokens - 1) / decode_s / 1e9, 1),
         "pct_of_hbm_peak": round(100 * bytes_per_token * (new_tokens - 1) / decode_s / 8e12, 2),

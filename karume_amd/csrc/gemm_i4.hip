@@ -1548,7 +1548,12 @@ void gemm_i4_rows_kernel(const XT* __restrict__ x, const uint8_t* __restrict__ w
   constexpr int BM = 32, BN = 32 * WN, kWaves = 8;
   constexpr int NA = OPERAND == kOperandSplit ? 2 : 1;
   constexpr int kChunk = 128;
-  constexpr int kRowA = kChunk * 2 + 16;          // bytes of a parked x row
+  // The split form with 64-column tiles parks the x rows of a chunk in two parts of 64 codes
+  // (hi and lo planes of 128 codes for eight waves would not fit the LDS next to 64 weight
+  // rows); every other form parks the chunk at once.
+  constexpr int kParts = (OPERAND == kOperandSplit && WN == 2) ? 2 : 1;
+  constexpr int kPartCodes = kChunk / kParts;
+  constexpr int kRowA = kPartCodes * 2 + 16;      // bytes of a parked x row
   constexpr int kPlane = BM * kRowA;
   constexpr int kRowB = kChunk / 2 + 16;          // bytes of a parked weight row
   constexpr int kWords = BN * kRowB;
@@ -1556,9 +1561,11 @@ void gemm_i4_rows_kernel(const XT* __restrict__ x, const uint8_t* __restrict__ w
   constexpr int kStageBytes = NA * kPlane + kWords;
   constexpr int kWaveBytes = kStageBytes > kSumBytes ? kStageBytes : kSumBytes;
   constexpr int kPieceCodes = RowPiece<XT, OPERAND>::kCodes;
-  constexpr int kLanesPerRow = kChunk / kPieceCodes;          // 32 (f32) or 16 (fp16)
+  constexpr int kLanesPerRow = kPartCodes / kPieceCodes;      // 32 (f32), 16 (fp16, f32 in parts)
   constexpr int kRowsPerLoad = 64 / kLanesPerRow;             // 2 or 4
-  constexpr int kActLoads = BM / kRowsPerLoad;                // 16 or 8
+  constexpr int kPartLoads = BM / kRowsPerLoad;               // loads of one part: 16 or 8
+  constexpr int kActLoads = kPartLoads * kParts;
+  static_assert(kWaves * kWaveBytes + 1024 <= 160 * 1024, "the waves' areas fit the LDS");
   constexpr int kWordLoads = BN / 16;                         // 16 rows x 4 pieces a load
   static_assert(OPERAND == kOperandF16 || sizeof(XT) == 4, "only f32 activations are split");
   __shared__ __align__(16) uint8_t s_wave[kWaves][kWaveBytes];
@@ -1609,12 +1616,15 @@ void gemm_i4_rows_kernel(const XT* __restrict__ x, const uint8_t* __restrict__ w
     float ws[WN][2];  // the scales of the chunk's first and second 64 codes
   };
   auto load_chunk = [&](uint32_t c, Staged& d) {
-    const uint32_t at = c * kChunk + a_piece * kPieceCodes;
-    const uint32_t off = at < k ? at : 0u;
 #pragma unroll
-    for (int i = 0; i < kActLoads; ++i)
-      d.a[i].raw = *reinterpret_cast<const uint4*>(
-          x + ((size_t)(min(x_row0 + (uint32_t)(kRowsPerLoad * i), m - 1) * k) + off));
+    for (int part = 0; part < kParts; ++part) {
+      const uint32_t at = c * kChunk + part * kPartCodes + a_piece * kPieceCodes;
+      const uint32_t off = at < k ? at : 0u;
+#pragma unroll
+      for (int i = 0; i < kPartLoads; ++i)
+        d.a[part * kPartLoads + i].raw = *reinterpret_cast<const uint4*>(
+            x + ((size_t)(min(x_row0 + (uint32_t)(kRowsPerLoad * i), m - 1) * k) + off));
+    }
     const uint32_t bat = c * (kChunk / 2) + b_piece * 16u;
     const uint32_t boff = bat < (k >> 1) ? bat : 0u;
 #pragma unroll
@@ -1628,15 +1638,19 @@ void gemm_i4_rows_kernel(const XT* __restrict__ x, const uint8_t* __restrict__ w
       d.ws[nt][1] = load_scale_f32<ST>(srow[nt], c1 >> group_shift);
     }
   };
-  auto park_chunk = [&](uint32_t c, const Staged& d) {
-    const uint32_t keep = c * kChunk + a_piece * kPieceCodes < k ? 0xFFFFFFFFu : 0u;  // past K: 0
+  auto park_rows = [&](uint32_t c, const Staged& d, int part) {
+    const uint32_t keep =  // past K: zeros
+        c * kChunk + part * kPartCodes + a_piece * kPieceCodes < k ? 0xFFFFFFFFu : 0u;
 #pragma unroll
-    for (int i = 0; i < kActLoads; ++i) {
+    for (int i = 0; i < kPartLoads; ++i) {
       const uint32_t at = (kRowsPerLoad * i + a_row) * kRowA + a_piece * (kPieceCodes * 2);
       float up = 1.0f;
       if constexpr (OPERAND == kOperandSplit) up = s_up[kRowsPerLoad * i + a_row];
-      d.a[i].park(mine + at, mine + kPlane + at, up, keep);
+      d.a[part * kPartLoads + i].park(mine + at, mine + kPlane + at, up, keep);
     }
+  };
+  auto park_chunk = [&](uint32_t c, const Staged& d) {
+    park_rows(c, d, 0);
 #pragma unroll
     for (int i = 0; i < kWordLoads; ++i)
       *reinterpret_cast<uint4*>(my_words + (16 * i + b_row) * kRowB + b_piece * 16u) = d.b[i];
@@ -1679,15 +1693,25 @@ void gemm_i4_rows_kernel(const XT* __restrict__ x, const uint8_t* __restrict__ w
       ws[nt][0] = staged[cur].ws[nt][0];
       ws[nt][1] = staged[cur].ws[nt][1];
     }
-    if (c + kDepth < c_end) load_chunk(c + kDepth, staged[cur]);
+    if constexpr (kParts == 1) {
+      if (c + kDepth < c_end) load_chunk(c + kDepth, staged[cur]);
+    }
     wave_sync();
 #pragma unroll
     for (int j = 0; j < 8; ++j) {  // step j: codes 16 j + 8 h .. + 7 of the chunk
+      if constexpr (kParts == 2) {
+        if (j == 4) {  // the second 64 codes of the x rows take the first ones' place
+          wave_sync();
+          park_rows(c, staged[cur], 1);
+          if (c + kDepth < c_end) load_chunk(c + kDepth, staged[cur]);
+          wave_sync();
+        }
+      }
       half8_t a[NA];
 #pragma unroll
       for (int copy = 0; copy < NA; ++copy)
         a[copy] = *reinterpret_cast<const half8_t*>(mine + copy * kPlane + frag_row * kRowA +
-                                                    32 * j + 16 * frag_h);
+                                                    32 * (j % (8 / kParts)) + 16 * frag_h);
 #pragma unroll
       for (int nt = 0; nt < WN; ++nt) {
         const uint32_t word = *reinterpret_cast<const uint32_t*>(
@@ -1838,12 +1862,9 @@ int32_t linear_i4_gemm_rows(krm_ctx* ctx, krm_buf x, krm_buf w, krm_buf scales, 
     if (scale_dtype == KRM_F16) KRM_ROWS(__half, __half, kOperandF16);
     KRM_ROWS(__half, float, kOperandF16);
   }
-  if (split) {  // (hi and lo planes of eight waves leave no LDS for 64 columns)
-    if (scale_dtype == KRM_F16)
-      return launch_rows<float, __half, kOperandSplit, 1>(ctx, x, w, scales, bias, out, m, n, k,
-                                                          group_shift, fuse);
-    return launch_rows<float, float, kOperandSplit, 1>(ctx, x, w, scales, bias, out, m, n, k,
-                                                       group_shift, fuse);
+  if (split) {
+    if (scale_dtype == KRM_F16) KRM_ROWS(float, __half, kOperandSplit);
+    KRM_ROWS(float, float, kOperandSplit);
   }
   if (scale_dtype == KRM_F16) KRM_ROWS(float, __half, kOperandF16);
   KRM_ROWS(float, float, kOperandF16);

@@ -1074,9 +1074,8 @@ int32_t krm_linear_i4(krm_ctx* ctx, krm_buf x, krm_buf w, krm_buf scales, krm_bu
   // workgroups make at most three rounds over the CUs (measured: 128 x 11264 x 2048 28.5 us
   // against 34.2 us, 512 x 2560 x 2048 29.2 against 33.9; 256 x 11264 x 2048 53.7 against 37.7).
   {
-    const bool split = compute == KRM_COMPUTE_F32 && io_dtype == KRM_F32;
     uint64_t workgroups = (uint64_t)((m + 31) / 32) * ((n + 31) / 32);
-    if (!split && workgroups > (uint64_t)ctx->num_cus) workgroups = (workgroups + 1) / 2;
+    if (workgroups > (uint64_t)ctx->num_cus) workgroups = (workgroups + 1) / 2;
     if (workgroups <= 3ull * (uint64_t)ctx->num_cus) {
       KRM_TRY(linear_i4_gemm_rows(ctx, x, w, scales, bias, out, m, n, k, group, io_dtype,
                                   scale_dtype, compute, RowsFusion{}, &handled));

@@ -248,6 +248,7 @@ def run_rows(ctx, x, packed, scale, bias, n, k, group, compute, residual=None,
 ROWS_SHAPES = [(128, 2560, 2048, 128),   # a 128-row chunk of the benchmark decoder: [q; k; v]
                (128, 2048, 5632, 128),   # its down-projection: 44 groups over 8 waves
                (40, 512, 1024, 128), (100, 129, 320, 64), (257, 96, 4096, 256),
+               (100, 2700, 1088, 64),    # 64-column tiles; K ends inside a chunk's second half
                (17, 33, 192, 64),        # fewer 64-code chunks than waves
                (1, 64, 2048, 128)]
 
