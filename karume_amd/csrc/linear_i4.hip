@@ -1165,8 +1165,9 @@ int32_t krm_linear_i4_rows(krm_ctx* ctx, krm_buf x, krm_buf w, krm_buf scales, k
                               compute, fuse, &handled));
   if (handled) return KRM_OK;
   return fail(ctx, KRM_ERR_VALIDATION,
-              "krm_linear_i4_rows: covers group_size >= 64, k %% 32 == 0 and 16-byte aligned x and "
-              "w (group %u, k %u); use krm_linear_i4 and the separate ops", group, k);
+              "krm_linear_i4_rows: covers group_size >= 64, k %% 32 == 0, 16-byte aligned x and w, "
+              "m * k and n * k / 2 below 2^32 and, in the f32 class, m <= 65536 (m %u, n %u, "
+              "group %u, k %u); use krm_linear_i4 and the separate ops", m, n, group, k);
 }
 
 int32_t krm_prefill_qkv(krm_ctx* ctx, krm_buf x, krm_buf w, krm_buf scales, krm_buf bias,
@@ -1216,8 +1217,9 @@ int32_t krm_prefill_qkv(krm_ctx* ctx, krm_buf x, krm_buf w, krm_buf scales, krm_
                               compute, fuse, &handled));
   if (handled) return KRM_OK;
   return fail(ctx, KRM_ERR_VALIDATION,
-              "krm_prefill_qkv: covers group_size >= 64, k %% 32 == 0 and 16-byte aligned x and w "
-              "(group %u, k %u); use krm_linear_i4, krm_rope_half and krm_transpose_01", group, k);
+              "krm_prefill_qkv: covers group_size >= 64, k %% 32 == 0, 16-byte aligned x and w, "
+              "m * k and n * k / 2 below 2^32 and, in the f32 class, m <= 65536 (m %u, group %u, "
+              "k %u); use krm_linear_i4, krm_rope_half and krm_transpose_01", m, group, k);
 }
 
 int32_t krm_decode_qkv(krm_ctx* ctx, krm_buf x, krm_buf norm_weight_f32, float norm_eps,

@@ -273,7 +273,7 @@ class LlamaDecoderSession:
         if m == 1 and self.fuse_decode:
             self._forward_fused_row(context, past, lengths)
             return
-        if m > 16 and self.fuse_decode and self._rows_form_covers():
+        if m > 16 and self.fuse_decode and self._rows_form_covers(m):
             self._forward_rows(context, m, past, query, lengths)
             self._head(last_row)
             return
@@ -350,11 +350,12 @@ class LlamaDecoderSession:
                 g.state_append_lengths(src, slot, kv_planes=c.kv_heads, lengths=lengths,
                                        x_dtype=io, slot_dtype=self.kv_dtype, **spec)
 
-    def _rows_form_covers(self) -> bool:
-        """The chunk-of-rows launches need groups of 64 codes or more and K a multiple of 32."""
+    def _rows_form_covers(self, m: int) -> bool:
+        """The chunk-of-rows launches need groups of 64 codes or more, K a multiple of 32 and
+        (their limit for the f32 class and for 32-bit element offsets) no more than 65536 rows."""
         c = self.config
         return (c.group_size >= 64 and c.d_model % 32 == 0 and c.ffn % 32 == 0
-                and (c.heads * c.head_dim) % 32 == 0)
+                and (c.heads * c.head_dim) % 32 == 0 and m <= 65536)
 
     def _forward_rows(self, context: GenerationContext, m: int, past: int, query: int,
                       lengths: Optional[DeviceBuffer]) -> None:

@@ -108,7 +108,7 @@ def test_decode_split_k(gpu_ctx, case, io, kv):
 
 ROWS_CASES = [
     # chunks of rows with D = 64 / 128: the matrix-core form (32 query rows a workgroup, key
-    # blocks of 32 dealt to four waves)
+    # blocks of 32 dealt to the waves: eight for D = 64, four for D = 128)
     StateCase("rows D64 M128 P0 r8 (decoder prefill)", 1, 32, 4, 128, 64, 256, 0, 0, 128),
     StateCase("rows D64 M40 Q33 P100 pad + slot/ins straddle", 2, 8, 2, 40, 64, 192, 0, 100, 33),
     StateCase("rows D128 M64 P31 r1", 1, 4, 4, 64, 128, 128, 0, 31, 64),
@@ -117,6 +117,10 @@ ROWS_CASES = [
     StateCase("rows D64 sliding W16 M64 Q50 gt W", 1, 4, 4, 64, 64, 16, 16, 7, 50),
     StateCase("rows D128 sliding W100 C128 P1000", 1, 8, 2, 35, 128, 128, 100, 1000, 20),
     StateCase("rows D64 M2 Q1 P5", 1, 4, 2, 2, 64, 16, 0, 5, 1),
+    # more key blocks than waves, D = 64
+    StateCase("rows D64 M64 P300, 12 blocks", 1, 8, 2, 64, 64, 512, 0, 300, 64),
+    StateCase("rows D64 M40 Q37 P1000, 33 blocks", 2, 4, 1, 40, 64, 1100, 0, 1000, 37),
+    StateCase("rows D64 sliding W300 P900", 1, 4, 2, 48, 64, 300, 300, 900, 48),
 ]
 
 
