@@ -176,23 +176,25 @@ __global__ __launch_bounds__(kThreads) void attention_generic_kernel(
 
 // ------------------------------------------------------------------- chunks of rows, MFMA
 //
-// A chunk of M > 1 rows with D = 64 or 128 (a prefill step): workgroup = (plane z, 32 query
-// rows), WAVES waves; the key columns the 32 rows can see are walked in blocks of 32 and wave w
-// takes blocks w, w + WAVES, ...  All arithmetic is f32 (v_mfma_f32_32x32x2_f32: f32 products, f32
-// sums), the operand roundings are the generic kernel's: q * scale and k * scale are rounded
-// before the product.
-//   S^T = K Q^T    A = the K block (row = key), B = Q^T (column = query row): a lane ends up
-//                  with 16 scores of ONE query row (lane % 32), so the running maximum and sum
-//                  of the online softmax are per lane, plus one exchange between the two
-//                  half-waves;
-//   O^T += V^T P^T the scores a lane holds (keys 8 (i / 4) + 4 (lane / 32) + i % 4, i < 16) are
-//                  exactly a B operand if MFMA step i is given those keys, so the probabilities
-//                  never move; V^T is the A operand, read from the parked V block with the
-//                  same key per step.  The result again has the query row in lane % 32.
+// A chunk of M > 1 rows with D = 64 or 128 (a prefill step): workgroup = (plane z, 16 query
+// rows), WAVES waves; the key columns the 16 rows can see are walked in blocks of 32 and wave w
+// takes blocks w, w + WAVES, ...  All arithmetic is f32 (v_mfma_f32_16x16x4_f32: f32 products,
+// f32 sums), the operand roundings are the generic kernel's: q * scale and k * scale are
+// rounded before the product.  With g = lane / 16:
+//   S^T = K Q^T    two tiles of 16 keys; A = the K tile (row = key, lane group g walks dims
+//                  g D/4 ..), B = Q^T (column = query row): a lane ends up with the scores of
+//                  ONE query row (lane % 16) against keys 16 t + 4 g + i (t < 2, i < 4), so the
+//                  running maximum and sum of the online softmax are per lane, plus an
+//                  exchange between the four lane groups;
+//   O^T += V^T P^T the scores a lane holds are exactly a B operand if MFMA step (t, i) is
+//                  given the keys 16 t + 4 g + i, so the probabilities never move; V^T is the A
+//                  operand, read from the parked V block with the same key per step.  The
+//                  result again has the query row in lane % 16 (dims 16 dt + 4 g + 0..3).
 // K and V blocks are parked in the wave's own LDS area (coalesced 16-byte loads; a block may
-// straddle the state slot and this step's rows).  The waves' (max, sum, O) are merged in
-// LDS at the end; rows >= query are written as +0.
-typedef float float16v_t __attribute__((ext_vector_type(16)));
+// straddle the state slot and this step's rows).  The waves' (max, sum, O) are merged in LDS
+// at the end; rows >= query are written as +0.  Sixteen rows a workgroup (not 32) so that a
+// 128-row chunk of 32 heads is 256 workgroups, one per CU.
+typedef float float4v_t __attribute__((ext_vector_type(4)));
 
 template <typename T>
 __device__ inline float4 load4_f32(const T* p);
@@ -207,25 +209,26 @@ __device__ inline float4 load4_f32<__half>(const __half* p) {
   return make_float4(__low2float(a), __high2float(a), __low2float(b), __high2float(b));
 }
 
-template <typename XT, typename ST, int D, int WAVES>
+template <typename XT, typename ST, int D, int WAVES, int RB>
 __global__ __launch_bounds__(64 * WAVES) void attention_rows_kernel(
     const XT* __restrict__ q, const XT* __restrict__ ins_k, const XT* __restrict__ ins_v,
     ST* __restrict__ slot_k, ST* __restrict__ slot_v, XT* __restrict__ out,
     GenericArgs a, uint32_t flags) {
+  constexpr uint32_t kBlock = 64u * WAVES;
+  constexpr int kRows = 16 * RB;              // query rows of a workgroup: RB blocks of 16
   constexpr int kRow = D + 4;                 // floats of a parked row
-  constexpr int NT = D / 32;
-  constexpr int kHalf = D / 2;                // dims a half-wave walks
+  constexpr int DT = D / 16;                  // output tiles of 16 dims
+  constexpr int kQuarter = D / 4;             // dims a lane group walks
   constexpr int kPieces = D / 4;              // 4-element pieces of a row
   constexpr int kRowsPerLoad = 64 / kPieces;
   constexpr int kLoads = 32 / kRowsPerLoad;
-  constexpr uint32_t kBlock = 64u * WAVES;
   __shared__ __align__(16) float s_k[WAVES][32 * kRow];
   __shared__ __align__(16) float s_v[WAVES][32 * kRow];
-  __shared__ float s_m[WAVES][32], s_l[WAVES][32];
+  __shared__ float s_m[WAVES][kRows], s_l[WAVES][kRows];
 
-  const uint32_t z = blockIdx.x, row0 = blockIdx.y * 32u;
+  const uint32_t z = blockIdx.x, row0 = blockIdx.y * (uint32_t)kRows;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int r = lane & 31, h = lane >> 5;
+  const int r = lane & 15, g = lane >> 4;
   uint32_t past = a.past, query = a.query;
   if (!device_lengths(a.lengths, a.chunk_rows, a.capacity, a.window, past, query)) return;
 
@@ -242,7 +245,7 @@ __global__ __launch_bounds__(64 * WAVES) void attention_rows_kernel(
   // touches them: slot rows are read for columns < past only, these are rows past + row.
   if ((flags & KRM_CHUNK_APPEND) && z % (a.heads / a.kv_heads) == 0) {
     const uint32_t plane = z / (a.heads / a.kv_heads);
-    for (uint32_t i = tid; i < 32u * kPieces; i += kBlock) {
+    for (uint32_t i = tid; i < (uint32_t)kRows * kPieces; i += kBlock) {
       const uint32_t rr = i / kPieces, piece = i - rr * kPieces;
       const uint32_t row = row0 + rr;
       if (row >= query) continue;
@@ -256,7 +259,7 @@ __global__ __launch_bounds__(64 * WAVES) void attention_rows_kernel(
     }
   }
   if (row0 >= query) {  // a block of pad rows: exact zeros, nothing is read
-    for (uint32_t i = tid; i < 32u * D; i += kBlock) {
+    for (uint32_t i = tid; i < (uint32_t)kRows * D; i += kBlock) {
       const uint32_t row = row0 + i / D;
       if (row < a.chunk_rows) st_f32<XT>(out, out_index(row, i % D), 0.0f);
     }
@@ -264,8 +267,8 @@ __global__ __launch_bounds__(64 * WAVES) void attention_rows_kernel(
   }
   const uint32_t kv_plane = z / (a.heads / a.kv_heads);
 
-  // Q block -> LDS (scaled), then each lane's B operands: Q[r][h * D/2 + s]
-  for (uint32_t i = tid; i < 32u * kPieces; i += kBlock) {
+  // Q block -> LDS (scaled), then each lane's B operands: Q[r][g * D/4 + s]
+  for (uint32_t i = tid; i < (uint32_t)kRows * kPieces; i += kBlock) {
     const uint32_t rr = i / kPieces, piece = i - rr * kPieces;
     const uint32_t row = min(row0 + rr, a.chunk_rows - 1);
     float4 v = load4_f32<XT>(q + ((size_t)z * a.chunk_rows + row) * D + 4 * piece);
@@ -273,21 +276,28 @@ __global__ __launch_bounds__(64 * WAVES) void attention_rows_kernel(
     *reinterpret_cast<float4*>(&s_k[0][rr * kRow + 4 * piece]) = v;
   }
   __syncthreads();
-  float qf[kHalf];
+  float qf[RB][kQuarter];
 #pragma unroll
-  for (int i = 0; i < kHalf / 4; ++i) {
-    const float4 v = *reinterpret_cast<const float4*>(&s_k[0][r * kRow + h * kHalf + 4 * i]);
-    qf[4 * i] = v.x; qf[4 * i + 1] = v.y; qf[4 * i + 2] = v.z; qf[4 * i + 3] = v.w;
-  }
+  for (int rb = 0; rb < RB; ++rb)
+#pragma unroll
+    for (int i = 0; i < kQuarter / 4; ++i) {
+      const float4 v = *reinterpret_cast<const float4*>(
+          &s_k[0][(16 * rb + r) * kRow + g * kQuarter + 4 * i]);
+      qf[rb][4 * i] = v.x; qf[rb][4 * i + 1] = v.y; qf[rb][4 * i + 2] = v.z; qf[rb][4 * i + 3] = v.w;
+    }
   __syncthreads();
 
   // columns the block's rows can see: [c_lo, limit_hi]
-  const uint32_t last_row = min(row0 + 31u, query - 1u);
+  const uint32_t last_row = min(row0 + (uint32_t)kRows - 1u, query - 1u);
   const uint64_t limit_hi = (uint64_t)past + last_row;
   const uint64_t c_lo = window_low(a.window, (uint64_t)past + row0);
   const uint32_t blocks = (uint32_t)((limit_hi - c_lo) / 32u) + 1u;
-  const uint64_t my_limit = (uint64_t)past + row0 + (uint32_t)r;
-  const uint64_t my_low = window_low(a.window, my_limit);
+  uint64_t my_limit[RB], my_low[RB];
+#pragma unroll
+  for (int rb = 0; rb < RB; ++rb) {
+    my_limit[rb] = (uint64_t)past + row0 + (uint32_t)(16 * rb + r);
+    my_low[rb] = window_low(a.window, my_limit[rb]);
+  }
 
   float* mk = s_k[wave];
   float* mv = s_v[wave];
@@ -297,12 +307,17 @@ __global__ __launch_bounds__(64 * WAVES) void attention_rows_kernel(
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
   };
 
-  float run_m = -INFINITY, run_l = 0.f;
-  float16v_t acc[NT];
+  float run_m[RB], run_l[RB];
+  float4v_t acc[RB][DT];
 #pragma unroll
-  for (int nt = 0; nt < NT; ++nt)
+  for (int rb = 0; rb < RB; ++rb) {
+    run_m[rb] = -INFINITY;
+    run_l[rb] = 0.f;
 #pragma unroll
-    for (int i = 0; i < 16; ++i) acc[nt][i] = 0.f;
+    for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) acc[rb][dt][i] = 0.f;
+  }
 
   for (uint32_t kb = (uint32_t)wave; kb < blocks; kb += (uint32_t)WAVES) {
     const uint64_t c0 = c_lo + (uint64_t)kb * 32u;
@@ -334,71 +349,91 @@ __global__ __launch_bounds__(64 * WAVES) void attention_rows_kernel(
     }
     wave_sync();
 
-    // S^T[key][query row]: A = K[key = r][h * D/2 + s], B = Q^T
-    float16v_t st;
 #pragma unroll
-    for (int i = 0; i < 16; ++i) st[i] = 0.f;
+    for (int rb = 0; rb < RB; ++rb) {
+      // (a block past every column these 16 rows can see is skipped: the workgroup's other
+      // rows see further)
+      if (c0 > (uint64_t)past + row0 + (uint32_t)(16 * rb + 15)) continue;
+      // S^T[key][query row], tile t = keys 16 t ..: A = K[16 t + r][g * D/4 + s], B = Q^T
+      float4v_t st[2];
 #pragma unroll
-    for (int i = 0; i < kHalf / 4; ++i) {
-      const float4 kf = *reinterpret_cast<const float4*>(&mk[r * kRow + h * kHalf + 4 * i]);
-      st = __builtin_amdgcn_mfma_f32_32x32x2f32(kf.x, qf[4 * i], st, 0, 0, 0);
-      st = __builtin_amdgcn_mfma_f32_32x32x2f32(kf.y, qf[4 * i + 1], st, 0, 0, 0);
-      st = __builtin_amdgcn_mfma_f32_32x32x2f32(kf.z, qf[4 * i + 2], st, 0, 0, 0);
-      st = __builtin_amdgcn_mfma_f32_32x32x2f32(kf.w, qf[4 * i + 3], st, 0, 0, 0);
-    }
-    // this lane: query row r, keys 8 (i / 4) + 4 h + i % 4
-    float block_max = -INFINITY;
-    bool valid[16];
+      for (int t = 0; t < 2; ++t) {
 #pragma unroll
-    for (int i = 0; i < 16; ++i) {
-      const uint64_t c = c0 + (uint32_t)(8 * (i / 4) + 4 * h + (i % 4));
-      valid[i] = c <= my_limit && c >= my_low;
-      block_max = fmaxf(block_max, valid[i] ? st[i] : -INFINITY);
-    }
-    block_max = fmaxf(block_max, __shfl_xor(block_max, 32, kWave));
-    const float new_m = fmaxf(run_m, block_max);
-    const float ref = new_m == -INFINITY ? 0.f : new_m;  // nothing seen yet: exp(-inf - 0) = 0
-    const float alpha = expf(run_m - ref);
-    float p[16], sum = 0.f;
+        for (int i = 0; i < 4; ++i) st[t][i] = 0.f;
 #pragma unroll
-    for (int i = 0; i < 16; ++i) {
-      p[i] = valid[i] ? expf(st[i] - ref) : 0.f;
-      sum += p[i];
-    }
-    run_l = run_l * alpha + sum;
-    run_m = new_m;
-    // O^T[d][query row] = alpha * O^T + V^T P^T: step i carries the keys of register i
+        for (int i = 0; i < kQuarter / 4; ++i) {
+          const float4 kf =
+              *reinterpret_cast<const float4*>(&mk[(16 * t + r) * kRow + g * kQuarter + 4 * i]);
+          st[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(kf.x, qf[rb][4 * i], st[t], 0, 0, 0);
+          st[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(kf.y, qf[rb][4 * i + 1], st[t], 0, 0, 0);
+          st[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(kf.z, qf[rb][4 * i + 2], st[t], 0, 0, 0);
+          st[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(kf.w, qf[rb][4 * i + 3], st[t], 0, 0, 0);
+        }
+      }
+      // this lane: query row 16 rb + r, keys 16 t + 4 g + i
+      float block_max = -INFINITY;
+      bool valid[2][4];
 #pragma unroll
-    for (int nt = 0; nt < NT; ++nt) {
+      for (int t = 0; t < 2; ++t)
 #pragma unroll
-      for (int i = 0; i < 16; ++i) acc[nt][i] *= alpha;
+        for (int i = 0; i < 4; ++i) {
+          const uint64_t c = c0 + (uint32_t)(16 * t + 4 * g + i);
+          valid[t][i] = c <= my_limit[rb] && c >= my_low[rb];
+          block_max = fmaxf(block_max, valid[t][i] ? st[t][i] : -INFINITY);
+        }
+      block_max = fmaxf(block_max, __shfl_xor(block_max, 16, kWave));
+      block_max = fmaxf(block_max, __shfl_xor(block_max, 32, kWave));
+      const float new_m = fmaxf(run_m[rb], block_max);
+      const float ref = new_m == -INFINITY ? 0.f : new_m;  // nothing seen yet: exp(-inf - 0) = 0
+      const float alpha = expf(run_m[rb] - ref);
+      float p[2][4], sum = 0.f;
 #pragma unroll
-      for (int i = 0; i < 16; ++i) {
-        const float vf = mv[(8 * (i / 4) + 4 * h + (i % 4)) * kRow + 32 * nt + r];
-        acc[nt] = __builtin_amdgcn_mfma_f32_32x32x2f32(vf, p[i], acc[nt], 0, 0, 0);
+      for (int t = 0; t < 2; ++t)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          p[t][i] = valid[t][i] ? expf(st[t][i] - ref) : 0.f;
+          sum += p[t][i];
+        }
+      run_l[rb] = run_l[rb] * alpha + sum;
+      run_m[rb] = new_m;
+      // O^T[d][query row] = alpha * O^T + V^T P^T: step (t, i) carries the keys 16 t + 4 g + i
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) acc[rb][dt][i] *= alpha;
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            const float vf = mv[(16 * t + 4 * g + i) * kRow + 16 * dt + r];
+            acc[rb][dt] = __builtin_amdgcn_mfma_f32_16x16x4f32(vf, p[t][i], acc[rb][dt], 0, 0, 0);
+          }
       }
     }
     wave_sync();  // the block's rows have been read: the next block may be parked
   }
 
   // the wave's state: (max, sum) per query row and O[row][d] in its own area
-  run_l += __shfl_xor(run_l, 32, kWave);
-  if (h == 0) {
-    s_m[wave][r] = run_m;
-    s_l[wave][r] = run_l;
+#pragma unroll
+  for (int rb = 0; rb < RB; ++rb) {
+    run_l[rb] += __shfl_xor(run_l[rb], 16, kWave);
+    run_l[rb] += __shfl_xor(run_l[rb], 32, kWave);
+    if (g == 0) {
+      s_m[wave][16 * rb + r] = run_m[rb];
+      s_l[wave][16 * rb + r] = run_l[rb];
+    }
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt)  // registers 0..3: dims 16 dt + 4 g + 0..3
+      *reinterpret_cast<float4*>(&mk[(16 * rb + r) * kRow + 16 * dt + 4 * g]) =
+          make_float4(acc[rb][dt][0], acc[rb][dt][1], acc[rb][dt][2], acc[rb][dt][3]);
   }
-#pragma unroll
-  for (int nt = 0; nt < NT; ++nt)
-#pragma unroll
-    for (int g = 0; g < 4; ++g)  // registers 4g..4g+3: dims 32 nt + 8 g + 4 h + 0..3
-      *reinterpret_cast<float4*>(&mk[r * kRow + 32 * nt + 8 * g + 4 * h]) =
-          make_float4(acc[nt][4 * g], acc[nt][4 * g + 1], acc[nt][4 * g + 2], acc[nt][4 * g + 3]);
   __syncthreads();
 
-  // merge of the waves, wave order; 8 threads a row (the first 256 threads)
+  // merge of the waves, wave order; 16 threads a row (the first 256 threads)
   if (tid < 256) {
-    constexpr int kPer = D / 8;
-    const uint32_t rr = tid >> 3, d0 = (tid & 7u) * kPer;
+   for (uint32_t rb = 0; rb < (uint32_t)RB; ++rb) {
+    constexpr int kPer = D / 16;
+    const uint32_t rr = 16u * rb + (tid >> 4), d0 = (tid & 15u) * kPer;
     const uint32_t row = row0 + rr;
     float top = s_m[0][rr];
 #pragma unroll
@@ -419,6 +454,7 @@ __global__ __launch_bounds__(64 * WAVES) void attention_rows_kernel(
         st_f32<XT>(out, out_index(row, d0 + e), row < query ? o * inv : 0.0f);
       }
     }
+   }
   }
 }
 
@@ -1133,17 +1169,27 @@ template <typename XT, typename ST>
 int32_t launch_rows(krm_ctx* ctx, krm_buf q, krm_buf ins_k, krm_buf ins_v, krm_buf slot_k,
                     krm_buf slot_v, krm_buf out, uint32_t batch, const GenericArgs& a,
                     uint32_t flags) {
-  const dim3 grid(batch * a.heads, (a.chunk_rows + 31) / 32);
   // D = 64: eight waves, two a SIMD, so that one wave's softmax and LDS traffic run under the
-  // other's MFMAs (past 1024: 41 -> 31 us; no past: 8.3 -> 8.0 us); the parked blocks of eight
-  // waves of D = 128 would not fit the LDS.  The wave count depends on D only, so a row's bits
-  // do not depend on the past, the capacity or the lengths form.
-#define KRM_ROWS_ATTENTION(DEPTH, WAVES)                                                       \
-  attention_rows_kernel<XT, ST, DEPTH, WAVES><<<grid, dim3(64 * WAVES), 0, ctx->stream>>>(     \
+  // other's MFMAs; the parked blocks of eight waves of D = 128 would not fit the LDS.  A
+  // workgroup takes one block of 16 query rows, or two (the parked K / V blocks then serve
+  // both) once that still leaves two workgroups per CU.  A row's arithmetic is the same in
+  // both forms and the wave count depends on D only, so its bits depend neither on the chunk
+  // length, the batch, the past or the capacity nor on the lengths form.
+  const uint32_t row_blocks = (a.chunk_rows + 15) / 16;
+  // (with a window the key blocks start at the first row's lower bound, which a second row
+  // block would not share: one block a workgroup there)
+  const bool two = a.window == 0 &&
+                   (uint64_t)batch * a.heads * ((row_blocks + 1) / 2) >= 2ull * ctx->num_cus;
+  const dim3 grid(batch * a.heads, two ? (row_blocks + 1) / 2 : row_blocks);
+#define KRM_ROWS_ATTENTION(DEPTH, WAVES, RB)                                                   \
+  attention_rows_kernel<XT, ST, DEPTH, WAVES, RB><<<grid, dim3(64 * WAVES), 0, ctx->stream>>>( \
       ptr<const XT>(q), ptr<const XT>(ins_k), ptr<const XT>(ins_v), ptr<ST>(slot_k),           \
       ptr<ST>(slot_v), ptr<XT>(out), a, flags)
-  if (a.depth == 64) KRM_ROWS_ATTENTION(64, 8);
-  else KRM_ROWS_ATTENTION(128, 4);
+  if (a.depth == 64) {
+    if (two) KRM_ROWS_ATTENTION(64, 8, 2); else KRM_ROWS_ATTENTION(64, 8, 1);
+  } else {
+    if (two) KRM_ROWS_ATTENTION(128, 4, 2); else KRM_ROWS_ATTENTION(128, 4, 1);
+  }
 #undef KRM_ROWS_ATTENTION
   return launched(ctx, "attention_rows_kernel");
 }

@@ -150,6 +150,22 @@ def test_chunks_of_rows_on_the_matrix_cores(gpu_ctx, case, io, kv):
         assert np.all(err <= ulp + STATE_ATOL), float(np.max(err - ulp))
 
 
+def test_chunk_rows_do_not_depend_on_the_batch(gpu_ctx):
+    """A large grid puts two blocks of 16 query rows into one workgroup (the parked K / V blocks
+    serve both); a row's arithmetic is the same, so one sequence alone and the same sequence as
+    the first of eight give the same bits."""
+    big = StateCase("rows D64 M64 P70 B8", 8, 32, 32, 64, 64, 160, 0, 70, 61)
+    x = random_state_inputs(big, seed=3, f16_values=False)
+    whole = run_attention(gpu_ctx, big, x)
+    one = StateCase("rows D64 M64 P70 B1", 1, 32, 32, 64, 64, 160, 0, 70, 61)
+    first = {k: np.ascontiguousarray(v[:1]) for k, v in x.items()}
+    alone = run_attention(gpu_ctx, one, first)
+    assert np.array_equal(alone.view(np.uint32), whole[:1].view(np.uint32))
+    ok, fails, max_abs, worst = oracle.allclose(alone, oracle_state_attention(one, first),
+                                                atol=STATE_ATOL, rtol=0)
+    assert ok, (fails, max_abs, worst)
+
+
 def test_chunks_of_rows_with_device_lengths_and_mutation_witness(gpu_ctx):
     """The device-lengths form of a chunk equals the scalar form bit for bit, and a dropped
     window bound, a ring taken modulo the capacity, or an ignored kv repeat (the oracle's
