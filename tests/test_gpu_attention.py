@@ -107,7 +107,7 @@ def test_decode_split_k(gpu_ctx, case, io, kv):
 
 
 ROWS_CASES = [
-    # chunks of rows with D = 64 / 128: the matrix-core form (32 query rows a workgroup, key
+    # chunks of rows with D = 64 / 128: the matrix-core form (16 query rows a workgroup, key
     # blocks of 32 dealt to the waves: eight for D = 64, four for D = 128)
     StateCase("rows D64 M128 P0 r8 (decoder prefill)", 1, 32, 4, 128, 64, 256, 0, 0, 128),
     StateCase("rows D64 M40 Q33 P100 pad + slot/ins straddle", 2, 8, 2, 40, 64, 192, 0, 100, 33),
