@@ -59,7 +59,7 @@ export const KARUME_HIP_SYMBOLS = {
   krm_linear_i4_rows: {
     parameters: [
       "pointer", "u64", "u64", "u64", "u64", "u64", "u64", "u32", "u32", "u32", "u32", "i32",
-      "i32", "i32", "i32"
+      "i32", "i32", "i32", "i32"
     ],
     result: "i32",
   },
@@ -158,6 +158,12 @@ export const KARUME_HIP_SYMBOLS = {
     ],
     result: "i32",
   },
+  krm_rms_norm_cast: {
+    parameters: [
+      "pointer", "u64", "u64", "u64", "u32", "u32", "f32", "i32", "i32"
+    ],
+    result: "i32",
+  },
   krm_rope_half: {
     parameters: [
       "pointer", "u64", "u64", "u64", "u64", "u64", "u32", "u32", "u32", "u32", "i32", "i32"
@@ -174,7 +180,7 @@ export const KARUME_HIP_SYMBOLS = {
   krm_prefill_qkv: {
     parameters: [
       "pointer", "u64", "u64", "u64", "u64", "u64", "u64", "u64", "u64", "u64", "u64", "u32",
-      "u32", "u32", "u32", "u32", "u32", "u32", "i32", "i32", "i32"
+      "u32", "u32", "u32", "u32", "u32", "u32", "i32", "i32", "i32", "i32"
     ],
     result: "i32",
   },

@@ -197,6 +197,11 @@ int32_t krm_linear_i4_fused(krm_ctx* ctx, krm_buf x, krm_buf norm_weight_f32, fl
  *                             one thread)
  *   KRM_EPILOGUE_SILU_PAIRS : rows (2i, 2i+1) of w = (gate_i, up_i), out[m, i] = silu(gate) * up,
  *                             n_out = n / 2; gate and up are not rounded to io_dtype in between
+ * x_dtype is the element type of x: io_dtype, or KRM_F16 beside io_dtype KRM_F32 under
+ * KRM_COMPUTE_F16 — an fp16 copy of the activations (krm_rms_norm_cast, KRM_CHUNK_OUT_F16, an
+ * fp16-io call of this function write one) holding exactly what f32 activations are rounded to
+ * in that class, so the result is the same bit for bit and x costs half the bytes; bias,
+ * residual and out stay io_dtype.
  * Covers group_size >= 64, k % 32 == 0, 16-byte aligned x and w; anything else is rejected
  * (krm_linear_i4 + krm_silu_mul + krm_add remain).  A pure function of the shape and dtypes.
  * Fuses packages/runtime/src/kernels/linear.ts:34-64 with the elementwise add / silu-mul that
@@ -204,7 +209,7 @@ int32_t krm_linear_i4_fused(krm_ctx* ctx, krm_buf x, krm_buf norm_weight_f32, fl
 int32_t krm_linear_i4_rows(krm_ctx* ctx, krm_buf x, krm_buf w, krm_buf scales, krm_buf bias,
                            krm_buf residual, krm_buf out, uint32_t m, uint32_t n, uint32_t k,
                            uint32_t group, int32_t io_dtype, int32_t scale_dtype, int32_t compute,
-                           int32_t epilogue);
+                           int32_t epilogue, int32_t x_dtype);
 
 /* ---- states-form attention (Params 10 words + Lengths{past,query} + bindings:
  *      packages/runtime/src/kernels/state-attention.ts:169-180,190-193,284-294,476-487;
@@ -262,11 +267,15 @@ int32_t krm_attention_state_noalloc(krm_ctx* ctx, krm_buf q, krm_buf ins_k, krm_
  *                             slots (krm_state_append's result, same roundings).  window == 0
  *                             only: slot rows past.. are read by nobody in this launch, while a
  *                             ring would overwrite rows it still reads (docs/ir-v1.md:345-348).
+ *   KRM_CHUNK_OUT_F16       : `out` is fp16 whatever io_dtype is: the f32 result rounded once,
+ *                             i.e. what a KRM_COMPUTE_F16 product would round it to when it
+ *                             reads it (see x_dtype of krm_linear_i4_rows)
  * Fuses packages/runtime/src/kernels/state-attention.ts:169-552 with
  * packages/runtime/src/kernels/state-append.ts:47-96 and the permute of
  * tools/export-recipes/minicpm5/export_decode.py:14-35. */
 #define KRM_CHUNK_OUT_ROW_MAJOR 1u
 #define KRM_CHUNK_APPEND 2u
+#define KRM_CHUNK_OUT_F16 4u
 int32_t krm_attention_chunk(krm_ctx* ctx, krm_buf q, krm_buf ins_k, krm_buf ins_v, krm_buf slot_k,
                             krm_buf slot_v, krm_buf out, uint32_t batch, uint32_t heads,
                             uint32_t kv_heads, uint32_t chunk_rows, uint32_t depth,
@@ -383,6 +392,11 @@ int32_t krm_attention_varlen_planned(krm_ctx* ctx, krm_buf q, krm_buf ins_k, krm
  * packages/runtime/src/kernels/rms-norm.ts:35-91 */
 int32_t krm_rms_norm(krm_ctx* ctx, krm_buf x, krm_buf weight_f32, krm_buf out, uint32_t rows,
                      uint32_t dim, float eps, int32_t io_dtype);
+/* The same with the result stored as out_dtype: io_dtype, or KRM_F16 for f32 rows (the f32
+ * result rounded once — the copy a KRM_COMPUTE_F16 product reads through x_dtype; no
+ * counterpart in the reference, which has no mixed-type activations). */
+int32_t krm_rms_norm_cast(krm_ctx* ctx, krm_buf x, krm_buf weight_f32, krm_buf out, uint32_t rows,
+                          uint32_t dim, float eps, int32_t io_dtype, int32_t out_dtype);
 /* Half-split RoPE: out = x*cos[pos] + rotate_half(x)*sin[pos] with cos/sin rows [table_rows, D]
  * (f32) looked up by positions[row] (i32, device); both products are rounded before the add
  * (packages/runtime/src/kernels/rope.ts:5-20,52-80).  x is [rows, heads, D]; out is
@@ -432,7 +446,7 @@ int32_t krm_decode_qkv(krm_ctx* ctx, krm_buf x, krm_buf norm_weight_f32, float n
  * head-major layouts the attention reads:
  *   q_out [H, m, D]   k_out [Hkv, m, D]   v_out [Hkv, m, D]      (io_dtype)
  * The state appends stay separate calls (after the attention, as docs/ir-v1.md:345-348 orders
- * them).  Same coverage limits as krm_linear_i4_rows.
+ * them).  Same coverage limits and the same x_dtype rule as krm_linear_i4_rows.
  * Fuses packages/runtime/src/kernels/linear.ts:34-64, packages/runtime/src/kernels/rope.ts:5-20,
  * 52-80 and the permute nodes of tools/export-recipes/minicpm5/export_decode.py:14-35. */
 int32_t krm_prefill_qkv(krm_ctx* ctx, krm_buf x, krm_buf w, krm_buf scales, krm_buf bias,
@@ -440,7 +454,7 @@ int32_t krm_prefill_qkv(krm_ctx* ctx, krm_buf x, krm_buf w, krm_buf scales, krm_
                         krm_buf q_out, krm_buf k_out, krm_buf v_out, uint32_t m, uint32_t heads,
                         uint32_t kv_heads, uint32_t depth, uint32_t k, uint32_t group,
                         uint32_t table_rows, int32_t io_dtype, int32_t scale_dtype,
-                        int32_t compute);
+                        int32_t compute, int32_t x_dtype);
 /* ---- w4a8: `linear` with int4 weights on integer dot products (the reference's opt-in
  *      SessionOptions.linearCompute "i8a8" with int4-resident weights,
  *      packages/runtime/src/runtime/recipe-builder.ts:1320-1341,1407-1488;

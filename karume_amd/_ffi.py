@@ -49,9 +49,9 @@ PROTOTYPES = {
     "krm_linear_i4_fused": (i32, [c_ctx, c_buf, c_buf, C.c_float, c_buf, c_buf, c_buf, c_buf,
                                   c_buf, u32, u32, u32, u32, i32, i32, i32]),
     "krm_linear_i4_rows": (i32, [c_ctx, c_buf, c_buf, c_buf, c_buf, c_buf, c_buf, u32, u32, u32,
-                                 u32, i32, i32, i32, i32]),
+                                 u32, i32, i32, i32, i32, i32]),
     "krm_prefill_qkv": (i32, [c_ctx, c_buf, c_buf, c_buf, c_buf, c_buf, c_buf, c_buf, c_buf, c_buf,
-                              c_buf, u32, u32, u32, u32, u32, u32, u32, i32, i32, i32]),
+                              c_buf, u32, u32, u32, u32, u32, u32, u32, i32, i32, i32, i32]),
     "krm_quantize_rows": (i32, [c_ctx, c_buf, c_buf, c_buf, u32, u32]),
     "krm_linear_w4a8": (i32, [c_ctx, c_buf, c_buf, c_buf, c_buf, c_buf, c_buf, u32, u32, u32, u32,
                               i32]),
@@ -89,6 +89,7 @@ PROTOTYPES = {
     "krm_state_append_lengths": (i32, [c_ctx, c_buf, c_buf, u32, u32, u32, u32, u32, c_buf, i32,
                                        i32]),
     "krm_rms_norm": (i32, [c_ctx, c_buf, c_buf, c_buf, u32, u32, C.c_float, i32]),
+    "krm_rms_norm_cast": (i32, [c_ctx, c_buf, c_buf, c_buf, u32, u32, C.c_float, i32, i32]),
     "krm_rope_half": (i32, [c_ctx, c_buf, c_buf, c_buf, c_buf, c_buf, u32, u32, u32, u32, i32,
                             i32]),
     "krm_decode_rope_append": (i32, [c_ctx, c_buf, c_buf, c_buf, c_buf, c_buf, c_buf, c_buf, u32,

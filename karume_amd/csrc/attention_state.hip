@@ -233,6 +233,7 @@ __global__ __launch_bounds__(64 * WAVES) void attention_rows_kernel(
   if (!device_lengths(a.lengths, a.chunk_rows, a.capacity, a.window, past, query)) return;
 
   const bool row_major = (flags & KRM_CHUNK_OUT_ROW_MAJOR) != 0;
+  const bool out_f16 = (flags & KRM_CHUNK_OUT_F16) != 0;  // fp16 `out` beside f32 q / k / v
   auto out_index = [&](uint32_t row, uint32_t d) -> size_t {
     if (row_major) {  // [B, M, H, D]
       const uint32_t b = z / a.heads, head = z - b * a.heads;
@@ -261,7 +262,11 @@ __global__ __launch_bounds__(64 * WAVES) void attention_rows_kernel(
   if (row0 >= query) {  // a block of pad rows: exact zeros, nothing is read
     for (uint32_t i = tid; i < (uint32_t)kRows * D; i += kBlock) {
       const uint32_t row = row0 + i / D;
-      if (row < a.chunk_rows) st_f32<XT>(out, out_index(row, i % D), 0.0f);
+      if (row >= a.chunk_rows) continue;
+      if (out_f16)
+        st_f32<__half>(reinterpret_cast<__half*>(out), out_index(row, i % D), 0.0f);
+      else
+        st_f32<XT>(out, out_index(row, i % D), 0.0f);
     }
     return;
   }
@@ -451,7 +456,12 @@ __global__ __launch_bounds__(64 * WAVES) void attention_rows_kernel(
         float o = 0.f;
 #pragma unroll
         for (int wv = 0; wv < WAVES; ++wv) o = fmaf(wgt[wv], s_k[wv][rr * kRow + d0 + e], o);
-        st_f32<XT>(out, out_index(row, d0 + e), row < query ? o * inv : 0.0f);
+        float value = row < query ? o * inv : 0.0f;
+        if (out_f16 && sizeof(XT) == 4) value = rounded_f32(value);  // the f32 result, rounded again
+        if (out_f16)
+          st_f32<__half>(reinterpret_cast<__half*>(out), out_index(row, d0 + e), value);
+        else
+          st_f32<XT>(out, out_index(row, d0 + e), value);
       }
     }
    }
@@ -1371,7 +1381,8 @@ int32_t krm_attention_chunk(krm_ctx* ctx, krm_buf q, krm_buf ins_k, krm_buf ins_
                             uint32_t capacity, uint32_t window, float half_scale, uint32_t past,
                             uint32_t query, krm_buf lengths, int32_t io_dtype, int32_t kv_dtype,
                             uint32_t flags) {
-  KRM_REQUIRE(ctx, (flags & ~(uint32_t)(KRM_CHUNK_OUT_ROW_MAJOR | KRM_CHUNK_APPEND)) == 0,
+  KRM_REQUIRE(ctx, (flags & ~(uint32_t)(KRM_CHUNK_OUT_ROW_MAJOR | KRM_CHUNK_APPEND |
+                                        KRM_CHUNK_OUT_F16)) == 0,
               "krm_attention_chunk: unknown flags 0x%x", flags);
   KRM_REQUIRE(ctx, !(flags & KRM_CHUNK_APPEND) || window == 0,
               "krm_attention_chunk: the fused append needs window == 0 (a ring overwrites rows "

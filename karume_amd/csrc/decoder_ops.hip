@@ -39,13 +39,17 @@ __device__ inline float block_sum(float v, float* scratch) {
 
 // rms_norm: out = x * rsqrt(mean(x^2) + eps) * weight, one workgroup per row.
 // packages/runtime/src/kernels/rms-norm.ts:35-91 (no mean subtraction; weight is f32).
-template <typename XT>
+// OT: the type the result is stored in (XT, or fp16 beside f32 rows: a copy for a consumer
+// that would round the f32 result to fp16 anyway).
+template <typename XT, typename OT = XT>
 __global__ __launch_bounds__(kThreads) void rms_norm_kernel(const XT* __restrict__ x,
                                                            const float* __restrict__ weight,
-                                                           XT* __restrict__ out, uint32_t dim,
+                                                           OT* __restrict__ out, uint32_t dim,
                                                            float eps) {
   __shared__ float scratch[kThreads / kWave];
   const size_t base = (size_t)blockIdx.x * dim;
+  // the fp16 copy of an f32 row is the f32 result rounded again, never a product rounded once
+  auto keep_f32 = [](float v) { return sizeof(OT) == sizeof(XT) ? v : rounded_f32(v); };
   constexpr int kKeep = 16;  // rows up to 4096 elements stay in registers: one trip to memory
   if (dim <= (uint32_t)(kThreads * kKeep)) {
     float v[kKeep], wv[kKeep];
@@ -64,7 +68,7 @@ __global__ __launch_bounds__(kThreads) void rms_norm_kernel(const XT* __restrict
 #pragma unroll
     for (int j = 0; j < kKeep; ++j) {
       const uint32_t i = threadIdx.x + j * kThreads;
-      if (i < dim) st<XT>(out, base + i, v[j] * inv * wv[j]);
+      if (i < dim) st<OT>(out, base + i, keep_f32(v[j] * inv * wv[j]));
     }
     return;
   }
@@ -76,7 +80,7 @@ __global__ __launch_bounds__(kThreads) void rms_norm_kernel(const XT* __restrict
   const float total = block_sum(squares, scratch);
   const float inv = 1.0f / sqrtf(total / (float)dim + eps);
   for (uint32_t i = threadIdx.x; i < dim; i += kThreads)
-    st<XT>(out, base + i, ld<XT>(x, base + i) * inv * weight[i]);
+    st<OT>(out, base + i, keep_f32(ld<XT>(x, base + i) * inv * weight[i]));
 }
 
 // Half-split RoPE with the cos / sin rows looked up by absolute position:
@@ -317,6 +321,21 @@ int32_t krm_rms_norm(krm_ctx* ctx, krm_buf x, krm_buf weight_f32, krm_buf out, u
                   (rms_norm_kernel<__half><<<dim3(rows), dim3(kThreads), 0, ctx->stream>>>(
                       ptr<const __half>(x), ptr<const float>(weight_f32), ptr<__half>(out), dim,
                       eps)));
+  return launched(ctx, "rms_norm_kernel");
+}
+
+int32_t krm_rms_norm_cast(krm_ctx* ctx, krm_buf x, krm_buf weight_f32, krm_buf out, uint32_t rows,
+                          uint32_t dim, float eps, int32_t io_dtype, int32_t out_dtype) {
+  if (out_dtype == io_dtype) return krm_rms_norm(ctx, x, weight_f32, out, rows, dim, eps, io_dtype);
+  KRM_TRY(enter(ctx));
+  KRM_REQUIRE(ctx, io_dtype == KRM_F32 && out_dtype == KRM_F16,
+              "krm_rms_norm_cast: io_dtype %d -> out_dtype %d (f32 -> fp16, or the same type)",
+              io_dtype, out_dtype);
+  KRM_REQUIRE(ctx, dim >= 1 && std::isfinite(eps), "krm_rms_norm_cast: dim %u / eps", dim);
+  if (rows == 0) return KRM_OK;
+  KRM_REQUIRE(ctx, x && weight_f32 && out, "krm_rms_norm_cast: NULL buffer");
+  rms_norm_kernel<float, __half><<<dim3(rows), dim3(kThreads), 0, ctx->stream>>>(
+      ptr<const float>(x), ptr<const float>(weight_f32), ptr<__half>(out), dim, eps);
   return launched(ctx, "rms_norm_kernel");
 }
 

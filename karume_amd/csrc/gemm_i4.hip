@@ -1538,11 +1538,14 @@ struct RowPiece<__half, OPERAND> {
   }
 };
 
-template <typename XT, typename ST, int OPERAND, int WN>
+// XT: element type of x; OT: element type of bias, residual and out (the call's io type).  They
+// differ only for fp16 x with f32 io: an fp16 copy of the activations written by the producing
+// kernel, the same values the f32 activations are rounded to under KRM_COMPUTE_F16.
+template <typename XT, typename OT, typename ST, int OPERAND, int WN>
 __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2)))
 void gemm_i4_rows_kernel(const XT* __restrict__ x, const uint8_t* __restrict__ w,
-                         const ST* __restrict__ scales, const XT* __restrict__ bias,
-                         XT* __restrict__ out, uint32_t m, uint32_t n, uint32_t k,
+                         const ST* __restrict__ scales, const OT* __restrict__ bias,
+                         OT* __restrict__ out, uint32_t m, uint32_t n, uint32_t k,
                          uint32_t group_shift, uint32_t m_blocks, uint32_t tiles,
                          const float* __restrict__ row_scale, RowsFusion fuse) {
   constexpr int BM = 32, BN = 32 * WN, kWaves = 8;
@@ -1765,11 +1768,11 @@ void gemm_i4_rows_kernel(const XT* __restrict__ x, const uint8_t* __restrict__ w
       v0 *= s_inv[local];
       v1 *= s_inv[local];
     }
-    finish_pair<XT>(v0, v1, row, col, m, n, bias, out, fuse);
+    finish_pair<OT>(v0, v1, row, col, m, n, bias, out, fuse);
   }
 }
 
-template <typename XT, typename ST, int OPERAND, int WN>
+template <typename XT, typename OT, typename ST, int OPERAND, int WN>
 int32_t launch_rows(krm_ctx* ctx, krm_buf x, krm_buf w, krm_buf scales, krm_buf bias, krm_buf out,
                     uint32_t m, uint32_t n, uint32_t k, uint32_t group_shift,
                     const RowsFusion& fuse) {
@@ -1779,10 +1782,10 @@ int32_t launch_rows(krm_ctx* ctx, krm_buf x, krm_buf w, krm_buf scales, krm_buf 
   }
   const uint32_t m_blocks = (m + 31) / 32, n_blocks = (n + 32 * WN - 1) / (32 * WN);
   const uint32_t tiles = m_blocks * n_blocks;
-  gemm_i4_rows_kernel<XT, ST, OPERAND, WN>
+  gemm_i4_rows_kernel<XT, OT, ST, OPERAND, WN>
       <<<dim3(((tiles + 7) / 8) * 8), dim3(512), 0, ctx->stream>>>(
-          ptr<const XT>(x), ptr<const uint8_t>(w), ptr<const ST>(scales), ptr<const XT>(bias),
-          ptr<XT>(out), m, n, k, group_shift, m_blocks, tiles, ctx->row_scales, fuse);
+          ptr<const XT>(x), ptr<const uint8_t>(w), ptr<const ST>(scales), ptr<const OT>(bias),
+          ptr<OT>(out), m, n, k, group_shift, m_blocks, tiles, ctx->row_scales, fuse);
   return launched(ctx, "gemm_i4_rows_kernel");
 }
 
@@ -1841,8 +1844,10 @@ int32_t linear_i4_gemm_exact(krm_ctx* ctx, krm_buf x, krm_buf w, krm_buf scales,
 int32_t linear_i4_gemm_rows(krm_ctx* ctx, krm_buf x, krm_buf w, krm_buf scales, krm_buf bias,
                             krm_buf out, uint32_t m, uint32_t n, uint32_t k, uint32_t group,
                             int32_t io_dtype, int32_t scale_dtype, int32_t compute,
-                            const RowsFusion& fuse, bool* handled) {
+                            const RowsFusion& fuse, bool* handled, int32_t x_dtype) {
   *handled = false;
+  const bool half_x = x_dtype == KRM_F16 && io_dtype == KRM_F32;  // fp16 x, f32 bias / out
+  if (x_dtype != io_dtype && !(half_x && compute == KRM_COMPUTE_F16)) return KRM_OK;
   const bool split = compute == KRM_COMPUTE_F32 && io_dtype == KRM_F32;
   if (group < 64 || k % 32 != 0 || !aligned(w, 16) || !aligned(x, 16)) return KRM_OK;
   if (split && (m > kMaxSplitRows || !ctx->row_scales)) return KRM_OK;
@@ -1855,19 +1860,25 @@ int32_t linear_i4_gemm_rows(krm_ctx* ctx, krm_buf x, krm_buf w, krm_buf scales, 
   // 64 columns a workgroup once 32 would need more than one round of workgroups: fewer reads of
   // x for the same weights
   const bool wide = m_blocks * ((n + 31) / 32) > (uint64_t)ctx->num_cus;
-#define KRM_ROWS(XT, ST, OP)                                                                      \
-  return wide ? launch_rows<XT, ST, OP, 2>(ctx, x, w, scales, bias, out, m, n, k, group_shift, fuse) \
-              : launch_rows<XT, ST, OP, 1>(ctx, x, w, scales, bias, out, m, n, k, group_shift, fuse)
+#define KRM_ROWS(XT, OT, ST, OP)                                                                  \
+  return wide ? launch_rows<XT, OT, ST, OP, 2>(ctx, x, w, scales, bias, out, m, n, k, group_shift, \
+                                               fuse)                                              \
+              : launch_rows<XT, OT, ST, OP, 1>(ctx, x, w, scales, bias, out, m, n, k, group_shift, \
+                                               fuse)
   if (io_dtype == KRM_F16) {
-    if (scale_dtype == KRM_F16) KRM_ROWS(__half, __half, kOperandF16);
-    KRM_ROWS(__half, float, kOperandF16);
+    if (scale_dtype == KRM_F16) KRM_ROWS(__half, __half, __half, kOperandF16);
+    KRM_ROWS(__half, __half, float, kOperandF16);
+  }
+  if (half_x) {
+    if (scale_dtype == KRM_F16) KRM_ROWS(__half, float, __half, kOperandF16);
+    KRM_ROWS(__half, float, float, kOperandF16);
   }
   if (split) {
-    if (scale_dtype == KRM_F16) KRM_ROWS(float, __half, kOperandSplit);
-    KRM_ROWS(float, float, kOperandSplit);
+    if (scale_dtype == KRM_F16) KRM_ROWS(float, float, __half, kOperandSplit);
+    KRM_ROWS(float, float, float, kOperandSplit);
   }
-  if (scale_dtype == KRM_F16) KRM_ROWS(float, __half, kOperandF16);
-  KRM_ROWS(float, float, kOperandF16);
+  if (scale_dtype == KRM_F16) KRM_ROWS(float, float, __half, kOperandF16);
+  KRM_ROWS(float, float, float, kOperandF16);
 #undef KRM_ROWS
 }
 

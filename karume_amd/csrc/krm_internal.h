@@ -63,6 +63,16 @@ constexpr uint32_t kMaxSplitRows = 1u << 16;
 // Records the message on the context (or on the context-less slot) and returns `code`.
 int32_t fail(krm_ctx* ctx, int32_t code, const char* fmt, ...);
 
+#if defined(__HIPCC__)
+// `v` as the f32 it has been rounded to.  Without this the compiler may fold the product that
+// made `v` and a conversion to fp16 that follows into one mixed-precision instruction with a
+// single rounding — a different fp16 on ties than the f32 value stored and rounded later.
+__device__ inline float rounded_f32(float v) {
+  asm volatile("" : "+v"(v));
+  return v;
+}
+#endif
+
 // Maps a HIP runtime status to an error class; 0 when `status` is hipSuccess.
 int32_t hip_status(krm_ctx* ctx, hipError_t status, const char* what);
 

@@ -1039,7 +1039,7 @@ int32_t linear_i4_gemm_exact(krm_ctx* ctx, krm_buf x, krm_buf w, krm_buf scales,
 int32_t linear_i4_gemm_rows(krm_ctx* ctx, krm_buf x, krm_buf w, krm_buf scales, krm_buf bias,
                             krm_buf out, uint32_t m, uint32_t n, uint32_t k, uint32_t group,
                             int32_t io_dtype, int32_t scale_dtype, int32_t compute,
-                            const RowsFusion& fuse, bool* handled);
+                            const RowsFusion& fuse, bool* handled, int32_t x_dtype);
 int32_t linear_i4_gemm_f16(krm_ctx* ctx, krm_buf x, krm_buf w, krm_buf scales, krm_buf bias,
                            krm_buf out, uint32_t m, uint32_t n, uint32_t k, uint32_t group,
                            int32_t io_dtype, int32_t scale_dtype);
@@ -1078,7 +1078,7 @@ int32_t krm_linear_i4(krm_ctx* ctx, krm_buf x, krm_buf w, krm_buf scales, krm_bu
     if (workgroups > (uint64_t)ctx->num_cus) workgroups = (workgroups + 1) / 2;
     if (workgroups <= 3ull * (uint64_t)ctx->num_cus) {
       KRM_TRY(linear_i4_gemm_rows(ctx, x, w, scales, bias, out, m, n, k, group, io_dtype,
-                                  scale_dtype, compute, RowsFusion{}, &handled));
+                                  scale_dtype, compute, RowsFusion{}, &handled, io_dtype));
       if (handled) return KRM_OK;
     }
   }
@@ -1086,7 +1086,7 @@ int32_t krm_linear_i4(krm_ctx* ctx, krm_buf x, krm_buf w, krm_buf scales, krm_bu
                                scale_dtype, compute, &handled));
   if (handled) return KRM_OK;
   KRM_TRY(linear_i4_gemm_rows(ctx, x, w, scales, bias, out, m, n, k, group, io_dtype, scale_dtype,
-                              compute, RowsFusion{}, &handled));
+                              compute, RowsFusion{}, &handled, io_dtype));
   if (handled) return KRM_OK;
   if (compute == KRM_COMPUTE_F16)
     return linear_i4_gemm_f16(ctx, x, w, scales, bias, out, m, n, k, group, io_dtype,
@@ -1138,10 +1138,14 @@ int32_t krm_linear_i4_fused(krm_ctx* ctx, krm_buf x, krm_buf norm_weight_f32, fl
 int32_t krm_linear_i4_rows(krm_ctx* ctx, krm_buf x, krm_buf w, krm_buf scales, krm_buf bias,
                            krm_buf residual, krm_buf out, uint32_t m, uint32_t n, uint32_t k,
                            uint32_t group, int32_t io_dtype, int32_t scale_dtype, int32_t compute,
-                           int32_t epilogue) {
+                           int32_t epilogue, int32_t x_dtype) {
   KRM_TRY(enter(ctx));
   KRM_REQUIRE(ctx, valid_dtype(io_dtype) && valid_dtype(scale_dtype),
               "krm_linear_i4_rows: io_dtype %d / scale_dtype %d", io_dtype, scale_dtype);
+  KRM_REQUIRE(ctx, x_dtype == io_dtype ||
+                       (x_dtype == KRM_F16 && io_dtype == KRM_F32 && compute == KRM_COMPUTE_F16),
+              "krm_linear_i4_rows: x_dtype %d with io_dtype %d / compute %d (fp16 x beside f32 io "
+              "needs KRM_COMPUTE_F16)", x_dtype, io_dtype, compute);
   KRM_REQUIRE(ctx, compute == KRM_COMPUTE_F32 || compute == KRM_COMPUTE_F16,
               "krm_linear_i4_rows: compute %d", compute);
   KRM_REQUIRE(ctx, epilogue == KRM_EPILOGUE_NONE || epilogue == KRM_EPILOGUE_SILU_PAIRS,
@@ -1162,7 +1166,7 @@ int32_t krm_linear_i4_rows(krm_ctx* ctx, krm_buf x, krm_buf w, krm_buf scales, k
   fuse.mode = epilogue == KRM_EPILOGUE_SILU_PAIRS ? 1 : 0;
   bool handled = false;
   KRM_TRY(linear_i4_gemm_rows(ctx, x, w, scales, bias, out, m, n, k, group, io_dtype, scale_dtype,
-                              compute, fuse, &handled));
+                              compute, fuse, &handled, x_dtype));
   if (handled) return KRM_OK;
   return fail(ctx, KRM_ERR_VALIDATION,
               "krm_linear_i4_rows: covers group_size >= 64, k %% 32 == 0, 16-byte aligned x and w, "
@@ -1175,10 +1179,14 @@ int32_t krm_prefill_qkv(krm_ctx* ctx, krm_buf x, krm_buf w, krm_buf scales, krm_
                         krm_buf q_out, krm_buf k_out, krm_buf v_out, uint32_t m, uint32_t heads,
                         uint32_t kv_heads, uint32_t depth, uint32_t k, uint32_t group,
                         uint32_t table_rows, int32_t io_dtype, int32_t scale_dtype,
-                        int32_t compute) {
+                        int32_t compute, int32_t x_dtype) {
   KRM_TRY(enter(ctx));
   KRM_REQUIRE(ctx, valid_dtype(io_dtype) && valid_dtype(scale_dtype),
               "krm_prefill_qkv: io_dtype %d / scale_dtype %d", io_dtype, scale_dtype);
+  KRM_REQUIRE(ctx, x_dtype == io_dtype ||
+                       (x_dtype == KRM_F16 && io_dtype == KRM_F32 && compute == KRM_COMPUTE_F16),
+              "krm_prefill_qkv: x_dtype %d with io_dtype %d / compute %d (fp16 x beside f32 io "
+              "needs KRM_COMPUTE_F16)", x_dtype, io_dtype, compute);
   KRM_REQUIRE(ctx, compute == KRM_COMPUTE_F32 || compute == KRM_COMPUTE_F16,
               "krm_prefill_qkv: compute %d", compute);
   KRM_REQUIRE(ctx, is_pow2(group) && group >= 16 && k >= 1 && k % group == 0,
@@ -1214,7 +1222,7 @@ int32_t krm_prefill_qkv(krm_ctx* ctx, krm_buf x, krm_buf w, krm_buf scales, krm_
   const uint32_t n = (heads + 2 * kv_heads) * depth;
   bool handled = false;
   KRM_TRY(linear_i4_gemm_rows(ctx, x, w, scales, bias, q_out, m, n, k, group, io_dtype, scale_dtype,
-                              compute, fuse, &handled));
+                              compute, fuse, &handled, x_dtype));
   if (handled) return KRM_OK;
   return fail(ctx, KRM_ERR_VALIDATION,
               "krm_prefill_qkv: covers group_size >= 64, k %% 32 == 0, 16-byte aligned x and w, "

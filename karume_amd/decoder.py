@@ -163,6 +163,7 @@ class LlamaDecoderSession:
         self.kv_eb = 2 if kv_dtype == F16 else 4
         self.chunk_length = chunk_length
         self.prefill_compute = prefill_compute
+        self.half_activations = True  # fp16 copies of product-only activations (COMPUTE_F16)
         # One-row steps use the fused launches: rms_norm + [q;k;v], o + residual,
         # rms_norm + interleaved gate/up + silu*mul, down + residual.
         self.fuse_decode = fuse_decode
@@ -368,13 +369,19 @@ class LlamaDecoderSession:
         d, group, compute = c.d_model, c.group_size, self.prefill_compute
         spec = dict(chunk_rows=m, depth=c.head_dim, capacity=context.capacity,
                     window=context.window)
+        # COMPUTE_F16 rounds the f32 activations of every product to fp16: the three activations
+        # only a product reads (both norms' outputs, the attention's, silu(gate) * up) are then
+        # written as fp16 by their producers — the same values, half the bytes for the products
+        half = (self.half_activations and compute == COMPUTE_F16 and io == F32
+                and c.head_dim in (64, 128))
+        xd = F16 if half else io
         for li, lw in enumerate(self.layers):
-            g.rms_norm(b["h"], lw["attn_norm"], b["xn"], m, d, c.rms_eps, io)
+            g.rms_norm_cast(b["h"], lw["attn_norm"], b["xn"], m, d, c.rms_eps, io, xd)
             lin = lw["qkv"]
             g.prefill_qkv(b["xn"], lin.w, lin.s, b["pos"], self.rope_cos, self.rope_sin, b["qr"],
                           b["kr"], b["vt"], m=m, heads=c.heads, kv_heads=c.kv_heads,
                           depth=c.head_dim, k=d, group=group, table_rows=c.max_position,
-                          io_dtype=io, scale_dtype=lin.scale_dtype, compute=compute)
+                          io_dtype=io, scale_dtype=lin.scale_dtype, compute=compute, x_dtype=xd)
             if c.head_dim in (64, 128):
                 # attention + output permute (+ both appends when no window can wrap) in one launch
                 g.attention_chunk(b["qr"], b["kr"], b["vt"], context.slots_k[li],
@@ -382,7 +389,7 @@ class LlamaDecoderSession:
                                   kv_heads=c.kv_heads, half_scale=c.half_scale, past=past,
                                   query=query, lengths=lengths, io_dtype=io,
                                   kv_dtype=self.kv_dtype, row_major=True,
-                                  append=context.window == 0, **spec)
+                                  append=context.window == 0, out_f16=half, **spec)
                 if context.window != 0:
                     self._append_chunk(context, li, past, query, lengths, spec)
             else:
@@ -406,16 +413,17 @@ class LlamaDecoderSession:
             lin = lw["o"]
             g.linear_i4_rows(b["att2"], lin.w, lin.s, b["h"], m, lin.n, lin.k, group,
                              residual=b["h"], io_dtype=io, scale_dtype=lin.scale_dtype,
-                             compute=compute)
-            g.rms_norm(b["h"], lw["ffn_norm"], b["xn"], m, d, c.rms_eps, io)
+                             compute=compute, x_dtype=xd)
+            g.rms_norm_cast(b["h"], lw["ffn_norm"], b["xn"], m, d, c.rms_eps, io, xd)
             lin = lw["gate_up"]
+            # (fp16 in and out: silu(gate) * up is computed on the f32 sums and rounded once)
             g.linear_i4_rows(b["xn"], lin.w, lin.s, b["act"], m, lin.n, lin.k, group,
-                             io_dtype=io, scale_dtype=lin.scale_dtype, compute=compute,
+                             io_dtype=xd, scale_dtype=lin.scale_dtype, compute=compute,
                              epilogue=EPILOGUE_SILU_PAIRS)
             lin = lw["down"]
             g.linear_i4_rows(b["act"], lin.w, lin.s, b["h"], m, lin.n, lin.k, group,
                              residual=b["h"], io_dtype=io, scale_dtype=lin.scale_dtype,
-                             compute=compute)
+                             compute=compute, x_dtype=xd)
 
     def _replay_max_past(self, context: GenerationContext) -> int:
         """Largest pastLength the recorded step will be replayed with: sizes the attention

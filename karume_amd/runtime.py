@@ -21,7 +21,7 @@ COMPUTE_F16 = 1
 PROBE_EMPTY = 0
 PROBE_READ = 1
 EPILOGUE_NONE = 0
-CHUNK_OUT_ROW_MAJOR, CHUNK_APPEND = 1, 2
+CHUNK_OUT_ROW_MAJOR, CHUNK_APPEND, CHUNK_OUT_F16 = 1, 2, 4
 EPILOGUE_SILU_PAIRS = 1
 
 _NP_DTYPE_CODE = {np.dtype(np.float32): F32, np.dtype(np.float16): F16}
@@ -336,10 +336,11 @@ class GpuContext:
                         window: int, half_scale: float, past: int = 0, query: int = 0,
                         lengths: Optional[BufferLike] = None, io_dtype: int = F32,
                         kv_dtype: int = F32, row_major: bool = False,
-                        append: bool = False) -> None:
+                        append: bool = False, out_f16: bool = False) -> None:
         """The attention of a chunk of rows with the output permute and the state appends
-        folded in (D = 64 / 128)."""
-        flags = (CHUNK_OUT_ROW_MAJOR if row_major else 0) | (CHUNK_APPEND if append else 0)
+        folded in (D = 64 / 128); out_f16 stores the result as fp16 whatever io_dtype is."""
+        flags = ((CHUNK_OUT_ROW_MAJOR if row_major else 0) | (CHUNK_APPEND if append else 0)
+                 | (CHUNK_OUT_F16 if out_f16 else 0))
         self._check(self._lib.krm_attention_chunk(
             self._handle, _addr(q), _addr(ins_k), _addr(ins_v), _addr(slot_k), _addr(slot_v),
             _addr(out), batch, heads, kv_heads, chunk_rows, depth, capacity, window,
@@ -471,6 +472,13 @@ class GpuContext:
         self._check(self._lib.krm_rms_norm(self._handle, _addr(x), _addr(weight_f32), _addr(out),
                                            rows, dim, float(eps), io_dtype))
 
+    def rms_norm_cast(self, x: BufferLike, weight_f32: BufferLike, out: BufferLike, rows: int,
+                      dim: int, eps: float, io_dtype: int = F32, out_dtype: int = F16) -> None:
+        """rms_norm with the result stored as out_dtype (fp16 beside f32 rows)."""
+        self._check(self._lib.krm_rms_norm_cast(self._handle, _addr(x), _addr(weight_f32),
+                                                _addr(out), rows, dim, float(eps), io_dtype,
+                                                out_dtype))
+
     def rope_half(self, x: BufferLike, positions: BufferLike, cos_table: BufferLike,
                   sin_table: BufferLike, out: BufferLike, rows: int, heads: int, head_dim: int,
                   table_rows: int, to_head_major: bool = False, io_dtype: int = F32) -> None:
@@ -512,26 +520,29 @@ class GpuContext:
                        m: int, n: int, k: int, group: int, *, bias: Optional[BufferLike] = None,
                        residual: Optional[BufferLike] = None, io_dtype: int = F32,
                        scale_dtype: int = F32, compute: int = COMPUTE_F32,
-                       epilogue: int = EPILOGUE_NONE) -> None:
+                       epilogue: int = EPILOGUE_NONE, x_dtype: Optional[int] = None) -> None:
         """`linear` for a chunk of rows on the matrix cores, with the residual add or the
-        gate/up silu-mul folded in."""
+        gate/up silu-mul folded in.  x_dtype (default: io_dtype) may be F16 beside f32 io under
+        COMPUTE_F16: an fp16 copy of the activations, same result."""
         self._check(self._lib.krm_linear_i4_rows(
             self._handle, _addr(x), _addr(w), _addr(scales),
             _addr(bias) if bias is not None else 0, _addr(residual) if residual is not None else 0,
-            _addr(out), m, n, k, group, io_dtype, scale_dtype, compute, epilogue))
+            _addr(out), m, n, k, group, io_dtype, scale_dtype, compute, epilogue,
+            io_dtype if x_dtype is None else x_dtype))
 
     def prefill_qkv(self, x: BufferLike, w: BufferLike, scales: BufferLike, positions: BufferLike,
                     cos_table: BufferLike, sin_table: BufferLike, q_out: BufferLike,
                     k_out: BufferLike, v_out: BufferLike, *, m: int, heads: int, kv_heads: int,
                     depth: int, k: int, group: int, table_rows: int,
                     bias: Optional[BufferLike] = None, io_dtype: int = F32, scale_dtype: int = F32,
-                    compute: int = COMPUTE_F32) -> None:
+                    compute: int = COMPUTE_F32, x_dtype: Optional[int] = None) -> None:
         """Fused [q; k; v] projection of m rows + RoPE of q and k, written head-major."""
         self._check(self._lib.krm_prefill_qkv(
             self._handle, _addr(x), _addr(w), _addr(scales),
             _addr(bias) if bias is not None else 0, _addr(positions), _addr(cos_table),
             _addr(sin_table), _addr(q_out), _addr(k_out), _addr(v_out), m, heads, kv_heads, depth,
-            k, group, table_rows, io_dtype, scale_dtype, compute))
+            k, group, table_rows, io_dtype, scale_dtype, compute,
+            io_dtype if x_dtype is None else x_dtype))
 
     def transpose_01(self, x: BufferLike, out: BufferLike, a: int, b: int, d: int,
                      io_dtype: int = F32) -> None:

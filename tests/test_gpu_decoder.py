@@ -471,3 +471,105 @@ def test_prefill_qkv_equals_linear_rope_transpose(gpu_ctx, io, compute, m):
     q_host = got_q.download(io_np, (heads, m, d))
     assert np.all(np.isnan(q_host[:, m // 2])) and not np.any(np.isnan(np.delete(q_host, m // 2, 1)))
     assert not np.any(np.isnan(got_v.download(io_np, (kv_heads, m, d))))
+
+
+# ---- fp16 copies of the activations only a product reads (KRM_COMPUTE_F16 beside f32 io) ------
+
+def test_fp16_activation_copies_give_the_bits_of_the_f32_activations(gpu_ctx):
+    """KRM_COMPUTE_F16 rounds f32 activations to fp16 when a product reads them.  The producers
+    can store that rounding themselves (krm_rms_norm_cast, KRM_CHUNK_OUT_F16, an fp16-io
+    gate/up call) and the products read it through x_dtype: each piece equals the f32 route bit
+    for bit."""
+    rng = np.random.default_rng(77)
+    m, k, n, group = 70, 512, 384, 128
+    x = (rng.normal(size=(m, k)) * 3).astype(np.float32)
+    w = rng.normal(size=k).astype(np.float32)
+    dx, dw = gpu_ctx.upload(x), gpu_ctx.upload(w)
+    # rms_norm: the cast form stores the f32 result rounded once
+    n32, n16 = gpu_ctx.alloc(m * k * 4), gpu_ctx.alloc(m * k * 2)
+    gpu_ctx.rms_norm(dx, dw, n32, m, k, 1e-5, ka.F32)
+    gpu_ctx.rms_norm_cast(dx, dw, n16, m, k, 1e-5, ka.F32, ka.F16)
+    normed = n32.download(np.float32, (m, k))
+    assert np.array_equal(n16.download(np.float16, (m, k)).view(np.uint16),
+                          normed.astype(np.float16).view(np.uint16))
+    with pytest.raises(ka.GpuValidationError, match="f32 -> fp16"):
+        gpu_ctx.rms_norm_cast(dx, dw, n16, m, k, 1e-5, ka.F16, ka.F32)
+    # a product: f32 x under COMPUTE_F16 against the fp16 copy through x_dtype
+    packed, _q, scale = helpers.synthetic_int4(rng, n, k, group)
+    dpk, dsc = gpu_ctx.upload(packed), gpu_ctx.upload(scale)
+    res = rng.normal(size=(m, n)).astype(np.float32)
+    outs = []
+    for xbuf, xd in ((n32, ka.F32), (n16, ka.F16)):
+        out = gpu_ctx.upload(res)   # residual in place
+        gpu_ctx.linear_i4_rows(xbuf, dpk, dsc, out, m, n, k, group, residual=out,
+                               io_dtype=ka.F32, scale_dtype=ka.dtype_code(scale.dtype),
+                               compute=ka.COMPUTE_F16, x_dtype=xd)
+        outs.append(out.download(np.float32, (m, n)))
+    assert np.array_equal(outs[0].view(np.uint32), outs[1].view(np.uint32))
+    want = oracle.linear_i4(normed.astype(np.float16).astype(np.float32), packed,
+                            np.asarray(scale, np.float32), np.zeros(n, np.float32), n, k, group) + res
+    assert np.allclose(outs[1], want, rtol=1e-5, atol=2e-4)
+    # gate/up: fp16 in and out equals the f32 route's result rounded once
+    act32, act16 = gpu_ctx.alloc(m * (n // 2) * 4), gpu_ctx.alloc(m * (n // 2) * 2)
+    gpu_ctx.linear_i4_rows(n32, dpk, dsc, act32, m, n, k, group, io_dtype=ka.F32,
+                           scale_dtype=ka.dtype_code(scale.dtype), compute=ka.COMPUTE_F16,
+                           epilogue=ka.EPILOGUE_SILU_PAIRS)
+    gpu_ctx.linear_i4_rows(n16, dpk, dsc, act16, m, n, k, group, io_dtype=ka.F16,
+                           scale_dtype=ka.dtype_code(scale.dtype), compute=ka.COMPUTE_F16,
+                           epilogue=ka.EPILOGUE_SILU_PAIRS)
+    assert np.array_equal(act16.download(np.float16, (m, n // 2)).view(np.uint16),
+                          act32.download(np.float32, (m, n // 2)).astype(np.float16).view(np.uint16))
+    # the combinations the kernel does not have are rejected
+    with pytest.raises(ka.GpuValidationError, match="x_dtype"):
+        gpu_ctx.linear_i4_rows(n16, dpk, dsc, act32, m, n, k, group, io_dtype=ka.F32,
+                               scale_dtype=ka.dtype_code(scale.dtype), compute=ka.COMPUTE_F32,
+                               x_dtype=ka.F16)
+    with pytest.raises(ka.GpuValidationError, match="x_dtype"):
+        gpu_ctx.linear_i4_rows(n32, dpk, dsc, act16, m, n, k, group, io_dtype=ka.F16,
+                               scale_dtype=ka.dtype_code(scale.dtype), compute=ka.COMPUTE_F16,
+                               x_dtype=ka.F32)
+
+
+def test_attention_chunk_fp16_output_is_the_f32_output_rounded(gpu_ctx):
+    rng = np.random.default_rng(5)
+    heads, kvh, m, d, cap, past, query = 8, 2, 40, 64, 128, 50, 37
+    q = gpu_ctx.upload(rng.normal(size=(heads, m, d)).astype(np.float32))
+    ik = gpu_ctx.upload(rng.normal(size=(kvh, m, d)).astype(np.float32))
+    iv = gpu_ctx.upload(rng.normal(size=(kvh, m, d)).astype(np.float32))
+    sk = gpu_ctx.upload(rng.normal(size=(kvh, cap, d)).astype(np.float32))
+    sv = gpu_ctx.upload(rng.normal(size=(kvh, cap, d)).astype(np.float32))
+    o32 = gpu_ctx.upload(np.full(m * heads * d, 7.0, np.float32))
+    o16 = gpu_ctx.upload(np.full(m * heads * d, 7.0, np.float16))
+    spec = dict(batch=1, heads=heads, kv_heads=kvh, chunk_rows=m, depth=d, capacity=cap, window=0,
+                half_scale=oracle.half_scale(d), past=past, query=query, row_major=True)
+    gpu_ctx.attention_chunk(q, ik, iv, sk, sv, o32, **spec)
+    gpu_ctx.attention_chunk(q, ik, iv, sk, sv, o16, out_f16=True, **spec)
+    a = o32.download(np.float32, (m, heads, d))
+    b = o16.download(np.float16, (m, heads, d))
+    assert np.array_equal(b.view(np.uint16), a.astype(np.float16).view(np.uint16))
+    assert np.all(b[query:] == 0) and np.any(b[:query] != 0)
+
+
+def test_prefill_with_fp16_activation_copies_equals_prefill_without(gpu_ctx):
+    """A whole chunk through the decoder under KRM_COMPUTE_F16: logits and the appended state are
+    the same bits with and without the fp16 copies."""
+    config = LlamaConfig(layers=2, d_model=256, ffn=384, heads=4, kv_heads=2, head_dim=64,
+                         vocab=512, group_size=128, max_position=64)
+    weights = random_weights(config, seed=6)
+    rng = np.random.default_rng(2)
+    ids = rng.integers(0, config.vocab, size=(1, 40)).astype(np.int32)
+    pos = np.arange(40, dtype=np.int32).reshape(1, 40)
+    results = []
+    for copies in (True, False):
+        session = LlamaDecoderSession(gpu_ctx, weights, io_dtype=ka.F32, kv_dtype=ka.F32,
+                                      chunk_length=40, prefill_compute=ka.COMPUTE_F16)
+        session.half_activations = copies
+        ctx = session.create_generation_context(capacity=64, chunk_length=40)
+        token, logits = session.run(ids, pos, 36, context=ctx, query_length=37, want_logits=True)
+        state = ctx.slots_k[1].download(np.float32, (2, 64, 64))[:, :37].copy()
+        results.append((token.copy(), logits.copy(), state))
+        ctx.dispose()
+        session.close()
+    assert np.array_equal(results[0][1].view(np.uint32), results[1][1].view(np.uint32))
+    assert np.array_equal(results[0][2].view(np.uint32), results[1][2].view(np.uint32))
+    assert np.array_equal(results[0][0], results[1][0])
