@@ -348,8 +348,8 @@ def bench_gemm(timer: Timer, rng, steps: int, warmup: int, m: int, n: int, k: in
 
 def bench_prefill_chunk(timer: Timer, rng, steps: int, warmup: int, g: int):
     """A 128-row prefill chunk of the config-4 decoder, kernel by kernel: the four few-row
-    products of a layer (f32 activations as the model runs them, KRM_COMPUTE_F16; the f32 class
-    beside it) and the chunk's attention (32 heads, 4 kv heads, D = 64, past 0).  us per launch."""
+    products of a layer (f32 activations, KRM_COMPUTE_F16; the f32 class beside it; `x16`: the
+    same class reading the fp16 copy of the activations its producer wrote, as the decoder does) and the chunk's attention (32 heads, 4 kv heads, D = 64, past 0).  us per launch."""
     ctx, ka = timer.ctx, timer.ka
     m, d, ffn, heads, kv_heads, depth = 128, 2048, 5632, 32, 4, 64
     out = {}
@@ -365,15 +365,25 @@ def bench_prefill_chunk(timer: Timer, rng, steps: int, warmup: int, g: int):
         x = ctx.upload(rng.normal(size=(m, k)).astype(np.float32))
         y = ctx.alloc(m * n * 4)
         epilogue = ka.EPILOGUE_SILU_PAIRS if name == "gate_up" else ka.EPILOGUE_NONE
-        for label, compute in (("us", ka.COMPUTE_F16), ("f32class_us", ka.COMPUTE_F32)):
+        x16 = ctx.upload(rng.normal(size=(m, k)).astype(np.float16))
+        for label, compute in (("us", ka.COMPUTE_F16), ("f32class_us", ka.COMPUTE_F32),
+                               ("x16_us", ka.COMPUTE_F16)):
             def step(i: int) -> None:
                 j = i % copies
+                if label == "x16_us":
+                    # the form the decoder runs under KRM_COMPUTE_F16: x is the fp16 copy its
+                    # producer wrote; gate/up also writes fp16 (what the down-projection reads)
+                    io = ka.F16 if name == "gate_up" else ka.F32
+                    ctx.linear_i4_rows(x16, weights[j], scales[j], y, m, n, k, g, io_dtype=io,
+                                       scale_dtype=ka.F16, compute=compute, epilogue=epilogue,
+                                       x_dtype=ka.F16)
+                    return
                 ctx.linear_i4_rows(x, weights[j], scales[j], y, m, n, k, g, io_dtype=ka.F32,
                                    scale_dtype=ka.F16, compute=compute, epilogue=epilogue)
             res = timer.run(step, steps, warmup, replays=20)
             out[f"{name}_{label}"] = round(res["ms"] / steps * 1e3, 2)
         out[f"{name}_tflops"] = round(2.0 * m * n * k / (out[f"{name}_us"] * 1e-6) / 1e12, 1)
-        for b in weights + scales + [x, y]:
+        for b in weights + scales + [x, x16, y]:
             b.free()
     capacity = 2048
     q = ctx.upload(rng.normal(size=(heads, m, depth)).astype(np.float32))
