@@ -487,6 +487,24 @@ def bench_model(ctx, ka, io_dtype, kv_dtype, prompt_len: int = 128, new_tokens: 
         times.append((t_prefill - t_start, t_end - t_prefill))
         gen.dispose()
     prefill_s, decode_s = times[-1]
+    # The replayed tokens are checked before they are reported: the first eight must equal
+    # eight step-by-step runs (scalar lengths, a read-back per token) on a fresh context — the
+    # path tests/test_gpu_model_full.py checks against the CPU oracle at this size.
+    gen = session.create_generation_context(capacity=config.max_position,
+                                            chunk_length=prompt_len)
+    tok = int(session.run(prompt.reshape(1, prompt_len),
+                          np.arange(prompt_len, dtype=np.int32).reshape(1, prompt_len),
+                          prompt_len - 1, context=gen, query_length=prompt_len)[0, 0, 0])
+    stepwise = []
+    for i in range(8):
+        tok = int(session.run(np.array([[tok]], dtype=np.int32),
+                              np.array([[prompt_len + i]], dtype=np.int32), 0, context=gen,
+                              query_length=1)[0, 0, 0])
+        stepwise.append(tok)
+    gen.dispose()
+    if [int(t) for t in tokens[:8]] != stepwise:
+        raise SystemExit(f"[bench] config 4: the replayed decode produced {list(tokens[:8])}, "
+                         f"step-by-step runs {stepwise}")
     # the same prefill in the reference's default class (KRM_COMPUTE_F32: f32 x split hi + lo)
     session.prefill_compute = ka.COMPUTE_F32
     prefill_f32_s = None
@@ -511,6 +529,7 @@ def bench_model(ctx, ka, io_dtype, kv_dtype, prompt_len: int = 128, new_tokens: 
         "weight_gbs": round(bytes_per_token * (new_tokens - 1) / decode_s / 1e9, 1),
         "pct_of_hbm_peak": round(100 * bytes_per_token * (new_tokens - 1) / decode_s / 8e12, 2),
         "first_tokens": [int(t) for t in tokens[:8]],
+        "first_tokens_check": "equal to 8 step-by-step session.run calls on a fresh context",
     }
 
 

@@ -24,13 +24,6 @@ export const KARUME_HIP_SYMBOLS = {
   krm_event_record: { parameters: ["pointer", "pointer"], result: "i32" },
   krm_event_elapsed_ms: { parameters: ["pointer", "pointer", "pointer", "buffer"], result: "i32" },
   krm_event_destroy: { parameters: ["pointer", "pointer"], result: "i32" },
-  krm_probe_launch: { parameters: ["pointer", "i32", "u64", "usize", "u32", "u32"], result: "i32" },
-  krm_probe_exchange: {
-    parameters: [
-      "pointer", "u64", "usize", "u32", "u32", "u32"
-    ],
-    result: "i32",
-  },
   krm_graph_begin: { parameters: ["pointer"], result: "i32" },
   krm_graph_branch: { parameters: ["pointer", "u32"], result: "i32" },
   krm_graph_end: { parameters: ["pointer", "buffer"], result: "i32" },
@@ -223,3 +216,15 @@ export const KARUME_HIP_SYMBOLS = {
 } as const;
 
 export type KarumeHipLibrary = Deno.DynamicLibrary<typeof KARUME_HIP_SYMBOLS>;
+
+// Measurement probes (the DIAGNOSTICS section of the header): not ops of the runtime; bind them
+// only to reproduce bench.py's launch and read floors.
+export const KARUME_HIP_DIAGNOSTIC_SYMBOLS = {
+  krm_probe_launch: { parameters: ["pointer", "i32", "u64", "usize", "u32", "u32"], result: "i32" },
+  krm_probe_exchange: {
+    parameters: [
+      "pointer", "u64", "usize", "u32", "u32", "u32"
+    ],
+    result: "i32",
+  },
+} as const;

@@ -106,28 +106,6 @@ int32_t krm_event_record(krm_ctx* ctx, krm_event* ev);
 /* Waits for `stop`, then writes the milliseconds between the two recorded events. */
 int32_t krm_event_elapsed_ms(krm_ctx* ctx, krm_event* start, krm_event* stop, float* ms);
 int32_t krm_event_destroy(krm_ctx* ctx, krm_event* ev);
-/* Measurement floors for a launch of `grid` workgroups of `block` threads on the context's
- * stream (diagnostics like the timestamp queries above; no op of the reference):
- *   KRM_PROBE_EMPTY — a kernel that does nothing (what a launch of that grid costs);
- *   KRM_PROBE_READ  — every thread streams its share of `bytes` at `src` with 16-byte loads
- *                     and stores nothing (what reading that much costs); up to eight loads a
- *                     thread are requested before any is used, so a grid that covers `bytes`
- *                     in one pass pays one memory round trip. */
-#define KRM_PROBE_EMPTY 0
-#define KRM_PROBE_READ 1
-int32_t krm_probe_launch(krm_ctx* ctx, int32_t kind, krm_buf src, size_t bytes, uint32_t grid,
-                         uint32_t block);
-
-/* What an all-to-all hand-over of a vector of `entries` floats (2048, 4096 or 8192) costs
- * between the 256 workgroups of ONE persistent launch, `phases` times in a row: flags polled
- * and the vector read with agent-scope loads, results written with agent-scope stores (the
- * step a single-launch decode would pay at every op boundary).  `work` is scratch of at least
- * 2 * entries * 4 + 1040 bytes that the call clears; its last word written (offset
- * 2 * entries * 4 + 1024) is a fault flag: 1 if a poll exceeded `spin_limit` rounds (every wait
- * is bounded; the launch always ends).  Time it with events; no op of the reference. */
-int32_t krm_probe_exchange(krm_ctx* ctx, krm_buf work, size_t work_bytes, uint32_t entries,
-                           uint32_t phases, uint32_t spin_limit);
-
 /* ---- recorded launch sequences (the reference bakes a step's dispatch recipes once and
  *      replays them: executeBakedPlan, packages/runtime/src/runtime/recipe.ts:357-394) ------
  * Between krm_graph_begin and krm_graph_end the op entry points record instead of running
@@ -142,7 +120,14 @@ int32_t krm_graph_begin(krm_ctx* ctx);
  * main branch in krm_graph_end.  Ops on different branches must not depend on one another;
  * the device may run them at the same time (the recipes of one step that the reference
  * submits in one command buffer without barriers between independent dispatches,
- * packages/runtime/src/runtime/recipe.ts:385-394). */
+ * packages/runtime/src/runtime/recipe.ts:385-394).
+ * Ops that use the context's own scratch share it in launch order and therefore belong on the
+ * main branch; while a side branch is selected they fail with KRM_ERR_VALIDATION and record
+ * nothing: the decode attention when it splits the columns (more than four chunks),
+ * krm_attention_varlen / _planned, the unit-dealt MFMA GEMMs of krm_linear_i4 and every
+ * f32-class (KRM_COMPUTE_F32 with f32 x) MFMA product.  GEMVs (m <= 16), the fp16-operand
+ * few-row products, krm_attention_state_noalloc (its own scratch: still one call at a time per
+ * GPU) and the glue ops carry no such state. */
 int32_t krm_graph_branch(krm_ctx* ctx, uint32_t branch);
 int32_t krm_graph_end(krm_ctx* ctx, krm_graph** out);
 int32_t krm_graph_launch(krm_ctx* ctx, krm_graph* graph);
@@ -512,6 +497,33 @@ int32_t krm_embedding(krm_ctx* ctx, krm_buf table, krm_buf index_i32, krm_buf ou
  * (packages/runtime/src/kernels/argmax.ts:16-34). */
 int32_t krm_argmax(krm_ctx* ctx, krm_buf x, krm_buf out_i32, uint32_t rows, uint32_t dim,
                    int32_t io_dtype);
+
+/* ==== DIAGNOSTICS ============================================================================
+ * Not ops of the runtime: measurement probes that bench.py uses to state what a launch and a
+ * read of a given size cost on this machine.  A host binds them only if it wants those floors
+ * (include/karume_hip.ffi.ts lists them in a table of their own, KARUME_HIP_DIAGNOSTIC_SYMBOLS).
+ * ============================================================================================ */
+/* Measurement floors for a launch of `grid` workgroups of `block` threads on the context's
+ * stream (diagnostics like the timestamp queries above; no op of the reference):
+ *   KRM_PROBE_EMPTY — a kernel that does nothing (what a launch of that grid costs);
+ *   KRM_PROBE_READ  — every thread streams its share of `bytes` at `src` with 16-byte loads
+ *                     and stores nothing (what reading that much costs); up to eight loads a
+ *                     thread are requested before any is used, so a grid that covers `bytes`
+ *                     in one pass pays one memory round trip. */
+#define KRM_PROBE_EMPTY 0
+#define KRM_PROBE_READ 1
+int32_t krm_probe_launch(krm_ctx* ctx, int32_t kind, krm_buf src, size_t bytes, uint32_t grid,
+                         uint32_t block);
+
+/* What an all-to-all hand-over of a vector of `entries` floats (2048, 4096 or 8192) costs
+ * between the 256 workgroups of ONE persistent launch, `phases` times in a row: flags polled
+ * and the vector read with agent-scope loads, results written with agent-scope stores (the
+ * step a single-launch decode would pay at every op boundary).  `work` is scratch of at least
+ * 2 * entries * 4 + 1040 bytes that the call clears; its last word written (offset
+ * 2 * entries * 4 + 1024) is a fault flag: 1 if a poll exceeded `spin_limit` rounds (every wait
+ * is bounded; the launch always ends).  Time it with events; no op of the reference. */
+int32_t krm_probe_exchange(krm_ctx* ctx, krm_buf work, size_t work_bytes, uint32_t entries,
+                           uint32_t phases, uint32_t spin_limit);
 
 #ifdef __cplusplus
 }

@@ -1287,7 +1287,8 @@ static int32_t attention_state_impl(krm_ctx* ctx, krm_buf q, krm_buf ins_k, krm_
   const bool fast = !chunk_only && (dyn || query == 1) && chunk_rows == 1 && lpr &&
                     decode_repeat_ok(repeat) &&
                     aligned(slot_k, 16) && aligned(slot_v, 16) && aligned(q, 16) && batch <= 65535 &&
-                    heads <= 65535 && (uint64_t)batch * heads <= kTicketSlots;
+                    heads <= 65535 &&
+                    (uint64_t)batch * heads <= (tickets ? ticket_slots : kTicketSlots);
   if (fast) {
     const uint64_t low = window_low(window, past);
     const uint32_t nsplit = decode_splits((uint64_t)past - low, decode_split_columns(lpr));
@@ -1309,8 +1310,15 @@ static int32_t attention_state_impl(krm_ctx* ctx, krm_buf q, krm_buf ins_k, krm_
     L.args.lengths = ptr<uint32_t>(lengths);
     L.args.capacity = capacity;
     if (nsplit > 1) {
+      // split partials + arrival counters: the context's counters assume launch order
+      if (!tickets) KRM_TRY(needs_serial_scratch(ctx, "the split decode attention"));
       const size_t ml_floats = (size_t)batch * nsplit * heads * 2;
       const size_t need = (ml_floats + (size_t)batch * nsplit * heads * depth) * sizeof(float);
+      if (tickets && workspace_bytes < need + 16)
+        return fail(ctx, KRM_ERR_VALIDATION,
+                    "krm_attention_state_noalloc: this call needs %zu bytes of split partials, the "
+                    "built-in scratch holds %zu (use krm_attention_state with a workspace)",
+                    need + 16, workspace_bytes);
       KRM_REQUIRE(ctx, workspace && aligned(workspace, 16) && workspace_bytes >= need,
                   "krm_attention_state: workspace of %zu bytes, %zu needed", workspace_bytes,
                   need);
@@ -1491,6 +1499,7 @@ int32_t krm_attention_varlen(krm_ctx* ctx, krm_buf q, krm_buf ins_k, krm_buf ins
   L.ws_acc = L.ws_ml + ml_floats;
   L.grid_x = (uint32_t)splits;
   L.grid_z = 1;
+  KRM_TRY(needs_serial_scratch(ctx, "krm_attention_varlen"));
   L.args.tickets = ctx->tickets;
   return decode_dispatch<true>(ctx, L, repeat, lpr, io_dtype, kv_dtype);
 }
@@ -1617,6 +1626,7 @@ int32_t krm_attention_varlen_planned(krm_ctx* ctx, krm_buf q, krm_buf ins_k, krm
   L.ws_acc = L.ws_ml + ml_floats;
   L.grid_x = max_splits;
   L.grid_z = 1;
+  KRM_TRY(needs_serial_scratch(ctx, "krm_attention_varlen_planned"));
   L.args.tickets = ctx->tickets;
   return decode_dispatch<true>(ctx, L, repeat, lpr, io_dtype, kv_dtype);
 }
@@ -1659,6 +1669,15 @@ int32_t static_scratch(krm_ctx* ctx, unsigned char** out) {
 
 }  // namespace
 
+namespace krm {
+// Called when a context is created on a device, so that the address is known before any caller
+// starts recording a graph (the lookup is a runtime call that does not belong in a capture).
+int32_t resolve_static_scratch(krm_ctx* ctx) {
+  unsigned char* unused = nullptr;
+  return static_scratch(ctx, &unused);
+}
+}  // namespace krm
+
 extern "C" {
 
 int32_t krm_attention_state_noalloc(krm_ctx* ctx, krm_buf q, krm_buf ins_k, krm_buf ins_v,
@@ -1670,16 +1689,11 @@ int32_t krm_attention_state_noalloc(krm_ctx* ctx, krm_buf q, krm_buf ins_k, krm_
   KRM_TRY(enter(ctx));
   unsigned char* base = nullptr;
   KRM_TRY(static_scratch(ctx, &base));
-  // the same sizing rule as krm_attention_state_workspace, against the fixed array
-  size_t need = 0;
-  KRM_TRY(krm_attention_state_workspace(batch, heads, kv_heads, chunk_rows, depth, window, past,
-                                        query, &need));
+  // Only the split decode form needs scratch; it checks its partials against `room` and words
+  // the error for this entry.  Chunks of rows and head dims the decode form does not cover run
+  // without any, and a call with more heads than the array has counters takes the generic
+  // kernel.
   const size_t room = kStaticScratchBytes - kStaticTicketBytes;
-  if (need > room)
-    return fail(ctx, KRM_ERR_VALIDATION,
-                "krm_attention_state_noalloc: this call needs %zu bytes of split partials, the "
-                "built-in scratch holds %zu (use krm_attention_state with a workspace)",
-                need, room);
   return attention_state_impl(ctx, q, ins_k, ins_v, slot_k, slot_v, out, batch, heads, kv_heads,
                               chunk_rows, depth, capacity, window, half_scale, past, query, 0,
                               io_dtype, kv_dtype,

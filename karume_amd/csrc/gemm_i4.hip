@@ -1316,6 +1316,7 @@ template <typename XT, typename ST, int WM>
 int32_t launch_dealt(krm_ctx* ctx, krm_buf x, krm_buf w, krm_buf scales, krm_buf bias, krm_buf out,
                      uint32_t m, uint32_t n, uint32_t k, uint32_t group_shift, uint32_t grid,
                      const UnitDeal& deal) {
+  KRM_TRY(needs_serial_scratch(ctx, "the unit-dealt GEMM"));
   gemm_i4_f16_dealt_kernel<XT, ST, WM><<<dim3(grid), dim3(WM * 256), 0, ctx->stream>>>(
       ptr<const XT>(x), ptr<const uint8_t>(w), ptr<const ST>(scales), ptr<const XT>(bias),
       ptr<XT>(out), m, n, k, group_shift, (m + 127) / 128, deal);
@@ -1777,6 +1778,7 @@ int32_t launch_rows(krm_ctx* ctx, krm_buf x, krm_buf w, krm_buf scales, krm_buf 
                     uint32_t m, uint32_t n, uint32_t k, uint32_t group_shift,
                     const RowsFusion& fuse) {
   if constexpr (OPERAND == kOperandSplit) {
+    KRM_TRY(needs_serial_scratch(ctx, "the f32-class few-row GEMM"));
     row_scale_kernel<<<dim3(m), dim3(256), 0, ctx->stream>>>(ptr<const float>(x), ctx->row_scales, k);
     KRM_TRY(launched(ctx, "row_scale_kernel"));
   }
@@ -1793,6 +1795,7 @@ template <typename XT, typename ST, int OPERAND>
 int32_t launch_exact(krm_ctx* ctx, krm_buf x, krm_buf w, krm_buf scales, krm_buf bias, krm_buf out,
                      uint32_t m, uint32_t n, uint32_t k, uint32_t group_shift, uint32_t grid,
                      const UnitDeal& deal) {
+  KRM_TRY(needs_serial_scratch(ctx, "the unit-dealt GEMM"));
   if constexpr (OPERAND == kOperandSplit) {
     row_scale_kernel<<<dim3(m), dim3(256), 0, ctx->stream>>>(ptr<const float>(x), ctx->row_scales, k);
     KRM_TRY(launched(ctx, "row_scale_kernel"));

@@ -85,6 +85,12 @@ int32_t not_recording(krm_ctx* ctx, const char* what);
 // Error check of the launch that was just queued.
 int32_t launched(krm_ctx* ctx, const char* kernel);
 
+// The context's own scratch (arrival counters, GEMM partials, row scales) assumes that the ops
+// using it run one after the other, which only the main stream guarantees: ops recorded on a
+// side branch of a graph (krm_graph_branch) may run beside the main branch and beside each
+// other.  Entry points call this before they hand that scratch to a kernel.
+int32_t needs_serial_scratch(krm_ctx* ctx, const char* what);
+
 inline bool valid_dtype(int32_t dtype) { return dtype == KRM_F32 || dtype == KRM_F16; }
 inline size_t dtype_bytes(int32_t dtype) { return dtype == KRM_F16 ? 2 : 4; }
 inline bool is_pow2(uint32_t v) { return v != 0 && (v & (v - 1)) == 0; }

@@ -50,9 +50,22 @@ int32_t launched(krm_ctx* ctx, const char* kernel) {
   return hip_status(ctx, hipGetLastError(), kernel);
 }
 
+int32_t needs_serial_scratch(krm_ctx* ctx, const char* what) {
+  if (ctx->stream != ctx->main_stream)
+    return fail(ctx, KRM_ERR_VALIDATION,
+                "%s uses the context's scratch (arrival counters, partial sums or row scales), "
+                "which ops share in launch order: record it on the main branch, not on a side "
+                "branch of the graph", what);
+  return KRM_OK;
+}
+
 }  // namespace krm
 
 using namespace krm;
+
+namespace krm {
+int32_t resolve_static_scratch(krm_ctx* ctx);  // attention_state.hip
+}
 
 // Measurement floors: what a launch of a given grid costs when it does nothing, and when it
 // only streams `bytes` with 16-byte loads (every thread folds what it read into one word that
@@ -216,6 +229,10 @@ int32_t krm_ctx_create_on_stream(int32_t device, void* hip_stream, krm_ctx** out
     delete ctx;
     return hip_status(nullptr, st, "hipMalloc(tickets)");
   }
+  // The device address of the built-in scratch of krm_attention_state_noalloc is looked up now,
+  // with this device current, so that the entry's first call may already sit inside a graph
+  // recording.  A failure here is not fatal: the entry repeats the lookup and reports it.
+  if (resolve_static_scratch(ctx) != KRM_OK) ctx->error[0] = 0;
   *out = ctx;
   return KRM_OK;
 }

@@ -235,8 +235,14 @@ class LlamaDecoderSession:
             self.workspace = self.gpu.alloc(need)
         return ctx
 
-    def run(self, input_ids: np.ndarray, position_ids: np.ndarray, last_row: int, *,
+    def run(self, input_ids: np.ndarray, position_ids: np.ndarray, last_row: Optional[int], *,
             context: GenerationContext, query_length: int, want_logits: bool = False):
+        """One run of the decode graph over a chunk of M rows, of which the first
+        `query_length` are valid.  With `last_row` (the token-only exit of the reference's
+        default asset) the head runs on that row alone: token [1, 1, 1] (and logits [1, V]).
+        With `last_row=None` the session returns what the reference graph itself returns
+        (tools/export-recipes/minicpm5/export_decode.py:14-22): the argmax of every row,
+        [1, M, 1] (and logits [1, M, V]); rows past `query_length` are unspecified."""
         ids = np.ascontiguousarray(input_ids, dtype=np.int32)
         pos = np.ascontiguousarray(position_ids, dtype=np.int32)
         if ids.ndim != 2 or ids.shape[0] != 1 or pos.shape != ids.shape:
@@ -244,15 +250,24 @@ class LlamaDecoderSession:
                                  "[1, M]")
         m = ids.shape[1]
         past = context.begin_run(m, query_length)
-        if not 0 <= last_row < query_length:
+        all_rows = last_row is None
+        if not all_rows and not 0 <= last_row < query_length:
             raise ExecutionError(f"last_row {last_row} is outside the {query_length} valid rows")
         try:
             self.buf["ids"].upload(ids)
             self.buf["pos"].upload(pos)
-            self._forward(context, m, past, query_length, last_row, lengths=None)
-            token = self.buf["token"].download(np.int32, (1, 1, 1))
-            logits = (self.buf["logits"].download(self.io_np, self.logits_shape)
-                      if want_logits else None)
+            if all_rows and m > 1:
+                self._forward(context, m, past, query_length, None, lengths=None)
+                token = self.buf["tokens_all"].download(np.int32, (1, m, 1))
+                logits = (self.buf["logits_all"].download(self.io_np, (1, m, self.config.vocab))
+                          if want_logits else None)
+            else:
+                self._forward(context, m, past, query_length, 0 if all_rows else last_row,
+                              lengths=None)
+                token = self.buf["token"].download(np.int32, (1, 1, 1))
+                shape = (1, 1, self.config.vocab) if all_rows else self.logits_shape
+                logits = (self.buf["logits"].download(self.io_np, shape)
+                          if want_logits else None)
         except KarumeError:
             context.poison()  # a state write may already have happened: no rollback
             raise
@@ -265,8 +280,8 @@ class LlamaDecoderSession:
         self.gpu.linear_i4(x, lin.w, lin.s, None, out, m, lin.n, lin.k, self.config.group_size,
                            self.io_dtype, lin.scale_dtype, compute)
 
-    def _forward(self, context: GenerationContext, m: int, past: int, query: int, last_row: int,
-                 lengths: Optional[DeviceBuffer], ids: Optional[DeviceBuffer] = None) -> None:
+    def _forward(self, context: GenerationContext, m: int, past: int, query: int,
+                 last_row: Optional[int], lengths: Optional[DeviceBuffer], ids: Optional[DeviceBuffer] = None) -> None:
         g, c, b, io = self.gpu, self.config, self.buf, self.io_dtype
         d = c.d_model
         g.embedding(self.embedding, ids if ids is not None else b["ids"], b["h"], m, c.vocab, d,
@@ -276,7 +291,7 @@ class LlamaDecoderSession:
             return
         if m > 16 and self.fuse_decode and self._rows_form_covers(m):
             self._forward_rows(context, m, past, query, lengths)
-            self._head(last_row)
+            self._head(last_row, m)
             return
         for li, lw in enumerate(self.layers):
             g.rms_norm(b["h"], lw["attn_norm"], b["xn"], m, d, c.rms_eps, io)
@@ -330,11 +345,23 @@ class LlamaDecoderSession:
             g.silu_mul(b["g"], b["u"], b["act"], m * c.ffn, io)
             self._linear(b["act"], lw["down"], b["dn"], m)
             g.add(b["h"], b["dn"], b["h"], m * d, io)
-        self._head(last_row)
+        self._head(last_row, m)
 
-    def _head(self, last_row: int) -> None:
-        """Token-only exit: the head runs on the last valid row only."""
+    def _head(self, last_row: Optional[int], m: int = 1) -> None:
+        """Token-only exit: the head runs on the last valid row only.  `last_row=None`: the
+        head runs on all m rows of the chunk (the graph's own outputs)."""
         g, c, b, io = self.gpu, self.config, self.buf, self.io_dtype
+        if last_row is None:
+            if "logits_all" not in b or b["logits_all"].nbytes < m * c.vocab * self.eb:
+                for name in ("logits_all", "tokens_all"):
+                    if name in b:
+                        b.pop(name).free()
+                b["logits_all"] = g.alloc(self.chunk_length * c.vocab * self.eb)
+                b["tokens_all"] = g.alloc(self.chunk_length * 4)
+            g.rms_norm(b["h"], self.final_norm, b["xn"], m, c.d_model, c.rms_eps, io)
+            self._linear(b["xn"], self.lm_head, b["logits_all"], m)
+            g.argmax(b["logits_all"], b["tokens_all"], m, c.vocab, io)
+            return
         row = b["h"].offset(last_row * c.d_model * self.eb)
         g.rms_norm(row, self.final_norm, b["xn"], 1, c.d_model, c.rms_eps, io)
         self._linear(b["xn"], self.lm_head, b["logits"], 1)

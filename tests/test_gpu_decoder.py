@@ -313,6 +313,46 @@ def test_greedy_loop_and_replayed_decode_agree(gpu_ctx):
         seq.append(stepwise[step])
 
 
+def test_all_rows_exit_returns_what_the_graph_returns(gpu_ctx):
+    """`last_row=None`: the session returns the decode graph's own outputs, logits [1, M, V] and
+    token [1, M, 1] (tools/export-recipes/minicpm5/export_decode.py:14-22).  A padded chunk (5 of
+    8 rows valid) then a padded second chunk and a one-row step: every valid row's logits equal
+    the oracle's full re-forward (atol 2e-4, the gate of the last-row form) and its token the
+    oracle's argmax wherever the margin exceeds twice that; pad rows are unspecified.  The
+    greedy loop gives the same tokens through either exit."""
+    weights = random_weights(SMALL, seed=8)
+    ids = np.random.default_rng(12).integers(0, SMALL.vocab, size=12).astype(np.int32)
+    want = helpers.oracle_decoder_logits(weights, ids)
+    session = LlamaDecoderSession(gpu_ctx, weights, chunk_length=8)
+    ctx = session.create_generation_context(capacity=32, chunk_length=8)
+    position = 0
+    for n, m in ((5, 8), (6, 8), (1, 1)):
+        cid = np.zeros((1, m), dtype=np.int32)
+        cpos = np.zeros((1, m), dtype=np.int32)
+        cid[0, :n] = ids[position:position + n]
+        cpos[0, :n] = np.arange(position, position + n)
+        token, logits = session.run(cid, cpos, None, context=ctx, query_length=n,
+                                    want_logits=True)
+        assert token.shape == (1, m, 1) and token.dtype == np.int32
+        assert logits.shape == (1, m, SMALL.vocab)
+        for row in range(n):
+            ref = want[position + row]
+            assert float(np.max(np.abs(logits[0, row] - ref))) <= 2e-4, (position, row)
+            top = np.sort(ref)
+            if top[-1] - top[-2] > 4e-4:
+                assert int(token[0, row, 0]) == int(np.argmax(ref)), (position, row)
+        position += n
+    assert ctx.past == 12
+    ctx.dispose()
+    prompt = [int(t) for t in ids[:11]]
+    by_last_row = generate_greedy(session, prompt=prompt, max_new_tokens=6, chunk_length=8,
+                                  max_position=SMALL.max_position)
+    by_all_rows = generate_greedy(session, prompt=prompt, max_new_tokens=6, chunk_length=8,
+                                  max_position=SMALL.max_position, last_row=False)
+    assert by_all_rows == by_last_row
+    session.close()
+
+
 def test_fused_and_separate_decode_launches_agree(gpu_ctx):
     """The fused one-row step (5 launches per layer) and the op-by-op step (16 launches) give
     logits within 1e-4 of each other and the same tokens on a teacher-forced sequence."""

@@ -5,6 +5,11 @@ one-row decode steps, each run's last-row logits against the CPU oracle's full r
 without a KV cache (how the reference derives its greedy goldens,
 tools/export-recipes/_shared/decode_series.py:51-73).
 
+The replayed decode that bench.py times (`decode_tokens`: one recorded step replayed with the
+lengths, the position and the fed-back token on the device) is checked at the same size: 255
+free-running steps behind the 128-token prefill, bit-equal to 255 step-by-step runs, and equal
+to the oracle's argmax of a full re-forward over the generated sequence at sampled positions.
+
 Tolerance.  The random init lets the residual stream grow by about 2e4 per layer, so logits are
 of the order 1e5..1e6 and an absolute gate means nothing across seeds; the gate is relative to
 the largest |logit| of the row.  f32 arithmetic (KRM_COMPUTE_F32 prefill, the reference's
@@ -74,4 +79,76 @@ def test_full_size_teacher_forced_logits(gpu_ctx, full_model, label, compute, ga
     assert worst <= gate, worst
     assert disagreements == 0 and checked_tokens >= 1
     ctx.dispose()
+    session.close()
+
+
+REPLAY_STEPS = 255
+
+
+@pytest.mark.parametrize("label,kv,gate", [("f32 state", ka.F32, 1.2e-4),
+                                           ("fp16 state", ka.F16, 2.4e-4)])
+def test_full_size_replayed_decode_equals_stepwise_and_the_oracle(gpu_ctx, full_model, label, kv,
+                                                                  gate):
+    """bench.py's config-4 path at full size: prefill 128 (fp16-operand products), then
+    decode_tokens for 255 steps.  (i) The tokens equal those of 255 step-by-step session.run
+    calls on a second context, bit for bit (same kernels, scalar instead of device lengths,
+    a full-capacity instead of a replay-sized attention launch).  (ii) A full re-forward of the
+    generated sequence through the CPU oracle (no KV cache,
+    tools/export-recipes/_shared/decode_series.py:51-73) gives, at 8 sampled positions including
+    the last, the same argmax wherever its top-1 / top-2 margin exceeds twice the logits gate,
+    and the last step's logits (left in the session's buffer) lie within the gate.  Gates are
+    relative to the row's largest |logit|: 1.2e-4 with the f32 state (the teacher-forced test's
+    gate for this prefill; measured at the last step 9.6e-7), 2.4e-4 with the fp16 state (K and V
+    rounded to 11 bits; measured 1.3e-6).
+    (iii) The device's fault word stays 0 (decode_tokens raises otherwise) and the context ends
+    at pastLength 383."""
+    config, weights, _ids, _want = full_model
+    prompt = np.random.default_rng(44).integers(0, config.vocab, size=PROMPT).astype(np.int32)
+    session = LlamaDecoderSession(gpu_ctx, weights, io_dtype=ka.F32, kv_dtype=kv,
+                                  chunk_length=PROMPT, prefill_compute=ka.COMPUTE_F16)
+    pos = np.arange(PROMPT, dtype=np.int32)[None]
+
+    def prefill():
+        ctx = session.create_generation_context(capacity=config.max_position,
+                                                chunk_length=PROMPT)
+        token = session.run(prompt[None], pos, PROMPT - 1, context=ctx, query_length=PROMPT)
+        return ctx, int(token[0, 0, 0])
+
+    ctx, first = prefill()
+    replayed = [first] + session.decode_tokens(ctx, first, REPLAY_STEPS)
+    last_logits = session.buf["logits"].download(np.float32, (config.vocab,))
+    assert ctx.past == PROMPT + REPLAY_STEPS == 383
+    ctx.dispose()
+
+    ctx, token = prefill()
+    stepwise = [token]
+    for step in range(REPLAY_STEPS):
+        token = int(session.run(np.array([[token]], dtype=np.int32),
+                                np.array([[PROMPT + step]], dtype=np.int32), 0, context=ctx,
+                                query_length=1)[0, 0, 0])
+        stepwise.append(token)
+    ctx.dispose()
+    assert replayed == stepwise
+
+    # replayed[j] is the argmax of the logits at position PROMPT - 1 + j
+    sequence = np.concatenate([prompt, np.array(replayed[:-1], dtype=np.int32)])
+    sampled = sorted({0, 1, 17, 64, 128, 191, 254, REPLAY_STEPS})
+    t0 = time.perf_counter()
+    want = helpers.oracle_decoder_logits(weights, sequence,
+                                         rows=[PROMPT - 1 + j for j in sampled])
+    print(f"[config 4, replay, {label}] oracle re-forward of {sequence.size} rows: "
+          f"{time.perf_counter() - t0:.1f} s", flush=True)
+    checked = 0
+    for row, j in zip(want, sampled):
+        scale = float(np.max(np.abs(row)))
+        top = np.sort(row)
+        if (top[-1] - top[-2]) / scale > 2 * gate:
+            checked += 1
+            assert replayed[j] == int(np.argmax(row)), (j, replayed[j], int(np.argmax(row)))
+    err = float(np.max(np.abs(last_logits.astype(np.float64) - want[-1]))) / \
+        float(np.max(np.abs(want[-1])))
+    print(f"[config 4, replay, {label}] {checked} of {len(sampled)} sampled tokens had a decisive "
+          f"margin and agree; last step's logits error / max|logit| = {err:.3e}", flush=True)
+    assert err <= gate, err
+    assert checked >= 1
     session.close()
