@@ -650,8 +650,8 @@ def main() -> int:
     ap.add_argument("--no-graph", action="store_true",
                     help="issue plain launches instead of replaying recorded graphs")
     ap.add_argument("--only", default="",
-                    help="gemv | gemv16 | gemm | attention | ragged | prefill | w4a8 | model | traffic: run "
-                         "only that part besides the headline GEMV")
+                    help="gemv | gemv16 | gemm | attention | ragged | prefill | w4a8 | model | traffic | "
+                         "counters: run only that part besides the headline GEMV")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build measures one GPU only (--gpus 1); no multi-GPU figure is "
@@ -736,6 +736,10 @@ def main() -> int:
         result["gemv_n65536_us"] = round(big_us, 2)
         result["gemv_n65536_gbs"] = round(big["algo"] / big_us / 1e3, 1)
         result["gemv_n65536_pct_of_hbm_peak"] = round(100 * big["algo"] / big_us / 1e3 / 8000, 2)
+    if args.only == "counters":
+        # For `rocprofv3 --pmc <SQ counters>`: beside the headline launches, a few plain launches
+        # of the same kernel on N = 65536 rows (128 MiB of weights each, the streaming case).
+        bench_gemv(timer, rng, 8, 8, 1, 65536, k, g, 5)
     if args.only == "traffic":
         # For `rocprofv3 --pmc FETCH_SIZE` / `--pmc WRITE_SIZE`: a plain 8 MiB copy (known
         # traffic: 8 MiB read + 8 MiB written) beside the GEMV, a few launches of each.

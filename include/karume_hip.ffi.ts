@@ -99,6 +99,20 @@ export const KARUME_HIP_SYMBOLS = {
     ],
     result: "i32",
   },
+  krm_decode_head: {
+    parameters: [
+      "pointer", "u64", "u64", "f32", "u64", "u64", "u64", "u64", "u64", "usize", "buffer", "u32",
+      "u32", "u32", "i32", "i32"
+    ],
+    result: "i32",
+  },
+  krm_decode_tail: {
+    parameters: [
+      "pointer", "u64", "u32", "u64", "u64", "u64", "u32", "u64", "u64", "u32", "u32", "u64",
+      "i32", "i32"
+    ],
+    result: "i32",
+  },
   krm_attention_state_lengths: {
     parameters: [
       "pointer", "u64", "u64", "u64", "u64", "u64", "u64", "u32", "u32", "u32", "u32", "u32",

@@ -305,6 +305,26 @@ int32_t krm_lengths_log_token(krm_ctx* ctx, krm_buf lengths, krm_buf token_i32,
  * the end of a recorded one-row decode step, which leaves the next step's position behind. */
 int32_t krm_lengths_step_end(krm_ctx* ctx, krm_buf lengths, krm_buf token_i32,
                              krm_buf history_i32, uint32_t history_len, krm_buf positions_i32);
+/* The exit of a one-row decode step in two launches instead of four (final rms_norm + lm_head
+ * `linear`, `argmax`, the step's bookkeeping, the next step's `embedding`; graph order
+ * tools/export-recipes/minicpm5/export_decode.py:14-35, loop
+ * packages/models/src/generation/greedy.ts:245-252).
+ * krm_decode_head: krm_linear_i4_fused for one row (optional rms_norm in front, logits [n]
+ * written in full) whose workgroups also leave the argmax of the rows they stored in
+ * `partials` ({f32 value bits, u32 row} pairs, 8 bytes per 4 rows of n at most);
+ * *partial_count = how many pairs this launch writes (a function of the shape only).
+ * krm_decode_tail: the argmax over those pairs with krm_argmax's order (NaN is the maximum,
+ * ties go to the smallest index), then krm_lengths_step_end (token written to token_i32 and
+ * logged, lengths advanced, next position written) and krm_embedding of that token into
+ * `next_row` [hidden], in one launch.  The token equals krm_argmax of the logits bit for bit. */
+int32_t krm_decode_head(krm_ctx* ctx, krm_buf x, krm_buf norm_weight_f32, float norm_eps,
+                        krm_buf w, krm_buf scales, krm_buf bias, krm_buf logits, krm_buf partials,
+                        size_t partials_bytes, uint32_t* partial_count, uint32_t n, uint32_t k,
+                        uint32_t group, int32_t io_dtype, int32_t scale_dtype);
+int32_t krm_decode_tail(krm_ctx* ctx, krm_buf partials, uint32_t partial_count, krm_buf token_i32,
+                        krm_buf lengths, krm_buf history_i32, uint32_t history_len,
+                        krm_buf positions_i32, krm_buf table, uint32_t vocab, uint32_t hidden,
+                        krm_buf next_row, int32_t table_dtype, int32_t out_dtype);
 /* krm_attention_state with device lengths; `max_past` sizes the launch and the workspace.  A
  * replay whose device-side pastLength needs more column splits than `max_past` did raises the
  * fault word and writes nothing (neither `out` nor the workspace nor the arrival counters). */

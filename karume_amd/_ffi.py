@@ -83,6 +83,10 @@ PROTOTYPES = {
     "krm_lengths_positions": (i32, [c_ctx, c_buf, c_buf, u32]),
     "krm_lengths_log_token": (i32, [c_ctx, c_buf, c_buf, c_buf, u32]),
     "krm_lengths_step_end": (i32, [c_ctx, c_buf, c_buf, c_buf, u32, c_buf]),
+    "krm_decode_head": (i32, [c_ctx, c_buf, c_buf, C.c_float, c_buf, c_buf, c_buf, c_buf, c_buf,
+                              size_t, C.POINTER(u32), u32, u32, u32, i32, i32]),
+    "krm_decode_tail": (i32, [c_ctx, c_buf, u32, c_buf, c_buf, c_buf, u32, c_buf, c_buf, u32, u32,
+                              c_buf, i32, i32]),
     "krm_attention_state_lengths": (i32, [c_ctx, c_buf, c_buf, c_buf, c_buf, c_buf, c_buf, u32,
                                           u32, u32, u32, u32, u32, u32, C.c_float, c_buf, u32,
                                           i32, i32, c_buf, size_t]),

@@ -189,10 +189,7 @@ __global__ __launch_bounds__(kThreads) void embedding_kernel(const WT* __restric
 // gives 0 (packages/runtime/src/kernels/argmax.ts:16-34).  (value, index) pairs are ordered
 // lexicographically (value descending, index ascending), so the tree shape does not matter.
 __device__ inline bool beats(float va, uint32_t ia, float vb, uint32_t ib) {
-  const bool na = va != va, nb = vb != vb;
-  if (na != nb) return na;
-  if (!na && va != vb) return va > vb;
-  return ia < ib;
+  return argmax_beats(va, ia, vb, ib);
 }
 constexpr int kArgmaxThreads = 1024;
 constexpr int kArgmaxUnroll = 32;  // independent loads in flight per thread (one pass up to 32768)
@@ -286,6 +283,95 @@ __global__ __launch_bounds__(kArgmaxThreads) void argmax_kernel(const XT* __rest
     at = s_idx[w];
     fold_row();
     if (threadIdx.x == 0) out[blockIdx.x] = (int32_t)at;
+  }
+}
+
+// End of a one-row decode step in one launch: the argmax over the per-workgroup partials the
+// head projection left (krm_decode_head), the step's bookkeeping (what lengths_step_end_kernel
+// does: token logged, lengths advanced when the step ran clean, the next position written) and
+// the next step's embedding row.  One workgroup; the partials are a few thousand pairs.
+template <typename WT, typename XT>
+__global__ __launch_bounds__(kArgmaxThreads) void decode_tail_kernel(
+    const uint2* __restrict__ partials, uint32_t count, int32_t* __restrict__ token,
+    uint32_t* __restrict__ lengths, int32_t* __restrict__ history, uint32_t history_len,
+    int32_t* __restrict__ positions, const WT* __restrict__ table, uint32_t vocab,
+    uint32_t hidden, XT* __restrict__ next_row) {
+  __shared__ float s_val[kArgmaxThreads / kWave];
+  __shared__ uint32_t s_idx[kArgmaxThreads / kWave];
+  __shared__ uint32_t s_token;
+  // the bookkeeping words are requested now, beside the partials, not after the reduction
+  const uint32_t len_past = lengths[0], len_query = lengths[1], len_fault = lengths[2],
+                 len_slot = lengths[3];
+  float best = -INFINITY;
+  uint32_t at = 0xffffffffu;
+  constexpr int kWide = 8;
+  for (uint32_t p0 = threadIdx.x; p0 < count; p0 += kArgmaxThreads * kWide) {
+    uint2 v[kWide];
+#pragma unroll
+    for (int u = 0; u < kWide; ++u) {
+      const uint32_t p = p0 + u * kArgmaxThreads;
+      v[u] = partials[p < count ? p : p0];
+    }
+#pragma unroll
+    for (int u = 0; u < kWide; ++u) {
+      const uint32_t p = p0 + u * kArgmaxThreads;
+      if (p < count && beats(__uint_as_float(v[u].x), v[u].y, best, at)) {
+        best = __uint_as_float(v[u].x);
+        at = v[u].y;
+      }
+    }
+  }
+  auto take = [&](float ov, uint32_t oi) {
+    if (beats(ov, oi, best, at)) {
+      best = ov;
+      at = oi;
+    }
+  };
+  auto fold_row = [&]() {
+#define KRM_ARGMAX_DPP(CTRL)                                                                      \
+  take(__builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, best),   \
+                                                            CTRL, 0xf, 0xf, true)),              \
+       (uint32_t)__builtin_amdgcn_update_dpp(0, (int)at, CTRL, 0xf, 0xf, true))
+    KRM_ARGMAX_DPP(0xB1);
+    KRM_ARGMAX_DPP(0x4E);
+    KRM_ARGMAX_DPP(0x124);
+    KRM_ARGMAX_DPP(0x128);
+#undef KRM_ARGMAX_DPP
+  };
+  fold_row();
+  for (int off = 16; off <= 32; off <<= 1)
+    take(__shfl_xor(best, off, kWave), (uint32_t)__shfl_xor((int)at, off, kWave));
+  if ((threadIdx.x & 63) == 0) {
+    s_val[threadIdx.x >> 6] = best;
+    s_idx[threadIdx.x >> 6] = at;
+  }
+  __syncthreads();
+  if (threadIdx.x < kWave) {
+    const int w = threadIdx.x & 15;
+    best = s_val[w];
+    at = s_idx[w];
+    fold_row();
+    if (threadIdx.x == 0) {
+      // a row of -inf: every pair ties on the value and the smallest row index wins, which is
+      // 0 as in argmax_kernel; no partial at all (count == 0) cannot happen (n >= 1)
+      const int32_t tok = (int32_t)at;
+      token[0] = tok;
+      s_token = at;
+      if (len_slot < history_len) history[len_slot] = tok;
+      lengths[3] = len_slot + 1;
+      uint32_t past = len_past;
+      if (len_fault == 0u) {  // P advances by Q only when the step ran clean
+        past += len_query;
+        lengths[0] = past;
+      }
+      positions[0] = (int32_t)past;
+    }
+  }
+  __syncthreads();
+  const uint32_t pick = s_token;
+  for (uint32_t col = threadIdx.x; col < hidden; col += kArgmaxThreads) {
+    const float v = pick >= vocab ? NAN : ld<WT>(table, (size_t)pick * hidden + col);
+    st<XT>(next_row, col, v);
   }
 }
 
@@ -447,6 +533,37 @@ int32_t krm_argmax(krm_ctx* ctx, krm_buf x, krm_buf out_i32, uint32_t rows, uint
                   (argmax_kernel<__half><<<dim3(rows), dim3(kArgmaxThreads), 0, ctx->stream>>>(
                       ptr<const __half>(x), ptr<int32_t>(out_i32), dim)));
   return launched(ctx, "argmax_kernel");
+}
+
+int32_t krm_decode_tail(krm_ctx* ctx, krm_buf partials, uint32_t partial_count, krm_buf token_i32,
+                        krm_buf lengths, krm_buf history_i32, uint32_t history_len,
+                        krm_buf positions_i32, krm_buf table, uint32_t vocab, uint32_t hidden,
+                        krm_buf next_row, int32_t table_dtype, int32_t out_dtype) {
+  KRM_TRY(enter(ctx));
+  KRM_REQUIRE(ctx, valid_dtype(table_dtype) && valid_dtype(out_dtype),
+              "krm_decode_tail: table_dtype %d / out_dtype %d", table_dtype, out_dtype);
+  KRM_REQUIRE(ctx, partial_count >= 1 && vocab >= 1 && hidden >= 1,
+              "krm_decode_tail: partial_count %u / vocab %u / hidden %u", partial_count, vocab,
+              hidden);
+  KRM_REQUIRE(ctx, partials && token_i32 && lengths && history_i32 && positions_i32 && table &&
+                       next_row,
+              "krm_decode_tail: NULL buffer");
+  KRM_REQUIRE(ctx, aligned(partials, 8) && aligned(token_i32, 4) && aligned(lengths, 4) &&
+                       aligned(history_i32, 4) && aligned(positions_i32, 4) &&
+                       aligned(table, dtype_bytes(table_dtype)) &&
+                       aligned(next_row, dtype_bytes(out_dtype)),
+              "krm_decode_tail: misaligned buffer");
+#define KRM_TAIL(WT, XT)                                                                         \
+  decode_tail_kernel<WT, XT><<<dim3(1), dim3(kArgmaxThreads), 0, ctx->stream>>>(                 \
+      ptr<const uint2>(partials), partial_count, ptr<int32_t>(token_i32), ptr<uint32_t>(lengths), \
+      ptr<int32_t>(history_i32), history_len, ptr<int32_t>(positions_i32), ptr<const WT>(table), \
+      vocab, hidden, ptr<XT>(next_row))
+  if (table_dtype == KRM_F16 && out_dtype == KRM_F16) KRM_TAIL(__half, __half);
+  else if (table_dtype == KRM_F16) KRM_TAIL(__half, float);
+  else if (out_dtype == KRM_F16) KRM_TAIL(float, __half);
+  else KRM_TAIL(float, float);
+#undef KRM_TAIL
+  return launched(ctx, "decode_tail_kernel");
 }
 
 }  // extern "C"

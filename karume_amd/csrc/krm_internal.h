@@ -71,6 +71,16 @@ __device__ inline float rounded_f32(float v) {
   asm volatile("" : "+v"(v));
   return v;
 }
+
+// Order of (value, index) pairs for argmax: NaN counts as the maximum, larger values win, ties
+// go to the smaller index (packages/runtime/src/kernels/argmax.ts:16-34).  Lexicographic, so
+// any tree of pairwise comparisons gives the same winner.
+__device__ inline bool argmax_beats(float va, uint32_t ia, float vb, uint32_t ib) {
+  const bool na = va != va, nb = vb != vb;
+  if (na != nb) return na;
+  if (!na && va != vb) return va > vb;
+  return ia < ib;
+}
 #endif
 
 // Maps a HIP runtime status to an error class; 0 when `status` is hipSuccess.

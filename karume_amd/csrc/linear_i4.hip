@@ -493,6 +493,11 @@ struct GemvFusion {
   uint32_t* lengths;         // device {past, query, fault, ...} or null: `past` below
   uint32_t heads, kv_heads, depth, table_rows, capacity, window, past;
   int32_t slot_f16;          // slot element type: 1 = fp16, 0 = f32
+  // One row (M = 1), plain epilogue: every workgroup also writes the argmax of the outputs it
+  // stored, {value bits, row index}, to argmax_partial[blockIdx.x] (a workgroup without a row:
+  // {-inf, 0xffffffff}); the number of workgroups is reported through host_blocks.
+  uint2* argmax_partial;
+  uint32_t* host_blocks;     // host side only: where the launcher leaves its grid size
 };
 
 __device__ inline void slot_store(void* slot, int32_t is_f16, size_t i, float v) {
@@ -887,6 +892,43 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 4))) voi
       }
     }
   }
+  if constexpr (MB == 1) {
+    if (fuse.argmax_partial) {  // uniform over the launch
+      // the values as stored (the totals are uniform over the wave, so every lane can redo the
+      // few additions), best of the wave's rows, then best of the workgroup's waves
+      __shared__ float s_best[4];
+      __shared__ uint32_t s_at[4];
+      float best = -INFINITY;
+      uint32_t at = 0xffffffffu;
+#pragma unroll
+      for (int r = 0; r < ROWS; ++r) {
+        const uint32_t row = row0 + r;
+        if (row < n) {
+          float value = total[r][0] * inv[0] + (bias ? to_f32<XT>(bias[row]) : 0.f);
+          if (residual) value += to_f32<XT>(residual[row]);
+          value = to_f32<XT>(from_f32<XT>(value));
+          if (argmax_beats(value, row, best, at)) {
+            best = value;
+            at = row;
+          }
+        }
+      }
+      if (lane == 0) {
+        s_best[wave] = best;
+        s_at[wave] = at;
+      }
+      __syncthreads();
+      if (threadIdx.x == 0) {
+#pragma unroll
+        for (int q = 1; q < 4; ++q)
+          if (argmax_beats(s_best[q], s_at[q], best, at)) {
+            best = s_best[q];
+            at = s_at[q];
+          }
+        fuse.argmax_partial[blockIdx.x] = make_uint2(__float_as_uint(best), at);
+      }
+    }
+  }
 }
 
 template <typename XT, typename ST, int MB, int ROWS, int VEC, int NSTEP>
@@ -895,6 +937,7 @@ int32_t launch_gemv(krm_ctx* ctx, krm_buf x, krm_buf w, krm_buf scales, krm_buf 
                     const GemvFusion& fuse = GemvFusion{}) {
   const uint32_t rows_per_block = 4 * ROWS;
   const uint32_t blocks = (n + rows_per_block - 1) / rows_per_block;
+  if (fuse.host_blocks) *fuse.host_blocks = blocks;
 #define KRM_GEMV_LAUNCH(NORM, ROW)                                                              \
   gemv_i4_kernel<XT, ST, MB, ROWS, VEC, NSTEP, NORM, ROW>                                       \
       <<<dim3(blocks), dim3(256), 0, ctx->stream>>>(ptr<const XT>(x), ptr<const uint32_t>(w),  \
@@ -940,6 +983,12 @@ int32_t pick_rows(krm_ctx* ctx, krm_buf x, krm_buf w, krm_buf scales, krm_buf bi
   // stage the row once more, as long as every CU still gets a few.
   if constexpr (MB == 1 && sizeof(XT) == 4 && VEC == 4)
     if (k <= 4096 && (uint64_t)n >= cus * 4 * 4 * 2)
+      return pick_steps<XT, ST, MB, 4, VEC>(ctx, x, w, scales, bias, out, m, n, k, group_shift, fuse);
+  // fp16 activations, many rows (the streaming case: every SIMD still gets 8 waves or more):
+  // four rows a wave share the activations read from LDS and the per-wave bookkeeping, about a
+  // sixth of the instructions of a launch that the vector ALU bounds
+  if constexpr (MB == 1 && sizeof(XT) == 2 && VEC == 4)
+    if (k <= 4096 && (uint64_t)n >= cus * 4 * 4 * 8)
       return pick_steps<XT, ST, MB, 4, VEC>(ctx, x, w, scales, bias, out, m, n, k, group_shift, fuse);
   // (one row of x shared through LDS: below 32 rows a CU one row a wave — twice the waves —
   // measured 1.5 % more decode tokens/s and 1 % on the 4096 x 4096 GEMV)
@@ -1133,6 +1182,43 @@ int32_t krm_linear_i4_fused(krm_ctx* ctx, krm_buf x, krm_buf norm_weight_f32, fl
   fuse.residual = ptr<const void>(residual);
   fuse.pair_silu = epilogue == KRM_EPILOGUE_SILU_PAIRS ? 1u : 0u;
   return gemv_dispatch(ctx, x, w, scales, bias, out, m, n, k, group, io_dtype, scale_dtype, fuse);
+}
+
+int32_t krm_decode_head(krm_ctx* ctx, krm_buf x, krm_buf norm_weight_f32, float norm_eps,
+                        krm_buf w, krm_buf scales, krm_buf bias, krm_buf logits, krm_buf partials,
+                        size_t partials_bytes, uint32_t* partial_count, uint32_t n, uint32_t k,
+                        uint32_t group, int32_t io_dtype, int32_t scale_dtype) {
+  KRM_TRY(enter(ctx));
+  KRM_REQUIRE(ctx, valid_dtype(io_dtype) && valid_dtype(scale_dtype),
+              "krm_decode_head: io_dtype %d / scale_dtype %d", io_dtype, scale_dtype);
+  KRM_REQUIRE(ctx, is_pow2(group) && group >= 16 && k >= 1 && k % group == 0,
+              "krm_decode_head: group_size %u must be a power of two >= 16 dividing k = %u", group,
+              k);
+  KRM_REQUIRE(ctx, n >= 1 && n <= 0x7fffffffu, "krm_decode_head: n = %u", n);
+  KRM_REQUIRE(ctx, !norm_weight_f32 || std::isfinite(norm_eps), "krm_decode_head: eps");
+  KRM_REQUIRE(ctx, partial_count != nullptr, "krm_decode_head: partial_count is NULL");
+  KRM_REQUIRE(ctx, x && w && scales && logits && partials, "krm_decode_head: NULL buffer");
+  KRM_REQUIRE(ctx, aligned(x, 16) && aligned(norm_weight_f32, 16) && aligned(w, 4) &&
+                       aligned(logits, dtype_bytes(io_dtype)) &&
+                       aligned(bias, dtype_bytes(io_dtype)) &&
+                       aligned(scales, dtype_bytes(scale_dtype)) && aligned(partials, 8),
+              "krm_decode_head: x and norm weight must be 16-byte aligned, w 4-byte, partials "
+              "8-byte aligned");
+  // at most one workgroup per four rows, whatever rows-per-wave the launch picks
+  const size_t worst = ((size_t)n + 3) / 4 * sizeof(uint2);
+  KRM_REQUIRE(ctx, partials_bytes >= worst,
+              "krm_decode_head: partials of %zu bytes, %zu needed (8 bytes per 4 rows)",
+              partials_bytes, worst);
+  GemvFusion fuse{};
+  fuse.norm_weight = ptr<const float>(norm_weight_f32);
+  fuse.norm_eps = norm_eps;
+  fuse.argmax_partial = ptr<uint2>(partials);
+  uint32_t blocks = 0;
+  fuse.host_blocks = &blocks;
+  KRM_TRY(gemv_dispatch(ctx, x, w, scales, bias, logits, 1, n, k, group, io_dtype, scale_dtype,
+                        fuse));
+  *partial_count = blocks;
+  return KRM_OK;
 }
 
 int32_t krm_linear_i4_rows(krm_ctx* ctx, krm_buf x, krm_buf w, krm_buf scales, krm_buf bias,

@@ -197,6 +197,8 @@ class LlamaDecoderSession:
             "g": a(m * c.ffn * eb), "u": a(m * c.ffn * eb), "act": a(m * c.ffn * eb),
             "dn": a(m * d * eb), "logits": a(c.vocab * eb), "token": a(16),
             "qkv": a((hd + 2 * kvd) * eb), "qkr": a((hd + kvd) * eb),
+            # per-workgroup argmax pairs of the head projection (8 bytes per 4 rows at most)
+            "argmax_part": a((c.vocab + 3) // 4 * 8),
         }
         self.workspace: Optional[DeviceBuffer] = None
         self.logits_shape = (1, c.vocab)
@@ -281,14 +283,21 @@ class LlamaDecoderSession:
                            self.io_dtype, lin.scale_dtype, compute)
 
     def _forward(self, context: GenerationContext, m: int, past: int, query: int,
-                 last_row: Optional[int], lengths: Optional[DeviceBuffer], ids: Optional[DeviceBuffer] = None) -> None:
+                 last_row: Optional[int], lengths: Optional[DeviceBuffer], ids: Optional[DeviceBuffer] = None,
+                 step_end: Optional[tuple] = None) -> None:
+        """`step_end` = (history, history_len): a replayed one-row step whose input row is
+        already in the activation buffer (the previous step's exit wrote it) and whose exit
+        also does the step's bookkeeping and the next step's embedding."""
         g, c, b, io = self.gpu, self.config, self.buf, self.io_dtype
         d = c.d_model
-        g.embedding(self.embedding, ids if ids is not None else b["ids"], b["h"], m, c.vocab, d,
-                    F16, io)
+        if step_end is None:
+            g.embedding(self.embedding, ids if ids is not None else b["ids"], b["h"], m, c.vocab,
+                        d, F16, io)
         if m == 1 and self.fuse_decode:
-            self._forward_fused_row(context, past, lengths)
+            self._forward_fused_row(context, past, lengths, step_end)
             return
+        if step_end is not None:
+            raise ExecutionError("the fused step exit needs the fused one-row launches")
         if m > 16 and self.fuse_decode and self._rows_form_covers(m):
             self._forward_rows(context, m, past, query, lengths)
             self._head(last_row, m)
@@ -463,7 +472,8 @@ class LlamaDecoderSession:
                                  io_dtype=self.io_dtype, scale_dtype=lin.scale_dtype, **kw)
 
     def _forward_fused_row(self, context: GenerationContext, past: int,
-                           lengths: Optional[DeviceBuffer]) -> None:
+                           lengths: Optional[DeviceBuffer],
+                           step_end: Optional[tuple] = None) -> None:
         """One decode row (M = Q = 1), 5 launches per layer instead of 16."""
         from .runtime import EPILOGUE_SILU_PAIRS
         g, c, b, io, eb = self.gpu, self.config, self.buf, self.io_dtype, self.eb
@@ -500,9 +510,21 @@ class LlamaDecoderSession:
             self._fused(b["h"], lw["gate_up"], b["act"], norm_weight=lw["ffn_norm"],
                         norm_eps=c.rms_eps, epilogue=EPILOGUE_SILU_PAIRS)
             self._fused(b["act"], lw["down"], b["h"], residual=b["h"])
-        self._fused(b["h"], self.lm_head, b["logits"], norm_weight=self.final_norm,
-                    norm_eps=c.rms_eps)
-        g.argmax(b["logits"], b["token"], 1, c.vocab, io)
+        if step_end is None:
+            self._fused(b["h"], self.lm_head, b["logits"], norm_weight=self.final_norm,
+                        norm_eps=c.rms_eps)
+            g.argmax(b["logits"], b["token"], 1, c.vocab, io)
+            return
+        # the exit of a replayed step, two launches: head projection with argmax partials, then
+        # argmax + bookkeeping + the next step's embedding row (into the activation buffer)
+        history, history_len = step_end
+        lm = self.lm_head
+        count = g.decode_head(b["h"], lm.w, lm.s, b["logits"], b["argmax_part"], lm.n, lm.k,
+                              c.group_size, norm_weight=self.final_norm, norm_eps=c.rms_eps,
+                              io_dtype=io, scale_dtype=lm.scale_dtype)
+        g.decode_tail(b["argmax_part"], count, b["token"], lengths, history, history_len,
+                      b["pos"], self.embedding, c.vocab, c.d_model, b["h"], table_dtype=F16,
+                      out_dtype=io)
 
     # -- replayed decode ---------------------------------------------------------------------
     def decode_tokens(self, context: GenerationContext, first_token: int, count: int
@@ -528,10 +550,18 @@ class LlamaDecoderSession:
             g.lengths_set(context.lengths, context.past, 1)
             self._replay_last_past = context.past + count - 1
             g.lengths_positions(context.lengths, b["pos"], 1)
-            with g.record() as rec:
-                self._forward(context, 1, 0, 1, 0, lengths=context.lengths, ids=b["token"])
-                # token logged, lengths advanced, the next replay's position written: one launch
-                g.lengths_step_end(context.lengths, b["token"], history, count, b["pos"])
+            if self.fuse_decode:
+                # the first step's input row; every replay's exit leaves the next one's
+                g.embedding(self.embedding, b["token"], b["h"], 1, self.config.vocab,
+                            self.config.d_model, F16, self.io_dtype)
+                with g.record() as rec:
+                    self._forward(context, 1, 0, 1, 0, lengths=context.lengths,
+                                  step_end=(history, count))
+            else:
+                with g.record() as rec:
+                    self._forward(context, 1, 0, 1, 0, lengths=context.lengths, ids=b["token"])
+                    # token logged, lengths advanced, the next replay's position written
+                    g.lengths_step_end(context.lengths, b["token"], history, count, b["pos"])
             graph = rec.graph
             for _ in range(count):
                 graph.launch()

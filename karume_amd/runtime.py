@@ -443,6 +443,30 @@ class GpuContext:
                                                    _addr(history), history_len,
                                                    _addr(positions)))
 
+    def decode_head(self, x: BufferLike, w: BufferLike, scales: BufferLike, logits: BufferLike,
+                    partials: DeviceBuffer, n: int, k: int, group: int, *,
+                    norm_weight: BufferLike = None, norm_eps: float = 0.0,
+                    bias: BufferLike = None, io_dtype: int = F32, scale_dtype: int = F16) -> int:
+        """Final rms_norm + lm_head for one row, leaving per-workgroup argmax partials; returns
+        how many partials the launch writes."""
+        count = C.c_uint32()
+        self._check(self._lib.krm_decode_head(
+            self._handle, _addr(x), _addr(norm_weight), float(norm_eps), _addr(w), _addr(scales),
+            _addr(bias), _addr(logits), _addr(partials), partials.nbytes, C.byref(count), n, k,
+            group, io_dtype, scale_dtype))
+        return int(count.value)
+
+    def decode_tail(self, partials: BufferLike, partial_count: int, token: BufferLike,
+                    lengths: BufferLike, history: BufferLike, history_len: int,
+                    positions: BufferLike, table: BufferLike, vocab: int, hidden: int,
+                    next_row: BufferLike, *, table_dtype: int = F16, out_dtype: int = F32) -> None:
+        """argmax over the head's partials + the end of a recorded decode step + the next
+        step's embedding row, one launch."""
+        self._check(self._lib.krm_decode_tail(
+            self._handle, _addr(partials), partial_count, _addr(token), _addr(lengths),
+            _addr(history), history_len, _addr(positions), _addr(table), vocab, hidden,
+            _addr(next_row), table_dtype, out_dtype))
+
     def attention_state_lengths(self, q: BufferLike, ins_k: BufferLike, ins_v: BufferLike,
                                 slot_k: BufferLike, slot_v: BufferLike, out: BufferLike, *,
                                 batch: int, heads: int, kv_heads: int, chunk_rows: int,

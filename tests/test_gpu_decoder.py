@@ -353,6 +353,90 @@ def test_all_rows_exit_returns_what_the_graph_returns(gpu_ctx):
     session.close()
 
 
+@pytest.mark.parametrize("io,n,k", [(np.float32, 32000, 2048), (np.float32, 1003, 512),
+                                    (np.float16, 4096, 4096), (np.float32, 70000, 256)])
+def test_decode_head_and_tail_equal_the_separate_ops(gpu_ctx, io, n, k):
+    """krm_decode_head + krm_decode_tail against the four launches they stand for: the logits
+    are those of krm_linear_i4_fused bit for bit, the token is krm_argmax of them, the
+    bookkeeping is krm_lengths_step_end's and the next row is krm_embedding's."""
+    ctx = gpu_ctx
+    rng = np.random.default_rng(n + k)
+    g, hidden = 128, 96
+    packed, _q, scale = helpers.synthetic_int4(rng, n, k, g)
+    x = rng.normal(size=(1, k)).astype(io)
+    norm = rng.normal(size=k).astype(np.float32)
+    table = rng.normal(size=(n, hidden)).astype(np.float16)
+    dx, dw, ds, dn, dt = (ctx.upload(a) for a in (x, packed, scale, norm, table))
+    code = ka.dtype_code(io)
+    eb = np.dtype(io).itemsize
+    logits_a, logits_b = ctx.alloc(n * eb), ctx.alloc(n * eb)
+    ctx.linear_i4_fused(dx, dw, ds, logits_a, 1, n, k, g, norm_weight=dn, norm_eps=1e-5,
+                        io_dtype=code, scale_dtype=ka.F16)
+    token_a = ctx.alloc(16)
+    ctx.argmax(logits_a, token_a, 1, n, code)
+    partials = ctx.alloc((n + 3) // 4 * 8)
+    count = ctx.decode_head(dx, dw, ds, logits_b, partials, n, k, g, norm_weight=dn,
+                            norm_eps=1e-5, io_dtype=code, scale_dtype=ka.F16)
+    assert 1 <= count <= (n + 3) // 4
+    assert logits_b.download(io, (n,)).tobytes() == logits_a.download(io, (n,)).tobytes()
+    lengths = ctx.alloc(16)
+    ctx.lengths_set(lengths, 41, 1)
+    history = ctx.zeros(8 * 4)
+    token_b, pos, row = ctx.alloc(16), ctx.alloc(16), ctx.alloc(hidden * 4)
+    for step in range(2):  # two steps in a row: the log slot and the position advance
+        ctx.decode_tail(partials, count, token_b, lengths, history, 8, pos, dt, n, hidden, row,
+                        table_dtype=ka.F16, out_dtype=ka.F32)
+    want = int(token_a.download(np.int32, (1,))[0])
+    assert int(token_b.download(np.int32, (1,))[0]) == want
+    assert list(history.download(np.int32, (8,))[:3]) == [want, want, 0]
+    assert list(lengths.download(np.uint32, (4,))) == [43, 1, 0, 2]
+    assert int(pos.download(np.int32, (1,))[0]) == 43
+    assert np.array_equal(row.download(np.float32, (hidden,)), table[want].astype(np.float32))
+    for b in (dx, dw, ds, dn, dt, logits_a, logits_b, token_a, token_b, partials, lengths,
+              history, pos, row):
+        b.free()
+
+
+def test_decode_tail_orders_pairs_like_argmax(gpu_ctx):
+    """The tail's merge on hand-made pairs: ties go to the smallest row, NaN is the maximum
+    (the smallest row among NaNs), a row of -inf gives row 0; a faulted step keeps pastLength
+    (packages/runtime/src/kernels/argmax.ts:16-34, generation-context.ts:576-591)."""
+    ctx = gpu_ctx
+    hidden = 8
+    table = np.arange(6000 * hidden, dtype=np.float32).reshape(6000, hidden)
+    dt = ctx.upload(table)
+
+    def run(values, rows, fault=0):
+        pairs = np.empty((len(values), 2), dtype=np.uint32)
+        pairs[:, 0] = np.asarray(values, dtype=np.float32).view(np.uint32)
+        pairs[:, 1] = rows
+        dp = ctx.upload(pairs)
+        lengths = ctx.upload(np.array([10, 1, fault, 0], dtype=np.uint32))
+        history, token, pos, row = ctx.zeros(16), ctx.alloc(16), ctx.alloc(16), ctx.alloc(hidden * 4)
+        ctx.decode_tail(dp, len(values), token, lengths, history, 4, pos, dt, 6000, hidden, row,
+                        table_dtype=ka.F32, out_dtype=ka.F32)
+        out = (int(token.download(np.int32, (1,))[0]), list(lengths.download(np.uint32, (4,))),
+               int(pos.download(np.int32, (1,))[0]), row.download(np.float32, (hidden,)))
+        for b in (dp, lengths, history, token, pos, row):
+            b.free()
+        return out
+
+    many = 5000  # more pairs than threads: the strided walk and the tree both take part
+    rows = np.arange(many, dtype=np.uint32)[::-1].copy()   # descending rows: order must not matter
+    values = np.full(many, -1.0, dtype=np.float32)
+    values[[100, 4000]] = 7.0                               # rows 4899 and 999 tie
+    token, lengths, pos, row = run(values, rows)
+    assert token == 999 and lengths == [11, 1, 0, 1] and pos == 11
+    assert np.array_equal(row, table[999])
+    values[[7, 4500]] = np.nan                              # rows 4992 and 499
+    assert run(values, rows)[0] == 499
+    assert run(np.full(many, -np.inf, dtype=np.float32), rows)[0] == 0
+    # workgroups without a row leave {-inf, 0xffffffff}: they never win
+    assert run([-np.inf, -np.inf, -np.inf], [0xFFFFFFFF, 5, 0xFFFFFFFF])[0] == 5
+    token, lengths, pos, _ = run(values, rows, fault=1)
+    assert lengths == [10, 1, 1, 1] and pos == 10          # the fault keeps pastLength
+
+
 def test_fused_and_separate_decode_launches_agree(gpu_ctx):
     """The fused one-row step (5 launches per layer) and the op-by-op step (16 launches) give
     logits within 1e-4 of each other and the same tokens on a teacher-forced sequence."""
