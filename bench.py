@@ -404,6 +404,99 @@ def bench_prefill_chunk(timer: Timer, rng, steps: int, warmup: int, g: int):
     return out
 
 
+def bench_decode_step_kernels(timer: Timer, rng, steps: int, warmup: int, g: int):
+    """The launches of one config-4 decode step, each alone: the four GEMV forms of a layer and
+    the head projection (f32 activations, fp16 scales, the fused forms the decoder records), and
+    the one-row attention over a past of 255 columns.  Every GEMV runs over rotating weight
+    copies (a token reads 0.53 GB of weights, more than the 256 MB Infinity Cache holds, so a
+    layer's weights are cold when its launch starts).  `read_floor_us`: krm_probe_launch(READ)
+    on the same bytes of the same buffers with the launch's own grid (workgroups of 256
+    threads; rows per workgroup as the GEMV picks them: 8 for [q;k;v], 4 for o and down, 16 for
+    gate/up and the head) — what a kernel that only reads those weights costs."""
+    ctx, ka = timer.ctx, timer.ka
+    d, ffn, heads, kv_heads, depth, vocab, cap = 2048, 5632, 32, 4, 64, 32000, 512
+    qkv_n = (heads + 2 * kv_heads) * depth
+    forms = [("qkv", qkv_n, d, 8), ("o", d, heads * depth, 4), ("gate_up", 2 * ffn, d, 16),
+             ("down", d, ffn, 4), ("head", vocab, d, 16)]
+    norm = ctx.upload(np.ones(ffn, dtype=np.float32))
+    pos = ctx.upload(np.array([255], dtype=np.int32))
+    ang = np.arange(cap, dtype=np.float64)[:, None] * np.ones((1, depth))
+    cos, sin = ctx.upload(np.cos(ang).astype(np.float32)), ctx.upload(np.sin(ang).astype(np.float32))
+    slot_k = ctx.upload(rng.normal(size=(kv_heads, cap, depth)).astype(np.float32))
+    slot_v = ctx.upload(rng.normal(size=(kv_heads, cap, depth)).astype(np.float32))
+    rows = []
+    for name, n, k, rows_per_wg in forms:
+        copies = max(4, min(64, (600 << 20) // (n * k // 2)))
+        weights = [ctx.upload(rng.integers(0, 256, size=n * k // 2, dtype=np.uint8))
+                   for _ in range(copies)]
+        scales = [ctx.upload(np.maximum(
+            np.abs(rng.normal(0, 0.02, size=(n, k // g))).astype(np.float16),
+            np.float16(6.104e-05))) for _ in range(copies)]
+        x = ctx.upload(rng.normal(size=(1, k)).astype(np.float32))
+        y = ctx.alloc(max(n, d) * 4)
+        res_buf = ctx.upload(rng.normal(size=(1, n)).astype(np.float32))
+        part = ctx.alloc((n + 3) // 4 * 8)
+
+        def step(i: int) -> None:
+            j = i % copies
+            if name == "qkv":
+                ctx.decode_qkv(x, weights[j], scales[j], pos, cos, sin, y, slot_k, slot_v,
+                               heads=heads, kv_heads=kv_heads, depth=depth, k=k, group=g,
+                               table_rows=cap, capacity=cap, window=0, past=255, lengths=None,
+                               norm_weight=norm, norm_eps=1e-5, io_dtype=ka.F32,
+                               scale_dtype=ka.F16, kv_dtype=ka.F32)
+            elif name == "gate_up":
+                ctx.linear_i4_fused(x, weights[j], scales[j], y, 1, n, k, g, norm_weight=norm,
+                                    norm_eps=1e-5, epilogue=ka.EPILOGUE_SILU_PAIRS,
+                                    io_dtype=ka.F32, scale_dtype=ka.F16)
+            elif name == "head":
+                ctx.decode_head(x, weights[j], scales[j], y, part, n, k, g, norm_weight=norm,
+                                norm_eps=1e-5, io_dtype=ka.F32, scale_dtype=ka.F16)
+            else:
+                ctx.linear_i4_fused(x, weights[j], scales[j], y, 1, n, k, g, residual=res_buf,
+                                    io_dtype=ka.F32, scale_dtype=ka.F16)
+
+        grid = (n + rows_per_wg - 1) // rows_per_wg
+
+        def read(i: int) -> None:
+            ctx.probe_launch(ka.PROBE_READ, weights[i % copies], n * k // 2, grid=grid, block=256)
+
+        us = timer.run(step, steps, warmup, replays=20)["ms"] / steps * 1e3
+        floor = timer.run(read, steps, warmup, replays=20)["ms"] / steps * 1e3
+        rows.append({"kernel": name, "n": n, "k": k, "weight_bytes": n * k // 2,
+                     "us": round(us, 2), "read_floor_us": round(floor, 2),
+                     "ratio": round(us / floor, 2)})
+        for b in weights + scales + [x, y, res_buf, part]:
+            b.free()
+    # the one-row attention of the step: 32 heads, 4 kv heads, D = 64, f32 state, past 255
+    q = ctx.upload(rng.normal(size=(heads, depth)).astype(np.float32))
+    ik = ctx.upload(rng.normal(size=(kv_heads, depth)).astype(np.float32))
+    iv = ctx.upload(rng.normal(size=(kv_heads, depth)).astype(np.float32))
+    att = ctx.alloc(heads * depth * 4)
+    lengths = ctx.alloc(16)
+    ctx.lengths_set(lengths, 255, 1)
+    ws = ctx.alloc(ctx.attention_state_workspace(1, heads, kv_heads, 1, depth, 0, cap))
+
+    def attention(i: int) -> None:
+        ctx.attention_state_lengths(q, ik, iv, slot_k, slot_v, att, batch=1, heads=heads,
+                                    kv_heads=kv_heads, chunk_rows=1, depth=depth, capacity=cap,
+                                    window=0, half_scale=float(depth ** -0.25), lengths=lengths,
+                                    max_past=383, io_dtype=ka.F32, kv_dtype=ka.F32, workspace=ws)
+
+    def attention_read(i: int) -> None:
+        ctx.probe_launch(ka.PROBE_READ, slot_k, kv_heads * 256 * depth * 4 * 2, grid=heads,
+                         block=256)
+
+    us = timer.run(attention, steps, warmup, replays=20)["ms"] / steps * 1e3
+    floor = timer.run(attention_read, steps, warmup, replays=20)["ms"] / steps * 1e3
+    rows.append({"kernel": "attention (past 255, device lengths)", "kv_bytes": kv_heads * 256 * depth * 8,
+                 "us": round(us, 2), "read_floor_us": round(floor, 2),
+                 "ratio": round(us / floor, 2)})
+    for b in (norm, pos, cos, sin, slot_k, slot_v, q, ik, iv, att, lengths, ws):
+        b.free()
+    return rows
+
+
 def bench_w4a8(timer: Timer, rng, steps: int, warmup: int, m: int, n: int, k: int, g: int,
                copies: int):
     """w4a8 `linear` (int8 activations x int4 weights, integer dot products): one step = the
@@ -650,7 +743,7 @@ def main() -> int:
     ap.add_argument("--no-graph", action="store_true",
                     help="issue plain launches instead of replaying recorded graphs")
     ap.add_argument("--only", default="",
-                    help="gemv | gemv16 | gemm | attention | ragged | prefill | w4a8 | model | traffic | "
+                    help="gemv | gemv16 | gemm | attention | ragged | prefill | w4a8 | model | step | traffic | "
                          "counters: run only that part besides the headline GEMV")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -795,6 +888,9 @@ def main() -> int:
     if args.only in ("", "prefill"):
         log("[bench] 128-row prefill chunk of the config-4 decoder, kernel by kernel")
         result["prefill_chunk_m128"] = bench_prefill_chunk(timer, rng, 64, 64, g)
+    if args.only in ("", "model", "step"):
+        log("[bench] the launches of one config-4 decode step, each against its read floor")
+        result["decode_step_kernels"] = bench_decode_step_kernels(timer, rng, 64, 64, g)
     if args.only in ("", "w4a8"):
         log("[bench] w4a8 linear: M=1 GEMV and M=512 up/down-projections")
         ms_q, ms_p, ms_f = bench_w4a8(timer, rng, steps2, warm2, 1, n, k, g, copies)

@@ -434,6 +434,9 @@ int32_t krm_decode_rope_append(krm_ctx* ctx, krm_buf qkv, krm_buf positions_i32,
  * the v section keeps its natural order.  Roundings are those of the separate ops
  * (krm_linear_i4_fused, krm_rope_half, krm_state_append); `lengths` / `past` as in
  * krm_decode_rope_append, and like it this may precede the step's attention.
+ * kv_heads = 0 with both slots 0: a layer that attends over another layer's K / V (KV-sharing
+ * layers, tools/export-recipes/gemma4/export_decode.py:59-70) projects and rotates q alone,
+ * `out` = [q_rot], and nothing is appended.
  * Fuses packages/runtime/src/kernels/linear.ts:34-64, packages/runtime/src/kernels/rope.ts:5-20,
  * 52-80 and packages/runtime/src/kernels/state-append.ts:47-96. */
 int32_t krm_decode_qkv(krm_ctx* ctx, krm_buf x, krm_buf norm_weight_f32, float norm_eps,

@@ -568,7 +568,14 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 4))) voi
   // with the weights instead of after the reductions.
   float rope_cos[ROWS / 2 > 0 ? ROWS / 2 : 1][2], rope_sin[ROWS / 2 > 0 ? ROWS / 2 : 1][2];
   bool rope_in_table = false;
+  // run-time lengths of a recorded step: asked for here, used by the appends at the very end
+  // (a load in the epilogue would add a memory round trip behind the reductions)
+  uint32_t dev_past = 0, dev_query = 0;
   if constexpr (DECODE_ROW) {
+    if (fuse.lengths) {
+      dev_past = fuse.lengths[0];
+      dev_query = fuse.lengths[1];
+    }
     {
       const uint32_t half = fuse.depth >> 1;
       const uint32_t rope_pairs = (fuse.heads + fuse.kv_heads) * half;
@@ -828,8 +835,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 4))) voi
       uint32_t past = fuse.past;
       bool append = true;
       if (fuse.lengths) {  // run-time lengths read on the device; same checks as the scalar form
-        past = fuse.lengths[0];
-        append = fuse.lengths[1] == 1u && (uint64_t)past + 1 <= 0xffffffffull &&
+        past = dev_past;
+        append = dev_query == 1u && (uint64_t)past + 1 <= 0xffffffffull &&
                  (fuse.window != 0 || (uint64_t)past + 1 <= fuse.capacity);
         if (!append && row0 == 0 && lane == 0) fuse.lengths[2] = 1u;
       }
@@ -1330,10 +1337,13 @@ int32_t krm_decode_qkv(krm_ctx* ctx, krm_buf x, krm_buf norm_weight_f32, float n
   KRM_REQUIRE(ctx, is_pow2(group) && group >= 16 && k >= 1 && k % group == 0,
               "krm_decode_qkv: group_size %u must be a power of two >= 16 dividing k = %u", group,
               k);
-  KRM_REQUIRE(ctx, heads >= 1 && kv_heads >= 1 && depth >= 2 && depth % 2 == 0 && capacity >= 1 &&
-                       table_rows >= 1,
-              "krm_decode_qkv: H / Hkv / D / C / table rows (%u / %u / %u / %u / %u)", heads,
-              kv_heads, depth, capacity, table_rows);
+  KRM_REQUIRE(ctx, heads >= 1 && depth >= 2 && depth % 2 == 0 && capacity >= 1 && table_rows >= 1,
+              "krm_decode_qkv: H / D / C / table rows (%u / %u / %u / %u)", heads, depth, capacity,
+              table_rows);
+  // kv_heads == 0: a layer that reads another layer's K / V projects and rotates q alone and
+  // appends nothing (no slots)
+  KRM_REQUIRE(ctx, kv_heads >= 1 || (!slot_k && !slot_v),
+              "krm_decode_qkv: kv_heads = 0 (q only) takes no state slots");
   KRM_REQUIRE(ctx, ((uint64_t)heads + 2ull * kv_heads) * depth <= 0x7fffffffull,
               "krm_decode_qkv: the row is too long");
   KRM_REQUIRE(ctx, window <= capacity, "krm_decode_qkv: window %u exceeds capacity %u", window,
@@ -1343,7 +1353,7 @@ int32_t krm_decode_qkv(krm_ctx* ctx, krm_buf x, krm_buf norm_weight_f32, float n
     return fail(ctx, KRM_ERR_EXECUTION,
                 "krm_decode_qkv: pastLength %u + queryLength 1 exceeds capacity %u", past, capacity);
   KRM_REQUIRE(ctx, x && w && scales && positions_i32 && cos_table_f32 && sin_table_f32 && out &&
-                       slot_k && slot_v,
+                       (kv_heads == 0 || (slot_k && slot_v)),
               "krm_decode_qkv: NULL buffer");
   KRM_REQUIRE(ctx, aligned(x, 16) && aligned(norm_weight_f32, 16) && aligned(w, 4) &&
                        aligned(out, dtype_bytes(io_dtype)) && aligned(bias, dtype_bytes(io_dtype)) &&

@@ -40,10 +40,56 @@ class LlamaConfig:
     rms_eps: float = 1e-5
     rope_base: float = 10000.0
     max_position: int = 512
+    # Per-layer attention structure (empty = the same for every layer), as Gemma-4-style decoders
+    # declare it (tools/export-recipes/gemma4/export_decode.py:59-82,510-527):
+    #   layer_windows[l]   sliding window of layer l's state slots, 0 = full context
+    #   layer_head_dims[l] head dim of layer l (sliding and full layers differ there)
+    #   layer_kv_source[l] the layer whose K / V layer l attends over: l itself, or an earlier
+    #                      layer for a KV-sharing layer (which has no k / v projection and
+    #                      appends nothing: two readers, one append)
+    layer_windows: tuple = ()
+    layer_head_dims: tuple = ()
+    layer_kv_source: tuple = ()
+
+    def __post_init__(self):
+        for name in ("layer_windows", "layer_head_dims", "layer_kv_source"):
+            value = tuple(int(v) for v in getattr(self, name))
+            if value and len(value) != self.layers:
+                raise ValueError(f"{name} has {len(value)} entries for {self.layers} layers")
+            object.__setattr__(self, name, value)
+        for layer, source in enumerate(self.layer_kv_source):
+            if not 0 <= source <= layer or self.layer_kv_source[source] != source:
+                raise ValueError(f"layer {layer} takes its K / V from layer {source}, which is "
+                                 "not an earlier layer that owns its own")
+            if source != layer and (self.depth_of(source) != self.depth_of(layer)
+                                    or self.window_of(source) != self.window_of(layer)):
+                raise ValueError(f"layer {layer} shares the K / V of layer {source} but declares "
+                                 "another head dim or window")
 
     @property
     def half_scale(self) -> float:
         return float(np.float32(np.sqrt(1.0 / np.sqrt(float(self.head_dim)))))
+
+    def window_of(self, layer: int) -> int:
+        return self.layer_windows[layer] if self.layer_windows else 0
+
+    def depth_of(self, layer: int) -> int:
+        return self.layer_head_dims[layer] if self.layer_head_dims else self.head_dim
+
+    def owner_of(self, layer: int) -> int:
+        return self.layer_kv_source[layer] if self.layer_kv_source else layer
+
+    def half_scale_of(self, layer: int) -> float:
+        return float(np.float32(np.sqrt(1.0 / np.sqrt(float(self.depth_of(layer))))))
+
+    @property
+    def head_dims(self) -> tuple:
+        """The distinct head dims, ascending (one pair of RoPE tables each)."""
+        return tuple(sorted({self.depth_of(l) for l in range(self.layers)}))
+
+    def readers_of(self, layer: int) -> list:
+        """Layers that attend over the K / V of `layer` (itself first)."""
+        return [l for l in range(self.layers) if self.owner_of(l) == layer]
 
 
 @dataclass
@@ -64,6 +110,14 @@ class DecoderWeights:
     lm_head: Int4Linear = None
     rope_cos: np.ndarray = None                # [max_position, head_dim] float32
     rope_sin: np.ndarray = None
+    # layers of another head dim look their rotation up in tables of their own:
+    # head dim -> (cos, sin), each [max_position, head dim]; head_dim itself stays above
+    rope_by_depth: Dict[int, tuple] = field(default_factory=dict)
+
+    def rope_of(self, depth: int):
+        if depth == self.config.head_dim:
+            return self.rope_cos, self.rope_sin
+        return self.rope_by_depth[depth]
 
     @staticmethod
     def from_model(model) -> "DecoderWeights":
@@ -74,10 +128,10 @@ class DecoderWeights:
         return decoder_weights_from_model(model)
 
 
-def rope_tables(config: LlamaConfig):
+def rope_tables(config: LlamaConfig, depth: Optional[int] = None):
     """cos / sin rows for positions 0..max_position-1, half-split convention (the two halves of
     a row repeat the same angles), computed in float64 and stored as float32."""
-    half = config.head_dim // 2
+    half = (config.head_dim if depth is None else depth) // 2
     inv_freq = 1.0 / (config.rope_base ** (np.arange(half, dtype=np.float64) / half))
     angles = np.arange(config.max_position, dtype=np.float64)[:, None] * inv_freq[None, :]
     angles = np.concatenate([angles, angles], axis=1)
@@ -95,18 +149,26 @@ def random_weights(config: LlamaConfig, seed: int = 0) -> DecoderWeights:
                             .astype(np.float16), np.float16(6.104e-05))
         return Int4Linear(n, k, packed, scales)
 
-    d, kv = config.d_model, config.kv_heads * config.head_dim
+    d = config.d_model
     w = DecoderWeights(config, rng.normal(0, 0.02, size=(config.vocab, d)).astype(np.float16))
-    for _ in range(config.layers):
-        w.layers.append({
+    for layer in range(config.layers):
+        depth = config.depth_of(layer)
+        kv = config.kv_heads * depth
+        entry = {
             "attn_norm": np.ones(d, dtype=np.float32), "ffn_norm": np.ones(d, dtype=np.float32),
-            "q": lin(config.heads * config.head_dim, d), "k": lin(kv, d), "v": lin(kv, d),
-            "o": lin(d, config.heads * config.head_dim),
+            "q": lin(config.heads * depth, d), "k": lin(kv, d), "v": lin(kv, d),
+            "o": lin(d, config.heads * depth),
             "gate": lin(config.ffn, d), "up": lin(config.ffn, d), "down": lin(d, config.ffn),
-        })
+        }
+        if config.owner_of(layer) != layer:   # a KV-sharing layer projects q only
+            del entry["k"], entry["v"]
+        w.layers.append(entry)
     w.final_norm = np.ones(d, dtype=np.float32)
     w.lm_head = lin(config.vocab, d)
     w.rope_cos, w.rope_sin = rope_tables(config)
+    for depth in config.head_dims:
+        if depth != config.head_dim:
+            w.rope_by_depth[depth] = rope_tables(config, depth)
     return w
 
 
@@ -169,24 +231,39 @@ class LlamaDecoderSession:
         self.fuse_decode = fuse_decode
         self.embedding = gpu.upload(weights.embedding)
         self.layers = []
-        for lw in weights.layers:
+        # per-layer attention structure: head dim, owner of the K / V, readers of an owner
+        self.spec = []
+        for li in range(c.layers):
+            depth, owner = c.depth_of(li), c.owner_of(li)
+            readers = c.readers_of(li) if owner == li else []
+            self.spec.append({"depth": depth, "hd": c.heads * depth, "kvd": c.kv_heads * depth,
+                              "owner": owner, "last_reader": readers[-1] if readers else li,
+                              "shared": len(readers) > 1, "half_scale": c.half_scale_of(li)})
+        for li, lw in enumerate(weights.layers):
+            owns = c.owner_of(li) == li
+            names = ("q", "k", "v", "o", "gate", "up", "down") if owns else \
+                ("q", "o", "gate", "up", "down")
             entry = {
                 "attn_norm": gpu.upload(lw["attn_norm"]), "ffn_norm": gpu.upload(lw["ffn_norm"]),
-                **{name: _DeviceLinear(gpu, lw[name])
-                   for name in ("q", "k", "v", "o", "gate", "up", "down")},
+                **{name: _DeviceLinear(gpu, lw[name]) for name in names},
             }
             if fuse_decode:
-                entry["qkv"] = _DeviceLinear(gpu, _stack_rows(
-                    _rope_pair_rows(lw["q"], c.head_dim), _rope_pair_rows(lw["k"], c.head_dim),
-                    lw["v"]))
+                depth = c.depth_of(li)
+                if owns:
+                    entry["qkv"] = _DeviceLinear(gpu, _stack_rows(
+                        _rope_pair_rows(lw["q"], depth), _rope_pair_rows(lw["k"], depth), lw["v"]))
+                else:   # a KV-sharing layer: the fused launch carries the q rows only
+                    entry["qkv"] = _DeviceLinear(gpu, _rope_pair_rows(lw["q"], depth))
                 entry["gate_up"] = _DeviceLinear(gpu, _interleave_rows(lw["gate"], lw["up"]))
             self.layers.append(entry)
         self.final_norm = gpu.upload(weights.final_norm)
         self.lm_head = _DeviceLinear(gpu, weights.lm_head)
-        self.rope_cos = gpu.upload(weights.rope_cos)
-        self.rope_sin = gpu.upload(weights.rope_sin)
+        # RoPE tables, one pair per head dim
+        self.rope = {depth: tuple(gpu.upload(t) for t in weights.rope_of(depth))
+                     for depth in c.head_dims}
         m, d = chunk_length, c.d_model
-        hd, kvd = c.heads * c.head_dim, c.kv_heads * c.head_dim
+        hd = max(sp["hd"] for sp in self.spec)
+        kvd = max(sp["kvd"] for sp in self.spec)
         eb = self.eb
         a = gpu.alloc
         self.buf = {
@@ -200,6 +277,13 @@ class LlamaDecoderSession:
             # per-workgroup argmax pairs of the head projection (8 bytes per 4 rows at most)
             "argmax_part": a((c.vocab + 3) // 4 * 8),
         }
+        # An owner whose K / V other layers read keeps this step's rows in buffers of its own
+        # until its last reader has run (the shared scratch above is reused by every layer).
+        for li, sp in enumerate(self.spec):
+            if sp["shared"]:
+                self.buf[f"kr{li}"] = a(m * sp["kvd"] * eb)
+                self.buf[f"vt{li}"] = a(m * sp["kvd"] * eb)
+                self.buf[f"qkv{li}"] = a((sp["hd"] + 2 * sp["kvd"]) * eb)
         self.workspace: Optional[DeviceBuffer] = None
         self.logits_shape = (1, c.vocab)
 
@@ -212,8 +296,9 @@ class LlamaDecoderSession:
                     value.s.free()
                 else:
                     value.free()
+        tables = [t for pair in self.rope.values() for t in pair]
         for buf in list(self.buf.values()) + [self.embedding, self.final_norm, self.lm_head.w,
-                                              self.lm_head.s, self.rope_cos, self.rope_sin]:
+                                              self.lm_head.s] + tables:
             buf.free()
         if self.workspace is not None:
             self.workspace.free()
@@ -226,11 +311,20 @@ class LlamaDecoderSession:
             raise ExecutionError(f"chunkLength {chunk_length} differs from the session's "
                                  f"{self.chunk_length}")
         c = self.config
+        layers = range(c.layers)
+        for li in layers:
+            if c.window_of(li) > capacity:
+                raise ExecutionError(f"layer {li}: window {c.window_of(li)} exceeds capacity "
+                                     f"{capacity}")
         ctx = GenerationContext(self.gpu, layers=c.layers, kv_planes=c.kv_heads,
                                 depth=c.head_dim, capacity=capacity, chunk_length=chunk_length,
-                                kv_itemsize=self.kv_eb)
-        need = self.gpu.attention_state_workspace(1, c.heads, c.kv_heads, 1, c.head_dim, 0,
-                                                  capacity)
+                                kv_itemsize=self.kv_eb,
+                                layer_depths=[c.depth_of(li) for li in layers],
+                                layer_windows=[c.window_of(li) for li in layers],
+                                layer_owners=[c.owner_of(li) for li in layers])
+        need = max(self.gpu.attention_state_workspace(1, c.heads, c.kv_heads, 1, c.depth_of(li),
+                                                      c.window_of(li), capacity)
+                   for li in layers)
         if self.workspace is None or self.workspace.nbytes < need:
             if self.workspace is not None:
                 self.workspace.free()
@@ -302,47 +396,50 @@ class LlamaDecoderSession:
             self._forward_rows(context, m, past, query, lengths)
             self._head(last_row, m)
             return
+        pending = {}   # owner layer -> (k rows, v rows) whose appends wait for the last reader
         for li, lw in enumerate(self.layers):
+            sp = self.spec[li]
+            depth, owner = sp["depth"], sp["owner"]
+            cos, sin = self.rope[depth]
             g.rms_norm(b["h"], lw["attn_norm"], b["xn"], m, d, c.rms_eps, io)
             self._linear(b["xn"], lw["q"], b["q"], m)
-            self._linear(b["xn"], lw["k"], b["k"], m)
-            self._linear(b["xn"], lw["v"], b["v"], m)
-            g.rope_half(b["q"], b["pos"], self.rope_cos, self.rope_sin, b["qr"], m, c.heads,
-                        c.head_dim, c.max_position, True, io)
-            g.rope_half(b["k"], b["pos"], self.rope_cos, self.rope_sin, b["kr"], m, c.kv_heads,
-                        c.head_dim, c.max_position, True, io)
-            if m > 1:
-                g.transpose_01(b["v"], b["vt"], m, c.kv_heads, c.head_dim, io)
-                vt = b["vt"]
-            else:
-                vt = b["v"]
-            spec = dict(chunk_rows=m, depth=c.head_dim, capacity=context.capacity,
-                        window=context.window)
+            g.rope_half(b["q"], b["pos"], cos, sin, b["qr"], m, c.heads, depth, c.max_position,
+                        True, io)
+            if owner == li:
+                # this step's K / V rows: in buffers of the layer's own when later layers read them
+                kr = b[f"kr{li}"] if sp["shared"] else b["kr"]
+                vt = b[f"vt{li}"] if sp["shared"] else (b["vt"] if m > 1 else b["v"])
+                self._linear(b["xn"], lw["k"], b["k"], m)
+                self._linear(b["xn"], lw["v"], b["v"], m)
+                g.rope_half(b["k"], b["pos"], cos, sin, kr, m, c.kv_heads, depth, c.max_position,
+                            True, io)
+                if m > 1:
+                    g.transpose_01(b["v"], vt, m, c.kv_heads, depth, io)
+                elif sp["shared"]:
+                    g.copy(vt, b["v"], self._copy_bytes(sp["kvd"] * self.eb))
+                pending[li] = (kr, vt)
+            kr, vt = pending[owner]
+            spec = dict(chunk_rows=m, depth=depth, capacity=context.layer_capacity[li],
+                        window=context.layer_window[li])
             if lengths is None:
-                g.attention_state(b["qr"], b["kr"], vt, context.slots_k[li], context.slots_v[li],
+                g.attention_state(b["qr"], kr, vt, context.slots_k[li], context.slots_v[li],
                                   b["att"], batch=1, heads=c.heads, kv_heads=c.kv_heads,
-                                  half_scale=c.half_scale, past=past, query=query, io_dtype=io,
-                                  kv_dtype=self.kv_dtype, workspace=self.workspace, **spec)
-                # readers first, then the appends (docs/ir-v1.md:345-348)
-                g.state_append(b["kr"], context.slots_k[li], kv_planes=c.kv_heads, past=past,
-                               query=query, x_dtype=io, slot_dtype=self.kv_dtype, **spec)
-                g.state_append(vt, context.slots_v[li], kv_planes=c.kv_heads, past=past,
-                               query=query, x_dtype=io, slot_dtype=self.kv_dtype, **spec)
+                                  half_scale=sp["half_scale"], past=past, query=query,
+                                  io_dtype=io, kv_dtype=self.kv_dtype, workspace=self.workspace,
+                                  **spec)
             else:
-                g.attention_state_lengths(b["qr"], b["kr"], vt, context.slots_k[li],
+                g.attention_state_lengths(b["qr"], kr, vt, context.slots_k[li],
                                           context.slots_v[li], b["att"], batch=1, heads=c.heads,
-                                          kv_heads=c.kv_heads, half_scale=c.half_scale,
+                                          kv_heads=c.kv_heads, half_scale=sp["half_scale"],
                                           lengths=lengths, max_past=context.capacity - 1,
                                           io_dtype=io, kv_dtype=self.kv_dtype,
                                           workspace=self.workspace, **spec)
-                g.state_append_lengths(b["kr"], context.slots_k[li], kv_planes=c.kv_heads,
-                                       lengths=lengths, x_dtype=io, slot_dtype=self.kv_dtype,
-                                       **spec)
-                g.state_append_lengths(vt, context.slots_v[li], kv_planes=c.kv_heads,
-                                       lengths=lengths, x_dtype=io, slot_dtype=self.kv_dtype,
-                                       **spec)
+            # readers first, then the appends (docs/ir-v1.md:345-348): the append of a slot
+            # follows the last layer that reads it
+            if self.spec[owner]["last_reader"] == li:
+                self._append_pair(context, owner, pending.pop(owner), m, past, query, lengths)
             if m > 1:
-                g.transpose_01(b["att"], b["att2"], c.heads, m, c.head_dim, io)
+                g.transpose_01(b["att"], b["att2"], c.heads, m, depth, io)
                 att = b["att2"]
             else:
                 att = b["att"]
@@ -355,6 +452,25 @@ class LlamaDecoderSession:
             self._linear(b["act"], lw["down"], b["dn"], m)
             g.add(b["h"], b["dn"], b["h"], m * d, io)
         self._head(last_row, m)
+
+    @staticmethod
+    def _copy_bytes(nbytes: int) -> int:
+        """Device copies move whole 16-byte pieces (every buffer here is allocated in them)."""
+        return (nbytes + 15) // 16 * 16
+
+    def _append_pair(self, context: GenerationContext, li: int, rows: tuple, m: int, past: int,
+                     query: int, lengths: Optional[DeviceBuffer]) -> None:
+        """state_append of this step's K and V rows to the slots of layer `li`."""
+        g, c, io = self.gpu, self.config, self.io_dtype
+        spec = dict(chunk_rows=m, depth=self.spec[li]["depth"],
+                    capacity=context.layer_capacity[li], window=context.layer_window[li])
+        for src, slot in ((rows[0], context.slots_k[li]), (rows[1], context.slots_v[li])):
+            if lengths is None:
+                g.state_append(src, slot, kv_planes=c.kv_heads, past=past, query=query,
+                               x_dtype=io, slot_dtype=self.kv_dtype, **spec)
+            else:
+                g.state_append_lengths(src, slot, kv_planes=c.kv_heads, lengths=lengths,
+                                       x_dtype=io, slot_dtype=self.kv_dtype, **spec)
 
     def _head(self, last_row: Optional[int], m: int = 1) -> None:
         """Token-only exit: the head runs on the last valid row only.  `last_row=None`: the
@@ -376,80 +492,92 @@ class LlamaDecoderSession:
         self._linear(b["xn"], self.lm_head, b["logits"], 1)
         g.argmax(b["logits"], b["token"], 1, c.vocab, io)
 
-    def _append_chunk(self, context: GenerationContext, li: int, past: int, query: int,
-                      lengths: Optional[DeviceBuffer], spec: dict) -> None:
-        g, c, b, io = self.gpu, self.config, self.buf, self.io_dtype
-        for src, slot in ((b["kr"], context.slots_k[li]), (b["vt"], context.slots_v[li])):
-            if lengths is None:
-                g.state_append(src, slot, kv_planes=c.kv_heads, past=past, query=query,
-                               x_dtype=io, slot_dtype=self.kv_dtype, **spec)
-            else:
-                g.state_append_lengths(src, slot, kv_planes=c.kv_heads, lengths=lengths,
-                                       x_dtype=io, slot_dtype=self.kv_dtype, **spec)
-
     def _rows_form_covers(self, m: int) -> bool:
         """The chunk-of-rows launches need groups of 64 codes or more, K a multiple of 32 and
         (their limit for the f32 class and for 32-bit element offsets) no more than 65536 rows."""
         c = self.config
         return (c.group_size >= 64 and c.d_model % 32 == 0 and c.ffn % 32 == 0
-                and (c.heads * c.head_dim) % 32 == 0 and m <= 65536)
+                and all(sp["hd"] % 32 == 0 for sp in self.spec) and m <= 65536)
 
     def _forward_rows(self, context: GenerationContext, m: int, past: int, query: int,
                       lengths: Optional[DeviceBuffer]) -> None:
         """A chunk of m > 16 rows, 7 launches a layer: the [q; k; v] projection writes roped,
         head-major q / k / v, the attention writes row-major and appends the chunk's K / V rows,
         the o and down projections add the residual in place, the gate/up projection applies
-        silu * up."""
+        silu * up.  (A KV-sharing layer projects and rotates q alone, in two launches.)"""
         from .runtime import EPILOGUE_SILU_PAIRS
         g, c, b, io = self.gpu, self.config, self.buf, self.io_dtype
         d, group, compute = c.d_model, c.group_size, self.prefill_compute
-        spec = dict(chunk_rows=m, depth=c.head_dim, capacity=context.capacity,
-                    window=context.window)
         # COMPUTE_F16 rounds the f32 activations of every product to fp16: the three activations
         # only a product reads (both norms' outputs, the attention's, silu(gate) * up) are then
         # written as fp16 by their producers — the same values, half the bytes for the products
-        half = (self.half_activations and compute == COMPUTE_F16 and io == F32
-                and c.head_dim in (64, 128))
+        half = self.half_activations and compute == COMPUTE_F16 and io == F32
         xd = F16 if half else io
+        pending = {}   # owner layer -> (k rows, v rows) whose appends wait for the last reader
         for li, lw in enumerate(self.layers):
+            sp = self.spec[li]
+            depth, owner = sp["depth"], sp["owner"]
+            window = context.layer_window[li]
+            cos, sin = self.rope[depth]
+            spec = dict(chunk_rows=m, depth=depth, capacity=context.layer_capacity[li],
+                        window=window)
             g.rms_norm_cast(b["h"], lw["attn_norm"], b["xn"], m, d, c.rms_eps, io, xd)
-            lin = lw["qkv"]
-            g.prefill_qkv(b["xn"], lin.w, lin.s, b["pos"], self.rope_cos, self.rope_sin, b["qr"],
-                          b["kr"], b["vt"], m=m, heads=c.heads, kv_heads=c.kv_heads,
-                          depth=c.head_dim, k=d, group=group, table_rows=c.max_position,
-                          io_dtype=io, scale_dtype=lin.scale_dtype, compute=compute, x_dtype=xd)
-            if c.head_dim in (64, 128):
-                # attention + output permute (+ both appends when no window can wrap) in one launch
-                g.attention_chunk(b["qr"], b["kr"], b["vt"], context.slots_k[li],
-                                  context.slots_v[li], b["att2"], batch=1, heads=c.heads,
-                                  kv_heads=c.kv_heads, half_scale=c.half_scale, past=past,
-                                  query=query, lengths=lengths, io_dtype=io,
-                                  kv_dtype=self.kv_dtype, row_major=True,
-                                  append=context.window == 0, out_f16=half, **spec)
-                if context.window != 0:
-                    self._append_chunk(context, li, past, query, lengths, spec)
+            if owner == li:
+                kr = b[f"kr{li}"] if sp["shared"] else b["kr"]
+                vt = b[f"vt{li}"] if sp["shared"] else b["vt"]
+                lin = lw["qkv"]
+                g.prefill_qkv(b["xn"], lin.w, lin.s, b["pos"], cos, sin, b["qr"], kr, vt, m=m,
+                              heads=c.heads, kv_heads=c.kv_heads, depth=depth, k=d, group=group,
+                              table_rows=c.max_position, io_dtype=io, scale_dtype=lin.scale_dtype,
+                              compute=compute, x_dtype=xd)
+                pending[li] = (kr, vt)
+            else:
+                lin = lw["q"]
+                g.linear_i4_rows(b["xn"], lin.w, lin.s, b["q"], m, lin.n, lin.k, group,
+                                 io_dtype=io, scale_dtype=lin.scale_dtype, compute=compute,
+                                 x_dtype=xd)
+                g.rope_half(b["q"], b["pos"], cos, sin, b["qr"], m, c.heads, depth,
+                            c.max_position, True, io)
+            kr, vt = pending[owner]
+            last_reader = self.spec[owner]["last_reader"] == li
+            att_half = half and depth in (64, 128)
+            if depth in (64, 128):
+                # attention + output permute in one launch; it also appends the chunk's rows when
+                # it is the slot's last reader and no window can wrap (slot rows past.. are read
+                # by nobody in that launch)
+                fold = last_reader and window == 0
+                g.attention_chunk(b["qr"], kr, vt, context.slots_k[li], context.slots_v[li],
+                                  b["att2"], batch=1, heads=c.heads, kv_heads=c.kv_heads,
+                                  half_scale=sp["half_scale"], past=past, query=query,
+                                  lengths=lengths, io_dtype=io, kv_dtype=self.kv_dtype,
+                                  row_major=True, append=fold, out_f16=att_half, **spec)
+                if last_reader:
+                    rows = pending.pop(owner)
+                    if not fold:
+                        self._append_pair(context, owner, rows, m, past, query, lengths)
             else:
                 if lengths is None:
-                    g.attention_state(b["qr"], b["kr"], b["vt"], context.slots_k[li],
-                                      context.slots_v[li], b["att"], batch=1, heads=c.heads,
-                                      kv_heads=c.kv_heads, half_scale=c.half_scale, past=past,
-                                      query=query, io_dtype=io, kv_dtype=self.kv_dtype,
+                    g.attention_state(b["qr"], kr, vt, context.slots_k[li], context.slots_v[li],
+                                      b["att"], batch=1, heads=c.heads, kv_heads=c.kv_heads,
+                                      half_scale=sp["half_scale"], past=past, query=query,
+                                      io_dtype=io, kv_dtype=self.kv_dtype,
                                       workspace=self.workspace, **spec)
                 else:
-                    g.attention_state_lengths(b["qr"], b["kr"], b["vt"], context.slots_k[li],
+                    g.attention_state_lengths(b["qr"], kr, vt, context.slots_k[li],
                                               context.slots_v[li], b["att"], batch=1,
                                               heads=c.heads, kv_heads=c.kv_heads,
-                                              half_scale=c.half_scale, lengths=lengths,
+                                              half_scale=sp["half_scale"], lengths=lengths,
                                               max_past=context.capacity - 1, io_dtype=io,
                                               kv_dtype=self.kv_dtype, workspace=self.workspace,
                                               **spec)
                 # readers first, then the appends (docs/ir-v1.md:345-348)
-                self._append_chunk(context, li, past, query, lengths, spec)
-                g.transpose_01(b["att"], b["att2"], c.heads, m, c.head_dim, io)
+                if last_reader:
+                    self._append_pair(context, owner, pending.pop(owner), m, past, query, lengths)
+                g.transpose_01(b["att"], b["att2"], c.heads, m, depth, io)
             lin = lw["o"]
             g.linear_i4_rows(b["att2"], lin.w, lin.s, b["h"], m, lin.n, lin.k, group,
                              residual=b["h"], io_dtype=io, scale_dtype=lin.scale_dtype,
-                             compute=compute, x_dtype=xd)
+                             compute=compute, x_dtype=F16 if att_half else io)
             g.rms_norm_cast(b["h"], lw["ffn_norm"], b["xn"], m, d, c.rms_eps, io, xd)
             lin = lw["gate_up"]
             # (fp16 in and out: silu(gate) * up is computed on the f32 sums and rounded once)
@@ -477,32 +605,44 @@ class LlamaDecoderSession:
         """One decode row (M = Q = 1), 5 launches per layer instead of 16."""
         from .runtime import EPILOGUE_SILU_PAIRS
         g, c, b, io, eb = self.gpu, self.config, self.buf, self.io_dtype, self.eb
-        hd, kvd = c.heads * c.head_dim, c.kv_heads * c.head_dim
-        # the qkv launch leaves [q_rot; k_rot; v] in one buffer
-        q_r, k_r = b["qkv"], b["qkv"].offset(hd * eb)
-        v_row = b["qkv"].offset((hd + kvd) * eb)
-        spec = dict(chunk_rows=1, depth=c.head_dim, capacity=context.capacity,
-                    window=context.window)
+        step_rows = {}   # owner layer -> its [q_rot; k_rot; v] buffer of this step
         for li, lw in enumerate(self.layers):
+            sp = self.spec[li]
+            depth, owner, hd, kvd = sp["depth"], sp["owner"], sp["hd"], sp["kvd"]
+            cos, sin = self.rope[depth]
+            spec = dict(chunk_rows=1, depth=depth, capacity=context.layer_capacity[li],
+                        window=context.layer_window[li])
             # rms_norm + [q; k; v] + rope of q and k + both appends in one launch; a one-row
-            # step's attention never reads the slot row this writes, so it may go first
+            # step's attention never reads the slot row this writes (the row holds a column
+            # outside every window of this step), so it may go first — also for the later
+            # layers that read the same slots
             lin = lw["qkv"]
-            g.decode_qkv(b["h"], lin.w, lin.s, b["pos"], self.rope_cos, self.rope_sin, b["qkv"],
-                         context.slots_k[li], context.slots_v[li], heads=c.heads,
-                         kv_heads=c.kv_heads, depth=c.head_dim, k=lin.k, group=c.group_size,
-                         table_rows=c.max_position, capacity=context.capacity,
-                         window=context.window, past=past, lengths=lengths,
-                         norm_weight=lw["attn_norm"], norm_eps=c.rms_eps, io_dtype=io,
-                         scale_dtype=lin.scale_dtype, kv_dtype=self.kv_dtype)
+            owns = owner == li
+            out = b[f"qkv{li}"] if sp["shared"] else b["qkv"]
+            g.decode_qkv(b["h"], lin.w, lin.s, b["pos"], cos, sin, out,
+                         context.slots_k[li] if owns else None,
+                         context.slots_v[li] if owns else None, heads=c.heads,
+                         kv_heads=c.kv_heads if owns else 0, depth=depth, k=lin.k,
+                         group=c.group_size, table_rows=c.max_position,
+                         capacity=context.layer_capacity[li], window=context.layer_window[li],
+                         past=past, lengths=lengths, norm_weight=lw["attn_norm"],
+                         norm_eps=c.rms_eps, io_dtype=io, scale_dtype=lin.scale_dtype,
+                         kv_dtype=self.kv_dtype)
+            if owns:
+                step_rows[li] = out
+            # the launch leaves [q_rot; k_rot; v] in one buffer (a sharing layer: q_rot alone)
+            q_r = out
+            kv = step_rows[owner]
+            k_r, v_row = kv.offset(hd * eb), kv.offset((hd + kvd) * eb)
             if lengths is None:
                 g.attention_state(q_r, k_r, v_row, context.slots_k[li], context.slots_v[li],
                                   b["att"], batch=1, heads=c.heads, kv_heads=c.kv_heads,
-                                  half_scale=c.half_scale, past=past, query=1, io_dtype=io,
+                                  half_scale=sp["half_scale"], past=past, query=1, io_dtype=io,
                                   kv_dtype=self.kv_dtype, workspace=self.workspace, **spec)
             else:
                 g.attention_state_lengths(q_r, k_r, v_row, context.slots_k[li],
                                           context.slots_v[li], b["att"], batch=1, heads=c.heads,
-                                          kv_heads=c.kv_heads, half_scale=c.half_scale,
+                                          kv_heads=c.kv_heads, half_scale=sp["half_scale"],
                                           lengths=lengths, max_past=self._replay_max_past(context),
                                           io_dtype=io, kv_dtype=self.kv_dtype,
                                           workspace=self.workspace, **spec)

@@ -12,7 +12,15 @@ node order the export recipe emits (tools/export-recipes/minicpm5/export_decode.
                                   -> rms_norm -> gate/up linear -> silu(gate) * up -> down linear -> add ]
                    -> rms_norm -> lm_head linear -> argmax
 
-so loading is recognition, not compilation: every attention node is traced back to the
+Layers may differ the way a Gemma-4-style decoder's do (tools/export-recipes/gemma4/
+export_decode.py:59-82,510-527): a `window` attr on the attention and the appends of a sliding
+layer, a head dim (with RoPE tables of its own) per layer kind, and KV-sharing layers, whose
+attention reads the roped k / v rows and the state slots of an earlier layer and which append
+nothing (two readers, one append; the owner's appends must follow its last reader,
+docs/ir-v1.md:345-348).  What else such models add around the attention (per-layer embedding
+tables, q / k norms, GELU, logit soft-capping) is not this graph shape and is rejected.
+
+So loading is recognition, not compilation: every attention node is traced back to the
 linears that feed it and forward to the linears that consume it, and anything that does not fit
 the shape above is rejected by name (nothing is approximated or skipped silently).  RoPE is the
 exported 7-node half-split chain (slice, slice, neg, cat, mul, mul, add in either of the two
@@ -184,50 +192,93 @@ def decoder_weights_from_model(model: KarumeModel) -> DecoderWeights:
     if not others:
         raise GraphShapeError("the graph has no position input")
 
-    group_sizes, eps_values, scales_seen = set(), set(), set()
+    group_sizes, eps_values = set(), set()
     layers: List[Dict[str, object]] = []
-    cos_table = sin_table = positions = None
-    heads = kv_heads = depth = None
+    tables: Dict[int, Tuple[str, str]] = {}     # head dim -> (cos table, sin table)
+    positions = None
+    heads = kv_heads = None
+    depths: List[int] = []
+    windows: List[int] = []
+    owners: List[int] = []
+    kv_linear_owner: Dict[int, int] = {}        # index of a k / v linear node -> its layer
+    att_index = {id(node): index for index, node in enumerate(g.nodes)}
     for li, att in enumerate(attentions):
         what = f"layer {li}"
         states = att.get("states")
         if not isinstance(states, dict) or set(states) != {"k", "v"}:
             raise GraphShapeError(f"{what}: the attention node is not in states form")
-        if "window" in att.get("attrs", {}):
-            raise GraphShapeError(f"{what}: sliding-window layers are not covered by this session")
-        scales_seen.add(float(att["attrs"]["scale"]))
+        window = att.get("attrs", {}).get("window", 0)
+        if not isinstance(window, int) or isinstance(window, bool) or window < 0:
+            raise GraphShapeError(f"{what}: window {window!r} is not a positive integer")
         q_shape, k_shape = g.shape(att["ins"][0]), g.shape(att["ins"][1])
-        dims = (q_shape[1], k_shape[1], q_shape[3])
+        dims = (q_shape[1], k_shape[1])
+        depth = q_shape[3]
         if heads is None:
-            heads, kv_heads, depth = dims
-        elif dims != (heads, kv_heads, depth):
-            raise GraphShapeError(f"{what}: heads / kv heads / head dim {dims} differ from layer 0")
+            heads, kv_heads = dims
+        elif dims != (heads, kv_heads):
+            raise GraphShapeError(f"{what}: heads / kv heads {dims} differ from layer 0")
+        if not isinstance(depth, int) or k_shape[3] != depth or g.shape(att["ins"][2])[3] != depth:
+            raise GraphShapeError(f"{what}: q, k and v do not share one head dim")
+        want_scale = float(np.float32(np.sqrt(1.0 / np.sqrt(float(depth)))))
+        scale = float(att["attrs"]["scale"])
+        if abs(scale - want_scale) > 1e-6 * want_scale:
+            raise GraphShapeError(f"{what}: attention scale {scale} is not sqrt(1/sqrt({depth})) "
+                                  f"= {want_scale}")
 
         entry: Dict[str, object] = {}
         norm_inputs = set()
+        kv_nodes = []
         for slot, name in zip(("q", "k", "v"), att["ins"]):
-            source, tables = _rope_source(g, g.through_layout(name), f"{what}.{slot}")
-            if (tables is not None) != (slot != "v"):
+            source, found = _rope_source(g, g.through_layout(name), f"{what}.{slot}")
+            if (found is not None) != (slot != "v"):
                 raise GraphShapeError(f"{what}.{slot}: RoPE is expected on q and k and not on v")
-            if tables is not None:
+            if found is not None:
                 for other in others:
                     try:
-                        found = (_table_of(g, tables[0], other, what), _table_of(g, tables[1], other, what))
+                        pair = (_table_of(g, found[0], other, what), _table_of(g, found[1], other, what))
                     except GraphShapeError:
                         continue
-                    if cos_table is None:
-                        cos_table, sin_table, positions = found[0], found[1], other
-                    elif (cos_table, sin_table, positions) != (found[0], found[1], other):
-                        raise GraphShapeError(f"{what}.{slot}: a second pair of RoPE tables")
+                    if positions is None:
+                        positions = other
+                    if other != positions or tables.setdefault(depth, pair) != pair:
+                        raise GraphShapeError(f"{what}.{slot}: a second pair of RoPE tables for "
+                                              f"head dim {depth}")
                     break
                 else:
                     raise GraphShapeError(f"{what}.{slot}: cos / sin are not looked up by position")
-            node = g.node_of(g.through_layout(source))
-            if node is None:
+            node_index = g.producer.get(g.through_layout(source))
+            if node_index is None:
                 raise GraphShapeError(f"{what}.{slot}: no linear node behind '{source}'")
+            node = g.nodes[node_index]
+            if slot != "q":
+                kv_nodes.append(node_index)
+                if node_index in kv_linear_owner:
+                    continue          # the k / v rows of an earlier layer (checked below)
             entry[slot], group = _linear(g, node, resident, f"{what}.{slot}")
             group_sizes.add(group)
             norm_inputs.add(node["ins"][0])
+        shared_from = {kv_linear_owner.get(index) for index in kv_nodes}
+        if shared_from == {None}:
+            owner = li
+            for index in kv_nodes:
+                kv_linear_owner[index] = li
+        elif len(shared_from) == 1:
+            # a KV-sharing layer: k and v are the rows of ONE earlier layer, read from that
+            # layer's slots under the same window
+            owner = shared_from.pop()
+            owner_att = attentions[owner]
+            if owner_att["ins"][1] != att["ins"][1] or owner_att["ins"][2] != att["ins"][2] or \
+                    owner_att["states"] != states:
+                raise GraphShapeError(f"{what}: reads the k / v linears of layer {owner} but not "
+                                      "its roped rows and state slots")
+            if depths[owner] != depth or windows[owner] != window:
+                raise GraphShapeError(f"{what}: shares the K / V of layer {owner} under another "
+                                      "head dim or window")
+        else:
+            raise GraphShapeError(f"{what}: k and v come from different layers")
+        depths.append(depth)
+        windows.append(window)
+        owners.append(owner)
         if len(norm_inputs) != 1:
             raise GraphShapeError(f"{what}: q, k and v do not read one normalised row")
         norm = g.node_of(next(iter(norm_inputs)))
@@ -236,10 +287,6 @@ def decoder_weights_from_model(model: KarumeModel) -> DecoderWeights:
         entry["attn_norm"] = np.ascontiguousarray(_f32_initializer(g, norm["ins"][1], what),
                                                    dtype=np.float32)
         eps_values.add(float(norm["attrs"]["eps"]))
-        # both appends name this layer's slots
-        appended = {n["states"]["slot"] for n in g.nodes if n["op"] == "state_append"}
-        if states["k"] not in appended or states["v"] not in appended:
-            raise GraphShapeError(f"{what}: KV-sharing layers (no state_append) are not covered")
 
         # forward: attention -> o linear -> add -> rms_norm -> gate / up -> silu * up -> down -> add
         _, o_node = g.forward_through_layout(att["outs"][0], f"{what} attention output")
@@ -287,6 +334,35 @@ def decoder_weights_from_model(model: KarumeModel) -> DecoderWeights:
             raise GraphShapeError(f"{what}: the down projection does not feed a residual add")
         layers.append(entry)
 
+    # every owner's slots are appended once each, from its own roped k rows and v rows, under
+    # the layer's window, after the last attention that reads them (docs/ir-v1.md:345-348)
+    appends = {}
+    for index, node in enumerate(g.nodes):
+        if node["op"] == "state_append":
+            slot = node["states"]["slot"]
+            if slot in appends:
+                raise GraphShapeError(f"state slot '{slot}' is appended twice")
+            appends[slot] = (index, node)
+    for li, att in enumerate(attentions):
+        if owners[li] != li:
+            continue
+        readers = [index for index, other in enumerate(attentions) if owners[index] == li]
+        last_reader = max(att_index[id(attentions[index])] for index in readers)
+        for slot, source in ((att["states"]["k"], att["ins"][1]), (att["states"]["v"], att["ins"][2])):
+            if slot not in appends:
+                raise GraphShapeError(f"layer {li}: no state_append for slot '{slot}' (a layer "
+                                      "that appends nothing must read another layer's k / v)")
+            index, node = appends[slot]
+            if node["ins"][0] != source:
+                raise GraphShapeError(f"layer {li}: slot '{slot}' is appended from "
+                                      f"'{node['ins'][0]}', not from the rows the attention reads")
+            if node.get("attrs", {}).get("window", 0) != windows[li]:
+                raise GraphShapeError(f"layer {li}: the append of '{slot}' declares another window "
+                                      "than the attention")
+            if index < last_reader:
+                raise GraphShapeError(f"layer {li}: slot '{slot}' is appended before its last "
+                                      "reader")
+
     # exit: argmax <- lm_head linear <- rms_norm
     argmaxes = [n for n in g.nodes if n["op"] == "argmax"]
     if len(argmaxes) != 1:
@@ -307,24 +383,34 @@ def decoder_weights_from_model(model: KarumeModel) -> DecoderWeights:
         raise GraphShapeError("the lm_head does not read an rms_norm")
     eps_values.add(float(final["attrs"]["eps"]))
 
-    if len(group_sizes) != 1 or len(eps_values) != 1 or len(scales_seen) != 1:
-        raise GraphShapeError(f"group sizes {sorted(group_sizes)}, eps {sorted(eps_values)} and "
-                              f"attention scales {sorted(scales_seen)} must each be uniform")
-    cos = np.ascontiguousarray(_f32_initializer(g, cos_table, "RoPE cos table"), dtype=np.float32)
-    sin = np.ascontiguousarray(_f32_initializer(g, sin_table, "RoPE sin table"), dtype=np.float32)
-    if cos.shape != sin.shape or cos.ndim != 2 or cos.shape[1] != depth:
-        raise GraphShapeError(f"RoPE tables {cos.shape} / {sin.shape} are not [positions, {depth}]")
-    q_lin, k_lin = layers[0]["q"], layers[0]["k"]
-    if q_lin.n != heads * depth or k_lin.n != kv_heads * depth or q_lin.k != d_model:
-        raise GraphShapeError("projection shapes disagree with heads x head dim / d_model")
+    if len(group_sizes) != 1 or len(eps_values) != 1:
+        raise GraphShapeError(f"group sizes {sorted(group_sizes)} and eps {sorted(eps_values)} "
+                              "must each be uniform")
+    rope = {}
+    for depth, (cos_table, sin_table) in tables.items():
+        cos = np.ascontiguousarray(_f32_initializer(g, cos_table, "RoPE cos table"), dtype=np.float32)
+        sin = np.ascontiguousarray(_f32_initializer(g, sin_table, "RoPE sin table"), dtype=np.float32)
+        if cos.shape != sin.shape or cos.ndim != 2 or cos.shape[1] != depth:
+            raise GraphShapeError(f"RoPE tables {cos.shape} / {sin.shape} are not "
+                                  f"[positions, {depth}]")
+        rope[depth] = (cos, sin)
+    if len({cos.shape[0] for cos, _ in rope.values()}) != 1:
+        raise GraphShapeError("the RoPE tables of the layer kinds differ in length")
+    for li, entry in enumerate(layers):
+        if entry["q"].n != heads * depths[li] or entry["q"].k != d_model or \
+                (owners[li] == li and entry["k"].n != kv_heads * depths[li]):
+            raise GraphShapeError(f"layer {li}: projection shapes disagree with heads x head dim "
+                                  "/ d_model")
+    uniform = len(set(depths)) == 1 and not any(windows) and owners == list(range(len(layers)))
+    depth0 = depths[0]
     config = LlamaConfig(layers=len(layers), d_model=int(d_model), ffn=int(layers[0]["gate"].n),
-                         heads=int(heads), kv_heads=int(kv_heads), head_dim=int(depth),
+                         heads=int(heads), kv_heads=int(kv_heads), head_dim=int(depth0),
                          vocab=int(vocab), group_size=int(next(iter(group_sizes))),
-                         rms_eps=float(next(iter(eps_values))), max_position=int(cos.shape[0]))
-    scale = next(iter(scales_seen))
-    if abs(scale - config.half_scale) > 1e-6 * config.half_scale:
-        raise GraphShapeError(f"attention scale {scale} is not sqrt(1/sqrt({depth})) = "
-                              f"{config.half_scale}")
+                         rms_eps=float(next(iter(eps_values))),
+                         max_position=int(rope[depth0][0].shape[0]),
+                         layer_windows=() if uniform else tuple(windows),
+                         layer_head_dims=() if uniform else tuple(depths),
+                         layer_kv_source=() if uniform else tuple(owners))
     if lm_head.n != vocab or lm_head.k != d_model:
         raise GraphShapeError("the lm_head shape disagrees with the embedding table")
     weights = DecoderWeights(config, np.ascontiguousarray(embedding, dtype=np.float16))
@@ -335,7 +421,8 @@ def decoder_weights_from_model(model: KarumeModel) -> DecoderWeights:
     weights.final_norm = np.ascontiguousarray(_f32_initializer(g, final["ins"][1], "final norm"),
                                               dtype=np.float32)
     weights.lm_head = lm_head
-    weights.rope_cos, weights.rope_sin = cos, sin
+    weights.rope_cos, weights.rope_sin = rope[depth0]
+    weights.rope_by_depth = {depth: pair for depth, pair in rope.items() if depth != depth0}
     return weights
 
 

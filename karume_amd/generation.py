@@ -49,22 +49,52 @@ class GenerationContext:
     """KV state slots + lengths of one sequence."""
 
     def __init__(self, gpu: GpuContext, *, layers: int, kv_planes: int, depth: int,
-                 capacity: int, chunk_length: int, window: int = 0, kv_itemsize: int = 4):
+                 capacity: int, chunk_length: int, window: int = 0, kv_itemsize: int = 4,
+                 layer_depths: Optional[Sequence[int]] = None,
+                 layer_windows: Optional[Sequence[int]] = None,
+                 layer_owners: Optional[Sequence[int]] = None):
+        """`layer_depths` / `layer_windows` / `layer_owners` (each one entry per layer) describe
+        decoders whose layers differ: a sliding layer's slots are rings of `window` rows (their
+        capacity is the window, not the context's: the ring map is col % window whatever the
+        capacity, docs/ir-v1.md:296-351), and a layer whose owner is an earlier layer has no
+        slots of its own — it reads the owner's (KV-sharing: two readers, one append,
+        packages/runtime/tests/gpu_state_acceptance_test.ts:866-977)."""
         _assert_positive_integer(capacity, "capacity")
         _assert_positive_integer(chunk_length, "chunkLength")
-        if window > capacity:
-            raise ExecutionError(f"window {window} exceeds capacity {capacity}")
+        depths = [depth] * layers if layer_depths is None else [int(v) for v in layer_depths]
+        windows = [window] * layers if layer_windows is None else [int(v) for v in layer_windows]
+        owners = list(range(layers)) if layer_owners is None else [int(v) for v in layer_owners]
+        if not (len(depths) == len(windows) == len(owners) == layers):
+            raise ExecutionError("per-layer depths / windows / owners must have one entry per layer")
         self.gpu = gpu
         self.capacity = capacity
         self.chunk_length = chunk_length
-        self.window = window
+        # full layers bound the sequence by the capacity; a context of sliding layers only never
+        # runs out of rows
+        self.window = 0 if any(w == 0 for w in windows) else min(windows)
+        self.layer_window: List[int] = windows
+        self.layer_capacity: List[int] = [w if w else capacity for w in windows]
         self.past = 0
         self.poisoned = False
         self.disposed = False
-        slot_bytes = kv_planes * capacity * depth * kv_itemsize
-        # zero-initialised at creation (packages/runtime/tests/gpu_state_execution_test.ts:159-164)
-        self.slots_k: List[DeviceBuffer] = [gpu.zeros(slot_bytes) for _ in range(layers)]
-        self.slots_v: List[DeviceBuffer] = [gpu.zeros(slot_bytes) for _ in range(layers)]
+        self.slots_k: List[DeviceBuffer] = []
+        self.slots_v: List[DeviceBuffer] = []
+        self._owned: List[DeviceBuffer] = []
+        for layer in range(layers):
+            owner = owners[layer]
+            if owner != layer:
+                if not 0 <= owner < layer or owners[owner] != owner:
+                    raise ExecutionError(f"layer {layer} cannot share the slots of layer {owner}")
+                self.slots_k.append(self.slots_k[owner])
+                self.slots_v.append(self.slots_v[owner])
+                continue
+            slot_bytes = kv_planes * self.layer_capacity[layer] * depths[layer] * kv_itemsize
+            # zero-initialised at creation
+            # (packages/runtime/tests/gpu_state_execution_test.ts:159-164)
+            k, v = gpu.zeros(slot_bytes), gpu.zeros(slot_bytes)
+            self.slots_k.append(k)
+            self.slots_v.append(v)
+            self._owned += [k, v]
         self.lengths: DeviceBuffer = gpu.zeros(16)
 
     # -- run protocol (generation-context.ts:330-345,559-604) --------------------------------
@@ -103,7 +133,7 @@ class GenerationContext:
         if self.poisoned:
             raise GenerationContextError(
                 "the generation context is poisoned by a failed run; create a new one")
-        if self.window:
+        if any(self.layer_window):
             raise ExecutionError("a sliding-window context cannot be rewound")
         if position < 0 or position > self.past:
             raise ExecutionError(f"rewind position {position} is outside 0..{self.past}")
@@ -112,9 +142,9 @@ class GenerationContext:
     def dispose(self) -> None:
         if self.disposed:
             return
-        for buf in self.slots_k + self.slots_v + [self.lengths]:
+        for buf in self._owned + [self.lengths]:
             buf.free()
-        self.slots_k, self.slots_v = [], []
+        self.slots_k, self.slots_v, self._owned = [], [], []
         self.disposed = True
 
 

@@ -232,20 +232,27 @@ def oracle_decoder_logits(weights, ids, rows=None) -> np.ndarray:
                                 np.zeros(l.n, dtype=np.float32), l.n, l.k, g)
 
     h = oracle.embedding(weights.embedding.astype(np.float32), ids)          # [T, d]
-    cos, sin = weights.rope_cos[:t], weights.rope_sin[:t]
-    for lw in weights.layers:
+    step_kv = {}     # owner layer -> (roped k, v) of the whole sequence
+    for li, lw in enumerate(weights.layers):
+        depth, owner, window = c.depth_of(li), c.owner_of(li), c.window_of(li)
+        cos, sin = (table[:t] for table in weights.rope_of(depth))
         xn = oracle.rms_norm(h, lw["attn_norm"], c.rms_eps)
-        q = lin(xn, lw["q"]).reshape(t, c.heads, c.head_dim).transpose(1, 0, 2)
-        k = lin(xn, lw["k"]).reshape(t, c.kv_heads, c.head_dim).transpose(1, 0, 2)
-        v = lin(xn, lw["v"]).reshape(t, c.kv_heads, c.head_dim).transpose(1, 0, 2)
+        q = lin(xn, lw["q"]).reshape(t, c.heads, depth).transpose(1, 0, 2)
         q = oracle.rope_half(q[None], cos, sin)
-        k = oracle.rope_half(k[None], cos, sin)
-        zeros = np.zeros((1, c.kv_heads, t, c.head_dim), dtype=np.float32)
-        att = oracle.state_attention(q, k, np.ascontiguousarray(v[None]), zeros, zeros, batch=1,
-                                     heads=c.heads, kv_heads=c.kv_heads, chunk_rows=t,
-                                     depth=c.head_dim, capacity=t, window=0, past=0, query=t,
-                                     scale=np.float32(c.half_scale))
-        att = att[0].transpose(1, 0, 2).reshape(t, c.heads * c.head_dim)
+        if owner == li:
+            k = lin(xn, lw["k"]).reshape(t, c.kv_heads, depth).transpose(1, 0, 2)
+            v = lin(xn, lw["v"]).reshape(t, c.kv_heads, depth).transpose(1, 0, 2)
+            step_kv[li] = (oracle.rope_half(k[None], cos, sin), np.ascontiguousarray(v[None]))
+        k, v = step_kv[owner]     # a KV-sharing layer attends over its owner's rows
+        slot_rows = max(t, window)  # the slots stay unread (past = 0); window <= capacity holds
+        zeros = np.zeros((1, c.kv_heads, slot_rows, depth), dtype=np.float32)
+        # one causal pass over the whole sequence; `window` is the explicit band
+        # (col <= row and row - col < window), no ring involved: nothing comes from a slot
+        att = oracle.state_attention(q, k, v, zeros, zeros, batch=1, heads=c.heads,
+                                     kv_heads=c.kv_heads, chunk_rows=t, depth=depth,
+                                     capacity=slot_rows, window=window, past=0, query=t,
+                                     scale=np.float32(c.half_scale_of(li)))
+        att = att[0].transpose(1, 0, 2).reshape(t, c.heads * depth)
         h = (h + lin(att, lw["o"])).astype(np.float32)
         xn = oracle.rms_norm(h, lw["ffn_norm"], c.rms_eps)
         act = oracle.silu_mul(lin(xn, lw["gate"]), lin(xn, lw["up"]))

@@ -2,7 +2,12 @@
 the decode export recipe lays the graph out (tools/export-recipes/minicpm5/export_decode.py:
 14-35; node vocabulary docs/ir-v1.md:277-520): token-only exit, RoPE as the exported 7-node
 half-split chain over cos / sin rows looked up by position, states-form attention followed by
-both appends.  Test-side only: the product reads such files, it does not write them."""
+both appends.  Layers may differ the way a Gemma-4-style decoder's do
+(tools/export-recipes/gemma4/export_decode.py:59-82,510-527): a `window` attr on the attention
+and both appends of a sliding layer, a head dim (and RoPE tables) per layer kind, and KV-sharing
+layers that read an earlier layer's roped k / v rows and slots and append nothing — the owner's
+appends then follow its last reader in node order (docs/ir-v1.md:345-348).
+Test-side only: the product reads such files, it does not write them."""
 from __future__ import annotations
 
 import json
@@ -17,8 +22,7 @@ from karume_amd.format_model import IR_METADATA_KEY, build_safetensors
 def decoder_graph(weights: DecoderWeights, edit: Optional[Callable[[dict], None]] = None):
     """(graph dict, tensors list) for `weights`; `edit(graph)` may damage the graph first."""
     c = weights.config
-    d, H, Hkv, D, V = c.d_model, c.heads, c.kv_heads, c.head_dim, c.vocab
-    half = D // 2
+    d, H, Hkv, V = c.d_model, c.heads, c.kv_heads, c.vocab
     nodes: List[dict] = []
     values: Dict[str, dict] = {}
     inits: Dict[str, dict] = {}
@@ -57,7 +61,9 @@ def decoder_graph(weights: DecoderWeights, edit: Optional[Callable[[dict], None]
         node("linear", [x, name, f"{name}.bias"], [value(out, (*lead, lin.n))])
         return out
 
-    def rope(x, heads, tag):
+    def rope(x, heads, tag, D):
+        half = D // 2
+        cos, sin = f"cos{D}", f"sin{D}"
         shape_full, shape_half = (1, heads, "M", D), (1, heads, "M", half)
         a, b, nb, rot, direct, cross, out = (f"{tag}.{s}" for s in
                                              ("lo", "hi", "neg", "rot", "xc", "rs", "rope"))
@@ -65,8 +71,8 @@ def decoder_graph(weights: DecoderWeights, edit: Optional[Callable[[dict], None]
         node("slice", [x], [value(b, shape_half)], {"dim": 3, "start": half, "end": D})
         node("neg", [b], [value(nb, shape_half)])
         node("cat", [nb, a], [value(rot, shape_full)], {"dim": 3})
-        node("mul", [x, "cos"], [value(direct, shape_full)])
-        node("mul", [rot, "sin"], [value(cross, shape_full)])
+        node("mul", [x, cos], [value(direct, shape_full)])
+        node("mul", [rot, sin], [value(cross, shape_full)])
         node("add", [direct, cross], [value(out, shape_full)])
         return out
 
@@ -77,33 +83,41 @@ def decoder_graph(weights: DecoderWeights, edit: Optional[Callable[[dict], None]
     inits["embed"] = {"tensor": "embed", "storage": {"dtype": "f16"}}
     value("embed", (V, d))
     node("embedding", ["embed", "input_ids"], [value("h.in", (1, "M", d))], {"padding_idx": None})
-    for table, array in (("cos", weights.rope_cos), ("sin", weights.rope_sin)):
-        f32_init(f"rope.{table}", array)
-        node("embedding", [f"rope.{table}", "position_ids"], [value(f"{table}.rows", (1, "M", D))],
-             {"padding_idx": None})
-        node("reshape", [f"{table}.rows"], [value(table, (1, 1, "M", D))])
+    for D in c.head_dims:
+        for table, array in zip(("cos", "sin"), weights.rope_of(D)):
+            f32_init(f"rope.{table}{D}", array)
+            node("embedding", [f"rope.{table}{D}", "position_ids"],
+                 [value(f"{table}{D}.rows", (1, "M", D))], {"padding_idx": None})
+            node("reshape", [f"{table}{D}.rows"], [value(f"{table}{D}", (1, 1, "M", D))])
     states = {}
     h = "h.in"
+    step_kv = {}      # owner layer -> (roped k value, v value) of this step
     for li, lw in enumerate(weights.layers):
         p = f"l{li}"
-        states[f"{p}.k"] = {"dtype": "f32", "shape": [1, Hkv, "C", D]}
-        states[f"{p}.v"] = {"dtype": "f32", "shape": [1, Hkv, "C", D]}
+        D, owner, window = c.depth_of(li), c.owner_of(li), c.window_of(li)
+        window_attr = {"window": window} if window else {}
         f32_init(f"{p}.attn_norm", lw["attn_norm"])
         node("rms_norm", [h, f"{p}.attn_norm"], [value(f"{p}.xn", (1, "M", d))], {"eps": c.rms_eps})
         heads_of = {"q": H, "k": Hkv, "v": Hkv}
         head_major = {}
-        for slot in ("q", "k", "v"):
+        for slot in ("q", "k", "v") if owner == li else ("q",):
             flat = linear(f"{p}.xn", f"{p}.{slot}_proj", lw[slot], f"{p}.{slot}.flat", (1, "M"))
             node("reshape", [flat], [value(f"{p}.{slot}.rows", (1, "M", heads_of[slot], D))])
             node("permute", [f"{p}.{slot}.rows"],
                  [value(f"{p}.{slot}", (1, heads_of[slot], "M", D))], {"dims": [0, 2, 1, 3]})
             head_major[slot] = f"{p}.{slot}"
-        q_rot = rope(head_major["q"], H, f"{p}.q")
-        k_rot = rope(head_major["k"], Hkv, f"{p}.k")
-        node("attention", [q_rot, k_rot, head_major["v"]], [value(f"{p}.att", (1, H, "M", D))],
-             {"scale": float(np.float32(c.half_scale))}, {"k": f"{p}.k", "v": f"{p}.v"})
-        node("state_append", [k_rot], [], {}, {"slot": f"{p}.k"})
-        node("state_append", [head_major["v"]], [], {}, {"slot": f"{p}.v"})
+        q_rot = rope(head_major["q"], H, f"{p}.q", D)
+        if owner == li:
+            states[f"{p}.k"] = {"dtype": "f32", "shape": [1, Hkv, "C", D]}
+            states[f"{p}.v"] = {"dtype": "f32", "shape": [1, Hkv, "C", D]}
+            step_kv[li] = (rope(head_major["k"], Hkv, f"{p}.k", D), head_major["v"])
+        k_rot, v_rows = step_kv[owner]
+        node("attention", [q_rot, k_rot, v_rows], [value(f"{p}.att", (1, H, "M", D))],
+             {"scale": float(np.float32(c.half_scale_of(li))), **window_attr},
+             {"k": f"l{owner}.k", "v": f"l{owner}.v"})
+        if c.readers_of(owner)[-1] == li:   # the appends follow the slot's last reader
+            node("state_append", [k_rot], [], dict(window_attr), {"slot": f"l{owner}.k"})
+            node("state_append", [v_rows], [], dict(window_attr), {"slot": f"l{owner}.v"})
         node("permute", [f"{p}.att"], [value(f"{p}.att.rows", (1, "M", H, D))], {"dims": [0, 2, 1, 3]})
         node("reshape", [f"{p}.att.rows"], [value(f"{p}.att.flat", (1, "M", H * D))])
         o = linear(f"{p}.att.flat", f"{p}.o_proj", lw["o"], f"{p}.o", (1, "M"))

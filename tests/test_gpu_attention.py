@@ -669,3 +669,81 @@ def test_attention_chunk_equals_attention_transpose_and_appends(gpu_ctx, io, kv,
         gpu_ctx.attention_chunk(got["q"], got["ins_k"], got["ins_v"], got["slot_k"], got["slot_v"],
                                 out, half_scale=0.5, past=0, query=1, io_dtype=io_code,
                                 kv_dtype=kv_code, **{**geometry, "depth": 32})
+
+
+# ---- KV-sharing layers: two readers, one append -------------------------------------------------
+
+SHARED_SERIES = [
+    # packages/runtime/tests/gpu_state_acceptance_test.ts:846-864
+    dict(name="full", heads=2, kv_heads=2, depth=4, capacity=16, window=0, chunk=3,
+         steps=[(3, 3), (3, 3), (3, 3), (1, 1)], order_probe=None),
+    # a ring of W = C = 4: the append of step 1 (past 3, Q 3) writes physical rows 3, 0, 1, two of
+    # which the readers of the same step still have to read — the one place where the order of
+    # readers and append shows in the values
+    dict(name="sliding W=4", heads=2, kv_heads=2, depth=4, capacity=4, window=4, chunk=3,
+         steps=[(3, 3), (3, 3), (3, 3), (1, 1)], order_probe=1),
+]
+
+
+@pytest.mark.parametrize("series", SHARED_SERIES, ids=lambda s: s["name"])
+def test_two_readers_one_append(gpu_ctx, series):
+    """Two attention calls with different queries read the same K / V rows and the same state
+    slots, then ONE pair of appends follows (packages/runtime/tests/
+    gpu_state_acceptance_test.ts:866-977): both outputs equal the oracle on the slots as they
+    were BEFORE the append (atol 5e-6), differ from each other, and — where the ring wraps into
+    rows of the same step — differ from an oracle that appended first; the slot bytes after
+    every step equal the oracle's chained slots."""
+    ctx = gpu_ctx
+    H, Hkv, D, C, W, M = (series[k] for k in ("heads", "kv_heads", "depth", "capacity", "window",
+                                              "chunk"))
+    scale = oracle.half_scale(D)
+    slot_k = np.zeros((1, Hkv, C, D), dtype=np.float32)
+    slot_v = np.zeros((1, Hkv, C, D), dtype=np.float32)
+    dk, dv = ctx.upload(slot_k), ctx.upload(slot_v)
+    past = 0
+    for index, (rows, query) in enumerate(series["steps"]):
+        salt = 17 + index * 23
+        count = Hkv * rows * D
+        qs = [helpers.seeded(H * rows * D, lambda i, s=salt + 101 * r: helpers.QUERY(i + s))
+              .reshape(1, H, rows, D) for r in range(2)]
+        k = helpers.seeded(count, lambda i: helpers.KEY(i + salt)).reshape(1, Hkv, rows, D)
+        v = helpers.seeded(count, lambda i: helpers.VALUE(i + salt)).reshape(1, Hkv, rows, D)
+        common = dict(chunk_rows=rows, depth=D, capacity=C, window=W, past=past, query=query)
+
+        def read(q, sk, sv):
+            return oracle.state_attention(q, k, v, sk, sv, batch=1, heads=H, kv_heads=Hkv,
+                                          scale=scale, **common)
+
+        bk, bv = ctx.upload(k), ctx.upload(v)
+        outs = []
+        for q in qs:   # both readers first ...
+            bq, out = ctx.upload(q), ctx.alloc(q.nbytes)
+            ws = ctx.alloc(ctx.attention_state_workspace(1, H, Hkv, rows, D, W, past, query))
+            ctx.attention_state(bq, bk, bv, dk, dv, out, batch=1, heads=H, kv_heads=Hkv,
+                                half_scale=scale, workspace=ws, **common)
+            outs.append(out.download(np.float32, q.shape))
+            for b in (bq, out, ws):
+                b.free()
+        for src, slot in ((bk, dk), (bv, dv)):   # ... then the one pair of appends
+            ctx.state_append(src, slot, kv_planes=Hkv, **common)
+        for q, got in zip(qs, outs):
+            want = read(q, slot_k, slot_v)
+            assert np.any(np.abs(want) > 1e-3), "the expected output is trivial"
+            ok, fails, max_abs, worst = oracle.allclose(got, want, atol=STATE_ATOL, rtol=0)
+            assert ok, (series["name"], index, fails, max_abs, worst)
+        assert outs[0].tobytes() != outs[1].tobytes()
+        new_k = oracle.state_append(k, slot_k, kv_planes=Hkv, **common)
+        new_v = oracle.state_append(v, slot_v, kv_planes=Hkv, **common)
+        if series["order_probe"] == index:
+            for q, got in zip(qs, outs):
+                wrong = read(q, new_k, new_v)
+                ok, *_ = oracle.allclose(got, wrong, atol=STATE_ATOL, rtol=0)
+                assert not ok, "the probe step does not tell reader-first from append-first"
+        slot_k, slot_v = new_k, new_v
+        past += query
+        assert dk.download(np.float32, slot_k.shape).tobytes() == slot_k.tobytes()
+        assert dv.download(np.float32, slot_v.shape).tobytes() == slot_v.tobytes()
+        bk.free()
+        bv.free()
+    dk.free()
+    dv.free()

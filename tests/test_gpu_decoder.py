@@ -697,3 +697,97 @@ def test_prefill_with_fp16_activation_copies_equals_prefill_without(gpu_ctx):
     assert np.array_equal(results[0][1].view(np.uint32), results[1][1].view(np.uint32))
     assert np.array_equal(results[0][2].view(np.uint32), results[1][2].view(np.uint32))
     assert np.array_equal(results[0][0], results[1][0])
+
+
+# ---- layers that differ: sliding windows, head dims per layer kind, KV-sharing layers ----------
+# (tools/export-recipes/gemma4/export_decode.py:59-82,510-527).  Sliding layers: head dim 64,
+# window 8 (the sequence passes it, so the band and the ring both matter); full layers: head
+# dim 128 here, 32 in the second config (the attention's generic kernel); layers 3 and 4 read
+# the K / V rows and slots of layers 1 and 2.
+MIXED = LlamaConfig(layers=5, d_model=256, ffn=384, heads=8, kv_heads=2, head_dim=64, vocab=512,
+                    group_size=128, max_position=64,
+                    layer_windows=(8, 8, 0, 8, 0), layer_head_dims=(64, 64, 128, 64, 128),
+                    layer_kv_source=(0, 1, 2, 1, 2))
+MIXED_SMALL_DIMS = LlamaConfig(layers=4, d_model=256, ffn=384, heads=8, kv_heads=4, head_dim=32,
+                               vocab=512, group_size=128, max_position=64,
+                               layer_windows=(0, 12, 0, 12), layer_head_dims=(32, 16, 32, 16),
+                               layer_kv_source=(0, 1, 0, 1))
+
+
+@pytest.mark.parametrize("config,chunk", [(MIXED, 8), (MIXED, 32), (MIXED_SMALL_DIMS, 8),
+                                          (MIXED_SMALL_DIMS, 24)],
+                         ids=["chunks of 8", "chunks of 32 (few-row launches)",
+                              "small dims, chunks of 8", "small dims, chunks of 24"])
+def test_layers_that_differ_match_the_full_reforward(gpu_ctx, config, chunk):
+    """Session over a decoder whose layers differ against the oracle's full re-forward with the
+    explicit band mask (no state slots, no ring): prefill in chunks (the last one padded), then
+    one-row steps, teacher-forced; every run's last-row logits within atol 2e-4 (the gate of the
+    uniform chain test).  The sequence is longer than the windows, so sliding layers wrap their
+    rings; sharing layers must see their owner's rows of this step and its slots before the
+    append."""
+    weights = random_weights(config, seed=31)
+    total, prompt_len = 44, 29
+    ids = np.random.default_rng(17).integers(0, config.vocab, size=total).astype(np.int32)
+    want = helpers.oracle_decoder_logits(weights, ids)
+    session = LlamaDecoderSession(gpu_ctx, weights, chunk_length=chunk)
+    ctx = session.create_generation_context(capacity=64, chunk_length=chunk)
+    assert [ctx.layer_capacity[li] for li in range(config.layers)] == \
+        [config.window_of(li) or 64 for li in range(config.layers)]
+    worst = 0.0
+    for piece in plan_prefill_chunks(prompt_len, chunk):
+        n = piece.query_length
+        cid = np.zeros((1, chunk), dtype=np.int32)
+        cpos = np.zeros((1, chunk), dtype=np.int32)
+        cid[0, :n] = ids[piece.position:piece.position + n]
+        cpos[0, :n] = np.arange(piece.position, piece.position + n)
+        _tok, logits = session.run(cid, cpos, n - 1, context=ctx, query_length=n,
+                                   want_logits=True)
+        worst = max(worst, float(np.max(np.abs(logits[0] - want[piece.position + n - 1]))))
+    for pos in range(prompt_len, total):
+        token, logits = session.run(ids[pos:pos + 1][None], np.array([[pos]], dtype=np.int32), 0,
+                                    context=ctx, query_length=1, want_logits=True)
+        worst = max(worst, float(np.max(np.abs(logits[0] - want[pos]))))
+        top = np.sort(want[pos])
+        if top[-1] - top[-2] > 4e-4:
+            assert int(token[0, 0, 0]) == int(np.argmax(want[pos])), pos
+    assert ctx.past == total
+    assert worst <= 2e-4, worst
+    with pytest.raises(ka.ExecutionError, match="sliding"):
+        ctx.rewind(3)
+    ctx.dispose()
+    session.close()
+
+
+def test_layers_that_differ_replayed_decode_and_file_session(gpu_ctx):
+    """The recorded step of a decoder whose layers differ replays to the step-by-step tokens,
+    and a session built from the model file gives the session from arrays bit for bit."""
+    from model_file import decoder_model_file
+    weights = random_weights(MIXED, seed=32)
+    from karume_amd.decoder import DecoderWeights
+    loaded = DecoderWeights.from_model(ka.open_model(decoder_model_file(weights)))
+    assert loaded.config == MIXED
+    prompt = [int(t) for t in np.random.default_rng(5).integers(0, MIXED.vocab, size=13)]
+    new = 20
+    results = []
+    for w in (weights, loaded):
+        session = LlamaDecoderSession(gpu_ctx, w, chunk_length=8)
+        stepwise = generate_greedy(session, prompt=prompt, max_new_tokens=new, chunk_length=8,
+                                   max_position=MIXED.max_position)
+        ctx = session.create_generation_context(capacity=MIXED.max_position, chunk_length=8)
+        token = None
+        for piece in plan_prefill_chunks(len(prompt), 8):
+            n = piece.query_length
+            cid = np.zeros((1, 8), dtype=np.int32)
+            cpos = np.zeros((1, 8), dtype=np.int32)
+            cid[0, :n] = prompt[piece.position:piece.position + n]
+            cpos[0, :n] = np.arange(piece.position, piece.position + n)
+            token, logits = session.run(cid, cpos, n - 1, context=ctx, query_length=n,
+                                        want_logits=True)
+        first = int(token[0, 0, 0])
+        replayed = [first] + session.decode_tokens(ctx, first, new - 1)
+        assert replayed == stepwise
+        assert ctx.past == len(prompt) + new - 1
+        ctx.dispose()
+        session.close()
+        results.append((stepwise, logits.tobytes()))
+    assert results[0] == results[1]
