@@ -243,7 +243,7 @@ int32_t krm_attention_state_noalloc(krm_ctx* ctx, krm_buf q, krm_buf ins_k, krm_
                                     int32_t io_dtype, int32_t kv_dtype);
 
 /* The attention of a chunk of rows (a prefill step) with what a decoder layer does around it
- * folded in; D = 64 or 128 and 16-byte aligned buffers, anything else is rejected (the three
+ * folded in; D = 64, 128 or 256 and 16-byte aligned buffers, anything else is rejected (the three
  * separate calls remain).  Arguments as krm_attention_state; `lengths` != 0 reads past / query
  * on the device as krm_attention_state_lengths does.  No workspace.
  *   KRM_CHUNK_OUT_ROW_MAJOR : `out` is [B, M, H, D] (what the o-projection reads) instead of

@@ -434,11 +434,12 @@ __global__ __launch_bounds__(64 * WAVES) void attention_rows_kernel(
   }
   __syncthreads();
 
-  // merge of the waves, wave order; 16 threads a row (the first 256 threads)
-  if (tid < 256) {
+  // merge of the waves, wave order; 16 threads a row (256 row-part units, dealt over the
+  // workgroup's threads: a workgroup of two waves takes two rounds)
+  for (uint32_t unit = tid; unit < 256u; unit += kBlock) {
    for (uint32_t rb = 0; rb < (uint32_t)RB; ++rb) {
     constexpr int kPer = D / 16;
-    const uint32_t rr = 16u * rb + (tid >> 4), d0 = (tid & 15u) * kPer;
+    const uint32_t rr = 16u * rb + (unit >> 4), d0 = (unit & 15u) * kPer;
     const uint32_t row = row0 + rr;
     float top = s_m[0][rr];
 #pragma unroll
@@ -1104,7 +1105,10 @@ int32_t decode_by_repeat(krm_ctx* ctx, const DecodeLaunch& L, uint32_t per_block
     case 1: return launch_decode<XT, ST, 1, LPR, RAGGED>(ctx, L);
     case 2: return launch_decode<XT, ST, 2, LPR, RAGGED>(ctx, L);
     case 4: return launch_decode<XT, ST, 4, LPR, RAGGED>(ctx, L);
-    case 8: return launch_decode<XT, ST, 8, LPR, RAGGED>(ctx, L);
+    case 8:
+      // (rows that span a whole wave: eight heads' state does not fit the registers)
+      if constexpr (LPR < 64) return launch_decode<XT, ST, 8, LPR, RAGGED>(ctx, L);
+      [[fallthrough]];
     default: return fail(ctx, KRM_ERR_VALIDATION, "decode attention: %u heads per block", per_block);
   }
 }
@@ -1116,6 +1120,7 @@ int32_t decode_by_depth(krm_ctx* ctx, const DecodeLaunch& L, uint32_t per_block,
     case 8: return decode_by_repeat<XT, ST, 8, RAGGED>(ctx, L, per_block);
     case 16: return decode_by_repeat<XT, ST, 16, RAGGED>(ctx, L, per_block);
     case 32: return decode_by_repeat<XT, ST, 32, RAGGED>(ctx, L, per_block);
+    case 64: return decode_by_repeat<XT, ST, 64, RAGGED>(ctx, L, per_block);
     default: return fail(ctx, KRM_ERR_VALIDATION, "decode attention: %u lanes per row", lpr);
   }
 }
@@ -1128,7 +1133,7 @@ int32_t decode_dispatch(krm_ctx* ctx, DecodeLaunch& L, uint32_t repeat, uint32_t
                         int32_t io_dtype, int32_t kv_dtype) {
   uint32_t per_block = repeat;
   uint64_t blocks = (uint64_t)L.grid_x * L.grid_z * L.args.kv_heads;
-  while (per_block > 1 && blocks < 2ull * (uint64_t)ctx->num_cus) {
+  while (per_block > 1 && (blocks < 2ull * (uint64_t)ctx->num_cus || (lpr == 64 && per_block > 4))) {
     per_block >>= 1;
     blocks <<= 1;
   }
@@ -1158,7 +1163,7 @@ uint32_t decode_lanes_per_row(uint32_t depth, int32_t kv_dtype) {
   const uint32_t row_bytes = depth * (uint32_t)dtype_bytes(kv_dtype);
   if (row_bytes % 16) return 0;
   const uint32_t lpr = row_bytes / 16;
-  return (lpr == 4 || lpr == 8 || lpr == 16 || lpr == 32) ? lpr : 0;
+  return (lpr == 4 || lpr == 8 || lpr == 16 || lpr == 32 || lpr == 64) ? lpr : 0;
 }
 
 bool decode_repeat_ok(uint32_t repeat) {
@@ -1188,14 +1193,17 @@ int32_t launch_rows(krm_ctx* ctx, krm_buf q, krm_buf ins_k, krm_buf ins_v, krm_b
   const uint32_t row_blocks = (a.chunk_rows + 15) / 16;
   // (with a window the key blocks start at the first row's lower bound, which a second row
   // block would not share: one block a workgroup there)
-  const bool two = a.window == 0 &&
+  const bool two = a.window == 0 && a.depth != 256 &&
                    (uint64_t)batch * a.heads * ((row_blocks + 1) / 2) >= 2ull * ctx->num_cus;
   const dim3 grid(batch * a.heads, two ? (row_blocks + 1) / 2 : row_blocks);
 #define KRM_ROWS_ATTENTION(DEPTH, WAVES, RB)                                                   \
   attention_rows_kernel<XT, ST, DEPTH, WAVES, RB><<<grid, dim3(64 * WAVES), 0, ctx->stream>>>( \
       ptr<const XT>(q), ptr<const XT>(ins_k), ptr<const XT>(ins_v), ptr<ST>(slot_k),           \
       ptr<ST>(slot_v), ptr<XT>(out), a, flags)
-  if (a.depth == 64) {
+  if (a.depth == 256) {
+    // two waves: a parked block of 32 rows of 256 floats is 33 KB for K and as much for V
+    KRM_ROWS_ATTENTION(256, 2, 1);
+  } else if (a.depth == 64) {
     if (two) KRM_ROWS_ATTENTION(64, 8, 2); else KRM_ROWS_ATTENTION(64, 8, 1);
   } else {
     if (two) KRM_ROWS_ATTENTION(128, 4, 2); else KRM_ROWS_ATTENTION(128, 4, 1);
@@ -1334,7 +1342,8 @@ static int32_t attention_state_impl(krm_ctx* ctx, krm_buf q, krm_buf ins_k, krm_
   GenericArgs a{heads, kv_heads, chunk_rows, depth, capacity, window, past, query, half_scale,
                 ptr<uint32_t>(lengths)};
   // chunks of rows with the usual head dims: the MFMA form
-  if ((chunk_rows > 1 || chunk_only) && (depth == 64 || depth == 128) && aligned(q, 16) &&
+  if ((chunk_rows > 1 || chunk_only) && (depth == 64 || depth == 128 || depth == 256) &&
+      aligned(q, 16) &&
       aligned(ins_k, 16) && aligned(ins_v, 16) && aligned(slot_k, 16) && aligned(slot_v, 16) &&
       (uint64_t)batch * heads <= 0x7fffffffull && (chunk_rows + 31) / 32 <= 65535) {
     const uint32_t f = chunk_flags;
@@ -1348,7 +1357,7 @@ static int32_t attention_state_impl(krm_ctx* ctx, krm_buf q, krm_buf ins_k, krm_
   }
   if (chunk_only)
     return fail(ctx, KRM_ERR_VALIDATION,
-                "krm_attention_chunk: covers D = 64 or 128 and 16-byte aligned buffers (D = %u); "
+                "krm_attention_chunk: covers D = 64, 128 or 256 and 16-byte aligned buffers (D = %u); "
                 "use krm_attention_state, krm_state_append and krm_transpose_01", depth);
   if (io_dtype == KRM_F32 && kv_dtype == KRM_F32)
     return launch_generic<float, float>(ctx, q, ins_k, ins_v, slot_k, slot_v, out, batch, a);

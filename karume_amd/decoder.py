@@ -540,8 +540,8 @@ class LlamaDecoderSession:
                             c.max_position, True, io)
             kr, vt = pending[owner]
             last_reader = self.spec[owner]["last_reader"] == li
-            att_half = half and depth in (64, 128)
-            if depth in (64, 128):
+            att_half = half and depth in (64, 128, 256)
+            if depth in (64, 128, 256):
                 # attention + output permute in one launch; it also appends the chunk's rows when
                 # it is the slot's last reader and no window can wrap (slot rows past.. are read
                 # by nobody in that launch)

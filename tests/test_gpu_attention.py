@@ -665,7 +665,7 @@ def test_attention_chunk_equals_attention_transpose_and_appends(gpu_ctx, io, kv,
                                 out, half_scale=oracle.half_scale(d), past=case.past,
                                 query=case.query, io_dtype=io_code, kv_dtype=kv_code, append=True,
                                 **{**geometry, "window": 64})
-    with pytest.raises(ka.GpuValidationError, match="D = 64 or 128"):
+    with pytest.raises(ka.GpuValidationError, match="D = 64, 128 or 256"):
         gpu_ctx.attention_chunk(got["q"], got["ins_k"], got["ins_v"], got["slot_k"], got["slot_v"],
                                 out, half_scale=0.5, past=0, query=1, io_dtype=io_code,
                                 kv_dtype=kv_code, **{**geometry, "depth": 32})
@@ -747,3 +747,31 @@ def test_two_readers_one_append(gpu_ctx, series):
         bv.free()
     dk.free()
     dv.free()
+
+
+# ---- head dims of 256 (a sliding layer of a Gemma-4-style decoder) -------------------------------
+
+@pytest.mark.parametrize("case,io,kv", [
+    (StateCase("chunk 40 rows, past 70, D 256", 1, 4, 2, 40, 256, 128, 0, 70, 37), np.float32, np.float32),
+    (StateCase("chunk 33 rows, window 48, D 256", 2, 2, 1, 33, 256, 64, 48, 90, 33), np.float32, np.float32),
+    (StateCase("chunk 16 rows, D 256, fp16 state", 1, 8, 1, 16, 256, 64, 0, 20, 16), np.float32, np.float16),
+    (StateCase("decode, past 300, D 256", 1, 8, 2, 1, 256, 512, 0, 300, 1), np.float32, np.float32),
+    (StateCase("decode, 8:1, past 700, D 256", 1, 8, 1, 1, 256, 1024, 0, 700, 1), np.float32, np.float32),
+    (StateCase("decode, window 128, D 256", 2, 4, 4, 1, 256, 128, 128, 1000, 1), np.float32, np.float32),
+    (StateCase("decode, past 900, D 512 fp16", 1, 8, 1, 1, 512, 1024, 0, 900, 1), np.float16, np.float16),
+], ids=lambda v: v.name if isinstance(v, StateCase) else None)
+def test_head_dim_256_forms(gpu_ctx, case, io, kv):
+    """The chunk kernel's D = 256 form (two waves a workgroup) and the decode kernel with rows
+    that span a whole wave (f32 D = 256, fp16 D = 512) against the oracle: atol 5e-6 for f32
+    output (the reference's gate), one fp16 ulp for fp16 output; pad rows exact +0."""
+    x = random_state_inputs(case, seed=case.past + case.depth, f16_values=True)
+    want = oracle_state_attention(case, x)
+    got = run_attention(gpu_ctx, case, x, io=io, kv=kv)
+    if io == np.float32:
+        ok, fails, max_abs, worst = oracle.allclose(got, want, atol=STATE_ATOL, rtol=0)
+        assert ok, (case.name, fails, max_abs, worst)
+    else:
+        ref = want.astype(np.float16).astype(np.float32)
+        assert np.all(np.abs(got.astype(np.float32) - ref) <= np.abs(ref) * 2.0 ** -10 + 1e-6)
+    pad = got[:, :, case.query:, :]
+    assert not pad.size or (np.all(pad == 0) and not np.any(np.signbit(pad)))

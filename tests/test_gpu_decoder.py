@@ -714,10 +714,18 @@ MIXED_SMALL_DIMS = LlamaConfig(layers=4, d_model=256, ffn=384, heads=8, kv_heads
                                layer_kv_source=(0, 1, 0, 1))
 
 
+# head dims 256 (sliding, shared by layer 2) and 64: the sizes of a Gemma-4 sliding layer
+MIXED_256 = LlamaConfig(layers=3, d_model=256, ffn=384, heads=4, kv_heads=1, head_dim=256,
+                        vocab=512, group_size=128, max_position=64,
+                        layer_windows=(8, 0, 8), layer_head_dims=(256, 64, 256),
+                        layer_kv_source=(0, 1, 0))
+
+
 @pytest.mark.parametrize("config,chunk", [(MIXED, 8), (MIXED, 32), (MIXED_SMALL_DIMS, 8),
-                                          (MIXED_SMALL_DIMS, 24)],
+                                          (MIXED_SMALL_DIMS, 24), (MIXED_256, 8), (MIXED_256, 32)],
                          ids=["chunks of 8", "chunks of 32 (few-row launches)",
-                              "small dims, chunks of 8", "small dims, chunks of 24"])
+                              "small dims, chunks of 8", "small dims, chunks of 24",
+                              "head dim 256, chunks of 8", "head dim 256, chunks of 32"])
 def test_layers_that_differ_match_the_full_reforward(gpu_ctx, config, chunk):
     """Session over a decoder whose layers differ against the oracle's full re-forward with the
     explicit band mask (no state slots, no ring): prefill in chunks (the last one padded), then
