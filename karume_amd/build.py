@@ -24,6 +24,9 @@ FLAGS = [
     "-O3", "-std=c++17", "-fPIC", "--offload-arch=gfx950",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-fno-fast-math", "-ffp-contract=off", "-Wall", "-Wno-unused-function", "-Wno-unknown-warning-option",
+    # the first kernel arguments arrive in scalar registers with the wave (gfx950 preloads them)
+    # instead of through a load every kernel would wait for before its first address is known
+    "-mllvm", "-amdgpu-kernarg-preload-count=16",
 ]
 
 

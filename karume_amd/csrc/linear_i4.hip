@@ -528,9 +528,12 @@ constexpr bool share_x_in_lds() {
 // nor their registers (a run-time test at the top of the kernel cost the plain GEMV 8 %).
 template <typename XT, typename ST, int MB, int ROWS, int VEC, int NSTEP, bool NORM, bool DECODE_ROW>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 4))) void gemv_i4_kernel(
+    // Argument order: what the first addresses are made of comes first — the leading 14 dwords of
+    // the arguments arrive in scalar registers with the wave (kernel-argument preload), the rest
+    // through a load the kernel has to wait for.
     const XT* __restrict__ x, const uint32_t* __restrict__ w, const ST* __restrict__ scales,
-    const XT* __restrict__ bias, XT* __restrict__ out, uint32_t m, uint32_t n, uint32_t k,
-    uint32_t group_shift, GemvFusion fuse) {
+    const float* __restrict__ norm_weight, uint32_t n, uint32_t k, uint32_t group_shift, uint32_t m,
+    const XT* __restrict__ bias, XT* __restrict__ out, GemvFusion fuse) {
   constexpr int kLaneElems = VEC * 8;
   constexpr int kStepElems = kWave * kLaneElems;
   using Regs = typename Acts<XT>::template Regs<VEC>;
@@ -564,19 +567,20 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 4))) voi
     for (int r = 0; r < ROWS; ++r) acc[r][b] = 0.f;
   }
 
-  // Decode-row epilogue: the rotation's table entries are requested now, so that they arrive
-  // with the weights instead of after the reductions.
+  // Decode-row epilogue: the rotation's table entries and the run-time lengths of a recorded
+  // step are requested early, so that they arrive with the weights instead of costing a round
+  // trip of their own behind the reductions — but after the weight requests where the kernel
+  // asks for those at once: the addresses of x and of the weights come from arguments that
+  // arrive with the wave, these from arguments that have to be loaded first.
   float rope_cos[ROWS / 2 > 0 ? ROWS / 2 : 1][2], rope_sin[ROWS / 2 > 0 ? ROWS / 2 : 1][2];
   bool rope_in_table = false;
-  // run-time lengths of a recorded step: asked for here, used by the appends at the very end
-  // (a load in the epilogue would add a memory round trip behind the reductions)
   uint32_t dev_past = 0, dev_query = 0;
-  if constexpr (DECODE_ROW) {
-    if (fuse.lengths) {
-      dev_past = fuse.lengths[0];
-      dev_query = fuse.lengths[1];
-    }
-    {
+  auto request_decode_row = [&]() {
+    if constexpr (DECODE_ROW) {
+      if (fuse.lengths) {
+        dev_past = fuse.lengths[0];
+        dev_query = fuse.lengths[1];
+      }
       const uint32_t half = fuse.depth >> 1;
       const uint32_t rope_pairs = (fuse.heads + fuse.kv_heads) * half;
       const int32_t pos = fuse.positions[0];
@@ -592,7 +596,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 4))) voi
         rope_sin[p][1] = fuse.sin_table[rotates ? t + half : 0];
       }
     }
-  }
+  };
+  constexpr bool kRowAfterWeights = share_x_in_lds<XT, MB, NSTEP>() && VEC == 4;
+  if constexpr (!kRowAfterWeights) request_decode_row();
 
   // Lanes past the end of K (last step of a K that is not a multiple of the step) read the
   // row's first words and activations instead and their partial sum is dropped, so every load
@@ -618,7 +624,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 4))) voi
     const uint32_t k0 = step * kStepElems + lane * kLaneElems;
     const uint32_t xrow = min((uint32_t)b, m - 1);  // rows past M re-read the last row, unused
     const uint32_t kc = k0 < k ? k0 : 0u;
-    Acts<XT>::template load<VEC, NORM>(x + (size_t)xrow * k + kc, fuse.norm_weight + kc,
+    Acts<XT>::template load<VEC, NORM>(x + (size_t)xrow * k + kc, norm_weight + kc,
                                        k0 < k && counted, regs, squares[b]);
   };
   auto consume = [&](uint32_t step, const uint32_t (&cw)[ROWS][VEC], const float (&cs)[ROWS],
@@ -655,10 +661,11 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 4))) voi
         for (int step = 0; step < NSTEP; ++step) {
           const uint32_t q_k0 = (uint32_t)step * kStepElems + wave * 512 + lane * 8;
           const uint32_t q_kc = q_k0 < k ? q_k0 : 0u;
-          Acts<XT>::template request<1, NORM>(x + q_kc, fuse.norm_weight + q_kc, raw_q[step]);
+          Acts<XT>::template request<1, NORM>(x + q_kc, norm_weight + q_kc, raw_q[step]);
         }
 #pragma unroll
         for (int step = 0; step < NSTEP; ++step) fetch(step, all_w[step], all_s[step]);
+        request_decode_row();
 #pragma unroll
         for (int step = 0; step < NSTEP; ++step) {
           const uint32_t q_k0 = (uint32_t)step * kStepElems + wave * 512 + lane * 8;
@@ -687,7 +694,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 4))) voi
         const uint32_t x_k0 = (uint32_t)wave * kStepElems + lane * kLaneElems;
         const uint32_t x_kc = x_k0 < k ? x_k0 : 0u;
         if (wave < NSTEP)
-          Acts<XT>::template request<VEC, NORM>(x + x_kc, fuse.norm_weight + x_kc, raw_x);
+          Acts<XT>::template request<VEC, NORM>(x + x_kc, norm_weight + x_kc, raw_x);
 #pragma unroll
         for (int step = 0; step < NSTEP; ++step) fetch(step, all_w[step], all_s[step]);
         if (wave < NSTEP) {
@@ -948,8 +955,9 @@ int32_t launch_gemv(krm_ctx* ctx, krm_buf x, krm_buf w, krm_buf scales, krm_buf 
 #define KRM_GEMV_LAUNCH(NORM, ROW)                                                              \
   gemv_i4_kernel<XT, ST, MB, ROWS, VEC, NSTEP, NORM, ROW>                                       \
       <<<dim3(blocks), dim3(256), 0, ctx->stream>>>(ptr<const XT>(x), ptr<const uint32_t>(w),  \
-                                                    ptr<const ST>(scales), ptr<const XT>(bias), \
-                                                    ptr<XT>(out), m, n, k, group_shift, fuse)
+                                                    ptr<const ST>(scales), fuse.norm_weight, n, k, \
+                                                    group_shift, m, ptr<const XT>(bias),        \
+                                                    ptr<XT>(out), fuse)
   if constexpr (MB == 1 && ROWS % 2 == 0) {
     if (fuse.positions) {
       if (fuse.norm_weight) KRM_GEMV_LAUNCH(true, true); else KRM_GEMV_LAUNCH(false, true);
@@ -994,6 +1002,7 @@ int32_t pick_rows(krm_ctx* ctx, krm_buf x, krm_buf w, krm_buf scales, krm_buf bi
   // fp16 activations, many rows (the streaming case: every SIMD still gets 8 waves or more):
   // four rows a wave share the activations read from LDS and the per-wave bookkeeping, about a
   // sixth of the instructions of a launch that the vector ALU bounds
+  // (eight rows a wave measured slower again: 24.8 against 23.8 us on 65536 rows)
   if constexpr (MB == 1 && sizeof(XT) == 2 && VEC == 4)
     if (k <= 4096 && (uint64_t)n >= cus * 4 * 4 * 8)
       return pick_steps<XT, ST, MB, 4, VEC>(ctx, x, w, scales, bias, out, m, n, k, group_shift, fuse);
