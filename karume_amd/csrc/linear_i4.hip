@@ -492,6 +492,9 @@ struct GemvFusion {
   void* slot_v;
   uint32_t* lengths;         // device {past, query, fault, ...} or null: `past` below
   uint32_t heads, kv_heads, depth, table_rows, capacity, window, past;
+  uint32_t half_shift;       // log2(depth / 2) when that is a power of two, else 0xffffffff:
+                             // the epilogue's index arithmetic is then shifts and masks instead
+                             // of integer divisions (about 150 instructions behind the reductions)
   int32_t slot_f16;          // slot element type: 1 = fp16, 0 = f32
   // One row (M = 1), plain epilogue: every workgroup also writes the argmax of the outputs it
   // stored, {value bits, row index}, to argmax_partial[blockIdx.x] (a workgroup without a row:
@@ -528,12 +531,12 @@ constexpr bool share_x_in_lds() {
 // nor their registers (a run-time test at the top of the kernel cost the plain GEMV 8 %).
 template <typename XT, typename ST, int MB, int ROWS, int VEC, int NSTEP, bool NORM, bool DECODE_ROW>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 4))) void gemv_i4_kernel(
-    // Argument order: what the first addresses are made of comes first — the leading 14 dwords of
-    // the arguments arrive in scalar registers with the wave (kernel-argument preload), the rest
-    // through a load the kernel has to wait for.
+    // Argument order: what the first addresses and the final store are made of comes first — the
+    // leading 14 dwords of the arguments arrive in scalar registers with the wave
+    // (kernel-argument preload), the rest through a load the kernel has to wait for.
     const XT* __restrict__ x, const uint32_t* __restrict__ w, const ST* __restrict__ scales,
-    const float* __restrict__ norm_weight, uint32_t n, uint32_t k, uint32_t group_shift, uint32_t m,
-    const XT* __restrict__ bias, XT* __restrict__ out, GemvFusion fuse) {
+    const float* __restrict__ norm_weight, XT* __restrict__ out, uint32_t n, uint32_t k,
+    uint32_t group_shift, uint32_t m, const XT* __restrict__ bias, GemvFusion fuse) {
   constexpr int kLaneElems = VEC * 8;
   constexpr int kStepElems = kWave * kLaneElems;
   using Regs = typename Acts<XT>::template Regs<VEC>;
@@ -583,13 +586,15 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 4))) voi
       }
       const uint32_t half = fuse.depth >> 1;
       const uint32_t rope_pairs = (fuse.heads + fuse.kv_heads) * half;
-      const int32_t pos = fuse.positions[0];
+      // (a table of one row is this step's row: no position to look it up by)
+      const int32_t pos = fuse.table_rows == 1 ? 0 : fuse.positions[0];
       rope_in_table = pos >= 0 && (uint32_t)pos < fuse.table_rows;
 #pragma unroll
       for (int p = 0; p < ROWS / 2; ++p) {
         const uint32_t pair = (row0 >> 1) + p;
         const bool rotates = rope_in_table && pair < rope_pairs;
-        const size_t t = rotates ? (size_t)pos * fuse.depth + pair % half : 0;
+        const uint32_t j = fuse.half_shift != 0xffffffffu ? (pair & (half - 1u)) : pair % half;
+        const size_t t = rotates ? (size_t)pos * fuse.depth + j : 0;
         rope_cos[p][0] = fuse.cos_table[t];
         rope_sin[p][0] = fuse.sin_table[t];
         rope_cos[p][1] = fuse.cos_table[rotates ? t + half : 0];
@@ -847,7 +852,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 4))) voi
                  (fuse.window != 0 || (uint64_t)past + 1 <= fuse.capacity);
         if (!append && row0 == 0 && lane == 0) fuse.lengths[2] = 1u;
       }
-      const uint64_t prow = fuse.window ? (uint64_t)past % fuse.window : (uint64_t)past;
+      const uint32_t prow = fuse.window ? past % fuse.window : past;
+      const bool pow2 = fuse.half_shift != 0xffffffffu;
       const bool in_table = rope_in_table;
 #pragma unroll
       for (int p = 0; p < ROWS / 2; ++p) {
@@ -863,7 +869,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 4))) voi
         x0 = to_f32<XT>(from_f32<XT>(x0));
         x1 = to_f32<XT>(from_f32<XT>(x1));
         if (pair < rope_pairs) {
-          const uint32_t head = pair / half, j = pair - head * half;
+          const uint32_t head = pow2 ? pair >> fuse.half_shift : pair / half;
+          const uint32_t j = pair - head * half;
           float o0 = NAN, o1 = NAN;  // a position outside the table is never a valid rotation
           if (in_table) {
             o0 = __fadd_rn(__fmul_rn(x0, rope_cos[p][0]), __fmul_rn(-x1, rope_sin[p][0]));
@@ -883,7 +890,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 4))) voi
           out[at] = from_f32<XT>(x0);
           out[at + 1] = from_f32<XT>(x1);
           if (append) {
-            const uint32_t plane = e / fuse.depth, d = e - plane * fuse.depth;
+            const uint32_t plane = pow2 ? e >> (fuse.half_shift + 1u) : e / fuse.depth;
+            const uint32_t d = e - plane * fuse.depth;
             const size_t dst = ((size_t)plane * fuse.capacity + prow) * fuse.depth + d;
             slot_store(fuse.slot_v, fuse.slot_f16, dst, x0);
             slot_store(fuse.slot_v, fuse.slot_f16, dst + 1, x1);
@@ -955,9 +963,9 @@ int32_t launch_gemv(krm_ctx* ctx, krm_buf x, krm_buf w, krm_buf scales, krm_buf 
 #define KRM_GEMV_LAUNCH(NORM, ROW)                                                              \
   gemv_i4_kernel<XT, ST, MB, ROWS, VEC, NSTEP, NORM, ROW>                                       \
       <<<dim3(blocks), dim3(256), 0, ctx->stream>>>(ptr<const XT>(x), ptr<const uint32_t>(w),  \
-                                                    ptr<const ST>(scales), fuse.norm_weight, n, k, \
-                                                    group_shift, m, ptr<const XT>(bias),        \
-                                                    ptr<XT>(out), fuse)
+                                                    ptr<const ST>(scales), fuse.norm_weight,   \
+                                                    ptr<XT>(out), n, k, group_shift, m,         \
+                                                    ptr<const XT>(bias), fuse)
   if constexpr (MB == 1 && ROWS % 2 == 0) {
     if (fuse.positions) {
       if (fuse.norm_weight) KRM_GEMV_LAUNCH(true, true); else KRM_GEMV_LAUNCH(false, true);
@@ -1388,6 +1396,11 @@ int32_t krm_decode_qkv(krm_ctx* ctx, krm_buf x, krm_buf norm_weight_f32, float n
   fuse.window = window;
   fuse.past = past;
   fuse.slot_f16 = kv_dtype == KRM_F16 ? 1 : 0;
+  fuse.half_shift = 0xffffffffu;
+  if (is_pow2(depth >> 1)) {
+    fuse.half_shift = 0;
+    while ((1u << fuse.half_shift) < (depth >> 1)) ++fuse.half_shift;
+  }
   const uint32_t n = (heads + 2 * kv_heads) * depth;
   return gemv_dispatch(ctx, x, w, scales, bias, out, 1, n, k, group, io_dtype, scale_dtype, fuse);
 }
