@@ -989,8 +989,9 @@ int32_t pick_steps(krm_ctx* ctx, krm_buf x, krm_buf w, krm_buf scales, krm_buf b
       return launch_gemv<XT, ST, MB, ROWS, VEC, 1>(ctx, x, w, scales, bias, out, m, n, k, group_shift, fuse);
     if (steps == 2)
       return launch_gemv<XT, ST, MB, ROWS, VEC, 2>(ctx, x, w, scales, bias, out, m, n, k, group_shift, fuse);
-    if (steps == 3 && ROWS <= 2)
-      return launch_gemv<XT, ST, MB, ROWS, VEC, 3>(ctx, x, w, scales, bias, out, m, n, k, group_shift, fuse);
+    if constexpr (ROWS <= 2)
+      if (steps == 3)
+        return launch_gemv<XT, ST, MB, ROWS, VEC, 3>(ctx, x, w, scales, bias, out, m, n, k, group_shift, fuse);
   }
   return launch_gemv<XT, ST, MB, ROWS, VEC, 0>(ctx, x, w, scales, bias, out, m, n, k, group_shift, fuse);
 }
@@ -1002,17 +1003,26 @@ int32_t pick_rows(krm_ctx* ctx, krm_buf x, krm_buf w, krm_buf scales, krm_buf bi
   // Rows per wave: two rows share one fetch of the activations; one row per wave keeps more
   // waves in flight when N is small.  The choice never changes a row's reduction order.
   const uint64_t cus = (uint64_t)ctx->num_cus;
-  // f32 activations of one row in few steps: four rows a wave halve the workgroups that each
-  // stage the row once more, as long as every CU still gets a few.
+  // f32 activations of one row in one or two steps (K <= 4096): every workgroup stages the row
+  // once, so more rows a wave mean fewer of those.  With the rms_norm in front (the norm weight
+  // is staged too) that pays early; measured at K = 2048, us per launch with 1 / 2 / 4 rows a
+  // wave: N = 2048 2.53 / 2.42 / 2.86, 4096 3.03 / 2.95 / 3.22, 6144 4.35 / 3.52 / 4.04, 8192
+  // 5.03 / 4.05 / 4.23, 11264 - / 5.01 / 4.93, 32000 14.2 / 10.3 / 9.0.  Without it one row a
+  // wave stays ahead on few rows (N = 2048 with a residual: 2.57 against 2.80).
   if constexpr (MB == 1 && sizeof(XT) == 4 && VEC == 4)
-    if (k <= 4096 && (uint64_t)n >= cus * 4 * 4 * 2)
-      return pick_steps<XT, ST, MB, 4, VEC>(ctx, x, w, scales, bias, out, m, n, k, group_shift, fuse);
-  // fp16 activations, many rows (the streaming case: every SIMD still gets 8 waves or more):
+    if (k <= 4096) {
+      if ((uint64_t)n >= cus * (fuse.norm_weight ? 40 : 32))
+        return pick_steps<XT, ST, MB, 4, VEC>(ctx, x, w, scales, bias, out, m, n, k, group_shift, fuse);
+      if (fuse.norm_weight && (uint64_t)n >= cus * 8)
+        return pick_steps<XT, ST, MB, 2, VEC>(ctx, x, w, scales, bias, out, m, n, k, group_shift, fuse);
+    }
+  // fp16 activations, many rows (the streaming case: every SIMD still gets 4 waves or more):
   // four rows a wave share the activations read from LDS and the per-wave bookkeeping, about a
-  // sixth of the instructions of a launch that the vector ALU bounds
-  // (eight rows a wave measured slower again: 24.8 against 23.8 us on 65536 rows)
+  // sixth of the instructions of a launch that the vector ALU bounds (K = 4096, 1 / 2 / 4 rows a
+  // wave: N = 4096 3.62 / 3.75 / 4.31, 8192 5.74 / 5.09 / 5.48, 16384 9.50 / 8.46 / 8.06 us;
+  // eight rows a wave measured slower again: 24.8 against 23.8 us on 65536 rows)
   if constexpr (MB == 1 && sizeof(XT) == 2 && VEC == 4)
-    if (k <= 4096 && (uint64_t)n >= cus * 4 * 4 * 8)
+    if (k <= 4096 && (uint64_t)n >= cus * 4 * 4 * 4)
       return pick_steps<XT, ST, MB, 4, VEC>(ctx, x, w, scales, bias, out, m, n, k, group_shift, fuse);
   // (one row of x shared through LDS: below 32 rows a CU one row a wave — twice the waves —
   // measured 1.5 % more decode tokens/s and 1 % on the 4096 x 4096 GEMV)
