@@ -408,8 +408,8 @@ def bench_decode_step_kernels(timer: Timer, rng, steps: int, warmup: int, g: int
     """The launches of one config-4 decode step, each alone: the four GEMV forms of a layer and
     the head projection (f32 activations, fp16 scales, the fused forms the decoder records), and
     the one-row attention over a past of 255 columns.  Every GEMV runs over rotating weight
-    copies (a token reads 0.53 GB of weights, more than the 256 MB Infinity Cache holds, so a
-    layer's weights are cold when its launch starts).  `read_floor_us`: krm_probe_launch(READ)
+    copies, 640 MB of them per shape (a token reads 0.53 GB of weights, more than the 256 MB
+    Infinity Cache holds, so a layer's weights are cold when its launch starts).  `read_floor_us`: krm_probe_launch(READ)
     on the same bytes of the same buffers with the launch's own grid (workgroups of 256
     threads; rows per workgroup as the GEMV picks them: 8 for [q;k;v], 4 for o and down, 16 for
     gate/up and the head) — what a kernel that only reads those weights costs."""
@@ -426,12 +426,14 @@ def bench_decode_step_kernels(timer: Timer, rng, steps: int, warmup: int, g: int
     slot_v = ctx.upload(rng.normal(size=(kv_heads, cap, depth)).astype(np.float32))
     rows = []
     for name, n, k, rows_per_wg in forms:
-        copies = max(4, min(64, (600 << 20) // (n * k // 2)))
-        weights = [ctx.upload(rng.integers(0, 256, size=n * k // 2, dtype=np.uint8))
-                   for _ in range(copies)]
-        scales = [ctx.upload(np.maximum(
-            np.abs(rng.normal(0, 0.02, size=(n, k // g))).astype(np.float16),
-            np.float16(6.104e-05))) for _ in range(copies)]
+        # enough copies to exceed the Infinity Cache for the small shapes too (one host array
+        # uploaded `copies` times: distinct device addresses are what matters here)
+        copies = max(4, min(320, (640 << 20) // (n * k // 2)))
+        host_w = rng.integers(0, 256, size=n * k // 2, dtype=np.uint8)
+        host_s = np.maximum(np.abs(rng.normal(0, 0.02, size=(n, k // g))).astype(np.float16),
+                            np.float16(6.104e-05))
+        weights = [ctx.upload(host_w) for _ in range(copies)]
+        scales = [ctx.upload(host_s) for _ in range(copies)]
         x = ctx.upload(rng.normal(size=(1, k)).astype(np.float32))
         y = ctx.alloc(max(n, d) * 4)
         res_buf = ctx.upload(rng.normal(size=(1, n)).astype(np.float32))
