@@ -595,14 +595,19 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 4))) voi
   uint32_t dev_past = 0, dev_query = 0;
   auto request_decode_row = [&]() {
     if constexpr (DECODE_ROW) {
-      if (fuse.lengths) {
-        dev_past = fuse.lengths[0];
-        dev_query = fuse.lengths[1];
-      }
+      // The lengths and the position are asked for together and without a branch (a missing
+      // lengths buffer reads x instead and is dropped): one wait for both, where a branch
+      // around each made them two round trips in a row in front of the staging of x.
+      const uint32_t* lengths_or_x =
+          fuse.lengths ? fuse.lengths : reinterpret_cast<const uint32_t*>(x);
+      const uint32_t word0 = lengths_or_x[0], word1 = lengths_or_x[1];
+      const int32_t first_position = fuse.positions[0];
+      dev_past = fuse.lengths ? word0 : 0u;
+      dev_query = fuse.lengths ? word1 : 0u;
       const uint32_t half = fuse.depth >> 1;
       const uint32_t rope_pairs = (fuse.heads + fuse.kv_heads) * half;
       // (a table of one row is this step's row: no position to look it up by)
-      const int32_t pos = fuse.table_rows == 1 ? 0 : fuse.positions[0];
+      const int32_t pos = fuse.table_rows == 1 ? 0 : first_position;
       rope_in_table = pos >= 0 && (uint32_t)pos < fuse.table_rows;
 #pragma unroll
       for (int p = 0; p < ROWS / 2; ++p) {
