@@ -192,12 +192,14 @@ def test_linear_shapes_of_the_decoder(gpu_ctx, shape):
     assert ok, (fails, max_abs, worst)
 
 
-@pytest.mark.parametrize("k,io", [(2048, np.float32), (5632, np.float32), (4096, np.float16)])
-def test_row_bits_do_not_depend_on_rows_per_wave(gpu_ctx, k, io):
+@pytest.mark.parametrize("k,io,many", [(2048, np.float32, 8256), (5632, np.float32, 8256),
+                                       (4096, np.float16, 8256), (4096, np.float16, 16512)])
+def test_row_bits_do_not_depend_on_rows_per_wave(gpu_ctx, k, io, many):
     """A narrow output gives a wave one row, a wide one two (K = 5632, or fp16) or four
-    (K = 2048, f32) that are reduced together: the same weight row and x give the same bits
-    either way (one fixed order of additions for every form of the wave reduction)."""
-    g, few, many = 128, 64, 8256
+    (K = 2048 with f32 activations, fp16 activations from 16384 rows) that are reduced together:
+    the same weight row and x give the same bits either way (one fixed order of additions for
+    every form of the wave reduction)."""
+    g, few = 128, 64
     rng = np.random.default_rng(k)
     packed, _q, scale = helpers.synthetic_int4(rng, many, k, g)
     x = rng.normal(size=(1, k)).astype(io)
