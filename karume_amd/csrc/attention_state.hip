@@ -111,7 +111,8 @@ __global__ __launch_bounds__(kThreads) void attention_generic_kernel(
     if (valid) {
       float dot = 0.f;
       if (col < a.past) {
-        const uint64_t prow = a.window ? col % a.window : col;
+        // (a slot column is below `past`, a u32: the ring row is a 32-bit modulo)
+        const uint32_t prow = a.window ? (uint32_t)col % a.window : (uint32_t)col;
         const ST* kp = slot_k + ((size_t)kv_plane * a.capacity + prow) * D;
         for (uint32_t d = 0; d < D; ++d) dot = fmaf(s_q[d], ld_f32<ST>(kp, d) * a.scale, dot);
       } else {
@@ -155,7 +156,7 @@ __global__ __launch_bounds__(kThreads) void attention_generic_kernel(
         const uint64_t vc = lo + c0 + c;
         float v;
         if (vc < a.past) {
-          const uint64_t prow = a.window ? vc % a.window : vc;
+          const uint32_t prow = a.window ? (uint32_t)vc % a.window : (uint32_t)vc;
           v = ld_f32<ST>(slot_v, ((size_t)kv_plane * a.capacity + prow) * D + d);
         } else {
           v = ld_f32<XT>(ins_v, ((size_t)kv_plane * a.chunk_rows + (vc - a.past)) * D + d);
@@ -334,7 +335,7 @@ __global__ __launch_bounds__(64 * WAVES) void attention_rows_kernel(
       uint64_t c = c0 + key;
       c = c < limit_hi ? c : limit_hi;  // beyond the last column: any valid row, masked below
       if (c < past) {
-        const uint64_t prow = a.window ? c % a.window : c;
+        const uint32_t prow = a.window ? (uint32_t)c % a.window : (uint32_t)c;  // c < past: a u32
         const size_t at = ((size_t)kv_plane * a.capacity + prow) * D + 4 * piece;
         kraw[j] = load4_f32<ST>(slot_k + at);
         vraw[j] = load4_f32<ST>(slot_v + at);
