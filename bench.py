@@ -94,18 +94,27 @@ class Timer:
         self.evict_pass_ms = self.start.elapsed_ms(self.stop) / 4
 
     def run(self, fn, steps: int, warmup: int, *, after_evict=None, branches: int = 1,
-            replays: int = REPLAYS, min_launches: int = None) -> dict:
+            replays: int = REPLAYS, min_launches: int = None, series=None) -> dict:
         """{"ms": median ms of one pass of `steps` calls, "ms_min", "ms_max", "mode", ...}.
         `after_evict` (optional) queues untimed calls behind the eviction (e.g. to warm the
         caches again for a cache-resident figure)."""
         ctx = self.ctx
         if not USE_GRAPHS:
-            for i in range(warmup):
-                fn(i)
+            # `series(count)`: the same calls queued from one host call (krm_probe_linear_series),
+            # so that the launches follow each other the way a replayed recording's do; a Python
+            # loop leaves the device idle between launches that last a few microseconds
+            if series is not None:
+                series(warmup)
+            else:
+                for i in range(warmup):
+                    fn(i)
             ctx.sync()
             self.start.record()
-            for i in range(steps):
-                fn(i)
+            if series is not None:
+                series(steps)
+            else:
+                for i in range(steps):
+                    fn(i)
             self.stop.record()
             ms = self.start.elapsed_ms(self.stop)
             ctx.sync()
@@ -191,7 +200,10 @@ def bench_gemv(timer: Timer, rng, steps: int, warmup: int, m: int, n: int, k: in
     def step_read(i: int) -> None:
         ctx.probe_launch(ka.PROBE_READ, weights[i % copies], n * row_bytes, grid=grid, block=256)
 
-    res = {"rotating": timer.run(step, steps, warmup)}
+    def series(count: int) -> None:
+        ctx.probe_linear_series(x, weights, scales, outs[0], count, m, n, k, g, ka.F16, ka.F16)
+
+    res = {"rotating": timer.run(step, steps, warmup, series=series)}
     if extras:
         res["resident"] = timer.run(step_resident, steps, warmup,
                                     after_evict=lambda: [step_resident(0) for _ in range(3)])

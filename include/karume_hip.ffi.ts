@@ -241,4 +241,11 @@ export const KARUME_HIP_DIAGNOSTIC_SYMBOLS = {
     ],
     result: "i32",
   },
+  krm_probe_linear_series: {
+    parameters: [
+      "pointer", "u64", "buffer", "buffer", "u32", "u64", "u32", "u32", "u32", "u32", "u32", "i32",
+      "i32"
+    ],
+    result: "i32",
+  },
 } as const;

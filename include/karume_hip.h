@@ -547,6 +547,15 @@ int32_t krm_probe_launch(krm_ctx* ctx, int32_t kind, krm_buf src, size_t bytes, 
  * is bounded; the launch always ends).  Time it with events; no op of the reference. */
 int32_t krm_probe_exchange(krm_ctx* ctx, krm_buf work, size_t work_bytes, uint32_t entries,
                            uint32_t phases, uint32_t spin_limit);
+/* `count` launches of krm_linear_i4 (m rows, m <= 16) in a row from one call, launch i on the
+ * weights w_list[i % copies] / scales_list[i % copies] (host arrays of `copies` device
+ * addresses): what a host loop of krm_linear_i4 calls does, without the host's time per call
+ * between the launches, so that a kernel trace of plain launches sees them back to back the way
+ * a recorded run replays them.  Rejected while recording. */
+int32_t krm_probe_linear_series(krm_ctx* ctx, krm_buf x, const krm_buf* w_list,
+                                const krm_buf* scales_list, uint32_t copies, krm_buf out,
+                                uint32_t count, uint32_t m, uint32_t n, uint32_t k,
+                                uint32_t group, int32_t io_dtype, int32_t scale_dtype);
 
 #ifdef __cplusplus
 }

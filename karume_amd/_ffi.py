@@ -38,6 +38,8 @@ PROTOTYPES = {
     "krm_event_destroy": (i32, [c_ctx, c_evt]),
     "krm_probe_launch": (i32, [c_ctx, i32, c_buf, size_t, u32, u32]),
     "krm_probe_exchange": (i32, [c_ctx, c_buf, size_t, u32, u32, u32]),
+    "krm_probe_linear_series": (i32, [c_ctx, c_buf, C.POINTER(c_buf), C.POINTER(c_buf), u32, c_buf,
+                                      u32, u32, u32, u32, u32, i32, i32]),
     "krm_graph_begin": (i32, [c_ctx]),
     "krm_graph_branch": (i32, [c_ctx, u32]),
     "krm_graph_end": (i32, [c_ctx, C.POINTER(C.c_void_p)]),

@@ -1204,6 +1204,20 @@ int32_t krm_linear_i4(krm_ctx* ctx, krm_buf x, krm_buf w, krm_buf scales, krm_bu
   return KRM_OK;
 }
 
+int32_t krm_probe_linear_series(krm_ctx* ctx, krm_buf x, const krm_buf* w_list,
+                                const krm_buf* scales_list, uint32_t copies, krm_buf out,
+                                uint32_t count, uint32_t m, uint32_t n, uint32_t k,
+                                uint32_t group, int32_t io_dtype, int32_t scale_dtype) {
+  KRM_TRY(enter(ctx));
+  KRM_TRY(not_recording(ctx, "krm_probe_linear_series"));
+  KRM_REQUIRE(ctx, w_list && scales_list && copies >= 1, "krm_probe_linear_series: no weights");
+  KRM_REQUIRE(ctx, m >= 1 && m <= 16, "krm_probe_linear_series: m = %u (1..16)", m);
+  for (uint32_t i = 0; i < count; ++i)
+    KRM_TRY(krm_linear_i4(ctx, x, w_list[i % copies], scales_list[i % copies], 0, out, m, n, k,
+                          group, io_dtype, scale_dtype, KRM_COMPUTE_F32));
+  return KRM_OK;
+}
+
 int32_t krm_linear_i4_fused(krm_ctx* ctx, krm_buf x, krm_buf norm_weight_f32, float norm_eps,
                             krm_buf w, krm_buf scales, krm_buf bias, krm_buf residual,
                             krm_buf out, uint32_t m, uint32_t n, uint32_t k, uint32_t group,

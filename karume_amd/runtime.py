@@ -257,6 +257,18 @@ class GpuContext:
         self._check(self._lib.krm_probe_exchange(self._handle, _addr(work), work.nbytes, entries,
                                                  phases, spin_limit))
 
+    def probe_linear_series(self, x: BufferLike, weights: Sequence[BufferLike],
+                            scales: Sequence[BufferLike], out: BufferLike, count: int, m: int,
+                            n: int, k: int, group: int, io_dtype: int = F32,
+                            scale_dtype: int = F32) -> None:
+        """`count` plain launches of linear_i4 from one call, rotating over the weight copies."""
+        copies = len(weights)
+        w_list = (C.c_uint64 * copies)(*[_addr(b) for b in weights])
+        s_list = (C.c_uint64 * copies)(*[_addr(b) for b in scales])
+        self._check(self._lib.krm_probe_linear_series(
+            self._handle, _addr(x), w_list, s_list, copies, _addr(out), count, m, n, k, group,
+            io_dtype, scale_dtype))
+
     def borrow(self, address: int, nbytes: int) -> DeviceBuffer:
         """Wrap device memory owned by someone else (for example a torch tensor's data_ptr)."""
         return DeviceBuffer(self, address, nbytes, owned=False)

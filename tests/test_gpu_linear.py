@@ -311,6 +311,30 @@ def test_linear_from_a_model_file(gpu_ctx):
     assert ok, (fails, max_abs, worst)
 
 
+def test_probe_linear_series_is_a_loop_of_linear_calls(gpu_ctx):
+    """krm_probe_linear_series queues `count` plain linear_i4 launches over rotating weights:
+    the output is that of the last launch's weights, bit for bit; it refuses to be recorded."""
+    n, k, g = 256, 512, 128
+    rng = np.random.default_rng(77)
+    sets = [helpers.synthetic_int4(rng, n, k, g) for _ in range(3)]
+    x = rng.normal(size=(1, k)).astype(np.float16)
+    dx = gpu_ctx.upload(x)
+    dws = [gpu_ctx.upload(p) for p, _q, _s in sets]
+    dss = [gpu_ctx.upload(s) for _p, _q, s in sets]
+    out, ref = gpu_ctx.alloc(n * 2), gpu_ctx.alloc(n * 2)
+    gpu_ctx.probe_linear_series(dx, dws, dss, out, 5, 1, n, k, g, ka.F16, ka.F16)
+    last = (5 - 1) % 3
+    gpu_ctx.linear_i4(dx, dws[last], dss[last], None, ref, 1, n, k, g, ka.F16, ka.F16)
+    assert out.download(np.uint16, (n,)).tobytes() == ref.download(np.uint16, (n,)).tobytes()
+    with gpu_ctx.record() as rec:
+        with pytest.raises(ka.GpuValidationError):
+            gpu_ctx.probe_linear_series(dx, dws, dss, out, 2, 1, n, k, g, ka.F16, ka.F16)
+        gpu_ctx.linear_i4(dx, dws[0], dss[0], None, ref, 1, n, k, g, ka.F16, ka.F16)
+    rec.graph.destroy()
+    for b in [dx, out, ref] + dws + dss:
+        b.free()
+
+
 def test_probe_exchange_is_bounded_and_clean(gpu_ctx):
     """The in-kernel hand-over probe: every wait in it is bounded, so the launch ends whatever
     the spin limit is and the fault word is 0 (every poll succeeded) or 1 (some poll gave up).
